@@ -1,0 +1,180 @@
+"""Pins for the oracle's matmul, norm, RoPE, attention and whole-model composition: each is checked
+against a library routine, a closed form in float64, or a special case with a known answer."""
+import math
+
+import numpy as np
+import pytest
+import torch
+import torch.nn.functional as F
+
+from oracle import q40_oracle as O
+
+
+def _rand_q40(K, N, seed, std=0.02):
+    g = torch.Generator().manual_seed(seed)
+    v = (torch.randn((N, K), generator=g) * std).to(torch.float16)
+    return O.quantize_weight(v)
+
+
+def test_matmul_against_float64_and_one_hot():
+    K, N = 256, 384
+    w, s, _ = _rand_q40(K, N, 10)
+    g = torch.Generator().manual_seed(11)
+    a = torch.randn((5, K), generator=g).to(torch.float16)
+    deq = O.dequantize_q40(w, s, 64, (K, N))
+    want = (a.double() @ deq.double())
+    got = O.matmul_q40(a, w, s, (K, N))
+    assert torch.allclose(got.double(), want, rtol=1e-3, atol=1e-3)
+    # one-hot rows pick single dequantised rows exactly; zero input gives zero
+    eye = torch.zeros((3, K), dtype=torch.float16)
+    eye[0, 0] = 1; eye[1, 63] = 1; eye[2, K - 1] = 1
+    got = O.matmul_q40(eye, w, s, (K, N))
+    assert torch.equal(got[0], deq[0]) and torch.equal(got[1], deq[63]) and torch.equal(got[2], deq[K - 1])
+    assert torch.all(O.matmul_q40(torch.zeros((1, K), dtype=torch.float16), w, s, (K, N)) == 0)
+    # the torch-only CPU path (dequant + F.linear) is the same function
+    assert torch.equal(O.linear_q40_cpu_path(a, w, s, (N, K)), O.matmul_q40(a, w, s, (K, N)))
+
+
+def test_rmsnorm_closed_form():
+    g = torch.Generator().manual_seed(12)
+    x = torch.randn((3, 512), generator=g).to(torch.float16)
+    wt = (1 + 0.1 * torch.randn(512, generator=g)).to(torch.float16)
+    got = O.rmsnorm(x, wt, 1e-5)
+    xd = x.double()
+    want = xd / torch.sqrt((xd ** 2).mean(-1, keepdim=True) + 1e-5) * wt.double()
+    assert torch.allclose(got.double(), want, rtol=2e-3, atol=1e-4)
+    # constant row: x/|x| = 1 -> output equals the weight (eps negligible)
+    assert torch.equal(O.rmsnorm(torch.full((1, 512), 3.0, dtype=torch.float16), wt, 1e-12), wt[None])
+
+
+def test_rope_table_and_rotation():
+    D, T, theta = 128, 40, 1e6
+    fc = O.precompute_freqs_cis(D, T, theta)
+    assert fc.shape == (T, D // 2) and fc.dtype == torch.complex64
+    t = np.arange(T)[:, None].astype(np.float64)
+    inv = theta ** (-np.arange(0, D, 2).astype(np.float64) / D)
+    assert np.allclose(fc.real.numpy(), np.cos(t * inv), atol=2e-6)
+    assert np.allclose(fc.imag.numpy(), np.sin(t * inv), atol=2e-6)
+    g = torch.Generator().manual_seed(13)
+    q = torch.randn((2, T, 4, D), generator=g).to(torch.float16)
+    k = torch.randn((2, T, 2, D), generator=g).to(torch.float16)
+    qe, ke = O.apply_rotary_emb(q, k, fc)
+    # position 0 is the identity
+    assert torch.equal(qe[:, 0], q[:, 0]) and torch.equal(ke[:, 0], k[:, 0])
+    # each (i, i+64) pair is rotated by angle t*inv_i: check against float64 and norm preservation
+    qd = q.double()
+    c = torch.from_numpy(np.cos(t * inv))[None, :, None, :]
+    s_ = torch.from_numpy(np.sin(t * inv))[None, :, None, :]
+    x1, x2 = qd[..., :64], qd[..., 64:]
+    want = torch.cat((x1 * c - x2 * s_, x2 * c + x1 * s_), dim=-1)
+    assert torch.allclose(qe.double(), want, atol=6e-3, rtol=0)
+    n0 = (qd[..., :64] ** 2 + qd[..., 64:] ** 2)
+    n1 = (qe.double()[..., :64] ** 2 + qe.double()[..., 64:] ** 2)
+    assert torch.allclose(n0, n1, atol=3e-2, rtol=1e-2)
+
+
+def test_silu_mul():
+    g = torch.Generator().manual_seed(14)
+    a = torch.randn(1000, generator=g).to(torch.float16)
+    b = torch.randn(1000, generator=g).to(torch.float16)
+    want = a.double() / (1 + torch.exp(-a.double())) * b.double()
+    assert torch.allclose(O.silu_mul(a, b).double(), want, atol=2e-3, rtol=2e-3)
+    assert torch.equal(O.silu_mul(a, b), F.silu(a) * b)          # same rounding points as torch's fp16 ops
+
+
+def _attn_inputs(B, H, Hkv, D, P, S, seed):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn((B, H, D), generator=g).to(torch.float16)
+    pk = torch.randn((P, Hkv, D), generator=g).to(torch.float16)
+    pv = torch.randn((P, Hkv, D), generator=g).to(torch.float16)
+    sk = torch.randn((B, S, Hkv, D), generator=g).to(torch.float16)
+    sv = torch.randn((B, S, Hkv, D), generator=g).to(torch.float16)
+    lens = torch.randint(0, S + 1, (B,), generator=g).tolist()
+    return q, pk, pv, sk, sv, lens
+
+
+@pytest.mark.parametrize("Hkv", [4, 2])
+def test_attention_against_sdpa(Hkv):
+    B, H, D, P, S = 5, 4, 128, 37, 9
+    q, pk, pv, sk, sv, lens = _attn_inputs(B, H, Hkv, D, P, S, 20)
+    lens[0] = 0; lens[1] = S
+    got = O.shared_prefix_attention(q, pk, pv, sk, sv, lens)
+    n_rep = H // Hkv
+    for b in range(B):
+        k = torch.cat((pk, sk[b, :lens[b]]), 0).repeat_interleave(n_rep, 1).transpose(0, 1).float()
+        v = torch.cat((pv, sv[b, :lens[b]]), 0).repeat_interleave(n_rep, 1).transpose(0, 1).float()
+        want = F.scaled_dot_product_attention(q[b].float()[:, None, :], k, v)[:, 0]
+        assert torch.allclose(got[b].float(), want, atol=2e-3, rtol=1e-2)
+
+
+def test_attention_special_cases_and_split_invariance():
+    B, H, D, P, S = 3, 2, 128, 16, 8
+    q, pk, pv, sk, sv, lens = _attn_inputs(B, H, H, D, P, S, 21)
+    # all-equal scores (q = 0) -> mean of V over prefix + suffix
+    z = torch.zeros_like(q)
+    got = O.shared_prefix_attention(z, pk, pv, sk, sv, [S] * B)
+    for b in range(B):
+        want = torch.cat((pv, sv[b]), 0).float().mean(0)
+        assert torch.allclose(got[b].float(), want, atol=2e-3)
+    # one dominant key -> its V row
+    pk2 = pk.clone(); pk2[5] = 0; pk2[5, :, 0] = 200.0
+    q2 = torch.zeros_like(q); q2[..., 0] = 50.0
+    got = O.shared_prefix_attention(q2, pk2 * 0 + pk2, pv, None, None, None)
+    assert torch.allclose(got[0].float(), pv[5].float(), atol=1e-3)
+    # moving tokens from the prefix into every branch's suffix changes nothing
+    full = O.shared_prefix_attention(q, pk, pv, sk, sv, [S] * B)
+    cut = 11
+    sk2 = torch.cat((pk[cut:][None].expand(B, -1, -1, -1), sk), 1)
+    sv2 = torch.cat((pv[cut:][None].expand(B, -1, -1, -1), sv), 1)
+    moved = O.shared_prefix_attention(q, pk[:cut], pv[:cut], sk2, sv2, [S + P - cut] * B)
+    assert torch.allclose(full.float(), moved.float(), atol=1e-3)
+
+
+def test_causal_attention_against_sdpa():
+    S, H, D = 19, 2, 128
+    g = torch.Generator().manual_seed(22)
+    q, k, v = (torch.randn((S, H, D), generator=g).to(torch.float16) for _ in range(3))
+    got = O.causal_attention(q, k, v)
+    want = F.scaled_dot_product_attention(q.transpose(0, 1).float(), k.transpose(0, 1).float(),
+                                          v.transpose(0, 1).float(), is_causal=True).transpose(0, 1)
+    assert torch.allclose(got.float(), want, atol=2e-3, rtol=1e-2)
+
+
+TINY = dict(dim=256, n_layers=2, n_heads=2, vocab_size=320, multiple_of=128, max_batch_size=4,
+            max_seq_len=8, max_prompt_seq_len=16)
+
+
+def test_ffn_hidden_dim():
+    assert O.ffn_hidden_dim(4096, 256, None) == 11008
+    assert O.ffn_hidden_dim(8192, 4096, 1.3) == 28672
+
+
+def test_model_dense_equals_q40_path_and_branches_agree():
+    args = O.OracleArgs(**TINY)
+    sd = O.random_q40_state_dict(args, seed=30, std=0.05)
+    prompt = torch.randint(0, args.vocab_size, (1, 10), generator=torch.Generator().manual_seed(31))
+    dense = O.OracleTransformer(args, sd, dense=True)
+    q40 = O.OracleTransformer(args, sd, dense=False)
+    t_dense, margins = dense.greedy(prompt, 3, 6)
+    t_q40, _ = q40.greedy(prompt, 3, 6)
+    assert torch.equal(t_dense, t_q40)
+    assert torch.equal(t_dense[0], t_dense[1]) and torch.equal(t_dense[0], t_dense[2])
+    assert len(margins) == 6 and all(m >= 0 for m in margins)
+
+
+def test_model_incremental_equals_full_recompute_without_kv_quant():
+    """prefill(P) + decode steps give the logits of prefill(P+t) at the same positions when the suffix
+    KV is kept exact (the only approximation in the decode path is the Q4 KV round trip)."""
+    args = O.OracleArgs(**TINY)
+    sd = O.random_q40_state_dict(args, seed=32, std=0.05)
+    g = torch.Generator().manual_seed(33)
+    toks = torch.randint(0, args.vocab_size, (1, 13), generator=g)
+    m = O.OracleTransformer(args, sd, dense=True, quantize_kv=False)
+    full = m.forward(toks, 0)[0]                       # [13, vocab]
+    m.reset()
+    inc = [m.forward(toks[:, :10], 0)[0, -1]]
+    for t in range(10, 13):
+        inc.append(m.forward(toks[:, t:t + 1], t)[0, -1])
+    inc = torch.stack(inc)
+    assert torch.allclose(inc.float(), full[9:13].float(), atol=3e-2, rtol=3e-2)
+    assert torch.equal(inc.argmax(-1), full[9:13].argmax(-1))
