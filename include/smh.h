@@ -1,0 +1,134 @@
+/* smh.h - C ABI of the MI355X (gfx950) Q4_0 CodeLlama hot path.
+ *
+ * The reference (hongyihuang/spec-mcts) is pure Python + Triton and has no native boundary; each
+ * entry point below replaces one Python-level operator or model method of the reference, cited
+ * as file:line relative to the reference checkout.  A Python caller binds these with ctypes
+ * (spec_mcts_amd/_lib.py does exactly that).
+ *
+ * Conventions
+ *  - every pointer is a DEVICE pointer unless its name ends in _host;
+ *  - fp16 data is IEEE binary16, row-major, innermost dimension contiguous;
+ *  - Q4_0 data is the reference's layout (fp16_to_int4.py:52-96): 64-byte rows of packed signed
+ *    nibbles, two 64-value groups per row (group 2p in the high nibbles, group 2p+1 in the low
+ *    nibbles), one fp16 scale per group;  value = nibble * scale, nibble in [-8, 7];
+ *  - a Q4_0 weight is the quantised TRANSPOSE of the [N,K] linear weight (fp16_to_int4.py:173):
+ *    bytes viewed [K, N/2], scales viewed [K, N/64] (triton_kernels.py:481-482), N % 128 == 0;
+ *  - kernels are enqueued on `stream` and never synchronise; nothing is allocated or freed;
+ *  - return value: 0 on success, negative = invalid argument (see smh_last_error_string),
+ *    positive = hipError_t from the launch.
+ */
+#ifndef SMH_H
+#define SMH_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *smh_stream_t; /* hipStream_t */
+
+#define SMH_VERSION 1
+
+/* epilogues of the Q4_0 matmul */
+#define SMH_EPI_NONE 0     /* c = fp16(acc) */
+#define SMH_EPI_RESIDUAL 1 /* c = fp16(residual + fp16(acc))   (h + wo(..), hf_model_q40_kv_shared.py:463-466) */
+
+/* suffix KV formats of the decode attention */
+#define SMH_KV_NONE 0
+#define SMH_KV_FP16 1
+#define SMH_KV_Q40 2
+
+int smh_version(void);
+/* message of the last failing call on the calling thread ("" if none) */
+const char *smh_last_error_string(void);
+
+/* ---- Q4_0 codec --------------------------------------------------------------------------
+ * smh_q40_dequant replaces triton_deq_int40 / dequantize_q40 (triton_kernels.py:43-107):
+ * rows 64-byte rows -> rows*128 fp16 values, bit-exact nibble*scale.
+ * smh_q40_quantize replaces quantize_q40 (triton_kernels.py:12-41) for fp16 input with torch's
+ * rounding: scale = fp16(absmax/7), code = rint(fp16(x/scale)), 0/0 -> 0. groups must be even. */
+int smh_q40_dequant(const void *w, const void *s, void *out, long rows, smh_stream_t stream);
+int smh_q40_quantize(const void *in, void *w, void *s, long groups, smh_stream_t stream);
+
+/* ---- Q4_0 matmul ---------------------------------------------------------------------------
+ * c[M,N] = a[M,K] . deq(b_w, b_s)[K,N], fp16 operands, fp32 accumulation, one fp16 rounding;
+ * replaces matmul_q40 (triton_kernels.py:471-500) = LinearQ4_0.forward
+ * (hf_model_q40_kv_shared.py:228-236).  lda/ldc/ldr are row strides in elements.
+ * Requires N % 128 == 0 and K % 8 == 0.
+ * smh_q40_matmul picks the GEMV kernel (M <= SMH_GEMV_MAX_M) or the LDS/MFMA GEMM.
+ * workspace: smh_q40_matmul_workspace_bytes() bytes, zero-filled ONCE by the caller before first
+ * use; the kernels leave it zeroed again, so it can be reused by every later call on the same
+ * stream (calls that overlap on different streams need separate workspaces). */
+#define SMH_GEMV_MAX_M 16
+size_t smh_q40_matmul_workspace_bytes(int max_m, int max_n);
+int smh_q40_gemv(const void *a, int M, int K, long lda, const void *b_w, const void *b_s, int N,
+                 void *c, long ldc, int epilogue, const void *residual, long ldr,
+                 void *workspace, size_t workspace_bytes, smh_stream_t stream);
+int smh_q40_gemm(const void *a, int M, int K, long lda, const void *b_w, const void *b_s, int N,
+                 void *c, long ldc, int epilogue, const void *residual, long ldr,
+                 void *workspace, size_t workspace_bytes, smh_stream_t stream);
+int smh_q40_matmul(const void *a, int M, int K, long lda, const void *b_w, const void *b_s, int N,
+                   void *c, long ldc, int epilogue, const void *residual, long ldr,
+                   void *workspace, size_t workspace_bytes, smh_stream_t stream);
+
+/* ---- small fused ops -----------------------------------------------------------------------
+ * smh_rmsnorm: RMSNorm.forward (hf_model_q40_kv_shared.py:129-134): fp32 normalise -> fp16 ->
+ *   * weight -> fp16.  x,out [rows, dim].
+ * smh_silu_mul: F.silu(g) * u in fp16 (hf_model_q40_kv_shared.py:434).
+ * smh_argmax: greedy pick, lowest index on ties (hf_model_q40.py:517-519). logits [rows, vocab]
+ *   fp16 with row stride ld; out int64 [rows].
+ * smh_rope_append_kv: apply_rotary_emb (hf_model_q40_kv_shared.py:173-203) to q[B,H,D] and
+ *   k[B,Hkv,D] in place with the fp16 cos/sin row of position *pos_dev (+ b * pos_stride rows? no:
+ *   all branches share one position), then quantise the rotated k and v[B,Hkv,D] into row
+ *   *t_dev of each branch's Q4_0 suffix cache (hf_model_q40_kv_shared.py:365-371).
+ *   cos/sin: fp16 tables [T, D/2].  cache_k/v: bytes [Bmax, Smax, Hkv*D/128, 64],
+ *   cache_ks/vs: fp16 [Bmax, Smax, Hkv*D/64].  pos_dev, t_dev: int32 on the device so that a
+ *   captured graph can be replayed for successive positions.
+ * smh_kv_fork: Attention.fork (hf_model_q40_kv_shared.py:282-297): copy branch `origin`'s rows
+ *   to branches curr .. curr+forks-1 in one Q4_0 cache (bytes and scales).
+ */
+int smh_rmsnorm(const void *x, const void *weight, void *out, int rows, int dim, float eps,
+                smh_stream_t stream);
+int smh_silu_mul(const void *g, const void *u, void *out, long n, smh_stream_t stream);
+int smh_argmax(const void *logits, int rows, int vocab, long ld, int64_t *out, smh_stream_t stream);
+int smh_rope_append_kv(void *q, void *k, const void *v, int B, int H, int Hkv, int D,
+                       const void *cos_tab, const void *sin_tab, const int32_t *pos_dev,
+                       void *cache_k, void *cache_ks, void *cache_v, void *cache_vs,
+                       int Smax, const int32_t *t_dev, smh_stream_t stream);
+int smh_rope(void *q, void *k, int S, int H, int Hkv, int D, const void *cos_tab,
+             const void *sin_tab, int pos0, smh_stream_t stream);
+int smh_kv_fork(void *cache, void *cache_s, int Bmax, long row_bytes, long row_scales,
+                int origin, int curr, int forks, smh_stream_t stream);
+
+/* ---- attention -----------------------------------------------------------------------------
+ * smh_shared_prefix_attn: the decode attention of Attention.forward
+ * (hf_model_q40_kv_shared.py:375-405) without materialising or copying the prefix per branch:
+ * out[b,h,:] = softmax(q[b,h,:] . K_b^T / sqrt(D)) . V_b  with  K_b = [prefix (P rows, shared) ||
+ * suffix of branch b (lens[b] rows) || cur_k[b] (one exact fp16 row, optional)].
+ *   q, out      fp16 [B, H, D], D == 128
+ *   prefix_k/v  fp16 [P, Hkv, D]
+ *   suffix      SMH_KV_FP16: suffix_k/v fp16 [B, Smax, Hkv, D]
+ *               SMH_KV_Q40 : suffix_k/v bytes [B, Smax, Hkv*D/128, 64], suffix_ks/vs fp16 [B, Smax, Hkv*D/64]
+ *   lens        int32 [B] on the device (rows of the suffix that are valid); with len_offset
+ *               added to each (the model passes the step counter t for every branch)
+ *   cur_k/v     fp16 [B, Hkv, D] or NULL
+ *   workspace   smh_attn_workspace_bytes(B, H, P) bytes of scratch (no initialisation needed)
+ * smh_prefill_attn: causal attention over the prompt (hf_model_q40_kv_shared.py:499-504,405),
+ *   q [S,H,D], k,v [S,Hkv,D] -> out [S,H,D].
+ */
+size_t smh_attn_workspace_bytes(int B, int H, int P);
+int smh_shared_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int D,
+                           const void *prefix_k, const void *prefix_v, int P,
+                           int suffix_format, const void *suffix_k, const void *suffix_v,
+                           const void *suffix_ks, const void *suffix_vs, int Smax,
+                           const int32_t *lens, int lens_stride, const void *cur_k, const void *cur_v,
+                           void *workspace, size_t workspace_bytes, smh_stream_t stream);
+int smh_prefill_attn(const void *q, const void *k, const void *v, void *out, int S, int H, int Hkv,
+                     int D, smh_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* SMH_H */

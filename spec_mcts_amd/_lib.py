@@ -1,0 +1,69 @@
+"""ctypes binding of libsmh.so (the C ABI declared in include/smh.h).
+
+The library is built in-tree by spec_mcts_amd.build.  There is no fallback: if the library is
+missing, or a call fails, an exception is raised.
+"""
+from __future__ import annotations
+
+import ctypes
+import os
+from ctypes import c_char_p, c_float, c_int, c_long, c_size_t, c_void_p
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libsmh.so")
+
+SMH_EPI_NONE, SMH_EPI_RESIDUAL = 0, 1
+SMH_KV_NONE, SMH_KV_FP16, SMH_KV_Q40 = 0, 1, 2
+SMH_GEMV_MAX_M = 16
+
+_P = c_void_p
+# name -> (restype, argtypes); must list every symbol of include/smh.h
+SIGNATURES = {
+    "smh_version": (c_int, []),
+    "smh_last_error_string": (c_char_p, []),
+    "smh_q40_dequant": (c_int, [_P, _P, _P, c_long, _P]),
+    "smh_q40_quantize": (c_int, [_P, _P, _P, c_long, _P]),
+    "smh_q40_matmul_workspace_bytes": (c_size_t, [c_int, c_int]),
+    "smh_q40_gemv": (c_int, [_P, c_int, c_int, c_long, _P, _P, c_int, _P, c_long, c_int, _P, c_long, _P, c_size_t, _P]),
+    "smh_q40_gemm": (c_int, [_P, c_int, c_int, c_long, _P, _P, c_int, _P, c_long, c_int, _P, c_long, _P, c_size_t, _P]),
+    "smh_q40_matmul": (c_int, [_P, c_int, c_int, c_long, _P, _P, c_int, _P, c_long, c_int, _P, c_long, _P, c_size_t, _P]),
+    "smh_rmsnorm": (c_int, [_P, _P, _P, c_int, c_int, c_float, _P]),
+    "smh_silu_mul": (c_int, [_P, _P, _P, c_long, _P]),
+    "smh_argmax": (c_int, [_P, c_int, c_int, c_long, _P, _P]),
+    "smh_rope_append_kv": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, c_int, _P, _P]),
+    "smh_rope": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, _P]),
+    "smh_kv_fork": (c_int, [_P, _P, c_int, c_long, c_long, c_int, c_int, c_int, _P]),
+    "smh_attn_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
+    "smh_shared_prefix_attn": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, c_int, _P, _P, _P, _P, c_int,
+                                       _P, c_int, _P, _P, _P, c_size_t, _P]),
+    "smh_prefill_attn": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
+}
+
+_lib = None
+
+
+class SmhError(RuntimeError):
+    pass
+
+
+def load() -> ctypes.CDLL:
+    """Load libsmh.so and declare every entry point.  Raises if the library has not been built."""
+    global _lib
+    if _lib is not None:
+        return _lib
+    if not os.path.exists(LIB_PATH):
+        raise SmhError(f"{LIB_PATH} not found: build it with `python -m spec_mcts_amd.build` "
+                       "(there is no fallback path)")
+    lib = ctypes.CDLL(LIB_PATH)
+    for name, (res, args) in SIGNATURES.items():
+        fn = getattr(lib, name)
+        fn.restype = res
+        fn.argtypes = args
+    _lib = lib
+    return lib
+
+
+def check(status: int, what: str) -> None:
+    if status != 0:
+        msg = load().smh_last_error_string().decode()
+        raise SmhError(f"{what} failed with status {status}: {msg}")

@@ -1,0 +1,386 @@
+// Shared-prefix decode attention: one query per (branch, head) over
+//   [ prefix K/V (P rows, fp16, shared by all branches) || that branch's suffix (fp16 or Q4_0 rows)
+//     || the new token's exact fp16 K/V ].
+//
+// Two kernels.
+//  1. attn_prefix_kernel, grid (splits, kv heads): a workgroup stages one slice of the prefix for one
+//     kv head in LDS ONCE (K row-major, V transposed) and every branch's query for that head is
+//     multiplied against it on the matrix cores: the B queries are the N dimension of
+//     S^T = K . Q^T and of O^T = V^T . P^T, so the prefix is read from HBM once per head instead of
+//     once per branch.  Each (slice, query) leaves an un-normalised partial (max, sum, o[128]).
+//  2. attn_suffix_kernel, one wave per (branch, kv head): streams the branch's own suffix rows
+//     (HBM-bound; Q4_0 rows are decoded in registers), keeps an online softmax per 16-lane group,
+//     folds in the prefix partials and the new token, normalises and writes fp16.
+// Scores and softmax are fp32 throughout (exp2 of log2(e)-scaled scores); probabilities are rounded
+// to fp16 only as the operand of the P.V matrix product.
+//
+// Algorithmic HBM traffic: prefix 2*P*Hkv*D*2 B once + per branch its suffix rows
+// (512 B fp16 or 136 B Q4_0 per row and kv head) + q/out.
+#include "smh_common.hpp"
+
+namespace smh {
+
+constexpr int ATT_D = 128;
+constexpr int ATT_TW_MAX = 128;            // prefix rows per workgroup
+constexpr int ATT_KPITCH = 136;            // halves per LDS row of K (272 B: 16 rows hit distinct banks)
+constexpr int ATT_VPITCH = ATT_TW_MAX + 8; // halves per LDS row of V^T
+constexpr float LOG2E = 1.4426950408889634f;
+
+struct AttnParams {
+    const half_t *q;
+    half_t *out;
+    const half_t *prefix_k, *prefix_v;
+    const void *suffix_k, *suffix_v;
+    const half_t *suffix_ks, *suffix_vs;
+    const int32_t *lens;
+    const half_t *cur_k, *cur_v;
+    float *part_o;           // [splits][Hkv][Bq][128]
+    float *part_ml;          // [splits][Hkv][Bq][2]
+    long suffix_batch_stride_rows;   // rows (tokens) between consecutive branches of the suffix
+    int B, H, Hkv, n_rep, Bq;        // Bq = B * n_rep queries per kv head
+    int P, tw, splits;
+    int suffix_format, lens_stride;
+    int causal;                      // prefill mode: branch b attends to suffix rows 0..b
+    float scale_log2;                // log2(e) / sqrt(D)
+};
+
+// position of prefix row t (0..tw-1) inside an LDS row of V^T: within each block of 32 rows the
+// order is chosen so that the 8 probabilities a lane holds after two S^T tiles (rows 4g+r of tile 2j
+// and of tile 2j+1) are 8 consecutive halves.
+__device__ __forceinline__ int vt_pos(int t) {
+    const int blk = t & ~31, w = t & 31;
+    const int j2 = w >> 4, g = (w >> 2) & 3, r = w & 3;
+    return blk + 8 * g + 4 * j2 + r;
+}
+
+__global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
+    __shared__ __attribute__((aligned(16))) half_t ks[ATT_TW_MAX][ATT_KPITCH];
+    __shared__ __attribute__((aligned(16))) half_t vt[ATT_D][ATT_VPITCH];
+
+    const int split = blockIdx.x;
+    const int hk = blockIdx.y;
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
+    const int t0 = split * p.tw;
+    const int cnt = min(p.tw, p.P - t0);
+    const int tw32 = (cnt + 31) & ~31;          // rows actually touched by the matrix ops
+
+    // ---- stage K (row-major) and V (transposed) ----
+    for (int idx = tid; idx < tw32 * 16; idx += 256) {
+        const int t = idx >> 4, ch = idx & 15;
+        u32x4 kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
+        if (t < cnt) {
+            const long off = ((long)(t0 + t) * p.Hkv + hk) * ATT_D + ch * 8;
+            kv = *reinterpret_cast<const u32x4 *>(p.prefix_k + off);
+            vv = *reinterpret_cast<const u32x4 *>(p.prefix_v + off);
+        }
+        *reinterpret_cast<u32x4 *>(&ks[t][ch * 8]) = kv;
+        const int pos = vt_pos(t);
+        const h8 vh = __builtin_bit_cast(h8, vv);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) vt[ch * 8 + j][pos] = vh[j];
+    }
+    __syncthreads();
+
+    const int q_tiles = (p.Bq + 15) / 16;
+    const int t_tiles = tw32 / 16;
+    for (int qt = wave; qt < q_tiles; qt += 4) {
+        const int qr = min(qt * 16 + c, p.Bq - 1);
+        const int b = qr / p.n_rep, r_ = qr % p.n_rep;
+        const half_t *qp = p.q + ((long)b * p.H + hk * p.n_rep + r_) * ATT_D + 8 * g;
+        h8 qb[4];
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) qb[k4] = *reinterpret_cast<const h8 *>(qp + 32 * k4);
+
+        // S^T tiles: element r of st[j] is row t = 16j + 4g + r, column (query) c
+        f4 st[ATT_TW_MAX / 16];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < ATT_TW_MAX / 16; ++j) {
+            st[j] = f4{0.f, 0.f, 0.f, 0.f};
+            if (j < t_tiles) {
+#pragma unroll
+                for (int k4 = 0; k4 < 4; ++k4) {
+                    h8 ka = *reinterpret_cast<const h8 *>(&ks[16 * j + c][32 * k4 + 8 * g]);
+                    st[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qb[k4], st[j], 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const int t = 16 * j + 4 * g + r;
+                    const float sv = (t < cnt) ? st[j][r] * p.scale_log2 : -INFINITY;
+                    st[j][r] = sv;
+                    mx = fmaxf(mx, sv);
+                }
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < ATT_TW_MAX / 16; ++j) {
+            if (j < t_tiles) {
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    const float e = exp2f(st[j][r] - mx);      // masked rows: exp2(-inf) = 0
+                    st[j][r] = e;
+                    sum += e;
+                }
+            }
+        }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+
+        // O^T tiles: element r of ot[dt] is row d = 16dt + 4g + r, column (query) c
+        f4 ot[8];
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) ot[dt] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int jj = 0; jj < ATT_TW_MAX / 32; ++jj) {
+            if (2 * jj < t_tiles) {
+                h8 pb;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    pb[r] = (half_t)st[2 * jj][r];
+                    pb[4 + r] = (half_t)st[2 * jj + 1][r];
+                }
+#pragma unroll
+                for (int dt = 0; dt < 8; ++dt) {
+                    h8 va = *reinterpret_cast<const h8 *>(&vt[16 * dt + c][32 * jj + 8 * g]);
+                    ot[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb, ot[dt], 0, 0, 0);
+                }
+            }
+        }
+        const int qrow = qt * 16 + c;
+        if (qrow < p.Bq) {
+            const long base = ((long)split * p.Hkv + hk) * p.Bq + qrow;
+            float *po = p.part_o + base * ATT_D;
+#pragma unroll
+            for (int dt = 0; dt < 8; ++dt) *reinterpret_cast<f4 *>(po + 16 * dt + 4 * g) = ot[dt];
+            if (g == 0) {
+                p.part_ml[base * 2] = mx;
+                p.part_ml[base * 2 + 1] = sum;
+            }
+        }
+    }
+}
+
+// ---- suffix rows ----------------------------------------------------------------------------------------
+// A 16-lane group handles one row at a time; lane c of the group owns head dims 4c..4c+3 ("low half")
+// and 64+4c..64+4c+3 ("high half"), held as fp16 pairs in the order (0,2),(1,3) that nibble decoding
+// produces.
+struct RowRegs { h2 a02, a13, b02, b13; };   // a: dims 4c.., b: dims 64+4c..
+
+__device__ __forceinline__ RowRegs row_from_fp16(const half_t *row, int c) {
+    const u32x2 lo = *reinterpret_cast<const u32x2 *>(row + 4 * c);
+    const u32x2 hi = *reinterpret_cast<const u32x2 *>(row + 64 + 4 * c);
+    RowRegs r;
+    r.a02 = as_h2(pack_lo16(lo[0], lo[1]));
+    r.a13 = as_h2(pack_hi16(lo[0], lo[1]));
+    r.b02 = as_h2(pack_lo16(hi[0], hi[1]));
+    r.b13 = as_h2(pack_hi16(hi[0], hi[1]));
+    return r;
+}
+// bytes: this lane's dword of the packed row; sc: (scale of dims 0..63, scale of dims 64..127)
+__device__ __forceinline__ RowRegs row_from_q40(uint32_t bytes, uint32_t sc) {
+    const uint32_t u = bytes ^ NIBBLE_FLIP, u1 = u >> 8;
+    const h2 s_a = as_h2(pack_lo16(sc, sc)), s_b = as_h2(pack_hi16(sc, sc));
+    RowRegs r;
+    r.a02 = codes_high(u) * s_a;
+    r.a13 = codes_high(u1) * s_a;
+    r.b02 = codes_low(u) * s_b;
+    r.b13 = codes_low(u1) * s_b;
+    return r;
+}
+__device__ __forceinline__ float row_dot(const RowRegs &k, const RowRegs &q) {
+    float s = __builtin_amdgcn_fdot2(k.a02, q.a02, 0.f, false);
+    s = __builtin_amdgcn_fdot2(k.a13, q.a13, s, false);
+    s = __builtin_amdgcn_fdot2(k.b02, q.b02, s, false);
+    s = __builtin_amdgcn_fdot2(k.b13, q.b13, s, false);
+    return row16_sum(s);
+}
+
+struct SoftState {
+    float m, l;
+    float o[8];     // dims 4c+0, 4c+2, 4c+1, 4c+3, 64+4c+0, 64+4c+2, 64+4c+1, 64+4c+3
+};
+__device__ __forceinline__ void soft_add_row(SoftState &st, float score, const RowRegs &v) {
+    const float m_new = fmaxf(st.m, score);
+    const float corr = exp2f(st.m - m_new);          // st.m = -inf on first use: exp2(-inf) = 0
+    const float pr = exp2f(score - m_new);
+    st.m = m_new;
+    st.l = st.l * corr + pr;
+    st.o[0] = st.o[0] * corr + pr * (float)v.a02.x;
+    st.o[1] = st.o[1] * corr + pr * (float)v.a02.y;
+    st.o[2] = st.o[2] * corr + pr * (float)v.a13.x;
+    st.o[3] = st.o[3] * corr + pr * (float)v.a13.y;
+    st.o[4] = st.o[4] * corr + pr * (float)v.b02.x;
+    st.o[5] = st.o[5] * corr + pr * (float)v.b02.y;
+    st.o[6] = st.o[6] * corr + pr * (float)v.b13.x;
+    st.o[7] = st.o[7] * corr + pr * (float)v.b13.y;
+}
+// fold an un-normalised partial (m2, l2, o2) into st
+__device__ __forceinline__ void soft_merge(SoftState &st, float m2, float l2, const float *o2) {
+    const float m_new = fmaxf(st.m, m2);
+    if (m_new == -INFINITY) return;                  // both empty
+    const float c1 = exp2f(st.m - m_new), c2 = exp2f(m2 - m_new);
+    st.m = m_new;
+    st.l = st.l * c1 + l2 * c2;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) st.o[j] = st.o[j] * c1 + o2[j] * c2;
+}
+
+__global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
+    const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+    const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= (long)p.B * p.Hkv) return;
+    const int b = (int)(item / p.Hkv);
+    const int hk = (int)(item % p.Hkv);
+    int len = 0;
+    if (p.suffix_format != SMH_KV_NONE) len = p.causal ? b + 1 : p.lens[(long)b * p.lens_stride];
+    const long row0 = (long)b * p.suffix_batch_stride_rows;     // first suffix row of this branch
+
+    for (int rep = 0; rep < p.n_rep; ++rep) {
+        const int h = hk * p.n_rep + rep;
+        const half_t *qp = p.q + ((long)b * p.H + h) * ATT_D;
+        const RowRegs qr = row_from_fp16(qp, c);
+        SoftState st;
+        st.m = -INFINITY;
+        st.l = 0.f;
+#pragma unroll
+        for (int j = 0; j < 8; ++j) st.o[j] = 0.f;
+
+        // ---- this branch's suffix: group g takes rows g, g+4, ... ----
+        for (int t = g; t < len; t += 4) {
+            const long row = (row0 + t) * p.Hkv + hk;
+            RowRegs kr, vr;
+            if (p.suffix_format == SMH_KV_FP16) {
+                kr = row_from_fp16((const half_t *)p.suffix_k + row * ATT_D, c);
+                vr = row_from_fp16((const half_t *)p.suffix_v + row * ATT_D, c);
+            } else {
+                const uint32_t kb = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_k + row * 64 + 4 * c);
+                const uint32_t vb = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_v + row * 64 + 4 * c);
+                const uint32_t ksc = *reinterpret_cast<const uint32_t *>(p.suffix_ks + row * 2);
+                const uint32_t vsc = *reinterpret_cast<const uint32_t *>(p.suffix_vs + row * 2);
+                kr = row_from_q40(kb, ksc);
+                vr = row_from_q40(vb, vsc);
+            }
+            soft_add_row(st, row_dot(kr, qr) * p.scale_log2, vr);
+        }
+        // ---- the new token's exact K/V (group 0 only) ----
+        if (p.cur_k != nullptr && g == 0) {
+            const long off = ((long)b * p.Hkv + hk) * ATT_D;
+            const RowRegs kr = row_from_fp16(p.cur_k + off, c);
+            const RowRegs vr = row_from_fp16(p.cur_v + off, c);
+            soft_add_row(st, row_dot(kr, qr) * p.scale_log2, vr);
+        }
+        // ---- prefix partials: group g folds in splits g, g+4, ... ----
+        const int qrow = b * p.n_rep + rep;
+        for (int s = g; s < p.splits; s += 4) {
+            const long base = ((long)s * p.Hkv + hk) * p.Bq + qrow;
+            const f4 lo = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 4 * c);
+            const f4 hi = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 64 + 4 * c);
+            const float o2[8] = {lo[0], lo[2], lo[1], lo[3], hi[0], hi[2], hi[1], hi[3]};
+            soft_merge(st, p.part_ml[base * 2], p.part_ml[base * 2 + 1], o2);
+        }
+        // ---- merge the four groups (xor 16, xor 32) ----
+#pragma unroll
+        for (int sh = 16; sh <= 32; sh <<= 1) {
+            const float m2 = __shfl_xor(st.m, sh, 64);
+            const float l2 = __shfl_xor(st.l, sh, 64);
+            float o2[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o2[j] = __shfl_xor(st.o[j], sh, 64);
+            soft_merge(st, m2, l2, o2);
+        }
+        if (g == 0) {
+            const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
+            half_t *op = p.out + ((long)b * p.H + h) * ATT_D;
+            h4 lo = {(half_t)(st.o[0] * inv), (half_t)(st.o[2] * inv), (half_t)(st.o[1] * inv), (half_t)(st.o[3] * inv)};
+            h4 hi = {(half_t)(st.o[4] * inv), (half_t)(st.o[6] * inv), (half_t)(st.o[5] * inv), (half_t)(st.o[7] * inv)};
+            *reinterpret_cast<h4 *>(op + 4 * c) = lo;
+            *reinterpret_cast<h4 *>(op + 64 + 4 * c) = hi;
+        }
+    }
+}
+
+static int attn_plan_tw(int P, int Hkv) {
+    // rows of the prefix per workgroup: as large as fits while still giving the 256 CUs work
+    int tw = ATT_TW_MAX;
+    while (tw > 32 && (long)((P + tw - 1) / tw) * Hkv < 256) tw >>= 1;
+    return tw;
+}
+
+}  // namespace smh
+
+extern "C" size_t smh_attn_workspace_bytes(int B, int H, int P) {
+    if (P <= 0 || B <= 0 || H <= 0) return 256;
+    size_t splits = (size_t)(P + 31) / 32;          // worst case: 32 rows per workgroup
+    return splits * (size_t)B * (size_t)H * (smh::ATT_D + 2) * sizeof(float) + 256;
+}
+
+extern "C" int smh_shared_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int D,
+                                      const void *prefix_k, const void *prefix_v, int P,
+                                      int suffix_format, const void *suffix_k, const void *suffix_v,
+                                      const void *suffix_ks, const void *suffix_vs, int Smax,
+                                      const int32_t *lens, int lens_stride, const void *cur_k, const void *cur_v,
+                                      void *workspace, size_t workspace_bytes, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(D == ATT_D, "smh_shared_prefix_attn: head dim %d (only 128)", D);
+    SMH_REQUIRE(B >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0 && P >= 0, "smh_shared_prefix_attn: B=%d H=%d Hkv=%d P=%d", B, H, Hkv, P);
+    SMH_REQUIRE(suffix_format == SMH_KV_NONE || suffix_format == SMH_KV_FP16 || suffix_format == SMH_KV_Q40,
+                "smh_shared_prefix_attn: suffix_format=%d", suffix_format);
+    if (B == 0) return 0;
+    SMH_REQUIRE(q && out, "smh_shared_prefix_attn: null q/out");
+    SMH_REQUIRE(P == 0 || (prefix_k && prefix_v), "smh_shared_prefix_attn: null prefix");
+    if (suffix_format != SMH_KV_NONE) {
+        SMH_REQUIRE(suffix_k && suffix_v && lens && Smax > 0 && (lens_stride == 0 || lens_stride == 1),
+                    "smh_shared_prefix_attn: suffix arguments incomplete");
+        SMH_REQUIRE(suffix_format != SMH_KV_Q40 || (suffix_ks && suffix_vs), "smh_shared_prefix_attn: null suffix scales");
+    }
+    SMH_REQUIRE((cur_k == nullptr) == (cur_v == nullptr), "smh_shared_prefix_attn: cur_k/cur_v must both be given or both be null");
+    AttnParams p;
+    p.q = (const half_t *)q; p.out = (half_t *)out;
+    p.prefix_k = (const half_t *)prefix_k; p.prefix_v = (const half_t *)prefix_v;
+    p.suffix_k = suffix_k; p.suffix_v = suffix_v;
+    p.suffix_ks = (const half_t *)suffix_ks; p.suffix_vs = (const half_t *)suffix_vs;
+    p.lens = lens; p.lens_stride = lens_stride;
+    p.cur_k = (const half_t *)cur_k; p.cur_v = (const half_t *)cur_v;
+    p.suffix_batch_stride_rows = Smax;
+    p.B = B; p.H = H; p.Hkv = Hkv; p.n_rep = H / Hkv; p.Bq = B * p.n_rep;
+    p.P = P; p.suffix_format = suffix_format; p.causal = 0;
+    p.scale_log2 = LOG2E / sqrtf((float)D);
+    p.tw = attn_plan_tw(P, Hkv);
+    p.splits = P > 0 ? (P + p.tw - 1) / p.tw : 0;
+    size_t n_part = (size_t)p.splits * Hkv * p.Bq;
+    SMH_REQUIRE(p.splits == 0 || (workspace && workspace_bytes >= n_part * (ATT_D + 2) * sizeof(float)),
+                "smh_shared_prefix_attn: workspace %zu < %zu bytes", workspace_bytes, n_part * (ATT_D + 2) * sizeof(float));
+    p.part_o = (float *)workspace;
+    p.part_ml = p.part_o + n_part * ATT_D;
+    if (p.splits > 0)
+        hipLaunchKernelGGL(attn_prefix_kernel, dim3(p.splits, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+    long items = (long)B * Hkv;
+    hipLaunchKernelGGL(attn_suffix_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
+    return launch_status();
+}
+
+// Causal prefill attention, expressed as the suffix kernel with "branch" = query position:
+// query s attends to rows 0..s of the same K/V tensors (batch stride 0, no shared prefix).
+extern "C" int smh_prefill_attn(const void *q, const void *k, const void *v, void *out, int S, int H, int Hkv,
+                                int D, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(D == ATT_D, "smh_prefill_attn: head dim %d (only 128)", D);
+    SMH_REQUIRE(S >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "smh_prefill_attn: S=%d H=%d Hkv=%d", S, H, Hkv);
+    if (S == 0) return 0;
+    SMH_REQUIRE(q && k && v && out, "smh_prefill_attn: null pointer");
+    AttnParams p = {};
+    p.q = (const half_t *)q; p.out = (half_t *)out;
+    p.suffix_k = k; p.suffix_v = v;
+    p.suffix_batch_stride_rows = 0;
+    p.B = S; p.H = H; p.Hkv = Hkv; p.n_rep = H / Hkv; p.Bq = S * p.n_rep;
+    p.P = 0; p.splits = 0; p.tw = 32;
+    p.suffix_format = SMH_KV_FP16; p.causal = 1;
+    p.scale_log2 = LOG2E / sqrtf((float)D);
+    long items = (long)S * Hkv;
+    hipLaunchKernelGGL(attn_suffix_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
+    return launch_status();
+}

@@ -1,0 +1,127 @@
+// Flat Q4_0 codec kernels: 64-byte rows of packed signed nibbles <-> fp16.
+//
+// Both kernels are pure streaming (HBM-bound): dequant reads 68 B and writes 256 B per row,
+// quantise reads 256 B and writes 68 B per row.  One lane owns 16 bytes of a row, so a row is
+// covered by 4 neighbouring lanes and every access is a 128-bit load/store.
+#include "smh_common.hpp"
+
+namespace smh {
+
+// out[row*128 + j]      = code(high nibble of byte j) * s[2*row]
+// out[row*128 + 64 + j] = code(low  nibble of byte j) * s[2*row+1]      (one fp16 multiply each)
+__global__ __launch_bounds__(256) void q40_dequant_kernel(const u32x4 *__restrict__ w,
+                                                          const uint32_t *__restrict__ s,
+                                                          half_t *__restrict__ out, long rows) {
+    long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    long row = t >> 2;
+    int c = (int)(t & 3);
+    if (row >= rows) return;
+    u32x4 v = w[row * 4 + c];
+    uint32_t sp = s[row];                       // (s[2row], s[2row+1])
+    h2 s_hi = as_h2(pack_lo16(sp, sp));
+    h2 s_lo = as_h2(pack_hi16(sp, sp));
+    uint32_t hi[8], lo[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t u = v[j] ^ NIBBLE_FLIP;
+        uint32_t u1 = u >> 8;
+        // pairs (byte0, byte2) and (byte1, byte3) of this word
+        uint32_t h02 = as_u32(codes_high(u) * s_hi), h13 = as_u32(codes_high(u1) * s_hi);
+        uint32_t l02 = as_u32(codes_low(u) * s_lo), l13 = as_u32(codes_low(u1) * s_lo);
+        hi[2 * j] = pack_lo16(h02, h13);        // (byte0, byte1)
+        hi[2 * j + 1] = pack_hi16(h02, h13);    // (byte2, byte3)
+        lo[2 * j] = pack_lo16(l02, l13);
+        lo[2 * j + 1] = pack_hi16(l02, l13);
+    }
+    u32x4 *o_hi = reinterpret_cast<u32x4 *>(out + row * 128 + c * 16);
+    u32x4 *o_lo = reinterpret_cast<u32x4 *>(out + row * 128 + 64 + c * 16);
+    o_hi[0] = u32x4{hi[0], hi[1], hi[2], hi[3]};
+    o_hi[1] = u32x4{hi[4], hi[5], hi[6], hi[7]};
+    o_lo[0] = u32x4{lo[0], lo[1], lo[2], lo[3]};
+    o_lo[1] = u32x4{lo[4], lo[5], lo[6], lo[7]};
+}
+
+// One fp16 value -> code with torch's semantics: q = fp16(x / scale); code = rint(q) (to nearest
+// even); NaN (0/0) -> 0.  The division is a correctly rounded fp32 division rounded once more to fp16.
+__device__ __forceinline__ int q40_code(half_t x, float scale) {
+    half_t q = (half_t)((float)x / scale);
+    float qf = (float)q;
+    if (!(qf == qf)) return 0;
+    return (int)__builtin_rintf(qf);
+}
+
+// Lane layout: 8 lanes per 64-value group (8 values = one 128-bit load each), so a wave covers
+// 8 groups = 4 packed rows.  absmax is reduced over the 8 lanes of a group with xor-shuffles.
+__global__ __launch_bounds__(256) void q40_quantize_kernel(const u32x4 *__restrict__ in,
+                                                           uint8_t *__restrict__ w,
+                                                           half_t *__restrict__ s, long groups) {
+    long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    long g = t >> 3;
+    int c = (int)(t & 7);
+    bool live = g < groups;
+    u32x4 raw = live ? in[t] : u32x4{0, 0, 0, 0};
+    half_t x[8];
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        h2 p = as_h2(raw[j]);
+        x[2 * j] = p.x;
+        x[2 * j + 1] = p.y;
+    }
+    // |x| as bit patterns: for finite values the integer order is the magnitude order
+    uint32_t amax = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        uint32_t a = raw[j] & 0x7FFF7FFFu;
+        uint32_t m = max(a & 0xFFFFu, a >> 16);
+        amax = max(amax, m);
+    }
+#pragma unroll
+    for (int o = 4; o > 0; o >>= 1) amax = max(amax, (uint32_t)__shfl_xor((int)amax, o, 64));
+    half_t amax_h = __builtin_bit_cast(half_t, (uint16_t)amax);
+    half_t scale_h = (half_t)((float)amax_h / 7.0f);
+    float scale = (float)scale_h;
+    uint32_t nib = 0;   // 8 codes, value j in bits 4j..4j+3
+#pragma unroll
+    for (int j = 0; j < 8; ++j) nib |= (uint32_t)(q40_code(x[j], scale) & 15) << (4 * j);
+    // the partner group (g ^ 1) sits 8 lanes away; even groups supply high nibbles
+    uint32_t other = (uint32_t)__shfl_xor((int)nib, 8, 64);
+    if (!live) return;
+    if (c == 0) s[g] = scale_h;
+    if ((g & 1) == 0) {
+        uint32_t hi = nib, lo = other;
+        uint32_t b0 = 0, b1 = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            b0 |= ((((hi >> (4 * j)) & 15) << 4) | ((lo >> (4 * j)) & 15)) << (8 * j);
+            b1 |= ((((hi >> (4 * j + 16)) & 15) << 4) | ((lo >> (4 * j + 16)) & 15)) << (8 * j);
+        }
+        u32x2 *dst = reinterpret_cast<u32x2 *>(w + (g >> 1) * 64 + c * 8);
+        *dst = u32x2{b0, b1};
+    }
+}
+
+}  // namespace smh
+
+extern "C" int smh_q40_dequant(const void *w, const void *s, void *out, long rows, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(rows >= 0, "smh_q40_dequant: rows=%ld", rows);
+    if (rows == 0) return 0;
+    SMH_REQUIRE(w && s && out, "smh_q40_dequant: null pointer");
+    long threads = rows * 4;
+    dim3 grid((unsigned)((threads + 255) / 256));
+    hipLaunchKernelGGL(q40_dequant_kernel, grid, dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4 *)w, (const uint32_t *)s, (half_t *)out, rows);
+    return launch_status();
+}
+
+extern "C" int smh_q40_quantize(const void *in, void *w, void *s, long groups, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(groups >= 0 && (groups & 1) == 0, "smh_q40_quantize: groups=%ld must be even", groups);
+    if (groups == 0) return 0;
+    SMH_REQUIRE(in && w && s, "smh_q40_quantize: null pointer");
+    long threads = groups * 8;
+    dim3 grid((unsigned)((threads + 255) / 256));
+    hipLaunchKernelGGL(q40_quantize_kernel, grid, dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4 *)in, (uint8_t *)w, (half_t *)s, groups);
+    return launch_status();
+}

@@ -1,0 +1,364 @@
+"""Drop-in model API of the reference's live Q4_0 CodeLlama model, running on the HIP kernels.
+
+Mirrors hf_model_q40_kv_shared.py of the reference: ModelArgs (:58-72), LinearQ4_0 (:217-250),
+Attention with a shared fp16 prompt KV cache plus a per-branch Q4_0 suffix KV cache and fork
+(:252-409), FeedForward (:412-436), TransformerBlock (:439-467) and Transformer with
+forward(tokens, start_pos), fork, resetSeq, resetTimers, printTimers, generate (:470-613).
+
+Same attribute names (`layers[i].attention.wq.w/.s/.shape`, `tok_embeddings`, `norm`, `output`,
+`freqs_cis`, cache_* tensors), same call protocol (first call start_pos == 0 = prefill that stores
+the prompt KV from row 0; later calls one token per branch), same cast points.  What differs is
+the execution: every operator is a HIP kernel (spec_mcts_amd.kernels); the prompt KV is never
+copied or expanded per branch and the Q4_0 suffix is decoded inside the attention kernel instead
+of being dequantised to a [B, t, H, D] tensor each step.
+"""
+from __future__ import annotations
+
+import time
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+import torch.nn.functional as F
+from torch import nn
+
+from . import kernels as K
+
+INIT_DEVICE = "meta"
+DTYPE = torch.float16
+GROUP_SIZE = 64
+
+# wall-clock accumulators with the reference's names (hf_model_q40_kv_shared.py:17-23).  They are
+# only filled when Transformer.profile is True, in which case every section is bracketed by a
+# device synchronisation so that the numbers mean something.
+COMP_TIME = 0.0
+DEQ_TIME = 0.0
+QKVO_TIME = 0.0
+ATTN_TIME = 0.0
+MLP_TIME = 0.0
+Q_TIME = 0.0
+DQ_TIME = 0.0
+PROFILE = False
+
+
+def _tick() -> float:
+    if PROFILE:
+        torch.cuda.synchronize()
+        return time.time()
+    return 0.0
+
+
+@dataclass
+class ModelArgs:
+    dim: int = 4096
+    n_layers: int = 32
+    n_heads: int = 32
+    n_kv_heads: Optional[int] = None
+    vocab_size: int = 32016
+    multiple_of: int = 256  # make SwiGLU hidden layer size multiple of large power of 2
+    ffn_dim_multiplier: Optional[float] = None
+    norm_eps: float = 1e-5
+    rope_theta: float = 1000000.0
+
+    max_batch_size: int = 80
+    max_seq_len: int = 256
+    max_prompt_seq_len: int = 256
+
+
+def _cache_device() -> torch.device:
+    return torch.device("cuda") if torch.cuda.is_available() else torch.device("cpu")
+
+
+class RMSNorm(torch.nn.Module):
+    def __init__(self, dim: int, eps: float = 1e-6):
+        super().__init__()
+        self.eps = eps
+        self.weight = nn.Parameter(torch.ones(dim))
+
+    def forward(self, x):
+        return K.rmsnorm(x, self.weight, self.eps)
+
+
+def precompute_freqs_cis(dim: int, end: int, theta: float = 10000.0):
+    """complex64 [end, dim/2] rotation table, built on the host exactly as the reference does
+    (hf_model_q40_kv_shared.py:137-142); the kernels consume its fp16 cos/sin."""
+    freqs = 1.0 / (theta ** (torch.arange(0, dim, 2)[: (dim // 2)].float() / dim))
+    t = torch.arange(end, dtype=torch.float32)
+    freqs = torch.outer(t, freqs)
+    return torch.polar(torch.ones_like(freqs), freqs)
+
+
+class LinearQ4_0(torch.nn.Module):
+    """Q4_0 linear.  `.w` (int8 [K*N/128, 64]), `.s` (fp16 [K*N/64]) and `.shape` are plain
+    attributes filled by the loader, exactly as in the reference; after loading `.shape` is the
+    checkpoint's (out_features, in_features)."""
+
+    def __init__(self, in_features, out_features, group_size):
+        super().__init__()
+        self.group_size = group_size
+        self.w = torch.zeros((int(in_features * out_features / group_size / 2), group_size), dtype=torch.int8, device="cpu")
+        self.s = torch.zeros(int(in_features * out_features / group_size), dtype=DTYPE, device="cpu")
+        self.shape = (out_features, in_features)
+
+    def forward(self, x, residual=None):
+        shape = x.shape
+        x = x.reshape(shape[0] * shape[1], shape[2])
+        t0 = _tick()
+        if residual is not None:
+            residual = residual.reshape(shape[0] * shape[1], -1)
+        result = K.matmul_q40(x, self.w, self.s, (self.shape[1], self.shape[0]), residual=residual)
+        if PROFILE:
+            global COMP_TIME
+            COMP_TIME += _tick() - t0
+        return result.view((shape[0], shape[1], -1))
+
+
+class Attention(nn.Module):
+    def __init__(self, args: ModelArgs):
+        super().__init__()
+        self.args = args
+        self.n_kv_heads = args.n_heads if args.n_kv_heads is None else args.n_kv_heads
+        assert args.n_heads % self.n_kv_heads == 0
+        self.n_local_heads = args.n_heads
+        self.n_local_kv_heads = self.n_kv_heads
+        self.n_rep = self.n_local_heads // self.n_local_kv_heads
+        self.head_dim = args.dim // args.n_heads
+        assert self.head_dim == 128, "the attention kernels are written for head_dim 128"
+
+        self.wq = LinearQ4_0(args.dim, args.n_heads * self.head_dim, GROUP_SIZE)
+        self.wk = LinearQ4_0(args.dim, self.n_kv_heads * self.head_dim, GROUP_SIZE)
+        self.wv = LinearQ4_0(args.dim, self.n_kv_heads * self.head_dim, GROUP_SIZE)
+        self.wo = LinearQ4_0(args.n_heads * self.head_dim, args.dim, GROUP_SIZE)
+
+        dev = _cache_device()
+        prompt_shape = (1, args.max_prompt_seq_len, self.n_local_kv_heads, self.head_dim)
+        self.cache_prompt_k = torch.zeros(prompt_shape, dtype=DTYPE, device=dev)
+        self.cache_prompt_v = torch.zeros(prompt_shape, dtype=DTYPE, device=dev)
+        self.cache_prompt_len = 0
+
+        # per-branch suffix cache in Q4_0: one 64-byte row + 2 scales per (branch, position, kv head).
+        # All-zero bytes and scales decode to 0.0, the state the reference reaches by quantising zeros.
+        rows = args.max_batch_size * args.max_seq_len * self.n_local_kv_heads
+        self.cache_k = torch.zeros((rows, 64), dtype=torch.int8, device=dev)
+        self.cache_k_s = torch.zeros((rows * 2, 1), dtype=DTYPE, device=dev)
+        self.cache_v = torch.zeros((rows, 64), dtype=torch.int8, device=dev)
+        self.cache_v_s = torch.zeros((rows * 2, 1), dtype=DTYPE, device=dev)
+
+    def fork(self, origin: int, curr_batch: int, forks: int):
+        """Copy the suffix KV of branch `origin` to branches curr_batch .. curr_batch+forks-1."""
+        B = self.args.max_batch_size
+        K.kv_fork(self.cache_k, self.cache_k_s, B, origin, curr_batch, forks)
+        K.kv_fork(self.cache_v, self.cache_v_s, B, origin, curr_batch, forks)
+
+    def resetSeq(self):
+        """Sets sequence length = 0"""
+        self.cache_prompt_len = 0
+
+    def forward(self, x: torch.Tensor, start_pos: int, freqs_cis, mask, residual=None, step_state=None):
+        """x [B,S,dim] (already normalised); returns residual + wo(attention) when `residual` is given."""
+        bsz, seqlen, _ = x.shape
+        global QKVO_TIME, ATTN_TIME
+        t0 = _tick()
+        xq, xk, xv = self.wq(x), self.wk(x), self.wv(x)
+        H, Hkv, D = self.n_local_heads, self.n_local_kv_heads, self.head_dim
+        cos, sin = freqs_cis
+        if start_pos == 0:
+            # prefill: rotate, keep the prompt K/V of row 0 in fp16, causal attention per row
+            outs = []
+            for b in range(bsz):
+                q_b = xq[b].view(seqlen, H, D)
+                k_b = xk[b].view(seqlen, Hkv, D)
+                v_b = xv[b].view(seqlen, Hkv, D)
+                K.rope(q_b, k_b, cos, sin, 0)
+                if b == 0:
+                    self.cache_prompt_k[0, :seqlen] = k_b
+                    self.cache_prompt_v[0, :seqlen] = v_b
+                    self.cache_prompt_len = seqlen
+                t1 = _tick()
+                outs.append(K.prefill_attn(q_b, k_b, v_b).view(seqlen, H * D))
+            output = torch.stack(outs)
+        else:
+            assert seqlen == 1, "decode steps take one token per branch"
+            pos_dev, t_dev = step_state
+            q_b = xq.view(bsz, H, D)
+            k_b = xk.view(bsz, Hkv, D)
+            v_b = xv.view(bsz, Hkv, D)
+            K.rope_append_kv(q_b, k_b, v_b, cos, sin, pos_dev, self.cache_k, self.cache_k_s,
+                             self.cache_v, self.cache_v_s, self.args.max_seq_len, t_dev)
+            t1 = _tick()
+            output = K.shared_prefix_attn(
+                q_b, self.cache_prompt_k[0], self.cache_prompt_v[0], self.cache_prompt_len,
+                suffix_k=self.cache_k, suffix_v=self.cache_v, suffix_ks=self.cache_k_s, suffix_vs=self.cache_v_s,
+                Smax=self.args.max_seq_len, lens=t_dev, lens_stride=0, cur_k=k_b, cur_v=v_b)
+            output = output.view(bsz, 1, H * D)
+        if PROFILE:
+            t2 = _tick()
+            QKVO_TIME += t1 - t0
+            ATTN_TIME += t2 - t1
+        return self.wo(output, residual=residual)
+
+
+class FeedForward(nn.Module):
+    def __init__(self, dim: int, hidden_dim: int, multiple_of: int, ffn_dim_multiplier: Optional[float]):
+        super().__init__()
+        hidden_dim = int(2 * hidden_dim / 3)
+        if ffn_dim_multiplier is not None:
+            hidden_dim = int(ffn_dim_multiplier * hidden_dim)
+        hidden_dim = multiple_of * ((hidden_dim + multiple_of - 1) // multiple_of)
+
+        self.w1 = LinearQ4_0(dim, hidden_dim, GROUP_SIZE)
+        self.w2 = LinearQ4_0(hidden_dim, dim, GROUP_SIZE)
+        self.w3 = LinearQ4_0(dim, hidden_dim, GROUP_SIZE)
+
+    def forward(self, x, residual=None):
+        global MLP_TIME
+        t0 = _tick()
+        out = self.w2(K.silu_mul(self.w1(x), self.w3(x)), residual=residual)
+        if PROFILE:
+            MLP_TIME += _tick() - t0
+        return out
+
+
+class TransformerBlock(nn.Module):
+    def __init__(self, layer_id: int, args: ModelArgs):
+        super().__init__()
+        self.n_heads = args.n_heads
+        self.dim = args.dim
+        self.head_dim = args.dim // args.n_heads
+        self.attention = Attention(args)
+        self.feed_forward = FeedForward(dim=args.dim, hidden_dim=4 * args.dim, multiple_of=args.multiple_of,
+                                        ffn_dim_multiplier=args.ffn_dim_multiplier)
+        self.layer_id = layer_id
+        self.attention_norm = RMSNorm(args.dim, eps=args.norm_eps)
+        self.ffn_norm = RMSNorm(args.dim, eps=args.norm_eps)
+
+    def forward(self, x, start_pos, freqs_cis, mask, step_state=None):
+        # the residual adds are fused into the epilogues of wo and w2
+        h = self.attention.forward(self.attention_norm(x), start_pos, freqs_cis, mask, residual=x, step_state=step_state)
+        return self.feed_forward.forward(self.ffn_norm(h), residual=h)
+
+
+class Transformer(nn.Module):
+    def __init__(self, params: ModelArgs):
+        super().__init__()
+        self.params = params
+        self.vocab_size = params.vocab_size
+        self.n_layers = params.n_layers
+
+        self.tok_embeddings = nn.Embedding(params.vocab_size, params.dim, device=INIT_DEVICE)
+        self.layers = torch.nn.ModuleList()
+        for layer_id in range(params.n_layers):
+            self.layers.append(TransformerBlock(layer_id, params))
+        self.norm = RMSNorm(params.dim, eps=params.norm_eps)
+        self.output = nn.Linear(params.dim, params.vocab_size, bias=False, device=INIT_DEVICE)
+
+        self.freqs_cis = precompute_freqs_cis(self.params.dim // self.params.n_heads,
+                                              self.params.max_seq_len + self.params.max_prompt_seq_len,
+                                              params.rope_theta)
+        self._rope_tables = None      # (cos, sin) fp16 [T, 64] on the device
+        self._step_state = None       # int32 [2] on the device: (position, suffix index t)
+        self._step_host = None
+
+    # -- helpers -------------------------------------------------------------------------------
+    def _tables(self, device):
+        if self._rope_tables is None or self._rope_tables[0].device != device:
+            fc = self.freqs_cis.to("cpu")
+            cos = fc.real.to(DTYPE).contiguous().to(device)    # rounded to fp16 as the reference does (:193-194)
+            sin = fc.imag.to(DTYPE).contiguous().to(device)
+            self._rope_tables = (cos, sin)
+        return self._rope_tables
+
+    def _set_step(self, device, start_pos: int):
+        """Publish (position, suffix index) to the device for the decode kernels."""
+        if self._step_state is None or self._step_state.device != device:
+            self._step_state = torch.zeros(2, dtype=torch.int32, device=device)
+            self._step_host = torch.zeros(2, dtype=torch.int32).pin_memory() if device.type == "cuda" else torch.zeros(2, dtype=torch.int32)
+        prompt_len = self.layers[0].attention.cache_prompt_len
+        self._step_host[0] = start_pos
+        self._step_host[1] = start_pos - prompt_len
+        self._step_state.copy_(self._step_host, non_blocking=False)
+        return self._step_state[0:1], self._step_state[1:2]
+
+    # -- the hot path ----------------------------------------------------------------------------
+    @torch.inference_mode()
+    def forward(self, tokens: torch.Tensor, start_pos: int):
+        _bsz, seqlen = tokens.shape
+        h = self.tok_embeddings(tokens).to(DTYPE)
+        freqs = self._tables(h.device)
+        step_state = None
+        if start_pos != 0:
+            t = start_pos - self.layers[0].attention.cache_prompt_len
+            assert 0 <= t < self.params.max_seq_len, "suffix cache exhausted"
+            assert _bsz <= self.params.max_batch_size
+            step_state = self._set_step(h.device, start_pos)
+        else:
+            assert seqlen <= self.params.max_prompt_seq_len
+        for layer in self.layers:
+            h = layer(h, start_pos, freqs, None, step_state=step_state)
+        h = self.norm(h)
+        output = self.output(h).to(DTYPE)
+        return output
+
+    def fork(self, origin: int, curr_batch: int, forks: int):
+        """Forks the process, such that kv-cache is copied from origin batch number to all the list of new batches"""
+        for layer in self.layers:
+            layer.attention.fork(origin, curr_batch, forks)
+
+    def resetSeq(self):
+        """Sets all sequence length = 0"""
+        for layer in self.layers:
+            layer.attention.resetSeq()
+
+    def resetTimers(self):
+        global COMP_TIME, DEQ_TIME, QKVO_TIME, ATTN_TIME, MLP_TIME, Q_TIME, DQ_TIME
+        COMP_TIME, DEQ_TIME, QKVO_TIME, ATTN_TIME, MLP_TIME, Q_TIME, DQ_TIME = 0.0, 0.0, 0.0, 0.0, 0.0, 0.0, 0.0
+
+    def printTimers(self):
+        if not PROFILE:
+            print("Timers are off (set spec_mcts_amd.hf_model_q40_kv_shared.PROFILE = True to fill them)")
+            return
+        print("Times: QKVO_TIME, ATTN_TIME, MLP_TIME, Q_TIME, DQ_TIME, DEQ_TIME, COMP_TIME")
+        print("Times:", QKVO_TIME, ATTN_TIME, MLP_TIME, Q_TIME, DQ_TIME, DEQ_TIME, COMP_TIME)
+        print("Measured Sum: ", QKVO_TIME + ATTN_TIME + MLP_TIME)
+
+    # -- sampling loops ----------------------------------------------------------------------------
+    @torch.inference_mode()
+    def generate(self, idx, batch_size, max_new_tokens, temperature=1.0, top_k=32, enc=None):
+        """Flat-batch sampling loop of the reference (hf_model_q40_kv_shared.py:534-613) with one
+        change of execution, not of result: the prompt is prefilled once (B=1) and the branches
+        share its KV, instead of prefilling batch_size identical rows.  temperature == 0.0 selects
+        greedy decoding (hf_model_q40.py:517-519)."""
+        self.resetTimers()
+        self.resetSeq()
+        assert self.params.max_batch_size >= batch_size
+        idx = idx[:1]
+        max_new_tokens = min(max_new_tokens, self.params.max_seq_len)
+        results = torch.zeros(batch_size, max_new_tokens, dtype=torch.int64, device=idx.device)
+        results_len = torch.zeros(batch_size, dtype=torch.int32, device=idx.device)
+        results_mask = results_len == 0
+        curr_pos = 0
+        for num_new_tokens in range(max_new_tokens):
+            if curr_pos == 0:
+                idx_cond = idx if idx.size(1) <= self.params.max_prompt_seq_len else idx[:, -self.params.max_prompt_seq_len:]
+                logits = self(idx_cond, 0)
+                curr_pos += idx_cond.shape[1]
+                logits = logits[:, -1, :].expand(batch_size, -1)
+            else:
+                logits = self(results[:, num_new_tokens - 1: num_new_tokens], curr_pos)
+                curr_pos += 1
+                logits = logits[:, -1, :]
+            if temperature == 0.0:
+                idx_next = K.argmax(logits.contiguous())[:, None]
+            else:
+                logits = logits / temperature
+                v, top_k_idx = torch.topk(logits, top_k)
+                probs = F.softmax(v, dim=-1)
+                sample = torch.multinomial(probs, num_samples=1, replacement=True)
+                idx_next = torch.gather(top_k_idx, 1, sample)
+            results[:, num_new_tokens] = idx_next[:, 0] * results_mask.int()
+            ends = (idx_next[:, 0] == 2)
+            results_len += (~ends).int() * results_mask * 1
+            results_mask = ~((ends) | ~results_mask)
+            if torch.sum(~results_mask) == batch_size:
+                return results[:, :num_new_tokens], results_len
+        return results, results_len

@@ -1,0 +1,273 @@
+"""Operator surface of the MI355X Q4_0 hot path: torch tensors in, torch tensors out, every
+operator a call through the C ABI into a hand-written HIP kernel.
+
+The names and argument meaning mirror the reference's operator file (triton_kernels.py):
+matmul_q40 (:471), triton_deq_int40 (:93), quantize_q40 (:12), dequantize_q40 (:43).  As there,
+inputs are borrowed, outputs are fresh tensors on the input's device, launches are asynchronous on
+the current stream and argument errors are assertions.  There is no CPU or eager fallback: tensors
+must live on the GPU and the library must be built.
+"""
+from __future__ import annotations
+
+import math
+from typing import Dict, Optional, Sequence, Tuple
+
+import torch
+
+from . import _lib
+from ._lib import SMH_EPI_NONE, SMH_EPI_RESIDUAL, SMH_KV_FP16, SMH_KV_NONE, SMH_KV_Q40, check
+from .quant import GROUP_SIZE, quantize_q40_torch
+
+DTYPE_torch = torch.float16
+
+_workspaces: Dict[Tuple[str, int], torch.Tensor] = {}
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _need_gpu(*tensors: torch.Tensor) -> None:
+    for t in tensors:
+        assert t.is_cuda, "spec_mcts_amd kernels need GPU tensors (there is no CPU fallback)"
+
+
+def matmul_workspace(device: torch.device, max_m: int = 16, max_n: int = 0) -> torch.Tensor:
+    """Per-device scratch for the K-split partial sums of the Q4_0 matmul.  Zero-filled once; the
+    kernels leave it zeroed.  Shared by all calls on the device: calls issued on different
+    streams at the same time need their own workspace."""
+    lib = _lib.load()
+    need = lib.smh_q40_matmul_workspace_bytes(int(max_m), int(max_n))
+    key = ("matmul", device.index if device.index is not None else torch.cuda.current_device())
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(need, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+def attn_workspace(device: torch.device, B: int, H: int, P: int) -> torch.Tensor:
+    lib = _lib.load()
+    need = lib.smh_attn_workspace_bytes(int(B), int(H), int(P))
+    key = ("attn", device.index if device.index is not None else torch.cuda.current_device())
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
+# ---------------------------------------------------------------------------------------------
+# Q4_0 matmul
+# ---------------------------------------------------------------------------------------------
+def matmul_q40(a: torch.Tensor, b_w: torch.Tensor, b_s: torch.Tensor, b_shape: Sequence[int],
+               residual: Optional[torch.Tensor] = None, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """c[M,N] = a[M,K] . deq(b_w, b_s)[K,N] in fp16 with fp32 accumulation
+    (reference: triton_kernels.py:471-500).  `residual` ([M,N] fp16) fuses the block's residual
+    add: c = residual + fp16(a . deq)."""
+    lib = _lib.load()
+    assert a.is_contiguous(), "Matrix A must be contiguous"
+    assert a.dtype == torch.float16 and a.dim() == 2
+    M, K = a.shape
+    K_b, N = int(b_shape[0]), int(b_shape[1])
+    assert K == K_b, "Incompatible dimensions"
+    _need_gpu(a, b_w, b_s)
+    assert b_w.is_contiguous() and b_s.is_contiguous()
+    assert b_w.dtype == torch.int8 and b_w.numel() == K * N // 2, "packed weight does not match b_shape"
+    assert b_s.dtype == torch.float16 and b_s.numel() == K * N // 64, "scales do not match b_shape"
+    assert a.data_ptr() % 16 == 0
+    c = out if out is not None else torch.empty((M, N), device=a.device, dtype=DTYPE_torch)
+    assert c.shape == (M, N) and c.is_contiguous() and c.dtype == torch.float16
+    epi = SMH_EPI_NONE
+    if residual is not None:
+        assert residual.shape == (M, N) and residual.is_contiguous() and residual.dtype == torch.float16
+        epi = SMH_EPI_RESIDUAL
+    ws = matmul_workspace(a.device, M, N)
+    check(lib.smh_q40_matmul(a.data_ptr(), M, K, K, b_w.data_ptr(), b_s.data_ptr(), N, c.data_ptr(), N,
+                             epi, _ptr(residual), N, ws.data_ptr(), ws.numel(), _stream()), "smh_q40_matmul")
+    return c
+
+
+# ---------------------------------------------------------------------------------------------
+# Q4_0 codec
+# ---------------------------------------------------------------------------------------------
+def deq_int40(w: torch.Tensor, s: torch.Tensor, group_size: int, shape, ptdtype=DTYPE_torch) -> torch.Tensor:
+    """Q4_0 -> fp16, bit-exact nibble*scale (reference: triton_kernels.py:93-107)."""
+    lib = _lib.load()
+    assert group_size == GROUP_SIZE and ptdtype == torch.float16
+    _need_gpu(w, s)
+    assert w.is_contiguous() and s.is_contiguous() and w.dtype == torch.int8 and s.dtype == torch.float16
+    n_elements = int(math.prod(shape))
+    assert n_elements % 128 == 0 and w.numel() == n_elements // 2 and s.numel() == n_elements // 64
+    out = torch.empty(n_elements, device=w.device, dtype=torch.float16)
+    check(lib.smh_q40_dequant(w.data_ptr(), s.data_ptr(), out.data_ptr(), n_elements // 128, _stream()),
+          "smh_q40_dequant")
+    return out.view(shape)
+
+
+def q_int40(w: torch.Tensor, group_size: int = GROUP_SIZE) -> Tuple[torch.Tensor, torch.Tensor]:
+    """fp16 -> Q4_0 on the GPU with the rounding of the torch quantiser (round-half-even of the fp16
+    quotient), NOT the +0.5-and-truncate of the reference's disabled Triton kernel
+    (triton_kernels.py:134)."""
+    lib = _lib.load()
+    assert group_size == GROUP_SIZE
+    _need_gpu(w)
+    assert w.dtype == torch.float16
+    w = w.contiguous()
+    n = w.numel()
+    assert n % 128 == 0
+    q = torch.empty((n // 128, 64), device=w.device, dtype=torch.int8)
+    s = torch.empty((n // 64, 1), device=w.device, dtype=torch.float16)
+    check(lib.smh_q40_quantize(w.data_ptr(), q.data_ptr(), s.data_ptr(), n // 64, _stream()), "smh_q40_quantize")
+    return q, s
+
+
+def quantize_q40(w: torch.Tensor, group_size: int = GROUP_SIZE) -> Tuple[torch.Tensor, torch.Tensor]:
+    """reference: triton_kernels.py:12-41.  fp16 GPU tensors use the HIP kernel; anything else
+    (checkpoint conversion of bf16/fp32 weights on the host) uses the torch formulation."""
+    if w.is_cuda and w.dtype == torch.float16:
+        return q_int40(w, group_size)
+    return quantize_q40_torch(w, group_size)
+
+
+dequantize_q40 = deq_int40
+triton_deq_int40 = deq_int40      # the reference's name for the same operator
+triton_q_int40 = q_int40
+
+
+# ---------------------------------------------------------------------------------------------
+# small fused ops
+# ---------------------------------------------------------------------------------------------
+def rmsnorm(x: torch.Tensor, weight: torch.Tensor, eps: float) -> torch.Tensor:
+    lib = _lib.load()
+    _need_gpu(x, weight)
+    assert x.is_contiguous() and x.dtype == torch.float16 and weight.dtype == torch.float16
+    dim = x.shape[-1]
+    assert weight.numel() == dim
+    out = torch.empty_like(x)
+    check(lib.smh_rmsnorm(x.data_ptr(), weight.data_ptr(), out.data_ptr(), x.numel() // dim, dim, float(eps),
+                          _stream()), "smh_rmsnorm")
+    return out
+
+
+def silu_mul(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
+    lib = _lib.load()
+    _need_gpu(g, u)
+    assert g.shape == u.shape and g.is_contiguous() and u.is_contiguous()
+    assert g.dtype == torch.float16 and u.dtype == torch.float16
+    out = torch.empty_like(g)
+    check(lib.smh_silu_mul(g.data_ptr(), u.data_ptr(), out.data_ptr(), g.numel(), _stream()), "smh_silu_mul")
+    return out
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """Greedy pick over the last dim of fp16 logits [rows, vocab]; lowest index on ties."""
+    lib = _lib.load()
+    _need_gpu(logits)
+    assert logits.dim() == 2 and logits.dtype == torch.float16 and logits.stride(1) == 1
+    rows, vocab = logits.shape
+    out = torch.empty(rows, device=logits.device, dtype=torch.int64)
+    check(lib.smh_argmax(logits.data_ptr(), rows, vocab, logits.stride(0), out.data_ptr(), _stream()), "smh_argmax")
+    return out
+
+
+def rope(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, pos0: int) -> None:
+    """In-place rotate-half RoPE of q [S,H,128] and k [S,Hkv,128]; token s is at position pos0+s."""
+    lib = _lib.load()
+    _need_gpu(q, k, cos, sin)
+    assert q.is_contiguous() and k.is_contiguous() and q.dtype == torch.float16 and k.dtype == torch.float16
+    S, H, D = q.shape
+    assert k.shape[0] == S and k.shape[2] == D and cos.shape[1] == D // 2 and pos0 + S <= cos.shape[0]
+    assert cos.dtype == torch.float16 and sin.dtype == torch.float16 and cos.is_contiguous() and sin.is_contiguous()
+    check(lib.smh_rope(q.data_ptr(), k.data_ptr(), S, H, k.shape[1], D, cos.data_ptr(), sin.data_ptr(), int(pos0),
+                       _stream()), "smh_rope")
+
+
+def rope_append_kv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                   pos_dev: torch.Tensor, cache_k: Optional[torch.Tensor], cache_ks: Optional[torch.Tensor],
+                   cache_v: Optional[torch.Tensor], cache_vs: Optional[torch.Tensor], Smax: int,
+                   t_dev: Optional[torch.Tensor]) -> None:
+    """Decode-step RoPE of q [B,H,128], k [B,Hkv,128] at position pos_dev[0] (int32 on the device),
+    then Q4_0 append of the rotated k and of v into row t_dev[0] of every branch's suffix cache."""
+    lib = _lib.load()
+    _need_gpu(q, k, v, pos_dev)
+    assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+    assert q.dtype == torch.float16 and k.dtype == torch.float16 and v.dtype == torch.float16
+    assert pos_dev.dtype == torch.int32 and (t_dev is None or t_dev.dtype == torch.int32)
+    B, H, D = q.shape
+    check(lib.smh_rope_append_kv(q.data_ptr(), k.data_ptr(), v.data_ptr(), B, H, k.shape[1], D,
+                                 cos.data_ptr(), sin.data_ptr(), pos_dev.data_ptr(),
+                                 _ptr(cache_k), _ptr(cache_ks), _ptr(cache_v), _ptr(cache_vs), int(Smax), _ptr(t_dev),
+                                 _stream()), "smh_rope_append_kv")
+
+
+def kv_fork(cache: torch.Tensor, cache_s: torch.Tensor, Bmax: int, origin: int, curr: int, forks: int) -> None:
+    """Copy branch `origin`'s Q4_0 cache rows to branches curr..curr+forks-1."""
+    lib = _lib.load()
+    _need_gpu(cache, cache_s)
+    assert cache.is_contiguous() and cache_s.is_contiguous()
+    row_bytes = cache.numel() * cache.element_size() // Bmax
+    row_scales = cache_s.numel() // Bmax
+    check(lib.smh_kv_fork(cache.data_ptr(), cache_s.data_ptr(), Bmax, row_bytes, row_scales, origin, curr, forks,
+                          _stream()), "smh_kv_fork")
+
+
+# ---------------------------------------------------------------------------------------------
+# attention
+# ---------------------------------------------------------------------------------------------
+def shared_prefix_attn(q: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix_v: Optional[torch.Tensor], P: int,
+                       suffix_k: Optional[torch.Tensor] = None, suffix_v: Optional[torch.Tensor] = None,
+                       suffix_ks: Optional[torch.Tensor] = None, suffix_vs: Optional[torch.Tensor] = None,
+                       Smax: int = 0, lens: Optional[torch.Tensor] = None, lens_stride: int = 1,
+                       cur_k: Optional[torch.Tensor] = None, cur_v: Optional[torch.Tensor] = None,
+                       n_kv_heads: Optional[int] = None) -> torch.Tensor:
+    """out[b,h] = softmax(q[b,h] . K_b^T / sqrt(D)) . V_b with K_b = prefix[:P] (shared) ||
+    suffix[b, :lens[b]] || cur_k[b].  The suffix is fp16 [B,Smax,Hkv,D] or Q4_0 (int8 rows +
+    fp16 scales, the model's cache layout); `lens` is int32 on the device."""
+    lib = _lib.load()
+    _need_gpu(q)
+    assert q.is_contiguous() and q.dtype == torch.float16 and q.dim() == 3
+    B, H, D = q.shape
+    if prefix_k is not None:
+        assert prefix_k.is_contiguous() and prefix_v.is_contiguous() and prefix_k.dtype == torch.float16
+        Hkv = prefix_k.shape[-2]
+        assert P <= prefix_k.shape[-3]
+    else:
+        assert P == 0
+        Hkv = n_kv_heads if n_kv_heads is not None else (cur_k.shape[1] if cur_k is not None else H)
+    fmt = SMH_KV_NONE
+    if suffix_k is not None:
+        assert suffix_k.is_contiguous() and suffix_v.is_contiguous() and lens is not None
+        assert lens.is_cuda and lens.dtype == torch.int32
+        if suffix_k.dtype == torch.float16:
+            fmt = SMH_KV_FP16
+        else:
+            assert suffix_k.dtype == torch.int8 and suffix_ks is not None and suffix_vs is not None
+            assert suffix_ks.dtype == torch.float16 and suffix_vs.dtype == torch.float16
+            fmt = SMH_KV_Q40
+    if cur_k is not None:
+        assert cur_k.is_contiguous() and cur_v.is_contiguous() and cur_k.dtype == torch.float16
+    out = torch.empty_like(q)
+    ws = attn_workspace(q.device, B, H, P)
+    check(lib.smh_shared_prefix_attn(q.data_ptr(), out.data_ptr(), B, H, Hkv, D, _ptr(prefix_k), _ptr(prefix_v), int(P),
+                                     fmt, _ptr(suffix_k), _ptr(suffix_v), _ptr(suffix_ks), _ptr(suffix_vs), int(Smax),
+                                     _ptr(lens), int(lens_stride), _ptr(cur_k), _ptr(cur_v),
+                                     ws.data_ptr(), ws.numel(), _stream()), "smh_shared_prefix_attn")
+    return out
+
+
+def prefill_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+    """Causal attention over one prompt: q [S,H,128], k/v [S,Hkv,128] -> [S,H,128]."""
+    lib = _lib.load()
+    _need_gpu(q, k, v)
+    assert q.is_contiguous() and k.is_contiguous() and v.is_contiguous()
+    assert q.dtype == torch.float16 and k.dtype == torch.float16 and v.dtype == torch.float16
+    S, H, D = q.shape
+    out = torch.empty_like(q)
+    check(lib.smh_prefill_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), S, H, k.shape[1], D,
+                               _stream()), "smh_prefill_attn")
+    return out

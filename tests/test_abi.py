@@ -1,0 +1,85 @@
+"""The C-ABI library loads and exports every symbol include/smh.h declares (no GPU needed)."""
+import ctypes
+import os
+import re
+
+import pytest
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def _declared():
+    text = open(os.path.join(ROOT, "include", "smh.h")).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(smh_[a-z0-9_]+)\s*\(", text)))
+
+
+def test_header_symbols_are_exported_and_bound():
+    from spec_mcts_amd import _lib
+    names = _declared()
+    assert len(names) >= 15
+    lib = _lib.load()
+    for n in names:
+        assert hasattr(lib, n), f"{n} declared in smh.h but not exported by libsmh.so"
+        assert n in _lib.SIGNATURES, f"{n} has no ctypes signature in spec_mcts_amd/_lib.py"
+    assert sorted(_lib.SIGNATURES) == names
+    assert lib.smh_version() == 1
+
+
+def test_argument_errors_are_reported_without_a_gpu():
+    from spec_mcts_amd import _lib
+    lib = _lib.load()
+    # N not a multiple of 128 is rejected before anything touches the device
+    st = lib.smh_q40_gemv(None, 1, 64, 64, None, None, 100, None, 100, 0, None, 0, None, 0, None)
+    assert st < 0 and b"multiple of 128" in lib.smh_last_error_string()
+    st = lib.smh_q40_quantize(None, None, None, 3, None)
+    assert st < 0 and b"even" in lib.smh_last_error_string()
+    with pytest.raises(_lib.SmhError):
+        _lib.check(st, "smh_q40_quantize")
+    assert lib.smh_q40_matmul_workspace_bytes(16, 4096) >= 16384 + 16 * 131072 * 4
+    assert lib.smh_attn_workspace_bytes(64, 32, 1024) >= 32 * 64 * 32 * 130 * 4
+
+
+def test_host_quantiser_matches_oracle():
+    """spec_mcts_amd.quant (the converter's quantiser) against the oracle on the host"""
+    import torch
+    from oracle import q40_oracle as O
+    from spec_mcts_amd import quant
+    g = torch.Generator().manual_seed(5)
+    v = (torch.randn((256, 128), generator=g) * 0.02).to(torch.float16)
+    w, s, shp = quant.quantize_linear_weight(v)
+    w2, s2, shp2 = O.quantize_weight(v)
+    assert torch.equal(w, w2) and torch.equal(s, s2) and shp == shp2
+    assert torch.equal(quant.dequantize_q40_torch(w, s, 64, (128, 256)), O.dequantize_q40(w, s, 64, (128, 256)))
+    vb = v.to(torch.bfloat16)
+    wb, sb = quant.quantize_q40_torch(vb.t(), 64)
+    wb2, sb2 = O.quantize_q40(vb.t(), 64)
+    assert torch.equal(wb, wb2) and torch.equal(sb, sb2)
+
+
+def test_converter_and_loader_host_logic():
+    import torch
+    from spec_mcts_amd import fp16_to_int4 as C
+    from spec_mcts_amd.load_q40 import load_q40
+    from spec_mcts_amd import ModelArgs
+    g = torch.Generator().manual_seed(6)
+    hf = {"model.embed_tokens.weight": torch.randn((320, 256), generator=g).half(),
+          "model.norm.weight": torch.ones(256).half(), "lm_head.weight": torch.randn((320, 256), generator=g).half()}
+    for name, shape in (("self_attn.q_proj", (256, 256)), ("self_attn.k_proj", (256, 256)), ("self_attn.v_proj", (256, 256)),
+                        ("self_attn.o_proj", (256, 256)), ("mlp.gate_proj", (768, 256)), ("mlp.down_proj", (256, 768)),
+                        ("mlp.up_proj", (768, 256))):
+        hf[f"model.layers.0.{name}.weight"] = (torch.randn(shape, generator=g) * 0.02).half()
+    hf["model.layers.0.input_layernorm.weight"] = torch.ones(256).half()
+    hf["model.layers.0.post_attention_layernorm.weight"] = torch.ones(256).half()
+    sd = C.quantize_state_dict(C.remap_state_dict(hf))
+    assert "layers.0.attention.wq.w" in sd and "layers.0.feed_forward.w2.shape" in sd and "tok_embeddings.weight" in sd
+    assert "layers.0.attention.wq.weight" not in sd and tuple(sd["layers.0.feed_forward.w1.shape"]) == (768, 256)
+    args = ModelArgs(dim=256, n_layers=1, n_heads=2, vocab_size=320, multiple_of=128, max_batch_size=2, max_seq_len=4,
+                     max_prompt_seq_len=8)
+    model = load_q40(sd, args, device="cpu")
+    lin = model.layers[0].feed_forward.w2
+    assert tuple(lin.shape) == (256, 768) and lin.w.shape == (768 * 256 // 128, 64) and lin.s.numel() == 768 * 256 // 64
+    assert model.tok_embeddings.weight.dtype == torch.float16 and model.output.weight.shape == (320, 256)
+    # the hot path refuses to run without a GPU instead of falling back
+    with pytest.raises(AssertionError):
+        model(torch.zeros((1, 4), dtype=torch.int64), 0)

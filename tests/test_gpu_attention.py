@@ -1,0 +1,127 @@
+"""GPU parity of the shared-prefix decode attention and the causal prefill attention against the
+oracle (explicit fp32 softmax attention).  Tolerance: 1e-2 relative + 2e-3 absolute."""
+import pytest
+import torch
+
+from oracle import q40_oracle as O
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-2, 2e-3
+
+
+def _g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+def _check(got, want):
+    got, want = got.float().cpu(), want.float()
+    err = (got - want).abs()
+    tol = ATOL + RTOL * want.abs()
+    assert bool((err <= tol).all()), f"max err {err.max():.4e}, worst excess {(err - tol).max():.4e}"
+
+
+def _inputs(B, H, Hkv, D, P, S, seed, std=1.0):
+    g = _g(seed)
+    q = (torch.randn((B, H, D), generator=g) * std).to(torch.float16)
+    pk = (torch.randn((max(P, 1), Hkv, D), generator=g) * std).to(torch.float16)
+    pv = (torch.randn((max(P, 1), Hkv, D), generator=g) * std).to(torch.float16)
+    sk = (torch.randn((B, max(S, 1), Hkv, D), generator=g) * std).to(torch.float16)
+    sv = (torch.randn((B, max(S, 1), Hkv, D), generator=g) * std).to(torch.float16)
+    lens = torch.randint(0, S + 1, (B,), generator=g, dtype=torch.int32)
+    return q, pk, pv, sk, sv, lens
+
+
+def test_config2_fp16_suffix():
+    """B=64 branches, 32 heads, D=128, shared 1024-token prefix, ragged suffix 0..256, seed 2"""
+    from spec_mcts_amd import kernels as K
+    B, H, D, P, S = 64, 32, 128, 1024, 256
+    q, pk, pv, sk, sv, lens = _inputs(B, H, H, D, P, S, 2)
+    lens[0] = 0; lens[1] = S
+    got = K.shared_prefix_attn(q.cuda(), pk.cuda(), pv.cuda(), P, suffix_k=sk.cuda(), suffix_v=sv.cuda(),
+                               Smax=S, lens=lens.cuda(), lens_stride=1)
+    want = O.shared_prefix_attention(q, pk, pv, sk, sv, lens.tolist())
+    _check(got, want)
+
+
+def test_config2_q40_suffix_as_the_model_stores_it():
+    from spec_mcts_amd import kernels as K
+    B, H, D, P, S = 64, 32, 128, 1024, 256
+    q, pk, pv, sk, sv, lens = _inputs(B, H, H, D, P, S, 3)
+    wk, sks = O.quantize_q40(sk, 64)
+    wv, svs = O.quantize_q40(sv, 64)
+    sk_deq = O.dequantize_q40(wk, sks, 64, sk.shape)
+    sv_deq = O.dequantize_q40(wv, svs, 64, sv.shape)
+    got = K.shared_prefix_attn(q.cuda(), pk.cuda(), pv.cuda(), P, suffix_k=wk.cuda(), suffix_v=wv.cuda(),
+                               suffix_ks=sks.cuda(), suffix_vs=svs.cuda(), Smax=S, lens=lens.cuda(), lens_stride=1)
+    want = O.shared_prefix_attention(q, pk, pv, sk_deq, sv_deq, lens.tolist())
+    _check(got, want)
+
+
+@pytest.mark.parametrize("B,H,Hkv,P,S", [(1, 2, 2, 1, 0), (3, 8, 2, 100, 5), (100, 8, 1, 512, 3), (17, 4, 4, 33, 9),
+                                         (5, 2, 2, 0, 7), (2, 64, 8, 2048, 4)])
+def test_shapes_gqa_empty_prefix_and_current_token(B, H, Hkv, P, S):
+    from spec_mcts_amd import kernels as K
+    D = 128
+    q, pk, pv, sk, sv, lens = _inputs(B, H, Hkv, D, P, S, 10 + B)
+    g = _g(99)
+    ck = torch.randn((B, Hkv, D), generator=g).to(torch.float16)
+    cv = torch.randn((B, Hkv, D), generator=g).to(torch.float16)
+    # the new token is one more exact row after each branch's suffix
+    sk2 = torch.cat((sk, torch.zeros_like(sk[:, :1])), 1); sv2 = torch.cat((sv, torch.zeros_like(sv[:, :1])), 1)
+    for b in range(B):
+        sk2[b, lens[b]] = ck[b]; sv2[b, lens[b]] = cv[b]
+    want = O.shared_prefix_attention(q, pk[:P], pv[:P], sk2, sv2, (lens + 1).tolist())
+    got = K.shared_prefix_attn(q.cuda(), pk.cuda() if P else None, pv.cuda() if P else None, P,
+                               suffix_k=sk.cuda(), suffix_v=sv.cuda(), Smax=max(S, 1), lens=lens.cuda(), lens_stride=1,
+                               cur_k=ck.cuda(), cur_v=cv.cuda(), n_kv_heads=Hkv)
+    _check(got, want)
+
+
+def test_uniform_length_from_device_counter():
+    """lens_stride 0: every branch uses the same device-side step counter, as the model does"""
+    from spec_mcts_amd import kernels as K
+    B, H, D, P, S = 6, 4, 128, 64, 8
+    q, pk, pv, sk, sv, _ = _inputs(B, H, H, D, P, S, 30)
+    t = torch.tensor([5], dtype=torch.int32).cuda()
+    got = K.shared_prefix_attn(q.cuda(), pk.cuda(), pv.cuda(), P, suffix_k=sk.cuda(), suffix_v=sv.cuda(), Smax=S,
+                               lens=t, lens_stride=0)
+    _check(got, O.shared_prefix_attention(q, pk, pv, sk, sv, [5] * B))
+
+
+def test_special_cases():
+    from spec_mcts_amd import kernels as K
+    B, H, D, P, S = 4, 2, 128, 96, 8
+    q, pk, pv, sk, sv, lens = _inputs(B, H, H, D, P, S, 31)
+    lens[:] = S
+    # q = 0 -> uniform weights -> mean of all V rows
+    got = K.shared_prefix_attn(torch.zeros_like(q).cuda(), pk.cuda(), pv.cuda(), P, suffix_k=sk.cuda(),
+                               suffix_v=sv.cuda(), Smax=S, lens=lens.cuda(), lens_stride=1).cpu()
+    for b in range(B):
+        assert torch.allclose(got[b].float(), torch.cat((pv, sv[b]), 0).float().mean(0), atol=2e-3)
+    # one dominant prefix key -> its V row
+    pk2 = pk.clone(); pk2[70] = 0; pk2[70, :, 0] = 200.0
+    q2 = torch.zeros_like(q); q2[..., 0] = 50.0
+    got = K.shared_prefix_attn(q2.cuda(), pk2.cuda(), pv.cuda(), P).cpu()
+    assert torch.allclose(got[0].float(), pv[70].float(), atol=2e-3)
+    # split invariance: moving the tail of the prefix into every branch's suffix changes nothing
+    full = K.shared_prefix_attn(q.cuda(), pk.cuda(), pv.cuda(), P, suffix_k=sk.cuda(), suffix_v=sv.cuda(), Smax=S,
+                                lens=lens.cuda(), lens_stride=1).cpu()
+    cut = 40
+    sk2 = torch.cat((pk[cut:][None].expand(B, -1, -1, -1), sk), 1).contiguous()
+    sv2 = torch.cat((pv[cut:][None].expand(B, -1, -1, -1), sv), 1).contiguous()
+    l2 = (lens + P - cut).to(torch.int32)
+    moved = K.shared_prefix_attn(q.cuda(), pk[:cut].contiguous().cuda(), pv[:cut].contiguous().cuda(), cut,
+                                 suffix_k=sk2.cuda(), suffix_v=sv2.cuda(), Smax=S + P - cut, lens=l2.cuda(),
+                                 lens_stride=1).cpu()
+    assert torch.allclose(full.float(), moved.float(), atol=2e-3, rtol=1e-2)
+
+
+@pytest.mark.parametrize("S,H,Hkv", [(1, 2, 2), (19, 4, 2), (512, 32, 32)])
+def test_prefill_causal(S, H, Hkv):
+    from spec_mcts_amd import kernels as K
+    g = _g(40 + S)
+    q = torch.randn((S, H, 128), generator=g).to(torch.float16)
+    k = torch.randn((S, Hkv, 128), generator=g).to(torch.float16)
+    v = torch.randn((S, Hkv, 128), generator=g).to(torch.float16)
+    got = K.prefill_attn(q.cuda(), k.cuda(), v.cuda())
+    _check(got, O.causal_attention(q, k, v))

@@ -1,0 +1,132 @@
+"""GPU parity of the fused Q4_0 dequant+matmul (GEMV for M<=16, LDS/MFMA GEMM above) against the
+oracle.  Tolerance is the one the task states for fp16 outputs: 1e-2 relative + 2e-3 absolute."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import q40_oracle as O
+
+pytestmark = pytest.mark.gpu
+RTOL, ATOL = 1e-2, 2e-3
+
+
+def _weights(N, K, seed, std=0.02):
+    g = torch.Generator().manual_seed(seed)
+    v = (torch.randn((N, K), generator=g) * std).to(torch.float16)
+    w, s, _ = O.quantize_weight(v)
+    return w, s
+
+
+def _acts(M, K, seed):
+    return torch.randn((M, K), generator=torch.Generator().manual_seed(seed)).to(torch.float16)
+
+
+def _check(got, want):
+    got, want = got.float().cpu(), want.float()
+    err = (got - want).abs()
+    tol = ATOL + RTOL * want.abs()
+    assert bool((err <= tol).all()), f"max err {err.max():.4e}, worst excess {(err - tol).max():.4e}"
+
+
+def test_config0_single_linear():
+    """x[1,4096] . W[11008,4096]^T, seed 0: dequant bit-exact, output within tolerance"""
+    from spec_mcts_amd import kernels as K
+    N, Kd = 11008, 4096
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((1, Kd), generator=g).to(torch.float16)
+    v = (torch.randn((N, Kd), generator=g) * 0.02).to(torch.float16)
+    w, s, shp = O.quantize_weight(v)
+    wd, sd_ = w.cuda(), s.cuda()
+    deq = K.deq_int40(wd, sd_, 64, (Kd, N))
+    assert torch.equal(deq.cpu().view(torch.int16), O.dequantize_q40(w, s, 64, (Kd, N)).view(torch.int16))
+    y = K.matmul_q40(x.cuda(), wd, sd_, (Kd, N))
+    assert y.shape == (1, N) and y.dtype == torch.float16
+    _check(y, O.matmul_q40(x, w, s, (Kd, N)))
+    _check(y, O.linear_q40_cpu_path(x, w, s, (N, Kd)))
+
+
+SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008), (32128, 4096)]   # 32016 padded to 251*128
+
+
+@pytest.mark.parametrize("idx", range(len(SHAPES)))
+def test_config1_sweep(idx):
+    from spec_mcts_amd import kernels as K
+    N, Kd = SHAPES[idx]
+    w, s = _weights(N, Kd, 1000 + idx)
+    wd, sd_ = w.cuda(), s.cuda()
+    deq = O.dequantize_q40(w, s, 64, (Kd, N)).float()
+    for M in (1, 10, 100):
+        a = _acts(M, Kd, 2000 + 10 * idx + M)
+        got = K.matmul_q40(a.cuda(), wd, sd_, (Kd, N))
+        want = (a.float() @ deq).to(torch.float16)
+        _check(got, want)
+        # a second launch reuses the self-cleaning workspace and must give the same bits
+        again = K.matmul_q40(a.cuda(), wd, sd_, (Kd, N))
+        assert torch.equal(got, again)
+
+
+@pytest.mark.parametrize("M", [1, 3, 16, 17, 100, 130, 300])
+def test_one_hot_rows_are_bit_exact(M):
+    """x = e_k returns row k of the dequantised matrix exactly (covers every column-block boundary)"""
+    from spec_mcts_amd import kernels as K
+    N, Kd = 384, 512
+    w, s = _weights(N, Kd, 7)
+    deq = O.dequantize_q40(w, s, 64, (Kd, N))
+    ks = torch.randint(0, Kd, (M,), generator=torch.Generator().manual_seed(M))
+    ks[0] = 0
+    ks[-1] = Kd - 1
+    a = torch.zeros((M, Kd), dtype=torch.float16)
+    a[torch.arange(M), ks] = 1.0
+    got = K.matmul_q40(a.cuda(), w.cuda(), s.cuda(), (Kd, N)).cpu()
+    assert torch.equal(got.view(torch.int16), deq[ks].view(torch.int16))
+    zero = K.matmul_q40(torch.zeros((M, Kd), dtype=torch.float16).cuda(), w.cuda(), s.cuda(), (Kd, N))
+    assert bool((zero == 0).all())
+
+
+@pytest.mark.parametrize("M,N,Kd", [(2, 128, 8), (5, 256, 40), (16, 128, 72), (40, 256, 200), (129, 128, 1000)])
+def test_ragged_k_and_small_shapes(M, N, Kd):
+    """K not a multiple of the 32-row step, single column block, M around the tile sizes"""
+    from spec_mcts_amd import kernels as K
+    w, s = _weights(N, Kd, 11, std=0.05)
+    a = _acts(M, Kd, 12)
+    got = K.matmul_q40(a.cuda(), w.cuda(), s.cuda(), (Kd, N))
+    _check(got, O.matmul_q40(a, w, s, (Kd, N)))
+
+
+@pytest.mark.parametrize("M", [4, 100])
+def test_residual_epilogue(M):
+    from spec_mcts_amd import kernels as K
+    N, Kd = 512, 1024
+    w, s = _weights(N, Kd, 13)
+    a = _acts(M, Kd, 14)
+    r = _acts(M, N, 15)
+    got = K.matmul_q40(a.cuda(), w.cuda(), s.cuda(), (Kd, N), residual=r.cuda())
+    want = r + O.matmul_q40(a, w, s, (Kd, N))            # fp16 add of the fp16 product, as h + wo(..)
+    _check(got, want)
+
+
+def test_linearity_at_full_size():
+    """size-independent property at a BASELINE shape: f(x1) + f(x2) ~ f(x1 + x2), f(2x) = 2 f(x) exactly"""
+    from spec_mcts_amd import kernels as K
+    N, Kd = 11008, 4096
+    w, s = _weights(N, Kd, 16)
+    wd, sd_ = w.cuda(), s.cuda()
+    x1, x2 = _acts(10, Kd, 17).cuda(), _acts(10, Kd, 18).cuda()
+    y1 = K.matmul_q40(x1, wd, sd_, (Kd, N)).float()
+    y2 = K.matmul_q40(x2, wd, sd_, (Kd, N)).float()
+    y12 = K.matmul_q40((x1.float() * 0.5 + x2.float() * 0.5).half(), wd, sd_, (Kd, N)).float()
+    assert torch.allclose(y12, 0.5 * (y1 + y2), rtol=RTOL, atol=2 * ATOL)
+    yd = K.matmul_q40(x1 * 2, wd, sd_, (Kd, N))
+    assert torch.equal(yd, (K.matmul_q40(x1, wd, sd_, (Kd, N)) * 2))      # scaling by 2 is exact in fp16/fp32
+
+
+def test_argument_errors():
+    from spec_mcts_amd import kernels as K
+    w, s = _weights(128, 64, 19)
+    a = _acts(2, 64, 20).cuda()
+    with pytest.raises(AssertionError):
+        K.matmul_q40(a, w.cuda(), s.cuda(), (32, 128))                    # K mismatch
+    with pytest.raises(AssertionError):
+        K.matmul_q40(a.t().contiguous().t(), w.cuda(), s.cuda(), (64, 128))  # non-contiguous A
+    with pytest.raises(AssertionError):
+        K.matmul_q40(a.cpu(), w, s, (64, 128))                            # no CPU fallback

@@ -1,0 +1,99 @@
+"""End-to-end parity of the drop-in model (prefill, shared-prefix decode, fork, greedy tokens)
+against the oracle's restatement of hf_model_q40_kv_shared.Transformer on small random-init models."""
+import pytest
+import torch
+
+from oracle import q40_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _build(cfg, seed, std=0.05):
+    from spec_mcts_amd import ModelArgs
+    from spec_mcts_amd.load_q40 import load_q40
+    oargs = O.OracleArgs(**cfg)
+    sd = O.random_q40_state_dict(oargs, seed=seed, std=std)
+    model = load_q40(dict(sd), ModelArgs(**cfg), device="cuda:0")
+    return oargs, sd, model
+
+
+def _greedy_gpu(model, prompt, batch, steps, fork_at=None):
+    """prefill at B=1, branches share the prompt; optional fork of branch 0 into the last row"""
+    from spec_mcts_amd import kernels as K
+    model.resetSeq()
+    dev = "cuda:0"
+    P = prompt.shape[1]
+    logits = model(prompt.to(dev), 0)[:, -1]
+    out = torch.zeros((batch, steps), dtype=torch.int64, device=dev)
+    out[:, 0] = K.argmax(logits.contiguous())[0]
+    live = batch if fork_at is None else batch - 1
+    for s in range(1, steps):
+        if fork_at is not None and s == fork_at:
+            model.fork(0, live, 1)
+            out[live] = out[0]
+            live = batch
+        lg = model(out[:live, s - 1:s], P + s - 1)[:, -1]
+        out[:live, s] = K.argmax(lg.contiguous())
+    return out.cpu()
+
+
+SMALL = dict(dim=256, n_layers=2, n_heads=2, vocab_size=320, multiple_of=128, max_batch_size=4, max_seq_len=24,
+             max_prompt_seq_len=32)
+GQA = dict(dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=384, multiple_of=128, max_batch_size=4,
+           max_seq_len=16, max_prompt_seq_len=48)
+
+
+@pytest.mark.parametrize("cfg,seed", [(SMALL, 30), (GQA, 31)])
+def test_prefill_and_decode_logits(cfg, seed):
+    oargs, sd, model = _build(cfg, seed)
+    oracle = O.OracleTransformer(oargs, sd, dense=True)
+    prompt = torch.randint(0, cfg["vocab_size"], (1, 21), generator=torch.Generator().manual_seed(seed + 100))
+    want = oracle.forward(prompt, 0)
+    got = model(prompt.cuda(), 0).cpu()
+    assert got.shape == want.shape and got.dtype == torch.float16
+    assert torch.allclose(got.float(), want.float(), rtol=2e-2, atol=2e-2)
+    nxt = want[:, -1].float().argmax(-1, keepdim=True).expand(3, 1).contiguous()
+    oracle.fork(0, 1, 2)
+    want2 = oracle.forward(nxt, 21)
+    got2 = model(nxt.cuda(), 21).cpu()
+    assert torch.allclose(got2.float(), want2.float(), rtol=2e-2, atol=2e-2)
+    assert torch.equal(got2[0], got2[1]) and torch.equal(got2[0], got2[2])     # identical branches, identical rows
+
+
+@pytest.mark.parametrize("cfg,seed", [(SMALL, 32), (GQA, 33)])
+def test_greedy_tokens_match_oracle(cfg, seed):
+    oargs, sd, model = _build(cfg, seed)
+    oracle = O.OracleTransformer(oargs, sd, dense=True)
+    prompt = torch.randint(0, cfg["vocab_size"], (1, 17), generator=torch.Generator().manual_seed(seed + 100))
+    steps = 12
+    want, margins = oracle.greedy(prompt, 3, steps)
+    got = _greedy_gpu(model, prompt, 3, steps)
+    print("oracle top-1/top-2 margins:", ["%.3f" % m for m in margins])
+    assert torch.equal(got, want), f"tokens differ; oracle margins {margins}"
+
+
+def test_fork_mid_sequence():
+    """fork copies the suffix KV: the forked branch continues exactly like its origin"""
+    oargs, sd, model = _build(SMALL, 34)
+    prompt = torch.randint(0, SMALL["vocab_size"], (1, 9), generator=torch.Generator().manual_seed(134))
+    got = _greedy_gpu(model, prompt, 3, 10, fork_at=5)
+    assert torch.equal(got[0], got[1]) and torch.equal(got[0], got[2])
+    oracle = O.OracleTransformer(oargs, sd, dense=True)
+    want, _ = oracle.greedy(prompt, 1, 10)
+    assert torch.equal(got[0], want[0])
+
+
+def test_generate_greedy_and_sampling_api():
+    oargs, sd, model = _build(SMALL, 35)
+    prompt = torch.randint(3, SMALL["vocab_size"], (1, 8), generator=torch.Generator().manual_seed(135)).cuda()
+    res, lens = model.generate(prompt, 3, 6, temperature=0.0)
+    assert res.shape[0] == 3 and res.dtype == torch.int64 and lens.dtype == torch.int32
+    oracle = O.OracleTransformer(oargs, sd, dense=True)
+    want, _ = oracle.greedy(prompt.cpu(), 3, 6)
+    n = res.shape[1]
+    stop = (want[0] == 2).nonzero()
+    if len(stop) == 0:
+        assert torch.equal(res.cpu(), want[:, :n])
+    torch.manual_seed(0)
+    res2, _ = model.generate(prompt, 2, 4, temperature=0.8, top_k=8)
+    assert res2.shape[0] == 2 and int(res2.max()) < SMALL["vocab_size"]

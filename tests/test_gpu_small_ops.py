@@ -1,0 +1,109 @@
+"""GPU parity of the small fused kernels (RMSNorm, SiLU*up, argmax, RoPE + Q4_0 KV append, fork)."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import q40_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def _g(seed):
+    return torch.Generator().manual_seed(seed)
+
+
+@pytest.mark.parametrize("rows,dim", [(1, 4096), (10, 4096), (100, 4096), (3, 8192), (2, 256)])
+def test_rmsnorm(rows, dim):
+    from spec_mcts_amd import kernels as K
+    x = torch.randn((rows, dim), generator=_g(1)).to(torch.float16)
+    wt = (1 + 0.1 * torch.randn(dim, generator=_g(2))).to(torch.float16)
+    got = K.rmsnorm(x.cuda(), wt.cuda(), 1e-5).cpu()
+    want = O.rmsnorm(x, wt, 1e-5)
+    # same cast points; the only freedom is the order of the fp32 sum of squares (<= 1 fp16 ulp)
+    assert torch.allclose(got.float(), want.float(), rtol=2e-3, atol=1e-4)
+    assert (got != want).float().mean() < 0.01
+
+
+def test_silu_mul():
+    from spec_mcts_amd import kernels as K
+    a = (torch.randn(100 * 11008 + 3, generator=_g(3)) * 2).to(torch.float16)
+    b = torch.randn(100 * 11008 + 3, generator=_g(4)).to(torch.float16)
+    got = K.silu_mul(a.cuda(), b.cuda()).cpu()
+    want = O.silu_mul(a, b)
+    assert torch.allclose(got.float(), want.float(), rtol=2e-3, atol=1e-4)
+    assert (got != want).float().mean() < 0.01
+
+
+def test_argmax_lowest_index_on_ties():
+    from spec_mcts_amd import kernels as K
+    logits = torch.randn((100, 32016), generator=_g(5)).to(torch.float16)
+    logits[0, 31000] = 9.0; logits[0, 17] = 9.0; logits[0, 5000] = 9.0     # three-way tie -> 17
+    logits[1, 32015] = 50.0                                                  # last column
+    logits[2] = 0.25                                                         # all equal -> 0
+    got = K.argmax(logits.cuda()).cpu()
+    assert got.dtype == torch.int64
+    assert torch.equal(got, logits.float().argmax(-1))
+    assert got[0] == 17 and got[1] == 32015 and got[2] == 0
+    # strided rows (a [B,1,V] slice of a bigger buffer)
+    big = torch.randn((4, 40000), generator=_g(6)).to(torch.float16).cuda()
+    assert torch.equal(K.argmax(big[:, :32016]).cpu(), big[:, :32016].float().argmax(-1).cpu())
+
+
+def test_rope_prefill_bit_exact():
+    from spec_mcts_amd import kernels as K
+    S, H, Hkv, D = 37, 8, 2, 128
+    fc = O.precompute_freqs_cis(D, 64, 1e6)
+    q = torch.randn((1, S, H, D), generator=_g(7)).to(torch.float16)
+    k = torch.randn((1, S, Hkv, D), generator=_g(8)).to(torch.float16)
+    qe, ke = O.apply_rotary_emb(q, k, fc[3:3 + S])
+    cos, sin = fc.real.to(torch.float16).contiguous().cuda(), fc.imag.to(torch.float16).contiguous().cuda()
+    qd, kd = q[0].clone().cuda(), k[0].clone().cuda()
+    K.rope(qd, kd, cos, sin, 3)
+    assert torch.equal(qd.cpu().view(torch.int16), qe[0].view(torch.int16))
+    assert torch.equal(kd.cpu().view(torch.int16), ke[0].view(torch.int16))
+
+
+def test_rope_append_kv_bit_exact():
+    """decode step: rotate q,k at position pos; store Q4_0(k_rot), Q4_0(v) in row t of each branch"""
+    from spec_mcts_amd import kernels as K
+    B, H, Hkv, D, Smax, Bmax = 5, 8, 2, 128, 6, 7
+    pos, t = 21, 4
+    fc = O.precompute_freqs_cis(D, 64, 1e6)
+    q = torch.randn((B, 1, H, D), generator=_g(9)).to(torch.float16)
+    k = torch.randn((B, 1, Hkv, D), generator=_g(10)).to(torch.float16)
+    v = torch.randn((B, 1, Hkv, D), generator=_g(11)).to(torch.float16)
+    v[0, 0, 0, :64] = 0                                           # an all-zero group
+    qe, ke = O.apply_rotary_emb(q, k, fc[pos:pos + 1])
+    cos, sin = fc.real.to(torch.float16).contiguous().cuda(), fc.imag.to(torch.float16).contiguous().cuda()
+    rows = Bmax * Smax * Hkv
+    ck = torch.zeros((rows, 64), dtype=torch.int8).cuda(); cks = torch.zeros((rows * 2, 1), dtype=torch.float16).cuda()
+    cv = torch.zeros((rows, 64), dtype=torch.int8).cuda(); cvs = torch.zeros((rows * 2, 1), dtype=torch.float16).cuda()
+    qd, kd, vd = q[:, 0].clone().cuda(), k[:, 0].clone().cuda(), v[:, 0].clone().cuda()
+    state = torch.tensor([pos, t], dtype=torch.int32).cuda()
+    K.rope_append_kv(qd, kd, vd, cos, sin, state[0:1], ck, cks, cv, cvs, Smax, state[1:2])
+    assert torch.equal(qd.cpu().view(torch.int16), qe[:, 0].view(torch.int16))
+    assert torch.equal(kd.cpu().view(torch.int16), ke[:, 0].view(torch.int16))
+    wk, sk = O.quantize_q40(ke[:, 0], 64)                          # [B*Hkv, 64], [B*Hkv*2, 1]
+    wv, sv = O.quantize_q40(v[:, 0], 64)
+    ck4 = ck.cpu().view(Bmax, Smax, Hkv, 64); cks4 = cks.cpu().view(Bmax, Smax, Hkv, 2)
+    cv4 = cv.cpu().view(Bmax, Smax, Hkv, 64); cvs4 = cvs.cpu().view(Bmax, Smax, Hkv, 2)
+    assert torch.equal(ck4[:B, t], wk.view(B, Hkv, 64)) and torch.equal(cv4[:B, t], wv.view(B, Hkv, 64))
+    assert torch.equal(cks4[:B, t].view(torch.int16), sk.view(B, Hkv, 2).view(torch.int16))
+    assert torch.equal(cvs4[:B, t].view(torch.int16), sv.view(B, Hkv, 2).view(torch.int16))
+    # nothing else was touched
+    ck4[:B, t] = 0; cv4[:B, t] = 0
+    assert not ck4.any() and not cv4.any()
+
+
+def test_kv_fork_copies_rows():
+    from spec_mcts_amd import kernels as K
+    Bmax, Smax, Hkv = 6, 4, 2
+    rows = Bmax * Smax * Hkv
+    c = torch.randint(-128, 127, (rows, 64), generator=_g(12), dtype=torch.int8)
+    s = torch.randn((rows * 2, 1), generator=_g(13)).to(torch.float16)
+    cd, sd_ = c.clone().cuda(), s.clone().cuda()
+    K.kv_fork(cd, sd_, Bmax, 1, 3, 2)
+    want_c = c.view(Bmax, -1).clone(); want_s = s.view(Bmax, -1).clone()
+    want_c[3:5] = want_c[1]; want_s[3:5] = want_s[1]
+    assert torch.equal(cd.cpu().view(Bmax, -1), want_c)
+    assert torch.equal(sd_.cpu().view(Bmax, -1).view(torch.int16), want_s.view(torch.int16))
