@@ -1,0 +1,234 @@
+#!/usr/bin/env python3
+"""Benchmark of the Q4_0 CodeLlama-7B-architecture decode hot path on one MI355X.
+
+Workload (BASELINE.json configs[3]): random-init 7B architecture (32 layers, dim 4096, 32 heads,
+FFN 11008, vocab 32016), weights ~N(0,0.02) in Q4_0, fp16 embeddings and lm_head; one 512-token
+prompt prefilled once, then greedy decode with B = 1 / 10 / 100 branches sharing the prompt KV.
+A "step" is one decode step (one new token per branch) through all layers, lm_head and argmax.
+
+Prints ONE JSON line.  `value` is decode tokens/s at B=100 (all three batch sizes are in
+`by_batch`); `roofline` describes the dominant kernel, the Q4_0 GEMV, timed live with HIP events
+over one decode step's worth of weight matrices (224 distinct matrices, 3.44 GB, far larger than
+the 256 MB Infinity Cache); `cpu_baseline` is the reference's CPU path (torch dequantise +
+F.linear per linear, explicit softmax attention) timed on this box's host cores on one layer and
+scaled to the model.
+"""
+from __future__ import annotations
+
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+if ROOT not in sys.path:
+    sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
+PROMPT_LEN = 512
+BATCHES = (1, 10, 100)
+
+
+def q40_bytes(M, N, K):
+    """algorithmic bytes of one Q4_0 matmul: packed nibbles + fp16 scales + activations + outputs"""
+    return N * K // 2 + 2 * N * K // 64 + 2 * M * K + 2 * M * N
+
+
+def build_model(torch, args_kw, seed):
+    """Random-init Q4_0 model generated on the GPU (the host cannot hold or quantise 7B quickly)."""
+    from spec_mcts_amd import ModelArgs, Transformer, kernels as K
+    dev = torch.device("cuda:0")
+    g = torch.Generator(device=dev).manual_seed(seed)
+    params = ModelArgs(**args_kw)
+    model = Transformer(params)
+    sd = {"tok_embeddings.weight": (torch.randn((params.vocab_size, params.dim), device=dev, generator=g) * 0.02).half(),
+          "output.weight": (torch.randn((params.vocab_size, params.dim), device=dev, generator=g) * 0.02).half(),
+          "norm.weight": torch.ones(params.dim, device=dev, dtype=torch.float16)}
+    for i in range(params.n_layers):
+        sd[f"layers.{i}.attention_norm.weight"] = torch.ones(params.dim, device=dev, dtype=torch.float16)
+        sd[f"layers.{i}.ffn_norm.weight"] = torch.ones(params.dim, device=dev, dtype=torch.float16)
+    model.load_state_dict(sd, strict=False, assign=True)
+    for layer in model.layers:
+        for blk, names in (("attention", ("wq", "wk", "wv", "wo")), ("feed_forward", ("w1", "w2", "w3"))):
+            for name in names:
+                lin = getattr(getattr(layer, blk), name)
+                n_out, k_in = lin.shape
+                v = (torch.randn((n_out, k_in), device=dev, generator=g) * 0.02).half()
+                lin.w, lin.s = K.q_int40(v.t().contiguous(), 64)
+                lin.shape = torch.Size((n_out, k_in))
+    model.to(device=dev, dtype=torch.float16)
+    model.eval()
+    return model
+
+
+def time_region(torch, fn, iters):
+    """average milliseconds of fn() over `iters` calls, HIP events on the current stream"""
+    start, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+    fn()
+    torch.cuda.synchronize()
+    start.record()
+    for _ in range(iters):
+        fn()
+    end.record()
+    torch.cuda.synchronize()
+    return start.elapsed_time(end) / iters
+
+
+def gemv_roofline(torch, model, M, iters):
+    """All 224 Q4_0 matrices of one decode step, back to back, at batch M."""
+    from spec_mcts_amd import kernels as K
+    dev = torch.device("cuda:0")
+    lins = []
+    for layer in model.layers:
+        a, f = layer.attention, layer.feed_forward
+        lins += [a.wq, a.wk, a.wv, a.wo, f.w1, f.w3, f.w2]
+    xs = {}
+    for lin in lins:
+        k_in = lin.shape[1]
+        if k_in not in xs:
+            xs[k_in] = torch.randn((M, k_in), device=dev).half()
+    outs = {lin.shape[0]: torch.empty((M, lin.shape[0]), device=dev, dtype=torch.float16) for lin in lins}
+
+    def run():
+        for lin in lins:
+            K.matmul_q40(xs[lin.shape[1]], lin.w, lin.s, (lin.shape[1], lin.shape[0]), out=outs[lin.shape[0]])
+
+    # capture the sequence in a graph so that the timed region holds kernels, not Python
+    run()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run()
+    ms = time_region(torch, graph.replay, iters)
+    total_bytes = sum(q40_bytes(M, lin.shape[0], lin.shape[1]) for lin in lins)
+    n = len(lins)
+    return {"launches": n, "avg_us": ms * 1e3 / n, "bytes_per_launch": total_bytes / n,
+            "gbs": total_bytes / (ms * 1e-3) / 1e9}
+
+
+def cpu_baseline(torch, args_kw, budget_s=20.0):
+    """The reference's CPU PyTorch path on ONE transformer layer (dequantise + F.linear for each of
+    the 7 linears, explicit softmax attention over prompt + suffix), scaled by n_layers, plus the
+    fp16 lm_head.  Bounded to about `budget_s` seconds."""
+    from oracle import q40_oracle as O
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    oargs = O.OracleArgs(**{**args_kw, "n_layers": 1, "max_batch_size": 10})
+    sd = O.random_q40_state_dict(oargs, seed=7)
+    model = O.OracleTransformer(oargs, sd, dense=False)     # dense=False: dequantise on every call, as the reference does
+    P = 64                                                  # short prompt: the sample times the decode step, not prefill
+    prompt = torch.randint(0, oargs.vocab_size, (1, P))
+    model.forward(prompt, 0)
+    res = {}
+    t_start = time.perf_counter()
+    for B in (1, 10):
+        tok = torch.randint(0, oargs.vocab_size, (B, 1))
+        times = []
+        for i in range(3):
+            t0 = time.perf_counter()
+            model.forward(tok, P + i)
+            times.append(time.perf_counter() - t0)
+            if time.perf_counter() - t_start > budget_s:
+                break
+        res[B] = sorted(times)[len(times) // 2]
+        if time.perf_counter() - t_start > budget_s:
+            break
+    # one forward() above = embedding + 1 layer + lm_head; time the head alone to scale layers only
+    h = torch.randn((1, oargs.dim)).half()
+    t0 = time.perf_counter()
+    (h.float() @ sd["output.weight"].float().t()).half()
+    t_head = time.perf_counter() - t0
+    n_layers = args_kw["n_layers"]
+    out = {}
+    for B, t in res.items():
+        step = max(t - t_head, 0.0) * n_layers + t_head
+        out[B] = B / step
+    return out, cores, res
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=100)
+    ap.add_argument("--warmup", type=int, default=10)
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--layers", type=int, default=32, help="fewer layers for a quick functional run (INVALID as a result)")
+    a = ap.parse_args()
+    if a.gpus != 1:
+        sys.exit("bench.py: this build runs the Q4_0 decode path on ONE GPU; --gpus must be 1 "
+                 "(branches would shard data-parallel across GPUs, which this run does not exercise)")
+    import torch
+    from spec_mcts_amd.decode import GraphDecoder
+
+    assert torch.cuda.is_available(), "bench.py needs a GPU"
+    steps, warmup = a.steps, a.warmup
+    assert steps + warmup + 1 <= 128, "configs[3] decodes at most 128 tokens per branch"
+    args_kw = dict(dim=4096, n_layers=a.layers, n_heads=32, vocab_size=32016, multiple_of=256, norm_eps=1e-5,
+                   rope_theta=1e6, max_batch_size=100, max_seq_len=128, max_prompt_seq_len=PROMPT_LEN)
+    torch.manual_seed(3)
+    model = build_model(torch, args_kw, seed=3)
+    prompt = torch.randint(0, 32016, (1, PROMPT_LEN), generator=torch.Generator().manual_seed(3)).cuda()
+
+    by_batch = {}
+    for B in BATCHES:
+        dec = GraphDecoder(model, B, use_graph=not a.no_graph)
+        dec.prefill(prompt)
+        dec.capture()
+        dec.decode(warmup)
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        dec.decode(steps)
+        torch.cuda.synchronize()
+        dt = time.perf_counter() - t0
+        by_batch[B] = {"tok_s": B * steps / dt, "ms_per_step": dt / steps * 1e3}
+        del dec
+
+    # per-step algorithmic HBM bytes: Q4 linears + fp16 lm_head + shared prefix KV (once) + suffix KV (Q4 rows)
+    lin_bytes = sum(q40_bytes(0, n, k) for n, k in ((4096, 4096),) * 4 + ((11008, 4096),) * 2 + ((4096, 11008),)) * a.layers
+    head_bytes = 32016 * 4096 * 2
+    prefix_bytes = 2 * PROMPT_LEN * 4096 * 2 * a.layers
+    t_mid = warmup + steps // 2
+    for B in BATCHES:
+        step_bytes = lin_bytes + head_bytes + prefix_bytes + B * t_mid * a.layers * 2 * 32 * 68
+        by_batch[B]["hbm_frac"] = step_bytes / (by_batch[B]["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
+
+    rf1 = gemv_roofline(torch, model, 1, 5)
+    rf10 = gemv_roofline(torch, model, 10, 5)
+    rf100 = gemv_roofline(torch, model, 100, 3)
+    flops100 = sum(2 * 100 * n * k for n, k in ((4096, 4096),) * 4 + ((11008, 4096),) * 2 + ((4096, 11008),)) * a.layers
+    gemm_tflops = flops100 / (rf100["avg_us"] * rf100["launches"] * 1e-6) / 1e12
+
+    result = {
+        "metric": "Q4_0 7B decode tok/s at B=1/10/100; Q4_0 GEMV achieved HBM GB/s",
+        "value": by_batch[100]["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": by_batch[100]["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "codellama7b_arch_q40_decode_prompt512_shared_prefix", "branches": 100,
+                   "layers": a.layers, "graph": not a.no_graph},
+        "by_batch": {str(B): {k: round(v, 4) for k, v in d.items()} for B, d in by_batch.items()},
+        "roofline": {"kernel": "q40_gemv_kernel (M=1, the 224 Q4_0 matrices of one 7B decode step)", "bound": "hbm",
+                     "achieved": round(rf1["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(rf1["gbs"] / HBM_PEAK_GBS, 4), "traffic": None,
+                     "avg_launch_us": round(rf1["avg_us"], 3), "bytes_per_launch": round(rf1["bytes_per_launch"])},
+        "rooflines_other": [
+            {"kernel": "q40_gemv_kernel (M=10)", "bound": "hbm", "achieved": round(rf10["gbs"], 1), "peak": HBM_PEAK_GBS,
+             "unit": "GB/s", "frac": round(rf10["gbs"] / HBM_PEAK_GBS, 4), "avg_launch_us": round(rf10["avg_us"], 3)},
+            {"kernel": "q40_gemm_kernel (M=100)", "bound": "mfma", "achieved": round(gemm_tflops, 1),
+             "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(gemm_tflops / MFMA_F16_PEAK_TFLOPS, 4),
+             "hbm_gbs": round(rf100["gbs"], 1), "avg_launch_us": round(rf100["avg_us"], 3)},
+        ],
+    }
+    if not a.no_cpu_baseline:
+        cpu, cores, raw = cpu_baseline(torch, args_kw)
+        result["cpu_baseline"] = {"value": round(cpu.get(1, 0.0), 4), "unit": "tok/s", "cores": cores, "kind": "port",
+                                  "sample": "oracle CPU path (torch dequantise + F.linear, fp32 compute): one layer + lm_head, "
+                                            "median of 3 decode steps at B=1 (and B=10), 64-token prompt, layer time x n_layers",
+                                  "by_batch": {str(B): round(v, 4) for B, v in cpu.items()}}
+    print(json.dumps(result))
+
+
+if __name__ == "__main__":
+    main()

@@ -141,16 +141,8 @@ __global__ __launch_bounds__(GEMM_THREADS) void q40_gemm_kernel(GemmParams p) {
                 if (m < p.M)
                     store_coherent(p.partial + slice * slice_stride + (long)m * p.N + n_base + 64 * h, acc[h][t][r]);
             }
-    __threadfence();
-    __syncthreads();
     uint32_t *counter = p.counters + mb * p.nb + block;
-    if (tid == 0) {
-        uint32_t prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
-        s_last = (prev == (uint32_t)p.ksplit - 1u) ? 1u : 0u;
-    }
-    __syncthreads();
-    if (!s_last) return;
-    __threadfence();
+    if (!arrive_is_last(counter, (uint32_t)p.ksplit, &s_last)) return;
     // the last workgroup adds the slices in order; thread t handles column t%128, rows t/128, +2, ...
     const int n = block * 128 + (tid & 127);
     for (int mm = tid >> 7; mm < m_count; mm += 2) {
@@ -162,7 +154,7 @@ __global__ __launch_bounds__(GEMM_THREADS) void q40_gemm_kernel(GemmParams p) {
         if (p.epilogue == SMH_EPI_RESIDUAL) v = (half_t)((float)p.resid[(long)m * p.ldr + n] + (float)v);
         p.c[(long)m * p.ldc + n] = v;
     }
-    if (tid == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    arrive_reset(counter);
 }
 
 }  // namespace smh

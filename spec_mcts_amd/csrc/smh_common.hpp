@@ -96,14 +96,39 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-// ---- coherent accesses for cross-workgroup hand-off ---------------------------------------------
+// ---- cross-workgroup hand-off of partial sums ----------------------------------------------------
 // Partial results written by one workgroup and read by another (possibly on a different XCD, i.e.
-// behind a different L2) go through device-scope atomics so that no non-coherent cache line is used.
+// behind a different L2) travel as device-scope relaxed atomics: such stores write through to the
+// point of coherence and such loads never use a possibly stale cache line.  That makes full
+// device-scope fences unnecessary (they write back and invalidate the whole L2, which is ruinous
+// while other workgroups stream weights through it); all that is needed is that a workgroup's
+// stores have completed before its counter increment is issued.
 __device__ __forceinline__ void store_coherent(float *p, float v) {
     __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ float load_coherent(const float *p) {
     return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+// wait until every memory operation this wave has issued is complete (stores acknowledged)
+__device__ __forceinline__ void wait_memory_ops() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
+// Counts arrivals of the workgroups that share `counter`; returns true in the last one (uniform over
+// the workgroup).  Call after store_coherent() of this workgroup's partials; in the last workgroup,
+// read the others' partials with load_coherent() and then reset the counter with arrive_reset().
+__device__ __forceinline__ bool arrive_is_last(uint32_t *counter, uint32_t expected, uint32_t *s_flag) {
+    wait_memory_ops();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        uint32_t prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *s_flag = (prev == expected - 1u) ? 1u : 0u;
+    }
+    __syncthreads();
+    return *s_flag != 0u;
+}
+__device__ __forceinline__ void arrive_reset(uint32_t *counter) {
+    if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
 }  // namespace smh

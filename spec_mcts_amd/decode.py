@@ -1,0 +1,102 @@
+"""Greedy tree-branch decoding with the whole decode step captured in one HIP graph.
+
+A decode step of the 7B model is ~420 kernel launches of a few microseconds each; issued one by
+one from Python the step is launch-bound.  The kernels read the position and the suffix index
+from device memory, so one captured graph serves every step: replay, bump the two counters on the
+device, replay again.  No hipMemsetAsync node is recorded (the matmul workspace cleans itself).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import kernels as K
+from .hf_model_q40_kv_shared import Transformer
+
+
+class GraphDecoder:
+    """Prefill once at B=1, share the prompt KV between `batch_size` branches, then greedy-decode.
+
+    Equivalent to calling model(tokens, start_pos) + argmax step by step (the graph records exactly
+    those kernels); `use_graph=False` runs that eager loop instead.
+    """
+
+    def __init__(self, model: Transformer, batch_size: int, use_graph: bool = True):
+        assert batch_size <= model.params.max_batch_size
+        self.model = model
+        self.B = batch_size
+        self.use_graph = use_graph
+        self.device = model.norm.weight.device
+        self.tokens = torch.zeros((batch_size, 1), dtype=torch.int64, device=self.device)
+        self.state = torch.zeros(2, dtype=torch.int32, device=self.device)     # (position, suffix index)
+        self.one = torch.ones(2, dtype=torch.int32, device=self.device)
+        self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self.prompt_len = 0
+
+    def _step(self):
+        logits = self.model._forward_impl(self.tokens, 1, (self.state[0:1], self.state[1:2]))
+        nxt = K.argmax(logits.view(self.B, -1))
+        self.tokens.copy_(nxt.view(self.B, 1))
+        self.state.add_(self.one)
+
+    @torch.inference_mode()
+    def prefill(self, prompt: torch.Tensor) -> torch.Tensor:
+        """prompt int64 [1,P] -> first greedy token; resets the branch state."""
+        m = self.model
+        m.resetSeq()
+        logits = m(prompt[:1].to(self.device), 0)[:, -1]
+        self.prompt_len = prompt.shape[1]
+        first = K.argmax(logits.contiguous())
+        self.tokens.copy_(first.view(1, 1).expand(self.B, 1))
+        self._reset_state()
+        return first
+
+    def _reset_state(self):
+        self.state.copy_(torch.tensor([self.prompt_len, 0], dtype=torch.int32))
+
+    @torch.inference_mode()
+    def capture(self):
+        """Warm up (allocates workspaces, loads kernels) and record one decode step."""
+        saved = self.tokens.clone()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            for _ in range(2):
+                self._reset_state()
+                self._step()
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        self._reset_state()
+        self.tokens.copy_(saved)
+        if self.use_graph:
+            self.graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(self.graph):
+                self._step()
+            # the capture pass itself does not execute; state and tokens are untouched
+        torch.cuda.synchronize()
+
+    @torch.inference_mode()
+    def decode(self, steps: int, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Run `steps` decode steps; returns the tokens produced, int64 [B, steps]."""
+        if out is None:
+            out = torch.empty((self.B, steps), dtype=torch.int64, device=self.device)
+        for i in range(steps):
+            if self.graph is not None:
+                self.graph.replay()
+            else:
+                self._step()
+            out[:, i].copy_(self.tokens[:, 0])
+        return out
+
+    @torch.inference_mode()
+    def generate(self, prompt: torch.Tensor, steps: int) -> torch.Tensor:
+        """tokens [B, steps]: the first comes from the prefill logits, the rest from decode steps."""
+        first = self.prefill(prompt)
+        if self.graph is None and self.use_graph:
+            self.capture()
+        res = torch.empty((self.B, steps), dtype=torch.int64, device=self.device)
+        res[:, 0] = first
+        if steps > 1:
+            self.decode(steps - 1, res[:, 1:])
+        return res

@@ -280,24 +280,29 @@ class Transformer(nn.Module):
         return self._step_state[0:1], self._step_state[1:2]
 
     # -- the hot path ----------------------------------------------------------------------------
+    def _forward_impl(self, tokens: torch.Tensor, start_pos: int, step_state):
+        """Embedding -> blocks -> final norm -> lm_head.  For decode steps (start_pos != 0) the
+        position and suffix index are read by the kernels from `step_state` (device int32), so this
+        function issues no host-to-device traffic and can be captured in a HIP graph."""
+        h = self.tok_embeddings(tokens).to(DTYPE)
+        freqs = self._tables(h.device)
+        for layer in self.layers:
+            h = layer(h, start_pos, freqs, None, step_state=step_state)
+        h = self.norm(h)
+        return self.output(h).to(DTYPE)
+
     @torch.inference_mode()
     def forward(self, tokens: torch.Tensor, start_pos: int):
         _bsz, seqlen = tokens.shape
-        h = self.tok_embeddings(tokens).to(DTYPE)
-        freqs = self._tables(h.device)
         step_state = None
         if start_pos != 0:
             t = start_pos - self.layers[0].attention.cache_prompt_len
             assert 0 <= t < self.params.max_seq_len, "suffix cache exhausted"
             assert _bsz <= self.params.max_batch_size
-            step_state = self._set_step(h.device, start_pos)
+            step_state = self._set_step(tokens.device, start_pos)
         else:
             assert seqlen <= self.params.max_prompt_seq_len
-        for layer in self.layers:
-            h = layer(h, start_pos, freqs, None, step_state=step_state)
-        h = self.norm(h)
-        output = self.output(h).to(DTYPE)
-        return output
+        return self._forward_impl(tokens, start_pos, step_state)
 
     def fork(self, origin: int, curr_batch: int, forks: int):
         """Forks the process, such that kv-cache is copied from origin batch number to all the list of new batches"""
