@@ -56,11 +56,11 @@ int smh_q40_quantize(const void *in, void *w, void *s, long groups, smh_stream_t
  * c[M,N] = a[M,K] . deq(b_w, b_s)[K,N], fp16 operands, fp32 accumulation, one fp16 rounding;
  * replaces matmul_q40 (triton_kernels.py:471-500) = LinearQ4_0.forward
  * (hf_model_q40_kv_shared.py:228-236).  lda/ldc/ldr are row strides in elements.
- * Requires N % 128 == 0 and K % 8 == 0.
+ * Requires N % 128 == 0, K % 8 == 0, lda % 8 == 0, ldc % 4 == 0 and 16-byte aligned a.
  * smh_q40_matmul picks the GEMV kernel (M <= SMH_GEMV_MAX_M) or the LDS/MFMA GEMM.
- * workspace: smh_q40_matmul_workspace_bytes() bytes, zero-filled ONCE by the caller before first
- * use; the kernels leave it zeroed again, so it can be reused by every later call on the same
- * stream (calls that overlap on different streams need separate workspaces). */
+ * workspace: smh_q40_matmul_workspace_bytes() bytes of scratch (no initialisation needed) that
+ * holds the fp32 K-slice slabs between the producing kernel and the reduce kernel; calls that
+ * overlap on different streams need separate workspaces. */
 #define SMH_GEMV_MAX_M 16
 size_t smh_q40_matmul_workspace_bytes(int max_m, int max_n);
 int smh_q40_gemv(const void *a, int M, int K, long lda, const void *b_w, const void *b_s, int N,
@@ -72,6 +72,41 @@ int smh_q40_gemm(const void *a, int M, int K, long lda, const void *b_w, const v
 int smh_q40_matmul(const void *a, int M, int K, long lda, const void *b_w, const void *b_s, int N,
                    void *c, long ldc, int epilogue, const void *residual, long ldr,
                    void *workspace, size_t workspace_bytes, smh_stream_t stream);
+
+/* ---- fused decode-layer operators ------------------------------------------------------------
+ * The matmul kernels cut K into `ksplit` slices and leave one fp32 slab per slice,
+ * partial[ksplit][M][n_total]; the operator that FOLLOWS the linear in the model adds the slabs
+ * (in slice order), rounds once to fp16 - the value matmul_q40 returns - and carries on, so no
+ * kernel waits for another workgroup and a decode layer needs 4 weight-streaming launches.
+ * Up to 3 weights that share the input (wq|wk|wv of Attention.forward,
+ * hf_model_q40_kv_shared.py:313; w1|w3 of FeedForward.forward, :434) run as segments of one
+ * launch; their outputs are concatenated along the columns (n_total = sum of n[i]).
+ *
+ * smh_q40_matmul_plan         ksplit the kernels will use for these dimensions (depends on M, K, n only)
+ * smh_q40_matmul_partial      produce the slabs; partial_bytes >= ksplit * M * n_total * 4
+ * smh_partial_reduce          c[m][j] = fp16(sum) (+ residual) for columns col0 .. col0+N-1
+ * smh_partial_rmsnorm         h_out = h_in + fp16(sum) (residual add of TransformerBlock.forward,
+ *                             :463-466; h_in may be NULL), xn_out = RMSNorm(h_out) * weight (:129-134);
+ *                             with partial == NULL it is a plain RMSNorm of h_in
+ * smh_partial_silu_mul        slabs hold [w1 x | w3 x] (n_total = 2 * n_half): out = silu(.) * (.) (:434)
+ * smh_partial_rope_append_kv  slabs hold [q | k | v] (n_total = (H + 2 Hkv) * D): rounds to fp16,
+ *                             applies apply_rotary_emb (:173-203) to q and k at position *pos_dev,
+ *                             writes q [B,H,D], k, v [B,Hkv,D] and appends Q4_0(k), Q4_0(v) to row
+ *                             *t_dev of every branch's suffix cache (:365-371); cache_k may be NULL
+ */
+int smh_q40_matmul_plan(int M, int K, int nseg, const int *n);
+int smh_q40_matmul_partial(const void *a, int M, int K, long lda, int nseg, const void *const *w,
+                           const void *const *s, const int *n, void *partial, size_t partial_bytes,
+                           smh_stream_t stream);
+int smh_partial_reduce(const void *partial, int ksplit, int M, int n_total, int col0, int N, void *c,
+                       long ldc, int epilogue, const void *residual, long ldr, smh_stream_t stream);
+int smh_partial_rmsnorm(const void *partial, int ksplit, int M, int N, const void *h_in,
+                        const void *weight, float eps, void *h_out, void *xn_out, smh_stream_t stream);
+int smh_partial_silu_mul(const void *partial, int ksplit, int M, int n_half, void *out, smh_stream_t stream);
+int smh_partial_rope_append_kv(const void *partial, int ksplit, int B, int H, int Hkv, int D,
+                               void *q, void *k, void *v, const void *cos_tab, const void *sin_tab,
+                               const int32_t *pos_dev, void *cache_k, void *cache_ks, void *cache_v,
+                               void *cache_vs, int Smax, const int32_t *t_dev, smh_stream_t stream);
 
 /* ---- small fused ops -----------------------------------------------------------------------
  * smh_rmsnorm: RMSNorm.forward (hf_model_q40_kv_shared.py:129-134): fp32 normalise -> fp16 ->

@@ -1,0 +1,371 @@
+// Consumers of the Q4_0 matmul's K-slice slabs.
+//
+// The matmul kernels leave `ksplit` fp32 slabs partial[s][m][n]; every kernel here first forms
+// acc = sum_s partial[s][m][n] (slice order, so the result does not depend on scheduling), rounds
+// it ONCE to fp16 - the value the reference's matmul_q40 returns - and then applies the operator
+// that follows the linear in the model:
+//   partial_reduce_kernel      c = fp16(acc) (+ fp16 residual add)
+//   partial_rmsnorm_kernel     h = h_in + fp16(acc);  xn = RMSNorm(h) * weight
+//   partial_silu_mul_kernel    out = fp16(silu(fp16(acc_gate))) * fp16(acc_up)
+//   partial_rope_append_kernel q,k,v = fp16(acc); RoPE(q,k); Q4_0 append of k,v to the suffix cache
+// so a decode layer is 4 weight-streaming launches plus these small ones, and no kernel ever waits
+// for another workgroup.
+#include "q40_matmul.hpp"
+
+namespace smh {
+
+__device__ __forceinline__ float slab_sum(const float *p, long slab_stride, int ksplit) {
+    float v[SMH_MAX_KSPLIT];
+#pragma unroll
+    for (int s = 0; s < SMH_MAX_KSPLIT; ++s) v[s] = (s < ksplit) ? p[s * slab_stride] : 0.f;
+    float tot = 0.f;
+#pragma unroll
+    for (int s = 0; s < SMH_MAX_KSPLIT; ++s) tot += v[s];
+    return tot;
+}
+__device__ __forceinline__ f4 slab_sum4(const float *p, long slab_stride, int ksplit) {
+    f4 v[SMH_MAX_KSPLIT];
+#pragma unroll
+    for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
+        v[s] = (s < ksplit) ? *reinterpret_cast<const f4 *>(p + s * slab_stride) : f4{0.f, 0.f, 0.f, 0.f};
+    f4 tot = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s = 0; s < SMH_MAX_KSPLIT; ++s) tot += v[s];
+    return tot;
+}
+
+// ---- plain reduce (+ residual) ------------------------------------------------------------------
+__global__ __launch_bounds__(256) void partial_reduce_kernel(const float *__restrict__ partial, int ksplit, int M, int n_total,
+                                                             int col0, int N, half_t *__restrict__ c, long ldc, int epilogue,
+                                                             const half_t *__restrict__ resid, long ldr) {
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= (long)M * N) return;
+    const int m = (int)(i / N), n = (int)(i % N);          // N % 4 == 0: the 4 columns share a row
+    const f4 acc = slab_sum4(partial + (long)m * n_total + col0 + n, (long)M * n_total, ksplit);
+    h4 out;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        half_t v = (half_t)acc[j];
+        if (epilogue == SMH_EPI_RESIDUAL) v = (half_t)((float)resid[(long)m * ldr + n + j] + (float)v);
+        out[j] = v;
+    }
+    *reinterpret_cast<h4 *>(c + (long)m * ldc + n) = out;
+}
+
+// ---- residual add + RMSNorm ---------------------------------------------------------------------
+// one workgroup of 1024 threads per row; h_out = h_in + fp16(acc) (fp16 add), xn = fp16(fp16(h*r)*w)
+__global__ __launch_bounds__(1024) void partial_rmsnorm_kernel(const float *__restrict__ partial, int ksplit, int M, int N,
+                                                               const half_t *__restrict__ h_in, const half_t *__restrict__ wt,
+                                                               float eps, half_t *__restrict__ h_out, half_t *__restrict__ xn_out) {
+    __shared__ float s_part[16];
+    const int m = blockIdx.x;
+    const long slab = (long)M * N;
+    float ss = 0.f;
+    // each thread owns columns 4t, 4t+1, 4t+2, 4t+3 (+ 4096 per pass); values kept for the second pass
+    constexpr int MAXPASS = 4;      // N <= 16384
+    h4 hv[MAXPASS];
+#pragma unroll
+    for (int ps = 0; ps < MAXPASS; ++ps) {
+        const int n = (ps * 1024 + threadIdx.x) * 4;
+        if (n < N) {
+            h4 v;
+            if (partial != nullptr) {
+                const f4 acc = slab_sum4(partial + (long)m * N + n, slab, ksplit);
+#pragma unroll
+                for (int j = 0; j < 4; ++j) v[j] = (half_t)acc[j];
+                if (h_in != nullptr) {
+                    const h4 r = *reinterpret_cast<const h4 *>(h_in + (long)m * N + n);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) v[j] = (half_t)((float)r[j] + (float)v[j]);
+                }
+            } else {
+                v = *reinterpret_cast<const h4 *>(h_in + (long)m * N + n);
+            }
+            hv[ps] = v;
+            if (h_out != nullptr) *reinterpret_cast<h4 *>(h_out + (long)m * N + n) = v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) ss += (float)v[j] * (float)v[j];
+        }
+    }
+    ss = wave_sum(ss);
+    if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    float total = 0.f;
+#pragma unroll
+    for (int w = 0; w < 16; ++w) total += s_part[w];
+    const float r = 1.0f / sqrtf(total / (float)N + eps);
+#pragma unroll
+    for (int ps = 0; ps < MAXPASS; ++ps) {
+        const int n = (ps * 1024 + threadIdx.x) * 4;
+        if (n < N) {
+            const h4 w = *reinterpret_cast<const h4 *>(wt + n);
+            h4 o;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                half_t nv = (half_t)((float)hv[ps][j] * r);
+                o[j] = nv * w[j];
+            }
+            *reinterpret_cast<h4 *>(xn_out + (long)m * N + n) = o;
+        }
+    }
+}
+
+// ---- SwiGLU gate ------------------------------------------------------------------------------------
+// slabs hold [gate | up] (2 * n_half columns)
+__global__ __launch_bounds__(256) void partial_silu_mul_kernel(const float *__restrict__ partial, int ksplit, int M, int n_half,
+                                                               half_t *__restrict__ out) {
+    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
+    if (i >= (long)M * n_half) return;
+    const int m = (int)(i / n_half), n = (int)(i % n_half);
+    const long slab = (long)M * 2 * n_half;
+    const f4 ga = slab_sum4(partial + (long)m * 2 * n_half + n, slab, ksplit);
+    const f4 ua = slab_sum4(partial + (long)m * 2 * n_half + n_half + n, slab, ksplit);
+    h4 o;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const float gf = (float)(half_t)ga[j];
+        const half_t sl = (half_t)(gf / (1.0f + expf(-gf)));
+        o[j] = sl * (half_t)ua[j];
+    }
+    *reinterpret_cast<h4 *>(out + (long)m * n_half + n) = o;
+}
+
+// ---- RoPE + Q4_0 KV append from the fused q|k|v product ------------------------------------------------
+__device__ __forceinline__ void rope_pair2(half_t &x1, half_t &x2, half_t cs, half_t sn) {
+#pragma clang fp contract(off)      // the two products are rounded to fp16 before they are added
+    half_t a = x1 * cs, b = (-x2) * sn;
+    half_t c = x2 * cs, d = x1 * sn;
+    x1 = a + b;
+    x2 = c + d;
+}
+__device__ __forceinline__ int kv_code2(half_t x, float scale) {
+    float qf = (float)(half_t)((float)x / scale);
+    if (!(qf == qf)) return 0;
+    return (int)__builtin_rintf(qf);
+}
+__device__ __forceinline__ void kv_store_row2(half_t lo, half_t hi, uint8_t *row, half_t *scales, int lane) {
+    uint32_t a_lo = (uint32_t)(__builtin_bit_cast(uint16_t, lo) & 0x7FFFu);
+    uint32_t a_hi = (uint32_t)(__builtin_bit_cast(uint16_t, hi) & 0x7FFFu);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        a_lo = max(a_lo, (uint32_t)__shfl_xor((int)a_lo, o, 64));
+        a_hi = max(a_hi, (uint32_t)__shfl_xor((int)a_hi, o, 64));
+    }
+    half_t s0 = (half_t)((float)__builtin_bit_cast(half_t, (uint16_t)a_lo) / 7.0f);
+    half_t s1 = (half_t)((float)__builtin_bit_cast(half_t, (uint16_t)a_hi) / 7.0f);
+    int c0 = kv_code2(lo, (float)s0), c1 = kv_code2(hi, (float)s1);
+    row[lane] = (uint8_t)(((c0 & 15) << 4) | (c1 & 15));
+    if (lane == 0) { scales[0] = s0; scales[1] = s1; }
+}
+
+// one wave per (branch, head); heads 0..H-1 queries, H..H+Hkv-1 keys, H+Hkv.. values.
+// slab columns: [q (H*128) | k (Hkv*128) | v (Hkv*128)]
+__global__ __launch_bounds__(256) void partial_rope_append_kernel(const float *__restrict__ partial, int ksplit, int B, int H, int Hkv,
+                                                                  half_t *__restrict__ q, half_t *__restrict__ k, half_t *__restrict__ v,
+                                                                  const half_t *__restrict__ cos_tab, const half_t *__restrict__ sin_tab,
+                                                                  const int32_t *__restrict__ pos_dev,
+                                                                  uint8_t *__restrict__ cache_k, half_t *__restrict__ cache_ks,
+                                                                  uint8_t *__restrict__ cache_v, half_t *__restrict__ cache_vs,
+                                                                  int Smax, const int32_t *__restrict__ t_dev) {
+    const int lane = threadIdx.x & 63;
+    const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int heads = H + 2 * Hkv;
+    if (item >= (long)B * heads) return;
+    const int b = (int)(item / heads);
+    const int h = (int)(item % heads);
+    const int n_total = heads * 128;
+    const float *src = partial + (long)b * n_total + (long)h * 128;
+    const long slab = (long)B * n_total;
+    half_t x1 = (half_t)slab_sum(src + lane, slab, ksplit);
+    half_t x2 = (half_t)slab_sum(src + lane + 64, slab, ksplit);
+    const int t = (t_dev != nullptr) ? *t_dev : -1;
+    if (h >= H + Hkv) {                                      // value head: store, append
+        const int hk = h - H - Hkv;
+        half_t *pv = v + ((long)b * Hkv + hk) * 128;
+        pv[lane] = x1;
+        pv[lane + 64] = x2;
+        if (cache_v != nullptr && t >= 0 && t < Smax) {
+            const long row = ((long)b * Smax + t) * Hkv + hk;
+            kv_store_row2(x1, x2, cache_v + row * 64, cache_vs + row * 2, lane);
+        }
+        return;
+    }
+    const int pos = *pos_dev;
+    rope_pair2(x1, x2, cos_tab[(long)pos * 64 + lane], sin_tab[(long)pos * 64 + lane]);
+    if (h < H) {
+        half_t *pq = q + ((long)b * H + h) * 128;
+        pq[lane] = x1;
+        pq[lane + 64] = x2;
+        return;
+    }
+    const int hk = h - H;
+    half_t *pk = k + ((long)b * Hkv + hk) * 128;
+    pk[lane] = x1;
+    pk[lane + 64] = x2;
+    if (cache_k != nullptr && t >= 0 && t < Smax) {
+        const long row = ((long)b * Smax + t) * Hkv + hk;
+        kv_store_row2(x1, x2, cache_k + row * 64, cache_ks + row * 2, lane);
+    }
+}
+
+}  // namespace smh
+
+using namespace smh;
+
+// ---- host side: plan, produce, consume ----------------------------------------------------------------
+static int fill_params(MatmulParams &p, const void *a, int M, int K, long lda, int nseg, const void *const *w,
+                       const void *const *s, const int *n, const char *who) {
+    SMH_REQUIRE(M >= 0, "%s: M=%d", who, M);
+    SMH_REQUIRE(K > 0 && K % 8 == 0, "%s: K=%d must be a positive multiple of 8", who, K);
+    SMH_REQUIRE(nseg >= 1 && nseg <= SMH_MAX_SEGMENTS && n != nullptr, "%s: nseg=%d outside [1,%d]", who, nseg, SMH_MAX_SEGMENTS);
+    SMH_REQUIRE(lda >= K && lda % 8 == 0, "%s: lda=%ld must be >= K and a multiple of 8 (128-bit loads)", who, lda);
+    p = MatmulParams{};
+    p.a = (const half_t *)a;
+    p.M = M; p.K = K; p.lda = lda; p.nseg = nseg;
+    for (int i = 0; i < nseg; ++i) {
+        SMH_REQUIRE(n[i] > 0 && n[i] % 128 == 0, "%s: N=%d must be a positive multiple of 128", who, n[i]);
+        p.seg[i].w = w ? (const uint8_t *)w[i] : nullptr;
+        p.seg[i].s = s ? (const half_t *)s[i] : nullptr;
+        p.seg[i].N = n[i];
+    }
+    if (M <= SMH_GEMV_MAX_M) gemv_fill_plan(p); else gemm_fill_plan(p);
+    return 0;
+}
+
+extern "C" int smh_q40_matmul_plan(int M, int K, int nseg, const int *n) {
+    MatmulParams p;
+    if (M <= 0) return 1;
+    int st = fill_params(p, nullptr, M, K, (K + 7) / 8 * 8, nseg, nullptr, nullptr, n, "smh_q40_matmul_plan");
+    return st < 0 ? st : p.ksplit;
+}
+
+extern "C" size_t smh_q40_matmul_workspace_bytes(int max_m, int max_n) {
+    // K is split only while (column units x row blocks) < 512, so the slabs never exceed
+    // 512 tiles of 128 x 128 floats for the GEMM, or SMH_MAX_KSPLIT x 16 x N floats for the GEMV
+    size_t n = (size_t)(max_n < 128 ? 128 : max_n);
+    size_t m = (size_t)(max_m < 1 ? 1 : (max_m > SMH_GEMV_MAX_M ? SMH_GEMV_MAX_M : max_m));
+    size_t floats = n * m * SMH_MAX_KSPLIT;
+    if (max_m > SMH_GEMV_MAX_M && floats < (size_t)640 * 128 * 128) floats = (size_t)640 * 128 * 128;
+    return floats * sizeof(float) + 256;
+}
+
+extern "C" int smh_q40_matmul_partial(const void *a, int M, int K, long lda, int nseg, const void *const *w,
+                                      const void *const *s, const int *n, void *partial, size_t partial_bytes,
+                                      smh_stream_t stream) {
+    MatmulParams p;
+    int st = fill_params(p, a, M, K, lda, nseg, w, s, n, "smh_q40_matmul_partial");
+    if (st) return st;
+    if (M == 0) return 0;
+    SMH_REQUIRE(a && w && s && partial, "smh_q40_matmul_partial: null pointer");
+    for (int i = 0; i < nseg; ++i) SMH_REQUIRE(w[i] && s[i], "smh_q40_matmul_partial: null weight %d", i);
+    size_t need = (size_t)p.ksplit * M * p.n_total * sizeof(float);
+    SMH_REQUIRE(partial_bytes >= need, "smh_q40_matmul_partial: partial buffer %zu < %zu bytes", partial_bytes, need);
+    p.partial = (float *)partial;
+    p.direct = 0;
+    return M <= SMH_GEMV_MAX_M ? gemv_launch(p, (hipStream_t)stream) : gemm_launch(p, (hipStream_t)stream);
+}
+
+static int reduce_launch(const float *partial, int ksplit, int M, int n_total, int col0, int N, void *c, long ldc,
+                         int epilogue, const void *residual, long ldr, hipStream_t stream) {
+    long quads = ((long)M * N + 3) / 4;
+    hipLaunchKernelGGL(partial_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
+                       partial, ksplit, M, n_total, col0, N, (half_t *)c, ldc, epilogue, (const half_t *)residual, ldr);
+    return launch_status();
+}
+
+extern "C" int smh_partial_reduce(const void *partial, int ksplit, int M, int n_total, int col0, int N, void *c, long ldc,
+                                  int epilogue, const void *residual, long ldr, smh_stream_t stream) {
+    SMH_REQUIRE(ksplit >= 1 && ksplit <= SMH_MAX_KSPLIT, "smh_partial_reduce: ksplit=%d outside [1,%d]", ksplit, SMH_MAX_KSPLIT);
+    SMH_REQUIRE(M >= 0 && N > 0 && N % 4 == 0 && col0 >= 0 && col0 % 4 == 0 && col0 + N <= n_total && n_total % 4 == 0,
+                "smh_partial_reduce: M=%d N=%d col0=%d n_total=%d", M, N, col0, n_total);
+    SMH_REQUIRE(epilogue == SMH_EPI_NONE || epilogue == SMH_EPI_RESIDUAL, "smh_partial_reduce: epilogue=%d", epilogue);
+    if (M == 0) return 0;
+    SMH_REQUIRE(partial && c && ldc >= N && ldc % 4 == 0, "smh_partial_reduce: bad output");
+    SMH_REQUIRE(epilogue != SMH_EPI_RESIDUAL || (residual && ldr >= N), "smh_partial_reduce: residual missing");
+    return reduce_launch((const float *)partial, ksplit, M, n_total, col0, N, c, ldc, epilogue, residual, ldr, (hipStream_t)stream);
+}
+
+static int matmul_fp16(const void *a, int M, int K, long lda, const void *b_w, const void *b_s, int N, void *c, long ldc,
+                       int epilogue, const void *residual, long ldr, void *workspace, size_t workspace_bytes,
+                       smh_stream_t stream, const char *who, int force) {
+    SMH_REQUIRE(force != 1 || M <= SMH_GEMV_MAX_M, "%s: M=%d outside [0,%d]", who, M, SMH_GEMV_MAX_M);
+    SMH_REQUIRE(epilogue == SMH_EPI_NONE || epilogue == SMH_EPI_RESIDUAL, "%s: epilogue=%d", who, epilogue);
+    SMH_REQUIRE(ldc >= N, "%s: ldc=%ld too small", who, ldc);
+    MatmulParams p;
+    const void *ws[1] = {b_w};
+    const void *ss[1] = {b_s};
+    int st = fill_params(p, a, M, K, lda, 1, ws, ss, &N, who);
+    if (st) return st;
+    if (M == 0) return 0;
+    SMH_REQUIRE(a && b_w && b_s && c, "%s: null pointer", who);
+    SMH_REQUIRE(epilogue != SMH_EPI_RESIDUAL || (residual && ldr >= N), "%s: residual missing", who);
+    if (force == 2 && M <= SMH_GEMV_MAX_M) gemm_fill_plan(p);        // smh_q40_gemm on a small batch
+    const bool gemm = (force == 2) || M > SMH_GEMV_MAX_M;
+    p.c = (half_t *)c; p.ldc = ldc; p.resid = (const half_t *)residual; p.ldr = ldr; p.epilogue = epilogue;
+    if (p.ksplit == 1) {
+        p.direct = 1;
+        return gemm ? gemm_launch(p, (hipStream_t)stream) : gemv_launch(p, (hipStream_t)stream);
+    }
+    size_t need = (size_t)p.ksplit * M * N * sizeof(float);
+    SMH_REQUIRE(workspace && workspace_bytes >= need, "%s: workspace %zu < %zu bytes", who, workspace_bytes, need);
+    p.partial = (float *)workspace;
+    p.direct = 0;
+    st = gemm ? gemm_launch(p, (hipStream_t)stream) : gemv_launch(p, (hipStream_t)stream);
+    if (st) return st;
+    SMH_REQUIRE(ldc % 4 == 0, "%s: ldc=%ld must be a multiple of 4", who, ldc);
+    return reduce_launch(p.partial, p.ksplit, M, N, 0, N, c, ldc, epilogue, residual, ldr, (hipStream_t)stream);
+}
+
+extern "C" int smh_q40_gemv(const void *a, int M, int K, long lda, const void *b_w, const void *b_s, int N, void *c, long ldc,
+                            int epilogue, const void *residual, long ldr, void *workspace, size_t workspace_bytes, smh_stream_t stream) {
+    return matmul_fp16(a, M, K, lda, b_w, b_s, N, c, ldc, epilogue, residual, ldr, workspace, workspace_bytes, stream, "smh_q40_gemv", 1);
+}
+extern "C" int smh_q40_gemm(const void *a, int M, int K, long lda, const void *b_w, const void *b_s, int N, void *c, long ldc,
+                            int epilogue, const void *residual, long ldr, void *workspace, size_t workspace_bytes, smh_stream_t stream) {
+    return matmul_fp16(a, M, K, lda, b_w, b_s, N, c, ldc, epilogue, residual, ldr, workspace, workspace_bytes, stream, "smh_q40_gemm", 2);
+}
+extern "C" int smh_q40_matmul(const void *a, int M, int K, long lda, const void *b_w, const void *b_s, int N, void *c, long ldc,
+                              int epilogue, const void *residual, long ldr, void *workspace, size_t workspace_bytes, smh_stream_t stream) {
+    return matmul_fp16(a, M, K, lda, b_w, b_s, N, c, ldc, epilogue, residual, ldr, workspace, workspace_bytes, stream, "smh_q40_matmul", 0);
+}
+
+extern "C" int smh_partial_rmsnorm(const void *partial, int ksplit, int M, int N, const void *h_in, const void *weight, float eps,
+                                   void *h_out, void *xn_out, smh_stream_t stream) {
+    SMH_REQUIRE(partial == nullptr || (ksplit >= 1 && ksplit <= SMH_MAX_KSPLIT), "smh_partial_rmsnorm: ksplit=%d", ksplit);
+    SMH_REQUIRE(M >= 0 && N > 0 && N % 4 == 0 && N <= 16384, "smh_partial_rmsnorm: M=%d N=%d (N must be a multiple of 4, <= 16384)", M, N);
+    SMH_REQUIRE(partial != nullptr || h_in != nullptr, "smh_partial_rmsnorm: no input");
+    if (M == 0) return 0;
+    SMH_REQUIRE(weight && xn_out, "smh_partial_rmsnorm: null pointer");
+    hipLaunchKernelGGL(partial_rmsnorm_kernel, dim3(M), dim3(1024), 0, (hipStream_t)stream, (const float *)partial, ksplit, M, N,
+                       (const half_t *)h_in, (const half_t *)weight, eps, (half_t *)h_out, (half_t *)xn_out);
+    return launch_status();
+}
+
+extern "C" int smh_partial_silu_mul(const void *partial, int ksplit, int M, int n_half, void *out, smh_stream_t stream) {
+    SMH_REQUIRE(ksplit >= 1 && ksplit <= SMH_MAX_KSPLIT, "smh_partial_silu_mul: ksplit=%d", ksplit);
+    SMH_REQUIRE(M >= 0 && n_half > 0 && n_half % 4 == 0, "smh_partial_silu_mul: M=%d n_half=%d", M, n_half);
+    if (M == 0) return 0;
+    SMH_REQUIRE(partial && out, "smh_partial_silu_mul: null pointer");
+    long quads = (long)M * n_half / 4;
+    hipLaunchKernelGGL(partial_silu_mul_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const float *)partial, ksplit, M, n_half, (half_t *)out);
+    return launch_status();
+}
+
+extern "C" int smh_partial_rope_append_kv(const void *partial, int ksplit, int B, int H, int Hkv, int D, void *q, void *k, void *v,
+                                          const void *cos_tab, const void *sin_tab, const int32_t *pos_dev,
+                                          void *cache_k, void *cache_ks, void *cache_v, void *cache_vs, int Smax,
+                                          const int32_t *t_dev, smh_stream_t stream) {
+    SMH_REQUIRE(D == 128, "smh_partial_rope_append_kv: head dim %d (only 128)", D);
+    SMH_REQUIRE(ksplit >= 1 && ksplit <= SMH_MAX_KSPLIT, "smh_partial_rope_append_kv: ksplit=%d", ksplit);
+    SMH_REQUIRE(B >= 0 && H > 0 && Hkv > 0, "smh_partial_rope_append_kv: B=%d H=%d Hkv=%d", B, H, Hkv);
+    if (B == 0) return 0;
+    SMH_REQUIRE(partial && q && k && v && cos_tab && sin_tab && pos_dev, "smh_partial_rope_append_kv: null pointer");
+    SMH_REQUIRE(!cache_k || (cache_ks && cache_v && cache_vs && t_dev && Smax > 0), "smh_partial_rope_append_kv: cache arguments incomplete");
+    long items = (long)B * (H + 2 * Hkv);
+    hipLaunchKernelGGL(partial_rope_append_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+                       (const float *)partial, ksplit, B, H, Hkv, (half_t *)q, (half_t *)k, (half_t *)v,
+                       (const half_t *)cos_tab, (const half_t *)sin_tab, pos_dev, (uint8_t *)cache_k, (half_t *)cache_ks,
+                       (uint8_t *)cache_v, (half_t *)cache_vs, Smax, t_dev);
+    return launch_status();
+}

@@ -1,0 +1,50 @@
+// Shared host/device declarations of the Q4_0 matmul kernels (GEMV for M <= 16, GEMM above).
+//
+// Both kernels cut K into slices for occupancy and write one fp32 [M, n_total] slab per slice into
+// the caller's `partial` buffer; the slabs are added in slice order by the consuming kernel
+// (partial_ops.hip).  With a single slice and a plain epilogue the product is written directly.
+#pragma once
+
+#include "smh_common.hpp"
+
+#define SMH_MAX_KSPLIT 16
+#define SMH_MAX_SEGMENTS 3
+
+namespace smh {
+
+struct MatmulSegment {
+    const uint8_t *w;    // packed nibbles [K, N/2]
+    const half_t *s;     // scales [K, N/64]
+    int N;               // columns of this weight
+    int col0;            // first output column
+    int unit0;           // first work unit (column pair / column block) of this weight
+};
+
+struct MatmulParams {
+    const half_t *a;
+    half_t *c;               // direct output (ksplit == 1)
+    const half_t *resid;
+    float *partial;          // [ksplit][M][n_total]
+    MatmulSegment seg[SMH_MAX_SEGMENTS];
+    long lda, ldc, ldr;
+    int M, K;
+    int nseg, n_total;
+    int units, units_pad;    // column units over all segments (GEMV: padded to a multiple of 8)
+    int mblocks;             // GEMM: 128-row blocks
+    int ksplit, steps_per_slice;
+    int epilogue, direct;
+};
+
+__device__ __forceinline__ half_t matmul_epilogue(const MatmulParams &p, float acc, int m, int n) {
+    half_t v = (half_t)acc;
+    if (p.epilogue == SMH_EPI_RESIDUAL) v = (half_t)((float)p.resid[(long)m * p.ldr + n] + (float)v);
+    return v;
+}
+
+int env_int(const char *name, int dflt);
+void gemv_fill_plan(MatmulParams &p);
+int gemv_launch(const MatmulParams &p, hipStream_t stream);
+void gemm_fill_plan(MatmulParams &p);
+int gemm_launch(const MatmulParams &p, hipStream_t stream);
+
+}  // namespace smh

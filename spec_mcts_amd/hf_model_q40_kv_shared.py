@@ -258,6 +258,7 @@ class Transformer(nn.Module):
         self._rope_tables = None      # (cos, sin) fp16 [T, 64] on the device
         self._step_state = None       # int32 [2] on the device: (position, suffix index t)
         self._step_host = None
+        self.fused = True             # fused decode-layer launches; False runs module by module
 
     # -- helpers -------------------------------------------------------------------------------
     def _tables(self, device):
@@ -284,12 +285,62 @@ class Transformer(nn.Module):
         """Embedding -> blocks -> final norm -> lm_head.  For decode steps (start_pos != 0) the
         position and suffix index are read by the kernels from `step_state` (device int32), so this
         function issues no host-to-device traffic and can be captured in a HIP graph."""
+        if self.fused:
+            return self._forward_fused(tokens, start_pos, step_state)
         h = self.tok_embeddings(tokens).to(DTYPE)
         freqs = self._tables(h.device)
         for layer in self.layers:
             h = layer(h, start_pos, freqs, None, step_state=step_state)
         h = self.norm(h)
         return self.output(h).to(DTYPE)
+
+    def _forward_fused(self, tokens: torch.Tensor, start_pos: int, step_state):
+        """Same arithmetic as the module-by-module path, with the launches of a layer fused:
+        residual+RMSNorm | wq,wk,wv (one launch) | RoPE + Q4_0 KV append | attention | wo |
+        residual+RMSNorm | w1,w3 (one launch) | SiLU*up | w2.  Every linear leaves fp32 K-slice
+        slabs that the next small kernel adds and rounds to fp16 once, exactly where the
+        reference's matmul_q40 rounds."""
+        bsz, seqlen = tokens.shape
+        M = bsz * seqlen
+        p = self.params
+        h = self.tok_embeddings(tokens).to(DTYPE).reshape(M, p.dim)
+        cos, sin = self._tables(h.device)
+        pending = None                      # product of the previous layer's w2, not yet added to h
+        for layer in self.layers:
+            att, ff = layer.attention, layer.feed_forward
+            H, Hkv, D = att.n_local_heads, att.n_local_kv_heads, att.head_dim
+            h, xn = K.partial_rmsnorm(pending, h, layer.attention_norm.weight, layer.attention_norm.eps)
+            qkv = K.matmul_q40_partial(xn, [(att.wq.w, att.wq.s, att.wq.shape[0]), (att.wk.w, att.wk.s, att.wk.shape[0]),
+                                            (att.wv.w, att.wv.s, att.wv.shape[0])])
+            if start_pos == 0:
+                xq = K.partial_reduce(qkv, 0, H * D).view(bsz, seqlen, H, D)
+                xk = K.partial_reduce(qkv, H * D, Hkv * D).view(bsz, seqlen, Hkv, D)
+                xv = K.partial_reduce(qkv, (H + Hkv) * D, Hkv * D).view(bsz, seqlen, Hkv, D)
+                outs = []
+                for b in range(bsz):
+                    K.rope(xq[b], xk[b], cos, sin, 0)
+                    if b == 0:
+                        att.cache_prompt_k[0, :seqlen] = xk[b]
+                        att.cache_prompt_v[0, :seqlen] = xv[b]
+                        att.cache_prompt_len = seqlen
+                    outs.append(K.prefill_attn(xq[b], xk[b], xv[b]).view(seqlen, H * D))
+                o = outs[0] if bsz == 1 else torch.cat(outs, 0)
+            else:
+                assert seqlen == 1, "decode steps take one token per branch"
+                pos_dev, t_dev = step_state
+                q, k, v = K.partial_rope_append_kv(qkv, H, Hkv, D, cos, sin, pos_dev, att.cache_k, att.cache_k_s,
+                                                   att.cache_v, att.cache_v_s, p.max_seq_len, t_dev)
+                o = K.shared_prefix_attn(q, att.cache_prompt_k[0], att.cache_prompt_v[0], att.cache_prompt_len,
+                                         suffix_k=att.cache_k, suffix_v=att.cache_v, suffix_ks=att.cache_k_s,
+                                         suffix_vs=att.cache_v_s, Smax=p.max_seq_len, lens=t_dev, lens_stride=0,
+                                         cur_k=k, cur_v=v).view(M, H * D)
+            po = K.matmul_q40_partial(o, [(att.wo.w, att.wo.s, att.wo.shape[0])])
+            h, xn = K.partial_rmsnorm(po, h, layer.ffn_norm.weight, layer.ffn_norm.eps)
+            gu = K.matmul_q40_partial(xn, [(ff.w1.w, ff.w1.s, ff.w1.shape[0]), (ff.w3.w, ff.w3.s, ff.w3.shape[0])])
+            act = K.partial_silu_mul(gu)
+            pending = K.matmul_q40_partial(act, [(ff.w2.w, ff.w2.s, ff.w2.shape[0])])
+        _, hn = K.partial_rmsnorm(pending, h, self.norm.weight, self.norm.eps, want_h=False)
+        return self.output(hn.view(bsz, seqlen, p.dim)).to(DTYPE)
 
     @torch.inference_mode()
     def forward(self, tokens: torch.Tensor, start_pos: int):

@@ -37,15 +37,15 @@ def _need_gpu(*tensors: torch.Tensor) -> None:
 
 
 def matmul_workspace(device: torch.device, max_m: int = 16, max_n: int = 0) -> torch.Tensor:
-    """Per-device scratch for the K-split partial sums of the Q4_0 matmul.  Zero-filled once; the
-    kernels leave it zeroed.  Shared by all calls on the device: calls issued on different
-    streams at the same time need their own workspace."""
+    """Per-device scratch that carries the fp32 K-slice slabs from the matmul kernel to its reduce
+    kernel.  Shared by all calls on the device (calls run in stream order); calls issued on
+    different streams at the same time need their own workspace."""
     lib = _lib.load()
     need = lib.smh_q40_matmul_workspace_bytes(int(max_m), int(max_n))
     key = ("matmul", device.index if device.index is not None else torch.cuda.current_device())
     ws = _workspaces.get(key)
     if ws is None or ws.numel() < need:
-        ws = torch.zeros(need, dtype=torch.uint8, device=device)
+        ws = torch.empty(need, dtype=torch.uint8, device=device)
         _workspaces[key] = ws
     return ws
 
@@ -90,6 +90,115 @@ def matmul_q40(a: torch.Tensor, b_w: torch.Tensor, b_s: torch.Tensor, b_shape: S
     check(lib.smh_q40_matmul(a.data_ptr(), M, K, K, b_w.data_ptr(), b_s.data_ptr(), N, c.data_ptr(), N,
                              epi, _ptr(residual), N, ws.data_ptr(), ws.numel(), _stream()), "smh_q40_matmul")
     return c
+
+
+def matmul_plan(M: int, K: int, ns: Sequence[int]) -> int:
+    """Number of K slices the matmul kernels use for a [M,K] x [K, sum(ns)] product."""
+    import ctypes
+    lib = _lib.load()
+    arr = (ctypes.c_int * len(ns))(*[int(n) for n in ns])
+    ks = lib.smh_q40_matmul_plan(int(M), int(K), len(ns), arr)
+    if ks < 1:
+        check(ks, "smh_q40_matmul_plan")
+    return ks
+
+
+class PartialProduct:
+    """fp32 K-slice slabs [ksplit, M, n_total] left by matmul_q40_partial, to be consumed by one of
+    the partial_* operators."""
+    __slots__ = ("buf", "ksplit", "M", "n_total")
+
+    def __init__(self, buf, ksplit, M, n_total):
+        self.buf, self.ksplit, self.M, self.n_total = buf, ksplit, M, n_total
+
+
+def matmul_q40_partial(a: torch.Tensor, linears, out: Optional[torch.Tensor] = None) -> PartialProduct:
+    """One launch for up to 3 Q4_0 weights that share the input a [M,K]; `linears` is a sequence of
+    (w, s, N).  Leaves the un-reduced product; the columns of the weights are concatenated."""
+    import ctypes
+    lib = _lib.load()
+    assert a.is_contiguous() and a.dtype == torch.float16 and a.dim() == 2 and a.data_ptr() % 16 == 0
+    _need_gpu(a)
+    M, Kd = a.shape
+    ns = [int(n) for (_, _, n) in linears]
+    for (w, s, n) in linears:
+        _need_gpu(w, s)
+        assert w.is_contiguous() and s.is_contiguous() and w.dtype == torch.int8 and s.dtype == torch.float16
+        assert w.numel() == Kd * n // 2 and s.numel() == Kd * n // 64, "packed weight does not match [K, N]"
+    ks = matmul_plan(M, Kd, ns)
+    n_total = sum(ns)
+    need = ks * M * n_total
+    if out is None:
+        out = torch.empty(need, dtype=torch.float32, device=a.device)
+    assert out.dtype == torch.float32 and out.numel() >= need and out.is_contiguous()
+    nseg = len(linears)
+    wp = (ctypes.c_void_p * nseg)(*[w.data_ptr() for (w, _, _) in linears])
+    sp = (ctypes.c_void_p * nseg)(*[s.data_ptr() for (_, s, _) in linears])
+    na = (ctypes.c_int * nseg)(*ns)
+    check(lib.smh_q40_matmul_partial(a.data_ptr(), M, Kd, Kd, nseg, wp, sp, na, out.data_ptr(), out.numel() * 4, _stream()),
+          "smh_q40_matmul_partial")
+    return PartialProduct(out, ks, M, n_total)
+
+
+def partial_reduce(p: PartialProduct, col0: int = 0, N: Optional[int] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
+    lib = _lib.load()
+    N = p.n_total - col0 if N is None else N
+    c = torch.empty((p.M, N), dtype=torch.float16, device=p.buf.device)
+    epi = SMH_EPI_NONE
+    if residual is not None:
+        assert residual.shape == (p.M, N) and residual.is_contiguous() and residual.dtype == torch.float16
+        epi = SMH_EPI_RESIDUAL
+    check(lib.smh_partial_reduce(p.buf.data_ptr(), p.ksplit, p.M, p.n_total, col0, N, c.data_ptr(), N, epi, _ptr(residual), N,
+                                 _stream()), "smh_partial_reduce")
+    return c
+
+
+def partial_rmsnorm(p: Optional[PartialProduct], h_in: Optional[torch.Tensor], weight: torch.Tensor, eps: float,
+                    want_h: bool = True):
+    """h = h_in + fp16(product) (either may be absent), xn = RMSNorm(h) * weight.  Returns (h, xn)."""
+    lib = _lib.load()
+    ref = h_in if h_in is not None else None
+    if p is not None:
+        M, N = p.M, p.n_total
+        dev = p.buf.device
+    else:
+        M, N = ref.shape
+        dev = ref.device
+    if h_in is not None:
+        assert h_in.shape == (M, N) and h_in.is_contiguous() and h_in.dtype == torch.float16
+    assert weight.numel() == N and weight.dtype == torch.float16
+    h = torch.empty((M, N), dtype=torch.float16, device=dev) if (want_h and p is not None) else None
+    xn = torch.empty((M, N), dtype=torch.float16, device=dev)
+    check(lib.smh_partial_rmsnorm(p.buf.data_ptr() if p is not None else None, p.ksplit if p is not None else 1, M, N,
+                                  _ptr(h_in), weight.data_ptr(), float(eps), _ptr(h), xn.data_ptr(), _stream()),
+          "smh_partial_rmsnorm")
+    return (h if h is not None else h_in), xn
+
+
+def partial_silu_mul(p: PartialProduct) -> torch.Tensor:
+    lib = _lib.load()
+    n_half = p.n_total // 2
+    out = torch.empty((p.M, n_half), dtype=torch.float16, device=p.buf.device)
+    check(lib.smh_partial_silu_mul(p.buf.data_ptr(), p.ksplit, p.M, n_half, out.data_ptr(), _stream()), "smh_partial_silu_mul")
+    return out
+
+
+def partial_rope_append_kv(p: PartialProduct, H: int, Hkv: int, D: int, cos: torch.Tensor, sin: torch.Tensor,
+                           pos_dev: torch.Tensor, cache_k, cache_ks, cache_v, cache_vs, Smax: int, t_dev):
+    """q|k|v product -> fp16 q [B,H,D], k, v [B,Hkv,D] with RoPE applied to q and k, plus the Q4_0
+    append of k and v into row t_dev[0] of each branch's suffix cache."""
+    lib = _lib.load()
+    B = p.M
+    assert p.n_total == (H + 2 * Hkv) * D
+    dev = p.buf.device
+    q = torch.empty((B, H, D), dtype=torch.float16, device=dev)
+    k = torch.empty((B, Hkv, D), dtype=torch.float16, device=dev)
+    v = torch.empty((B, Hkv, D), dtype=torch.float16, device=dev)
+    check(lib.smh_partial_rope_append_kv(p.buf.data_ptr(), p.ksplit, B, H, Hkv, D, q.data_ptr(), k.data_ptr(), v.data_ptr(),
+                                         cos.data_ptr(), sin.data_ptr(), pos_dev.data_ptr(), _ptr(cache_k), _ptr(cache_ks),
+                                         _ptr(cache_v), _ptr(cache_vs), int(Smax), _ptr(t_dev), _stream()),
+          "smh_partial_rope_append_kv")
+    return q, k, v
 
 
 # ---------------------------------------------------------------------------------------------

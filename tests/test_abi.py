@@ -36,7 +36,12 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert st < 0 and b"even" in lib.smh_last_error_string()
     with pytest.raises(_lib.SmhError):
         _lib.check(st, "smh_q40_quantize")
-    assert lib.smh_q40_matmul_workspace_bytes(16, 4096) >= 16384 + 16 * 131072 * 4
+    assert lib.smh_q40_matmul_workspace_bytes(16, 4096) >= 16 * 16 * 4096 * 4
+    import ctypes
+    n = (ctypes.c_int * 3)(4096, 4096, 4096)
+    ks = lib.smh_q40_matmul_plan(1, 4096, 3, n)
+    assert 1 <= ks <= 16
+    assert lib.smh_q40_matmul_plan(1, 4096, 1, (ctypes.c_int * 1)(100)) < 0      # N not a multiple of 128
     assert lib.smh_attn_workspace_bytes(64, 32, 1024) >= 32 * 64 * 32 * 130 * 4
 
 

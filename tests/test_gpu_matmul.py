@@ -134,3 +134,64 @@ def test_argument_errors():
         K.matmul_q40(a.t().contiguous().t(), w.cuda(), s.cuda(), (64, 128))  # non-contiguous A
     with pytest.raises(AssertionError):
         K.matmul_q40(a.cpu(), w, s, (64, 128))                            # no CPU fallback
+
+
+@pytest.mark.parametrize("M", [1, 10, 100])
+def test_fused_segments_and_consumers(M):
+    """wq|wk|wv and w1|w3 as segments of one launch; slab consumers against the oracle's cast points"""
+    from spec_mcts_amd import kernels as K
+    Kd = 1024
+    ws = [_weights(n, Kd, 50 + i) for i, n in enumerate((512, 256, 256))]
+    a = _acts(M, Kd, 60 + M)
+    lin = [(w.cuda(), s.cuda(), n) for (w, s), n in zip(ws, (512, 256, 256))]
+    pp = K.matmul_q40_partial(a.cuda(), lin)
+    assert pp.n_total == 1024 and pp.M == M
+    want = torch.cat([O.matmul_q40(a, w, s, (Kd, n)) for (w, s), n in zip(ws, (512, 256, 256))], 1)
+    got = K.partial_reduce(pp)
+    _check(got, want)
+    # column windows and the residual epilogue
+    r = _acts(M, 256, 70)
+    _check(K.partial_reduce(pp, 512, 256, residual=r.cuda()), r + want[:, 512:768])
+    # SiLU(gate) * up with gate = columns [0,512), up = columns [512,1024)
+    got_act = K.partial_silu_mul(pp).cpu()
+    g16, u16 = got[:, :512].cpu(), got[:, 512:].cpu()
+    want_act = O.silu_mul(g16, u16)
+    assert torch.allclose(got_act.float(), want_act.float(), rtol=2e-3, atol=1e-4)
+    # residual + RMSNorm consumer on a [M, 1024] product
+    wt = (1 + 0.1 * torch.randn(1024, generator=torch.Generator().manual_seed(71))).to(torch.float16)
+    hin = _acts(M, 1024, 72)
+    h, xn = K.partial_rmsnorm(pp, hin.cuda(), wt.cuda(), 1e-5)
+    h_want = hin + got.cpu()
+    assert torch.equal(h.cpu(), h_want)
+    xn_want = O.rmsnorm(h_want, wt, 1e-5)
+    assert torch.allclose(xn.cpu().float(), xn_want.float(), rtol=2e-3, atol=1e-4)
+    assert (xn.cpu() != xn_want).float().mean() < 0.01
+
+
+def test_fused_rope_append_consumer_bit_exact():
+    from spec_mcts_amd import kernels as K
+    B, H, Hkv, D, Kd, Smax = 3, 4, 2, 128, 512, 4
+    ws = [_weights(n, Kd, 80 + i, std=0.05) for i, n in enumerate((H * D, Hkv * D, Hkv * D))]
+    a = _acts(B, Kd, 83)
+    lin = [(w.cuda(), s.cuda(), n) for (w, s), n in zip(ws, (H * D, Hkv * D, Hkv * D))]
+    pp = K.matmul_q40_partial(a.cuda(), lin)
+    flat = K.partial_reduce(pp).cpu()
+    q0 = flat[:, :H * D].view(B, 1, H, D); k0 = flat[:, H * D:(H + Hkv) * D].view(B, 1, Hkv, D)
+    v0 = flat[:, (H + Hkv) * D:].view(B, Hkv, D)
+    fc = O.precompute_freqs_cis(D, 32, 1e6)
+    pos, t = 9, 2
+    qe, ke = O.apply_rotary_emb(q0, k0, fc[pos:pos + 1])
+    cos, sin = fc.real.to(torch.float16).contiguous().cuda(), fc.imag.to(torch.float16).contiguous().cuda()
+    rows = B * Smax * Hkv
+    ck = torch.zeros((rows, 64), dtype=torch.int8).cuda(); cks = torch.zeros((rows * 2, 1), dtype=torch.float16).cuda()
+    cv = torch.zeros((rows, 64), dtype=torch.int8).cuda(); cvs = torch.zeros((rows * 2, 1), dtype=torch.float16).cuda()
+    st = torch.tensor([pos, t], dtype=torch.int32).cuda()
+    q, k, v = K.partial_rope_append_kv(pp, H, Hkv, D, cos, sin, st[0:1], ck, cks, cv, cvs, Smax, st[1:2])
+    assert torch.equal(q.cpu().view(torch.int16), qe[:, 0].view(torch.int16))
+    assert torch.equal(k.cpu().view(torch.int16), ke[:, 0].view(torch.int16))
+    assert torch.equal(v.cpu().view(torch.int16), v0.view(torch.int16))
+    wk, sk = O.quantize_q40(ke[:, 0], 64); wv, sv = O.quantize_q40(v0, 64)
+    assert torch.equal(ck.cpu().view(B, Smax, Hkv, 64)[:, t], wk.view(B, Hkv, 64))
+    assert torch.equal(cv.cpu().view(B, Smax, Hkv, 64)[:, t], wv.view(B, Hkv, 64))
+    assert torch.equal(cks.cpu().view(B, Smax, Hkv, 2)[:, t].view(torch.int16), sk.view(B, Hkv, 2).view(torch.int16))
+    assert torch.equal(cvs.cpu().view(B, Smax, Hkv, 2)[:, t].view(torch.int16), sv.view(B, Hkv, 2).view(torch.int16))

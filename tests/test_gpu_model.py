@@ -97,3 +97,21 @@ def test_generate_greedy_and_sampling_api():
     torch.manual_seed(0)
     res2, _ = model.generate(prompt, 2, 4, temperature=0.8, top_k=8)
     assert res2.shape[0] == 2 and int(res2.max()) < SMALL["vocab_size"]
+
+
+def test_fused_and_module_paths_are_bit_identical():
+    """the fused launches (slab consumers) round at the same points as the module-by-module path"""
+    oargs, sd, model = _build(GQA, 36)
+    prompt = torch.randint(0, GQA["vocab_size"], (1, 13), generator=torch.Generator().manual_seed(136)).cuda()
+    outs = {}
+    for fused in (True, False):
+        model.fused = fused
+        model.resetSeq()
+        a = model(prompt, 0)
+        nxt = a[:, -1].float().argmax(-1, keepdim=True).expand(3, 1).contiguous()
+        b = model(nxt, 13)
+        c = model(nxt, 14)
+        outs[fused] = (a.clone(), b.clone(), c.clone())
+    model.fused = True
+    for x, y in zip(outs[True], outs[False]):
+        assert torch.equal(x, y)
