@@ -10,7 +10,7 @@ import os
 from ctypes import c_char_p, c_float, c_int, c_long, c_size_t, c_void_p
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libsmh.so")
+LIB_PATH = os.environ.get("SMH_LIB", os.path.join(HERE, "libsmh.so"))
 
 SMH_EPI_NONE, SMH_EPI_RESIDUAL = 0, 1
 SMH_KV_NONE, SMH_KV_FP16, SMH_KV_Q40 = 0, 1, 2

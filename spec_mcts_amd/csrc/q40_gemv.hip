@@ -32,67 +32,118 @@ namespace smh {
 
 constexpr int GEMV_COLS = 256;             // columns per workgroup
 
-// registers of one 32-row step of one lane
-struct GemvStep {
-    u32x2 wv[8];     // 8 bytes of 8 consecutive rows
-    uint32_t sv[8];  // (scale of columns 0..63, scale of columns 64..127) of this lane's block, per row
-    h8 av;           // 8 activations of batch row c
+// ---- per-wave ring of 32-row steps in LDS ----------------------------------------------------------
+// The loads of a step go straight from global memory to LDS (global_load_lds, no VGPRs held while
+// they are in flight): 4 x 1 KB of packed nibbles (8 rows x 128 B each), the step's 32 x 4 scales
+// and the 16 x 32 tile of activations.  A wave keeps RING_STAGES steps in flight,
+// which is what hides the HBM latency; it needs no barrier in its main loop because the ring is
+// private to the wave (vmcnt orders the DMA against the wave's own LDS reads).
+#ifndef SMH_RING_STAGES
+#define SMH_RING_STAGES 3
+#endif
+constexpr int RING_STAGES = SMH_RING_STAGES;
+constexpr int STAGE_W_BYTES = 32 * 128;
+constexpr int STAGE_S_BYTES = 32 * 8;
+constexpr int STAGE_X_BYTES = 16 * 64;
+constexpr int STAGE_BYTES = STAGE_W_BYTES + STAGE_S_BYTES + STAGE_X_BYTES;   // 5376
+constexpr int RING_BYTES = RING_STAGES * STAGE_BYTES;                        // 16128 per wave
+
+typedef const __attribute__((address_space(1))) void *gptr_t;
+typedef __attribute__((address_space(3))) void *lptr_t;
+
+struct GemvLane {
+    const uint8_t *w_lane;   // weight address of this lane for row 0 of a step's first 8-row group
+    const half_t *s_lane;    // scale address of this lane for row 0 of a step
+    const half_t *x_lane;    // activation address of this lane for column 0 of a step
+    long w_row, s_row;       // row pitches: bytes / halves
+    int K;
 };
 
-__device__ __forceinline__ void gemv_load(GemvStep &st, int K, const uint8_t *wp, const half_t *sp,
-                                          const half_t *ap, long w_row, long s_row, int k0) {
+// 6 vector-memory instructions per step
+__device__ __forceinline__ void gemv_issue(const GemvLane &L, uint8_t *stage, int step, int lane) {
+    const int k0 = step * 32;
 #pragma unroll
-    for (int i = 0; i < 8; ++i) {
-        const int k = min(k0 + i, K - 1);
-        st.wv[i] = *reinterpret_cast<const u32x2 *>(wp + (long)k * w_row);
-        st.sv[i] = *reinterpret_cast<const uint32_t *>(sp + (long)k * s_row);
+    for (int j = 0; j < 4; ++j) {
+        const int row = min(k0 + 8 * j + (lane >> 3), L.K - 1);
+        __builtin_amdgcn_global_load_lds((gptr_t)(L.w_lane + (long)row * L.w_row), (lptr_t)(stage + j * 1024), 16, 0, 0);
     }
-    if (k0 < K) {
-        st.av = *reinterpret_cast<const h8 *>(ap + k0);
-    } else {
-#pragma unroll
-        for (int i = 0; i < 8; ++i) st.av[i] = (half_t)0.f;
+    {
+        // lane -> (row = lane / 2, block = lane % 2): one dword = (scale of columns 0..63, 64..127) of that block
+        const int row = min(k0 + (lane >> 1), L.K - 1);
+        __builtin_amdgcn_global_load_lds((gptr_t)(L.s_lane + (long)row * L.s_row), (lptr_t)(stage + STAGE_W_BYTES), 4, 0, 0);
+    }
+    {
+        const int col = min(k0 + 8 * (lane & 3), L.K - 8);
+        __builtin_amdgcn_global_load_lds((gptr_t)(L.x_lane + col), (lptr_t)(stage + STAGE_W_BYTES + STAGE_S_BYTES), 16, 0, 0);
     }
 }
 
-// acc[d][h][b]: dword d of the lane's 8 bytes, nibble half h (0 = high = columns 0..63 of the block),
-// byte b of the dword
-__device__ __forceinline__ void gemv_compute(const GemvStep &st, f4 (&acc)[2][2][4]) {
-    h2 s_hi[4], s_lo[4];
+// Decoding without a per-weight multiply or subtract.  With u = nibble ^ 8 = code + 8:
+//   high nibble: (bits & 0x00F0) | 0x5400 is the fp16 number 64 + u,   code = (64 + u) - 72
+//   low  nibble: (bits & 0x000F) | 0x6400 is the fp16 number 1024 + u, code = (1024 + u) - 1032
+// These offset codes go into the matrix core as they are.  The scales move to the other operand,
+// A[m][k] = fp16(x[m][k] * s[k]) for the (block, nibble half) the 16 columns of an MFMA share, and the
+// offsets are taken out at the end:  sum_k A (v - off) = sum_k A v - off * sum_k A,  where sum_k A
+// comes from one more MFMA per (block, half) against a B operand of ones.
+// acc[blk][h][b]: column 128*blk + 64*h + 4c + b;  corr[blk*2 + h] = sum_k A.
+__device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K, int c, int g,
+                                             f4 (&acc)[2][2][4], f4 (&corr)[4]) {
+    uint32_t u0[8], u1[8];
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        s_hi[j] = as_h2(pack_lo16(st.sv[2 * j], st.sv[2 * j + 1]));
-        s_lo[j] = as_h2(pack_hi16(st.sv[2 * j], st.sv[2 * j + 1]));
+    for (int i = 0; i < 8; ++i) {
+        u0[i] = *reinterpret_cast<const uint32_t *>(stage + (8 * g + i) * 128 + 4 * c) ^ NIBBLE_FLIP;
+        u1[i] = *reinterpret_cast<const uint32_t *>(stage + (8 * g + i) * 128 + 64 + 4 * c) ^ NIBBLE_FLIP;
     }
+    h8 xv = *reinterpret_cast<const h8 *>(stage + STAGE_W_BYTES + STAGE_S_BYTES + c * 64 + 16 * g);
+    if (k0 + 8 * g >= K) {
 #pragma unroll
-    for (int d = 0; d < 2; ++d) {
-        uint32_t u[8];
+        for (int i = 0; i < 8; ++i) xv[i] = (half_t)0.f;
+    }
+    // scales of this lane's 8 rows: sv[i] = ((hi, lo) of block 0, (hi, lo) of block 1); regroup them per
+    // (block, half) into the k-pair order of xv and scale the activations
+    u32x2 sv[8];
 #pragma unroll
-        for (int i = 0; i < 8; ++i) u[i] = st.wv[i][d] ^ NIBBLE_FLIP;
-#define SMH_GEMV_BYTE(B)                                                                        \
-        {                                                                                       \
-            h2 bh[4], bl[4];                                                                    \
-            _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                     \
-                uint32_t pr = pair_bytes<B>(u[2 * j], u[2 * j + 1]);                            \
-                bh[j] = codes_high(pr) * s_hi[j];                                               \
-                bl[j] = codes_low(pr) * s_lo[j];                                                \
-            }                                                                                   \
-            h8 vb_h = {bh[0].x, bh[0].y, bh[1].x, bh[1].y, bh[2].x, bh[2].y, bh[3].x, bh[3].y}; \
-            h8 vb_l = {bl[0].x, bl[0].y, bl[1].x, bl[1].y, bl[2].x, bl[2].y, bl[3].x, bl[3].y}; \
-            acc[d][0][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(st.av, vb_h, acc[d][0][B], 0, 0, 0); \
-            acc[d][1][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(st.av, vb_l, acc[d][1][B], 0, 0, 0); \
+    for (int i = 0; i < 8; ++i) sv[i] = *reinterpret_cast<const u32x2 *>(stage + STAGE_W_BYTES + (8 * g + i) * 8);
+    h8 a[4];
+#pragma unroll
+    for (int blk = 0; blk < 2; ++blk) {
+        u32x4 s_hi, s_lo;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            s_hi[j] = pack_lo16(sv[2 * j][blk], sv[2 * j + 1][blk]);
+            s_lo[j] = pack_hi16(sv[2 * j][blk], sv[2 * j + 1][blk]);
         }
-        SMH_GEMV_BYTE(0)
-        SMH_GEMV_BYTE(1)
-        SMH_GEMV_BYTE(2)
-        SMH_GEMV_BYTE(3)
-#undef SMH_GEMV_BYTE
+        a[2 * blk] = xv * __builtin_bit_cast(h8, s_hi);
+        a[2 * blk + 1] = xv * __builtin_bit_cast(h8, s_lo);
     }
+    const h8 ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
+#pragma unroll
+    for (int bh = 0; bh < 4; ++bh) corr[bh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[bh], ones, corr[bh], 0, 0, 0);
+#define SMH_GEMV_BYTE(U, BLK, B)                                                                 \
+    {                                                                                            \
+        u32x4 vh, vl;                                                                            \
+        _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                          \
+            const uint32_t pr = pair_bytes<B>(U[2 * j], U[2 * j + 1]);                           \
+            vh[j] = (pr & 0x00F000F0u) | 0x54005400u;                                            \
+            vl[j] = (pr & 0x000F000Fu) | 0x64006400u;                                            \
+        }                                                                                        \
+        acc[BLK][0][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * BLK], __builtin_bit_cast(h8, vh), acc[BLK][0][B], 0, 0, 0);     \
+        acc[BLK][1][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * BLK + 1], __builtin_bit_cast(h8, vl), acc[BLK][1][B], 0, 0, 0); \
+    }
+    SMH_GEMV_BYTE(u0, 0, 0)
+    SMH_GEMV_BYTE(u0, 0, 1)
+    SMH_GEMV_BYTE(u0, 0, 2)
+    SMH_GEMV_BYTE(u0, 0, 3)
+    SMH_GEMV_BYTE(u1, 1, 0)
+    SMH_GEMV_BYTE(u1, 1, 1)
+    SMH_GEMV_BYTE(u1, 1, 2)
+    SMH_GEMV_BYTE(u1, 1, 3)
+#undef SMH_GEMV_BYTE
 }
 
 template <int WAVES>
 __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
-    extern __shared__ float red[];          // [WAVES][M][256]
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // WAVES rings, then reused as red[WAVES][M][256]
     constexpr int THREADS = WAVES * 64;
 
     const int unit = blockIdx.x % p.units_pad;
@@ -110,42 +161,61 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     const int lane = tid & 63;
     const int c = lane & 15;
     const int g = lane >> 4;
-
-    const long w_row = seg.N / 2;          // bytes per k
-    const long s_row = seg.N / 64;         // scales per k
     const int col0 = pair * GEMV_COLS;     // first column (inside the segment) of this workgroup
-    // lanes c >= 8 belong to the second block of the pair; when N/128 is odd the last pair has none:
-    // such lanes re-read the first block (valid memory) and their results are dropped
-    const bool has_block = col0 + 128 * (c >> 3) < seg.N;
-    const int c_ld = has_block ? c : (c & 7);
-    const uint8_t *wp = seg.w + (long)pair * 128 + 8 * c_ld;
-    const half_t *sp = seg.s + (long)pair * 4 + 2 * (c_ld >> 3);
-    const int m_a = min(c, p.M - 1);       // row of A this lane feeds (rows >= M are never stored)
-    const half_t *ap = p.a + (long)m_a * p.lda;
+    // when N/128 is odd the last pair has no second block: its loads re-read the first block (valid
+    // memory) and the results of those columns are dropped
+    const bool two_blocks = col0 + 128 < seg.N;
 
-    f4 acc[2][2][4];
+    GemvLane L;
+    L.K = p.K;
+    L.w_row = seg.N / 2;
+    L.s_row = seg.N / 64;
+    {
+        const int chunk = lane & 7;                                   // 16-byte chunk of the 128-byte line
+        L.w_lane = seg.w + (long)pair * 128 + 16 * (two_blocks ? chunk : (chunk & 3));
+        L.s_lane = seg.s + (long)pair * 4 + 2 * (two_blocks ? (lane & 1) : 0);
+        L.x_lane = p.a + (long)min(lane >> 2, p.M - 1) * p.lda;
+    }
+    uint8_t *ring = lds + wave * RING_BYTES;
+
+    f4 acc[2][2][4], corr[4];
 #pragma unroll
     for (int d = 0; d < 2; ++d)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int b = 0; b < 4; ++b) acc[d][h][b] = f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int bh = 0; bh < 4; ++bh) corr[bh] = f4{0.f, 0.f, 0.f, 0.f};
 
+    // this wave's steps: first, first + WAVES, ...
     const int step0 = slice * p.steps_per_slice;
     const int step1 = min(step0 + p.steps_per_slice, (p.K + 31) / 32);
-    for (int step = step0 + 2 * wave; step < step1; step += 2 * WAVES) {
-        GemvStep s0, s1;
-        gemv_load(s0, p.K, wp, sp, ap, w_row, s_row, step * 32 + 8 * g);
-        const bool two = step + 1 < step1;
-        if (two) gemv_load(s1, p.K, wp, sp, ap, w_row, s_row, (step + 1) * 32 + 8 * g);
-        gemv_compute(s0, acc);
-        if (two) gemv_compute(s1, acc);
+    const int first = step0 + wave;
+    const int n_steps = first < step1 ? (step1 - first + WAVES - 1) / WAVES : 0;
+#pragma unroll
+    for (int i = 0; i < RING_STAGES; ++i)
+        if (i < n_steps) gemv_issue(L, ring + i * STAGE_BYTES, first + i * WAVES, lane);
+    int stage = 0;
+    for (int i = 0; i < n_steps; ++i) {
+        const int later = min(RING_STAGES - 1, n_steps - 1 - i);     // steps issued after step i and still in flight
+        if (later >= 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
+        else if (later == 1) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        const int step = first + i * WAVES;
+        gemv_consume(ring + stage * STAGE_BYTES, step * 32, p.K, c, g, acc, corr);
+        if (i + RING_STAGES < n_steps) {
+            asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");        // this stage's LDS reads are done
+            gemv_issue(L, ring + stage * STAGE_BYTES, first + (i + RING_STAGES) * WAVES, lane);
+        }
+        stage = (stage + 1 == RING_STAGES) ? 0 : stage + 1;
     }
+    __syncthreads();                        // every wave is done with its ring: reuse LDS for the sums
 
     // ---- add the waves' partial sums through LDS ----
-    // accumulator element r of acc[d][h][b] in lane (g, c) is row m = 4g + r,
-    // column 128*(c>>3) + 64h + 8*(c&7) + 4d + b of the workgroup's 256
-    const int col_lane = 128 * (c >> 3) + 8 * (c & 7);
+    // accumulator element r of acc[blk][h][b] in lane (g, c) is row m = 4g + r,
+    // column 128*blk + 64h + 4c + b of the workgroup's 256; the nibble offsets (72 / 1032) leave here
+    float *red = reinterpret_cast<float *>(lds);
 #pragma unroll
     for (int d = 0; d < 2; ++d)
 #pragma unroll
@@ -155,7 +225,9 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
                     const int m = 4 * g + r;
-                    if (m < p.M) red[(wave * p.M + m) * GEMV_COLS + col_lane + 64 * h + 4 * d + b] = acc[d][h][b][r];
+                    const float off = h ? 1032.f : 72.f;
+                    if (m < p.M)
+                        red[(wave * p.M + m) * GEMV_COLS + 128 * d + 64 * h + 4 * c + b] = acc[d][h][b][r] - off * corr[2 * d + h][r];
                 }
     __syncthreads();
 
@@ -183,28 +255,26 @@ int env_int(const char *name, int dflt) {
     return v ? atoi(v) : dflt;
 }
 
-// K is cut into at most SMH_MAX_KSPLIT slices so that about `target` workgroups are in flight
-// (256 CUs) while every wave still has a pair of steps to do.
+// K is cut into slices so that the launch fills the GPU in ONE round of workgroups: two
+// workgroups (two sets of LDS rings) fit a CU, 256 CUs, so at most 512 workgroups; a launch of a
+// few more than that would run a second, nearly empty round and take twice as long.
 void gemv_plan(int n_total_units, int K, int waves, int *ksplit, int *steps_per_slice) {
     const int steps = (K + 31) / 32;
-    static const int target_wgs = env_int("SMH_GEMV_WGS", 512);
-    const int unit = 2 * waves;
-    int want = (target_wgs + n_total_units - 1) / n_total_units;
-    int max_split = (steps + unit - 1) / unit;
-    int ks = want < 1 ? 1 : want;
-    if (ks > max_split) ks = max_split;
+    static const int capacity = env_int("SMH_GEMV_WGS", 512);
+    int ks = capacity / n_total_units;              // floor: never exceed one round
+    if (ks < 1) ks = 1;
     if (ks > SMH_MAX_KSPLIT) ks = SMH_MAX_KSPLIT;
-    int sps = (steps + ks - 1) / ks;
-    sps = (sps + unit - 1) / unit * unit;
-    ks = (steps + sps - 1) / sps;
-    *ksplit = ks;
+    int max_split = (steps + waves - 1) / waves;    // every wave should have a step
+    if (ks > max_split) ks = max_split;
+    const int sps = (steps + ks - 1) / ks;
+    *ksplit = (steps + sps - 1) / sps;
     *steps_per_slice = sps;
 }
 
 int gemv_waves(int M) {
     static const int waves_pref = env_int("SMH_GEMV_WAVES", 4);
     int waves = waves_pref;
-    while (waves > 2 && (size_t)waves * M * GEMV_COLS * sizeof(float) > 48 * 1024) waves >>= 1;   // LDS budget
+    (void)M;
     return waves;
 }
 
@@ -225,7 +295,9 @@ void gemv_fill_plan(MatmulParams &p) {
 int gemv_launch(const MatmulParams &p, hipStream_t stream) {
     const int waves = gemv_waves(p.M);
     dim3 grid((unsigned)(p.units_pad * p.ksplit));
-    size_t lds = (size_t)waves * p.M * GEMV_COLS * sizeof(float);
+    size_t lds = (size_t)waves * RING_BYTES;                       // rings, reused for the [waves][M][256] sums
+    const size_t red = (size_t)waves * p.M * GEMV_COLS * sizeof(float);
+    if (red > lds) lds = red;
     if (waves == 2) hipLaunchKernelGGL(q40_gemv_kernel<2>, grid, dim3(128), lds, stream, p);
     else if (waves == 8) hipLaunchKernelGGL(q40_gemv_kernel<8>, grid, dim3(512), lds, stream, p);
     else hipLaunchKernelGGL(q40_gemv_kernel<4>, grid, dim3(256), lds, stream, p);
