@@ -240,12 +240,12 @@ extern "C" int smh_q40_matmul_plan(int M, int K, int nseg, const int *n) {
 }
 
 extern "C" size_t smh_q40_matmul_workspace_bytes(int max_m, int max_n) {
-    // K is split only while (column units x row blocks) < 512, so the slabs never exceed
-    // 512 tiles of 128 x 128 floats for the GEMM, or SMH_MAX_KSPLIT x 16 x N floats for the GEMV
+    // K is split only while (column units x row blocks) <= 512, so the slabs never exceed
+    // 512 tiles of 128 x 256 floats for the GEMM, or SMH_MAX_KSPLIT x 16 x N floats for the GEMV
     size_t n = (size_t)(max_n < 128 ? 128 : max_n);
     size_t m = (size_t)(max_m < 1 ? 1 : (max_m > SMH_GEMV_MAX_M ? SMH_GEMV_MAX_M : max_m));
     size_t floats = n * m * SMH_MAX_KSPLIT;
-    if (max_m > SMH_GEMV_MAX_M && floats < (size_t)640 * 128 * 128) floats = (size_t)640 * 128 * 128;
+    if (max_m > SMH_GEMV_MAX_M && floats < (size_t)512 * 128 * 256) floats = (size_t)512 * 128 * 256;
     return floats * sizeof(float) + 256;
 }
 
@@ -304,6 +304,7 @@ static int matmul_fp16(const void *a, int M, int K, long lda, const void *b_w, c
     p.c = (half_t *)c; p.ldc = ldc; p.resid = (const half_t *)residual; p.ldr = ldr; p.epilogue = epilogue;
     if (p.ksplit == 1) {
         p.direct = 1;
+        SMH_REQUIRE(!gemm || ldc % 8 == 0, "%s: ldc=%ld must be a multiple of 8 for M > 16", who, ldc);
         return gemm ? gemm_launch(p, (hipStream_t)stream) : gemv_launch(p, (hipStream_t)stream);
     }
     size_t need = (size_t)p.ksplit * M * N * sizeof(float);

@@ -52,31 +52,57 @@ typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
 struct GemvLane {
-    const uint8_t *w_lane;   // weight address of this lane for row 0 of a step's first 8-row group
-    const half_t *s_lane;    // scale address of this lane for row 0 of a step
-    const half_t *x_lane;    // activation address of this lane for column 0 of a step
-    long w_row, s_row;       // row pitches: bytes / halves
-    int K;
+    const uint8_t *w_base;   // uniform: row 0 of this workgroup's 128-byte column
+    const uint8_t *s_base;   // uniform: row 0 of its scales
+    const uint8_t *x_base;   // uniform: the activations
+    uint32_t w_off, s_off, x_off;   // this lane's byte offsets inside a step
+    long w_row, s_row;       // row pitches in bytes
+    int K, lane;
+    bool two_blocks;
+    int m_row;
 };
 
-// 6 vector-memory instructions per step
-__device__ __forceinline__ void gemv_issue(const GemvLane &L, uint8_t *stage, int step, int lane) {
+// 6 vector-memory instructions per step.  For a full step the address is a uniform base (scalar
+// registers, advanced by scalar arithmetic) plus a per-lane offset that never changes; only the
+// last step of a K that is not a multiple of 32 clamps rows per lane.
+template <bool RAGGED>
+__device__ __forceinline__ void gemv_issue(const GemvLane &L, uint8_t *stage, int step) {
     const int k0 = step * 32;
+    if constexpr (!RAGGED) {
+        const uint8_t *wb = L.w_base + (long)k0 * L.w_row;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-        const int row = min(k0 + 8 * j + (lane >> 3), L.K - 1);
-        __builtin_amdgcn_global_load_lds((gptr_t)(L.w_lane + (long)row * L.w_row), (lptr_t)(stage + j * 1024), 16, 0, 0);
-    }
-    {
+        for (int j = 0; j < 4; ++j)
+            __builtin_amdgcn_global_load_lds((gptr_t)(wb + (long)(8 * j) * L.w_row + L.w_off), (lptr_t)(stage + j * 1024), 16, 0, 0);
         // lane -> (row = lane / 2, block = lane % 2): one dword = (scale of columns 0..63, 64..127) of that block
-        const int row = min(k0 + (lane >> 1), L.K - 1);
-        __builtin_amdgcn_global_load_lds((gptr_t)(L.s_lane + (long)row * L.s_row), (lptr_t)(stage + STAGE_W_BYTES), 4, 0, 0);
-    }
-    {
-        const int col = min(k0 + 8 * (lane & 3), L.K - 8);
-        __builtin_amdgcn_global_load_lds((gptr_t)(L.x_lane + col), (lptr_t)(stage + STAGE_W_BYTES + STAGE_S_BYTES), 16, 0, 0);
+        __builtin_amdgcn_global_load_lds((gptr_t)(L.s_base + (long)k0 * L.s_row + L.s_off), (lptr_t)(stage + STAGE_W_BYTES), 4, 0, 0);
+        // lane -> (batch row = lane / 4, 8 k-values at 8 * (lane % 4))
+        __builtin_amdgcn_global_load_lds((gptr_t)(L.x_base + 2 * k0 + L.x_off), (lptr_t)(stage + STAGE_W_BYTES + STAGE_S_BYTES), 16, 0, 0);
+    } else {
+        const int lane = L.lane;
+        const int chunk = L.two_blocks ? (lane & 7) : (lane & 3);
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int row = min(k0 + 8 * j + (lane >> 3), L.K - 1);
+            __builtin_amdgcn_global_load_lds((gptr_t)(L.w_base + (long)row * L.w_row + 16 * chunk), (lptr_t)(stage + j * 1024), 16, 0, 0);
+        }
+        {
+            const int row = min(k0 + (lane >> 1), L.K - 1);
+            __builtin_amdgcn_global_load_lds((gptr_t)(L.s_base + (long)row * L.s_row + (L.two_blocks ? 4 * (lane & 1) : 0)),
+                                             (lptr_t)(stage + STAGE_W_BYTES), 4, 0, 0);
+        }
+        {
+            const int col = min(k0 + 8 * (lane & 3), L.K - 8);
+            __builtin_amdgcn_global_load_lds((gptr_t)(L.x_base + (long)L.m_row + 2 * col), (lptr_t)(stage + STAGE_W_BYTES + STAGE_S_BYTES), 16, 0, 0);
+        }
     }
 }
+
+// The two masks and the two fp16 magic numbers of the decoder, held in registers the compiler cannot
+// see through: (bits & mask) | magic then becomes ONE v_and_or_b32 (that instruction takes no
+// literal operands, so with visible constants the compiler emits an AND and an OR).
+struct GemvConsts {
+    uint32_t mask_hi, mask_lo, magic_hi, magic_lo;
+};
 
 // Decoding without a per-weight multiply or subtract.  With u = nibble ^ 8 = code + 8:
 //   high nibble: (bits & 0x00F0) | 0x5400 is the fp16 number 64 + u,   code = (64 + u) - 72
@@ -86,7 +112,8 @@ __device__ __forceinline__ void gemv_issue(const GemvLane &L, uint8_t *stage, in
 // offsets are taken out at the end:  sum_k A (v - off) = sum_k A v - off * sum_k A,  where sum_k A
 // comes from one more MFMA per (block, half) against a B operand of ones.
 // acc[blk][h][b]: column 128*blk + 64*h + 4c + b;  corr[blk*2 + h] = sum_k A.
-__device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K, int c, int g,
+template <bool RAGGED>
+__device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K, int c, int g, const GemvConsts &C,
                                              f4 (&acc)[2][2][4], f4 (&corr)[4]) {
     uint32_t u0[8], u1[8];
 #pragma unroll
@@ -95,9 +122,11 @@ __device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K
         u1[i] = *reinterpret_cast<const uint32_t *>(stage + (8 * g + i) * 128 + 64 + 4 * c) ^ NIBBLE_FLIP;
     }
     h8 xv = *reinterpret_cast<const h8 *>(stage + STAGE_W_BYTES + STAGE_S_BYTES + c * 64 + 16 * g);
-    if (k0 + 8 * g >= K) {
+    if constexpr (RAGGED) {
+        if (k0 + 8 * g >= K) {
 #pragma unroll
-        for (int i = 0; i < 8; ++i) xv[i] = (half_t)0.f;
+            for (int i = 0; i < 8; ++i) xv[i] = (half_t)0.f;
+        }
     }
     // scales of this lane's 8 rows: sv[i] = ((hi, lo) of block 0, (hi, lo) of block 1); regroup them per
     // (block, half) into the k-pair order of xv and scale the activations
@@ -124,8 +153,8 @@ __device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K
         u32x4 vh, vl;                                                                            \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                          \
             const uint32_t pr = pair_bytes<B>(U[2 * j], U[2 * j + 1]);                           \
-            vh[j] = (pr & 0x00F000F0u) | 0x54005400u;                                            \
-            vl[j] = (pr & 0x000F000Fu) | 0x64006400u;                                            \
+            vh[j] = (pr & C.mask_hi) | C.magic_hi;                                               \
+            vl[j] = (pr & C.mask_lo) | C.magic_lo;                                               \
         }                                                                                        \
         acc[BLK][0][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * BLK], __builtin_bit_cast(h8, vh), acc[BLK][0][B], 0, 0, 0);     \
         acc[BLK][1][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * BLK + 1], __builtin_bit_cast(h8, vl), acc[BLK][1][B], 0, 0, 0); \
@@ -157,7 +186,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     const int pair = unit - seg.unit0;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const int lane = tid & 63;
     const int c = lane & 15;
     const int g = lane >> 4;
@@ -168,15 +197,22 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
 
     GemvLane L;
     L.K = p.K;
+    L.lane = lane;
+    L.two_blocks = two_blocks;
     L.w_row = seg.N / 2;
-    L.s_row = seg.N / 64;
-    {
-        const int chunk = lane & 7;                                   // 16-byte chunk of the 128-byte line
-        L.w_lane = seg.w + (long)pair * 128 + 16 * (two_blocks ? chunk : (chunk & 3));
-        L.s_lane = seg.s + (long)pair * 4 + 2 * (two_blocks ? (lane & 1) : 0);
-        L.x_lane = p.a + (long)min(lane >> 2, p.M - 1) * p.lda;
-    }
+    L.s_row = seg.N / 32;
+    L.w_base = seg.w + (long)pair * 128;
+    L.s_base = reinterpret_cast<const uint8_t *>(seg.s) + (long)pair * 8;
+    L.x_base = reinterpret_cast<const uint8_t *>(p.a);
+    L.m_row = (int)(min(lane >> 2, p.M - 1) * p.lda * 2);
+    L.w_off = (uint32_t)((lane >> 3) * (seg.N / 2) + 16 * (two_blocks ? (lane & 7) : (lane & 3)));
+    L.s_off = (uint32_t)((lane >> 1) * (seg.N / 32) + (two_blocks ? 4 * (lane & 1) : 0));
+    L.x_off = (uint32_t)(L.m_row + 16 * (lane & 3));
     uint8_t *ring = lds + wave * RING_BYTES;
+
+    GemvConsts C{0x00F000F0u, 0x000F000Fu, 0x54005400u, 0x64006400u};
+    asm volatile("" : "+s"(C.mask_hi), "+s"(C.mask_lo));
+    asm volatile("" : "+v"(C.magic_hi), "+v"(C.magic_lo));
 
     f4 acc[2][2][4], corr[4];
 #pragma unroll
@@ -193,22 +229,33 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     const int step1 = min(step0 + p.steps_per_slice, (p.K + 31) / 32);
     const int first = step0 + wave;
     const int n_steps = first < step1 ? (step1 - first + WAVES - 1) / WAVES : 0;
+    const int full_steps = p.K / 32;        // steps below this index have all their 32 rows
+    auto issue = [&](uint8_t *stage, int step) {
+        if (step < full_steps) gemv_issue<false>(L, stage, step);
+        else gemv_issue<true>(L, stage, step);
+    };
 #pragma unroll
     for (int i = 0; i < RING_STAGES; ++i)
-        if (i < n_steps) gemv_issue(L, ring + i * STAGE_BYTES, first + i * WAVES, lane);
+        if (i < n_steps) issue(ring + i * STAGE_BYTES, first + i * WAVES);
+    // the one step that may lack rows is the last step of K, hence the last one of its wave; it is
+    // peeled off so that the loop has a single decoder in it
+    const int n_full = first < full_steps ? min(n_steps, (full_steps - first + WAVES - 1) / WAVES) : 0;
     int stage = 0;
-    for (int i = 0; i < n_steps; ++i) {
+    for (int i = 0; i < n_full; ++i) {
         const int later = min(RING_STAGES - 1, n_steps - 1 - i);     // steps issued after step i and still in flight
         if (later >= 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
         else if (later == 1) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        const int step = first + i * WAVES;
-        gemv_consume(ring + stage * STAGE_BYTES, step * 32, p.K, c, g, acc, corr);
+        gemv_consume<false>(ring + stage * STAGE_BYTES, 0, p.K, c, g, C, acc, corr);
         if (i + RING_STAGES < n_steps) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");        // this stage's LDS reads are done
-            gemv_issue(L, ring + stage * STAGE_BYTES, first + (i + RING_STAGES) * WAVES, lane);
+            issue(ring + stage * STAGE_BYTES, first + (i + RING_STAGES) * WAVES);
         }
         stage = (stage + 1 == RING_STAGES) ? 0 : stage + 1;
+    }
+    if (n_full < n_steps) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        gemv_consume<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, c, g, C, acc, corr);
     }
     __syncthreads();                        // every wave is done with its ring: reuse LDS for the sums
 

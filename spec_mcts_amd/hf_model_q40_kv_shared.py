@@ -345,6 +345,7 @@ class Transformer(nn.Module):
     @torch.inference_mode()
     def forward(self, tokens: torch.Tensor, start_pos: int):
         _bsz, seqlen = tokens.shape
+        K._need_gpu(tokens, self.tok_embeddings.weight)
         step_state = None
         if start_pos != 0:
             t = start_pos - self.layers[0].attention.cache_prompt_len

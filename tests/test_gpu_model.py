@@ -129,4 +129,3 @@ def test_fused_and_module_paths_agree():
     model.fused = True
     for x, y in zip(outs[True], outs[False]):
         assert torch.allclose(x.float(), y.float(), rtol=1e-2, atol=1e-2)
-        assert (x != y).float().mean() < 0.5
