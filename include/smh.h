@@ -163,6 +163,46 @@ int smh_shared_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int 
 int smh_prefill_attn(const void *q, const void *k, const void *v, void *out, int S, int H, int Hkv,
                      int D, smh_stream_t stream);
 
+/* ---- whole decode step ------------------------------------------------------------------------
+ * smh_decode_step: one decode step (start_pos != 0) of Transformer.forward
+ * (hf_model_q40_kv_shared.py:481-512) up to, not including, the final norm and lm_head, for
+ * 1..16 branches, as ONE persistent kernel: embedding, then per layer RMSNorm -> wq|wk|wv -> RoPE
+ * + Q4_0 KV append -> shared-prefix attention -> wo (+residual) -> RMSNorm -> w1|w3 -> SiLU*up ->
+ * w2 (+residual), i.e. TransformerBlock.forward (:456-467) with Attention.forward (:313-405) and
+ * FeedForward.forward (:431-436).  Same arithmetic and rounding points as the operator entry
+ * points above.  Multi-head attention only (H == Hkv); dim, ffn multiples of 256.
+ *   layers_dev  DEVICE array of n_layers descriptors; matrices in the order wq wk wv wo w1 w3 w2
+ *               (packed bytes w[i], fp16 scales s[i], checkpoint layout), norm weights fp16 [dim],
+ *               prefix_k/v fp16 [P, Hkv, 128], suffix cache as in smh_rope_append_kv
+ *   tokens      int64 [M] on the device;  emb fp16 [vocab, dim]
+ *   pos_dev, t_dev  int32 on the device: RoPE position and suffix row of this step
+ *   h_out       fp16 [M, dim]: hidden state after the last layer (input of the final norm)
+ *   workspace   smh_decode_step_workspace_bytes(...) bytes, 256-byte aligned, owned by the step
+ *               kernel from smh_decode_prepare on.
+ * smh_decode_prepare validates the configuration, clears the workspace and uploads the parameter
+ * block into it (synchronous; once per configuration, e.g. after each prefill).  smh_decode_step
+ * launches one step on `stream` (asynchronous, capturable in a graph); tokens, pos_dev, t_dev and
+ * the caches are read at execution time.  smh_decode_status copies three status words to the
+ * host (synchronous): [2] is nonzero if a bounded wait inside a step ran out - the workgroups of
+ * a launch must all be resident at once - and the results are then invalid.
+ * Steps that share a workspace must not overlap in time.
+ */
+typedef struct smh_decode_layer {
+    const void *w[7];
+    const void *s[7];
+    const void *attn_norm, *ffn_norm;
+    const void *prefix_k, *prefix_v;
+    void *cache_k, *cache_v;
+    void *cache_ks, *cache_vs;
+} smh_decode_layer;
+size_t smh_decode_step_workspace_bytes(int n_layers, int M, int dim, int H, int Hkv, int ffn, int P, int Smax);
+int smh_decode_prepare(const smh_decode_layer *layers_dev, int n_layers, int M, int dim, int H, int Hkv,
+                       int ffn, int P, int Smax, float eps, const int64_t *tokens, const void *emb,
+                       const void *cos_tab, const void *sin_tab, const int32_t *pos_dev,
+                       const int32_t *t_dev, void *h_out, void *workspace, size_t workspace_bytes);
+int smh_decode_step(void *workspace, smh_stream_t stream);
+int smh_decode_status(const void *workspace, uint32_t *status3);
+
 #ifdef __cplusplus
 }
 #endif

@@ -44,6 +44,11 @@ SIGNATURES = {
     "smh_shared_prefix_attn": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, c_int, _P, _P, _P, _P, c_int,
                                        _P, c_int, _P, _P, _P, c_size_t, _P]),
     "smh_prefill_attn": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
+    "smh_decode_step_workspace_bytes": (c_size_t, [c_int] * 8),
+    "smh_decode_prepare": (c_int, [_P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, _P, _P, _P, _P, _P, _P,
+                                   c_size_t]),
+    "smh_decode_step": (c_int, [_P, _P]),
+    "smh_decode_status": (c_int, [_P, _P]),
 }
 
 _lib = None

@@ -259,6 +259,8 @@ class Transformer(nn.Module):
         self._step_state = None       # int32 [2] on the device: (position, suffix index t)
         self._step_host = None
         self.fused = True             # fused decode-layer launches; False runs module by module
+        self.persistent = True        # decode steps of <= 16 branches as one persistent kernel (needs fused)
+        self._step_kernels = {}       # branches -> K.DecodeStepKernel
 
     # -- helpers -------------------------------------------------------------------------------
     def _tables(self, device):
@@ -303,6 +305,13 @@ class Transformer(nn.Module):
         bsz, seqlen = tokens.shape
         M = bsz * seqlen
         p = self.params
+        if start_pos != 0 and seqlen == 1 and self.persistent:
+            sk = self._step_kernel(bsz, tokens.device)
+            if sk is not None:
+                pos_dev, t_dev = step_state
+                sk.prepare(self.layers[0].attention.cache_prompt_len, pos_dev, t_dev)
+                hn = K.rmsnorm(sk.launch(tokens), self.norm.weight, self.norm.eps)
+                return self.output(hn.view(bsz, 1, p.dim)).to(DTYPE)
         h = self.tok_embeddings(tokens).to(DTYPE).reshape(M, p.dim)
         cos, sin = self._tables(h.device)
         pending = None                      # product of the previous layer's w2, not yet added to h
@@ -341,6 +350,35 @@ class Transformer(nn.Module):
             pending = K.matmul_q40_partial(act, [(ff.w2.w, ff.w2.s, ff.w2.shape[0])])
         _, hn = K.partial_rmsnorm(pending, h, self.norm.weight, self.norm.eps, want_h=False)
         return self.output(hn.view(bsz, seqlen, p.dim)).to(DTYPE)
+
+    def _step_kernel(self, bsz: int, device):
+        """The persistent decode kernel for `bsz` branches, or None when the model shape is outside it."""
+        if bsz in self._step_kernels:
+            return self._step_kernels[bsz]
+        p = self.params
+        att0, ff0 = self.layers[0].attention, self.layers[0].feed_forward
+        H, Hkv, ffn = att0.n_local_heads, att0.n_local_kv_heads, ff0.w1.shape[0]
+        sk = None
+        if K.DecodeStepKernel.supports(bsz, p.dim, H, Hkv, ffn):
+            rows = []
+            for layer in self.layers:
+                a, f = layer.attention, layer.feed_forward
+                lins = [a.wq, a.wk, a.wv, a.wo, f.w1, f.w3, f.w2]
+                rows.append([l.w.data_ptr() for l in lins] + [l.s.data_ptr() for l in lins] +
+                            [layer.attention_norm.weight.data_ptr(), layer.ffn_norm.weight.data_ptr(),
+                             a.cache_prompt_k.data_ptr(), a.cache_prompt_v.data_ptr(),
+                             a.cache_k.data_ptr(), a.cache_v.data_ptr(), a.cache_k_s.data_ptr(), a.cache_v_s.data_ptr()])
+            cos, sin = self._tables(device)
+            sk = K.DecodeStepKernel(rows, bsz, p.dim, H, Hkv, ffn, p.max_seq_len, p.max_prompt_seq_len, self.norm.eps,
+                                    self.tok_embeddings.weight, cos, sin)
+        self._step_kernels[bsz] = sk
+        return sk
+
+    def check_step_kernels(self):
+        """Raises if a persistent decode step reported a time-out (call after synchronising)."""
+        for sk in self._step_kernels.values():
+            if sk is not None and sk.bound is not None:
+                sk.check_status()
 
     @torch.inference_mode()
     def forward(self, tokens: torch.Tensor, start_pos: int):

@@ -380,3 +380,68 @@ def prefill_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Ten
     check(lib.smh_prefill_attn(q.data_ptr(), k.data_ptr(), v.data_ptr(), out.data_ptr(), S, H, k.shape[1], D,
                                _stream()), "smh_prefill_attn")
     return out
+
+
+class DecodeStepKernel:
+    """One decode step (embedding + every layer) of up to 16 branches as a single persistent kernel.
+
+    Owns the layer descriptor table, the workspace and the output buffer; `prepare` binds a prompt
+    length and the device-side step state, `launch` runs one step on the current stream and returns
+    the hidden state that enters the final norm.  The caller checks `status()` after synchronising.
+    """
+
+    MAX_BRANCHES = 16
+
+    @staticmethod
+    def supports(M: int, dim: int, H: int, Hkv: int, ffn: int) -> bool:
+        return 1 <= M <= DecodeStepKernel.MAX_BRANCHES and H == Hkv and dim % 256 == 0 and ffn % 256 == 0 and (H * 128) % 256 == 0
+
+    def __init__(self, layer_rows: Sequence[Sequence[int]], M: int, dim: int, H: int, Hkv: int, ffn: int, Smax: int,
+                 P_max: int, eps: float, emb: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor):
+        lib = _lib.load()
+        _need_gpu(emb, cos, sin)
+        self.dev = emb.device
+        self.M, self.dim, self.H, self.Hkv, self.ffn, self.Smax, self.eps = M, dim, H, Hkv, ffn, Smax, float(eps)
+        self.n_layers = len(layer_rows)
+        assert all(len(r) == 22 for r in layer_rows), "a layer descriptor is 22 pointers"
+        self.table = torch.tensor(layer_rows, dtype=torch.int64).to(self.dev)
+        need = lib.smh_decode_step_workspace_bytes(self.n_layers, M, dim, H, Hkv, ffn, P_max, Smax)
+        if need == 0:
+            raise _lib.SmhError("smh_decode_step_workspace_bytes: " + lib.smh_last_error_string().decode())
+        self.workspace = torch.zeros(need + 256, dtype=torch.uint8, device=self.dev)
+        off = (-self.workspace.data_ptr()) % 256
+        self.ws_ptr = self.workspace.data_ptr() + off
+        self.ws_bytes = need
+        self.tokens = torch.zeros(M, dtype=torch.int64, device=self.dev)
+        self.h = torch.empty((M, dim), dtype=torch.float16, device=self.dev)
+        self.emb, self.cos, self.sin = emb, cos, sin
+        self.bound = None
+
+    def prepare(self, P: int, pos_dev: torch.Tensor, t_dev: torch.Tensor) -> None:
+        key = (P, pos_dev.data_ptr(), t_dev.data_ptr())
+        if self.bound == key:
+            return
+        lib = _lib.load()
+        check(lib.smh_decode_prepare(self.table.data_ptr(), self.n_layers, self.M, self.dim, self.H, self.Hkv, self.ffn, P,
+                                     self.Smax, self.eps, self.tokens.data_ptr(), self.emb.data_ptr(), self.cos.data_ptr(),
+                                     self.sin.data_ptr(), pos_dev.data_ptr(), t_dev.data_ptr(), self.h.data_ptr(),
+                                     self.ws_ptr, self.ws_bytes), "smh_decode_prepare")
+        self.bound = key
+
+    def launch(self, tokens: torch.Tensor) -> torch.Tensor:
+        assert self.bound is not None, "prepare() first"
+        self.tokens.copy_(tokens.reshape(-1))
+        check(_lib.load().smh_decode_step(self.ws_ptr, _stream()), "smh_decode_step")
+        return self.h
+
+    def status(self) -> Tuple[int, int, int]:
+        import ctypes
+        out = (ctypes.c_uint32 * 3)()
+        check(_lib.load().smh_decode_status(self.ws_ptr, out), "smh_decode_status")
+        return int(out[0]), int(out[1]), int(out[2])
+
+    def check_status(self) -> None:
+        st = self.status()
+        if st[2] != 0:
+            raise _lib.SmhError("the persistent decode kernel timed out waiting for its own workgroups "
+                                "(they must all be resident at once); results are invalid")
