@@ -15,7 +15,7 @@
 //
 // Phases of a layer (a grid barrier after each):
 //   QKV   x = RMSNorm(h)            . [wq|wk|wv]   finisher: RoPE, q / exact k,v out, Q4_0 KV append
-//   ATT   softmax(q K^T) V over the shared fp16 prefix (64-row chunks) and the branch's Q4_0 suffix
+//   ATT   softmax(q K^T) V over the shared fp16 prefix (in chunks) and the branch's Q4_0 suffix
 //   O     x = attention output     . wo          finisher: h += fp16(sum), sum of squares of h
 //   W13   x = RMSNorm(h)            . [w1|w3]     finisher: fp16(silu(gate)) * up
 //   W2    x = SiLU product          . w2          finisher: h += fp16(sum), sum of squares of h
@@ -39,6 +39,12 @@
 #include "attn_rows.hpp"
 #include "rope_kv.hpp"
 
+#ifdef SMH_MEGA_DEBUG
+__device__ unsigned long long smh_mega_trace[8][4096];
+#define MTR(slotbase, k) do { if (trace_on && lane0 == 0) smh_mega_trace[slotbase][trace_i++ & 4095] = ((unsigned long long)(k) << 56) | (__builtin_readcyclecounter() & 0xFFFFFFFFFFFFFFull); } while (0)
+#else
+#define MTR(slotbase, k) do {} while (0)
+#endif
 namespace smh {
 
 int env_int(const char *name, int dflt);
@@ -51,9 +57,9 @@ constexpr int MK_STAGE_S = 32 * 8;                   // 32 rows x 4 scales
 constexpr int MK_STAGE = MK_STAGE_W + MK_STAGE_S;
 constexpr int MK_MAX_STAGES = 8;
 constexpr int MK_MAX_M = 16;
-constexpr int MK_ATT_ROWS = 64;                      // prefix rows per attention item
 constexpr int MK_PART = 132;                         // floats per attention partial: o[128], m, l, pad
 constexpr int MK_LDS_LIMIT = 160 * 1024;
+constexpr int MK_SYNC_BYTES = 2048;                  // status words + barrier counters at the head of the workspace
 
 enum { MK_QKV = 0, MK_O = 1, MK_W13 = 2, MK_W2 = 3, MK_MATRIX_PHASES = 4 };
 enum { MK_X_NORM_ATTN = 0, MK_X_ATTN_OUT = 1, MK_X_NORM_FFN = 2, MK_X_ACT = 3 };
@@ -91,6 +97,7 @@ struct MegaParams {
     MegaMatrix mat[MK_MATRIX_PHASES];
     int n_layers, M, dim, H, Hkv, ffn, P, Smax, G;
     int stages, max_units, chunks;  // ring depth; counter stride; prefix chunks per head
+    int att_rows;                   // prefix rows per attention item (multiple of 16)
     int xbuf_off, red_off, flag_off;// LDS layout (bytes)
     int mr;                         // row groups of 4: ceil(M/4)
     int spin_limit;
@@ -154,7 +161,12 @@ __device__ __forceinline__ f4 ld_f4(const float *p) {
 }
 __device__ __forceinline__ h4 ld_h4(const half_t *p) { return __builtin_bit_cast(h4, ld_u64(p)); }
 __device__ __forceinline__ void st_h4(half_t *p, h4 v) { st_u64(p, __builtin_bit_cast(u32x2, v)); }
-__device__ __forceinline__ void wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
+__device__ __forceinline__ void wait_vmem() {
+#ifdef SMH_MEGA_RELEASE_FENCE
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
+#endif
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+}
 // workgroup barrier that does not wait for the ring loads in flight (LDS traffic only)
 __device__ __forceinline__ void wg_sync() {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
@@ -162,22 +174,49 @@ __device__ __forceinline__ void wg_sync() {
     asm volatile("" ::: "memory");
 }
 
-// ---- grid barrier (control waves; one arrival per control wave) ----------------------------------------
-__device__ __forceinline__ void grid_arrive(CParams &p, int lane) {
+// ---- grid barrier (control waves) ------------------------------------------------------------------------
+// A thousand atomics on one address take tens of microseconds, so arrivals go up a tree: the control
+// waves of a workgroup count in LDS, the last of them increments the counter of the workgroup's group
+// (16 groups, one cache line each), and the arrival that completes a group increments the top counter.
+// Counters only grow; "complete" is a multiple of the group size.  One wave per workgroup polls the top
+// counter and releases the other control waves through LDS.
+// LDS words at flag_off: [0] attention finisher flag, [1] control-wave arrivals, [2] last barrier passed.
+constexpr int MK_GROUPS = 16;
+constexpr int MK_GROUP_WORD0 = 32, MK_GROUP_STRIDE = 16;      // uint32 index of group g's counter: 32 + 16 g
+__device__ __forceinline__ void grid_arrive(CParams &p, uint32_t *words, int w, int lane) {
     wait_vmem();
-    if (lane == 0) __hip_atomic_fetch_add(p.sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void grid_wait(CParams &p, uint32_t target) {
-    int it = 0;
-    while (true) {
-        const uint32_t v = ld_u32(p.sync);
-        if ((int32_t)(v - target) >= 0) break;
-        if (ld_u32(p.sync + 2) != 0u) break;
-        if (++it > p.spin_limit) {
-            st_u32(p.sync + 2, 1u);
-            break;
+    if (lane == 0) {
+        const uint32_t old = __hip_atomic_fetch_add(words + 1, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (((old + 1u) & (MK_CONTROL_WAVES - 1)) == 0u) {
+            const int g = w & (MK_GROUPS - 1);
+            const uint32_t size = (uint32_t)((p.G - g + MK_GROUPS - 1) / MK_GROUPS);
+            const uint32_t prev = __hip_atomic_fetch_add(p.sync + MK_GROUP_WORD0 + MK_GROUP_STRIDE * g, 1u, __ATOMIC_RELAXED,
+                                                         __HIP_MEMORY_SCOPE_AGENT);
+            if ((prev + 1u) % size == 0u) __hip_atomic_fetch_add(p.sync, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        __builtin_amdgcn_s_sleep(1);
+    }
+}
+__device__ __forceinline__ void grid_wait(CParams &p, uint32_t *words, int cw, uint32_t target, uint32_t barrier_no) {
+    int it = 0;
+    if (cw == 0) {
+        while (true) {
+            const uint32_t v = ld_u32(p.sync);
+            if ((int32_t)(v - target) >= 0) break;
+            if ((it & 63) == 63 && ld_u32(p.sync + 2) != 0u) break;
+            if (++it > p.spin_limit) {
+                st_u32(p.sync + 2, 1u);
+                break;
+            }
+            __builtin_amdgcn_s_sleep(1);
+        }
+        __hip_atomic_store(words + 2, barrier_no, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    } else {
+        while (true) {
+            const uint32_t v = __hip_atomic_load(words + 2, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+            if ((int32_t)(v - barrier_no) >= 0) break;
+            if (++it > p.spin_limit) break;
+            __builtin_amdgcn_s_sleep(1);
+        }
     }
 }
 
@@ -652,11 +691,11 @@ __device__ __forceinline__ void attention_item(CParams &p, CLayer &L, int item, 
             SoftState st;
             soft_init(st);
             if (ck < p.chunks) {
-                const int r0 = ck * MK_ATT_ROWS;
-#pragma unroll
-                for (int qd = 0; qd < MK_ATT_ROWS / 4 / MK_STREAM_WAVES; ++qd) {
-                    const int r = r0 + 4 * (wave + MK_STREAM_WAVES * qd) + g;
-                    if (r < p.P) {
+                const int r0 = ck * p.att_rows, r1 = min(r0 + p.att_rows, p.P);
+#pragma unroll 4
+                for (int rq = r0 + 4 * wave; rq < r1; rq += 4 * MK_STREAM_WAVES) {
+                    const int r = rq + g;
+                    if (r < r1) {
                         const long off = ((long)r * p.Hkv + h) * 128;
                         const RowRegs kr = row_from_fp16(L.prefix_k + off, c);
                         const RowRegs vr = row_from_fp16(L.prefix_v + off, c);
@@ -765,6 +804,13 @@ __device__ __forceinline__ void stream_role(CParams &p, uint8_t *lds, int w, int
     ring.base = (uint32_t)(wave * (p.stages * MK_STAGE));
     ring.stages = p.stages;
     ring_fill(ring, cur, p, lds, w, wave, lane0);
+    wg_sync();                                                   // [init]
+#ifdef SMH_MEGA_DEBUG
+    const bool trace_on = wave == 0 && (w == 0 || w == 131);
+    const int trace_slot = w == 0 ? 0 : 1;
+    int trace_i = 0;
+#endif
+    MTR(trace_slot, 1);
 
     for (int layer = 0; layer < p.n_layers; ++layer) {
         CLayer &L = layer_of(p, layer);
@@ -775,13 +821,16 @@ __device__ __forceinline__ void stream_role(CParams &p, uint8_t *lds, int w, int
             const int c = lane & 15, g = lane >> 4;
             if (phase == 1) {
                 wg_sync();                                           // [att] inputs are visible
+                MTR(trace_slot, 10);
                 const int items = p.H * (p.chunks + 1);
                 for (int item = w; item < items; item += p.G) attention_item(p, L, item, reinterpret_cast<float *>(xbuf), flag, wave, lane);
+                MTR(trace_slot, 11);
                 continue;
             }
             const int ph = matrix_phase(phase);
             const PhaseWork k = phase_work(matrix_of(p, ph), w);
             wg_sync();                                               // [x] activations are in LDS
+            MTR(trace_slot, 20 + phase);
             int j = wave;
             for (int ui = 0; ui < k.n_units; ++ui) {
                 const int j_end = ui == 0 ? k.nA : k.n;
@@ -793,16 +842,6 @@ __device__ __forceinline__ void stream_role(CParams &p, uint8_t *lds, int w, int
                 const int row = min(c, M - 1);
                 for (; j < j_end; j += MK_STREAM_WAVES) {
                     ring_wait_head(ring);
-#ifdef SMH_MEGA_DEBUG
-                    if (phase == 4 && layer == 0 && w == 0 && wave == 0 && j == 0) {
-                        uint32_t *dbg = reinterpret_cast<uint32_t *>(p.slabs + 200 * 2 * M * 256);
-                        const uint32_t *st = reinterpret_cast<const uint32_t *>(lds + ring.base + ring.head * MK_STAGE);
-                        for (int i = lane; i < MK_STAGE / 4; i += 64) dbg[i] = st[i];
-                        const uint32_t *xt = reinterpret_cast<const uint32_t *>(xbuf);
-                        if (lane < 16) dbg[MK_STAGE / 4 + lane] = xt[lane];
-                        dbg[MK_STAGE / 4 + 16] = ring.base; dbg[MK_STAGE / 4 + 17] = ring.head; dbg[MK_STAGE / 4 + 18] = ring.inflight;
-                    }
-#endif
                     step_consume(lds + ring.base + ring.head * MK_STAGE, xbuf + (long)j * M * 64, c, g, row, C, val, corr);
                     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");            // the stage has been read
                     ring.head = uni((ring.head + 1 == ring.stages) ? 0 : ring.head + 1);
@@ -815,15 +854,10 @@ __device__ __forceinline__ void stream_role(CParams &p, uint8_t *lds, int w, int
                     const int bh = t >> 2;
                     val[t] -= ((bh & 1) ? 1032.f : 72.f) * corr[bh];
                 }
-#ifdef SMH_MEGA_DEBUG
-                if (phase == 4 && layer == 0 && w == 0 && wave == 0) {
-                    float *dbg = p.slabs + 220 * 2 * M * 256;
-                    for (int t = 0; t < 16; ++t)
-                        for (int r = 0; r < 4; ++r) dbg[(lane * 16 + t) * 4 + r] = val[t][r];
-                }
-#endif
+                MTR(trace_slot, 30 + phase);
                 wg_fold(val, red, p.mr, wave, lane);           // [fold rounds] ... [sum ready]
                 wg_sync();                                           // [sum taken] the image may be overwritten
+                MTR(trace_slot, 40 + phase);
             }
         }
     }
@@ -833,8 +867,14 @@ __device__ __forceinline__ void control_role(CParams &p, uint8_t *lds, int w, in
     uint8_t *xbuf = lds + p.xbuf_off;
     const float *red = reinterpret_cast<const float *>(lds + p.red_off);
     const int M = p.M;
-    const uint32_t arrivals = (uint32_t)(p.G * MK_CONTROL_WAVES);      // per grid barrier
+    uint32_t *words = reinterpret_cast<uint32_t *>(lds + p.flag_off);
+    const uint32_t arrivals = (uint32_t)(p.G < MK_GROUPS ? p.G : MK_GROUPS);   // top-counter increments per grid barrier
     const uint32_t base = ld_u32(p.sync + 1);
+    if (cw == 0 && lane0 == 0) {
+        words[1] = 0u;
+        words[2] = 0u;
+    }
+    wg_sync();                                                   // [init]
     uint32_t barrier_no = 0;
 
     // ---- embedding: unit u of the hidden state by workgroup u ----
@@ -850,14 +890,22 @@ __device__ __forceinline__ void control_role(CParams &p, uint8_t *lds, int w, in
             if (lane0 == 0) st_f32(p.ssq + ((long)(p.dim / 256) + w) * M + m, ss);
         }
     }
-    grid_arrive(p, lane0);
+    grid_arrive(p, words, w, lane0);
+#ifdef SMH_MEGA_DEBUG
+    const bool trace_on = cw == 0 && (w == 0 || w == 131);
+    const int trace_slot = w == 0 ? 2 : 3;
+    int trace_i = 0;
+#endif
+    MTR(trace_slot, 1);
 
     for (int layer = 0; layer < p.n_layers; ++layer) {
         CLayer &L = layer_of(p, layer);
         for (int phase = 0; phase < 5; ++phase) {
             const int lane = launder(lane0);
             ++barrier_no;
-            grid_wait(p, base + barrier_no * arrivals);
+            MTR(trace_slot, 50 + phase);
+            grid_wait(p, words, cw, base + barrier_no * arrivals, barrier_no);
+            MTR(trace_slot, 60 + phase);
             if (phase == 1) {
                 wg_sync();                                           // [att]
                 const int items = p.H * (p.chunks + 1);
@@ -867,12 +915,13 @@ __device__ __forceinline__ void control_role(CParams &p, uint8_t *lds, int w, in
                     wg_sync();
                     wg_sync();
                 }
-                grid_arrive(p, lane);
+                grid_arrive(p, words, w, lane);
                 continue;
             }
             const int ph = matrix_phase(phase);
             const PhaseWork k = phase_work(matrix_of(p, ph), w);
             if (k.n > 0) load_x(p, L, ph, xbuf, k.n, k.nA, k.kA0, cw * 64 + lane, lane);
+            MTR(trace_slot, 70 + phase);
             wg_sync();                                               // [x]
             for (int ui = 0; ui < k.n_units; ++ui) {
                 wg_fold_barriers();                              // [fold rounds] ... [sum ready]
@@ -890,21 +939,17 @@ __device__ __forceinline__ void control_role(CParams &p, uint8_t *lds, int w, in
                         }
                     }
                 }
-#ifdef SMH_MEGA_DEBUG
-                if (phase == 4 && layer == 0 && w == 0 && cw == 0) {
-                    float *dbg = p.slabs + 230 * 2 * M * 256;
-                    for (int i = lane; i < 16 * MK_IMG_PITCH; i += 64) dbg[i] = red[i];
-                    for (int bb = 0; bb < 4; ++bb) dbg[2048 + lane * 4 + bb] = rows[0][bb];
-                }
-#endif
                 wg_sync();                                           // [sum taken]
+                MTR(trace_slot, 80 + phase);
                 control_unit(p, L, ph, k.uA + ui, ui, w, cw, lane, rows);
+                MTR(trace_slot, 90 + phase);
             }
-            grid_arrive(p, lane);
+            grid_arrive(p, words, w, lane);
+            MTR(trace_slot, 100 + phase);
         }
     }
     ++barrier_no;
-    grid_wait(p, base + barrier_no * arrivals);
+    grid_wait(p, words, cw, base + barrier_no * arrivals, barrier_no);
     if (w == 0 && cw == 0 && lane0 == 0) st_u32(p.sync + 1, base + barrier_no * arrivals);
     wait_vmem();
 }
@@ -943,7 +988,15 @@ int mega_plan(MegaPlan &pl, int n_layers, int M, int dim, int H, int Hkv, int ff
     MegaParams &p = pl.p;
     p = MegaParams{};
     p.n_layers = n_layers; p.M = M; p.dim = dim; p.H = H; p.Hkv = Hkv; p.ffn = ffn; p.P = P; p.Smax = Smax; p.G = G;
-    p.chunks = (P + MK_ATT_ROWS - 1) / MK_ATT_ROWS;
+    // attention items per head: prefix chunks + the suffix; sized so that one round of workgroups covers them
+    {
+        int want = G / H - 1;
+        if (want < 1) want = 1;
+        int rows = ((P + want - 1) / want + 15) / 16 * 16;
+        if (rows < 16) rows = 16;
+        p.att_rows = rows;
+        p.chunks = (P + rows - 1) / rows;
+    }
     auto set = [&](int ph, int nseg, const int *ids, const int *ns, int K) {
         MegaMatrix &g = p.mat[ph];
         g.nseg = nseg;
@@ -997,7 +1050,7 @@ int mega_plan(MegaPlan &pl, int n_layers, int M, int dim, int H, int Hkv, int ff
     p.spin_limit = 1 << 22;
     size_t o = 0;
     auto take = [&](size_t bytes) { size_t at = o; o = align_up(o + bytes, 256); return at; };
-    pl.off_sync = take(64);          // the status words come first, then the parameter block (offset 256)
+    pl.off_sync = take(MK_SYNC_BYTES);   // status words and barrier counters come first, then the parameter block
     pl.off_params = take(sizeof(MegaParams));
     pl.off_q = take((size_t)M * H * 128 * 2);
     pl.off_k = take((size_t)M * Hkv * 128 * 2);
@@ -1093,7 +1146,7 @@ extern "C" int smh_decode_step(void *workspace, smh_stream_t stream) {
         SMH_REQUIRE(it != g_prepared.end(), "smh_decode_step: workspace %p was not prepared (smh_decode_prepare)", workspace);
         pr = it->second;
     }
-    const MegaParams *params = reinterpret_cast<const MegaParams *>((const uint8_t *)workspace + 256);
+    const MegaParams *params = reinterpret_cast<const MegaParams *>((const uint8_t *)workspace + MK_SYNC_BYTES);
     hipLaunchKernelGGL(decode_mega_kernel, dim3((unsigned)pr.G), dim3(MK_THREADS), pr.lds_bytes, (hipStream_t)stream, params);
     return launch_status();
 }
@@ -1117,3 +1170,9 @@ extern "C" int smhdbg_decode_offsets(int n_layers, int M, int dim, int H, int Hk
     out[8] = pl.p.stages; out[9] = pl.lds_bytes;
     return 0;
 }
+
+#ifdef SMH_MEGA_DEBUG
+extern "C" int smhdbg_read_trace(unsigned long long *out) {
+    return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(smh_mega_trace), sizeof(unsigned long long) * 8 * 4096);
+}
+#endif
