@@ -237,58 +237,79 @@ __device__ __forceinline__ void unit_contributors(const MegaMatrix &g, int u, in
 }
 
 // ---- the stream of weight steps of one wave -------------------------------------------------------------
+// The position is kept as running addresses: issuing a step costs five loads and a few scalar adds;
+// geometry and layer pointers are looked up only when the cursor enters a phase or a new unit.
 struct Cursor {
     int layer, ph;          // layer, matrix phase
     int j, n;               // next step of the workgroup's range this wave takes; length of the range
-    int unit, kstep;        // position of that step
+    int unit, kstep, steps; // position of that step; steps per unit in this phase
+    const uint8_t *wb, *sb; // nibbles / scales of row 32*kstep of the unit (uniform)
+    uint32_t rowb, srow;    // row pitches in bytes
+    uint32_t w_off, s_off;  // this lane's byte offsets inside a step
 };
-__device__ __forceinline__ void cursor_enter(Cursor &c, CParams &p, int w, int wave) {
-    const MegaMatrix g = matrix_of(p, c.ph);
-    int a, b;
-    wg_range(g, w, a, b);
-    c.n = b - a;
-    c.j = wave;
-    const uint32_t t = (uint32_t)(a + wave);
-    c.unit = (int)(t / (uint32_t)g.steps);
-    c.kstep = (int)(t - (uint32_t)c.unit * g.steps);
+__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
+__device__ __forceinline__ const uint8_t *uni(const uint8_t *ptr) {
+    const uint64_t v = reinterpret_cast<uint64_t>(ptr);
+    const uint32_t lo = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)v);
+    const uint32_t hi = (uint32_t)__builtin_amdgcn_readfirstlane((int)(uint32_t)(v >> 32));
+    return reinterpret_cast<const uint8_t *>(((uint64_t)hi << 32) | lo);
 }
-// moves to the next phase until the cursor points at a step; false when the model is exhausted
-__device__ __forceinline__ bool cursor_settle(Cursor &c, CParams &p, int w, int wave) {
-    while (c.layer < p.n_layers && c.j >= c.n) {
-        if (++c.ph == MK_MATRIX_PHASES) {
-            c.ph = 0;
-            ++c.layer;
-        }
-        if (c.layer < p.n_layers) cursor_enter(c, p, w, wave);
-    }
-    return c.layer < p.n_layers;
-}
-// 5 direct-to-LDS loads: 4 x (8 rows x 128 B) of nibbles + 32 rows x 8 B of scales; then advance by 8 steps
-__device__ __forceinline__ void cursor_issue(Cursor &c, CParams &p, uint8_t *stage, int lane) {
+// addresses of the cursor's (layer, phase, unit, kstep)
+__device__ __forceinline__ void cursor_locate(Cursor &c, CParams &p, int lane) {
     const MegaMatrix g = matrix_of(p, c.ph);
     int sg = 0;
     if (g.nseg > 1 && c.unit >= g.unit0[1]) sg = 1;
     if (g.nseg > 2 && c.unit >= g.unit0[2]) sg = 2;
     CLayer &L = layer_of(p, c.layer);
     const int id = pick3(g.seg_id, sg);
-    const uint8_t *wp = L.w[id];
-    const uint8_t *sp = reinterpret_cast<const uint8_t *>(L.s[id]);
     const int N = pick3(g.seg_n, sg);
-    const long rowb = N / 2, srow = N / 32;
     const int ul = c.unit - pick3(g.unit0, sg);
-    const uint8_t *wb = wp + (long)c.kstep * 32 * rowb + (long)ul * 128;
-    const uint32_t w_off = (uint32_t)((lane >> 3) * (int)rowb + 16 * (lane & 7));
+    c.rowb = (uint32_t)uni(N / 2);
+    c.srow = (uint32_t)uni(N / 32);
+    c.wb = uni(L.w[id] + (long)c.kstep * 32 * c.rowb + (long)ul * 128);
+    c.sb = uni(reinterpret_cast<const uint8_t *>(L.s[id]) + (long)c.kstep * 32 * c.srow + (long)ul * 8);
+    c.w_off = (uint32_t)(lane >> 3) * c.rowb + 16u * (uint32_t)(lane & 7);
+    c.s_off = (uint32_t)(lane >> 1) * c.srow + 4u * (uint32_t)(lane & 1);
+}
+__device__ __forceinline__ void cursor_enter(Cursor &c, CParams &p, int w, int wave, int lane) {
+    const MegaMatrix g = matrix_of(p, c.ph);
+    int a, b;
+    wg_range(g, w, a, b);
+    c.n = uni(b - a);
+    c.j = wave;
+    c.steps = uni(g.steps);
+    const uint32_t t = (uint32_t)(a + wave);
+    c.unit = uni((int)(t / (uint32_t)g.steps));
+    c.kstep = uni((int)(t - (uint32_t)c.unit * g.steps));
+    if (c.j < c.n) cursor_locate(c, p, lane);
+}
+// moves to the next phase until the cursor points at a step; false when the model is exhausted
+__device__ __forceinline__ bool cursor_settle(Cursor &c, CParams &p, int w, int wave, int lane) {
+    while (c.layer < p.n_layers && c.j >= c.n) {
+        c.ph = uni(c.ph + 1);
+        if (c.ph == MK_MATRIX_PHASES) {
+            c.ph = 0;
+            c.layer = uni(c.layer + 1);
+        }
+        if (c.layer < p.n_layers) cursor_enter(c, p, w, wave, lane);
+    }
+    return c.layer < p.n_layers;
+}
+// 5 direct-to-LDS loads: 4 x (8 rows x 128 B) of nibbles + 32 rows x 8 B of scales; then on to the wave's next step
+__device__ __forceinline__ void cursor_issue(Cursor &c, CParams &p, uint8_t *stage, int lane) {
 #pragma unroll
     for (int q = 0; q < 4; ++q)
-        __builtin_amdgcn_global_load_lds((gptr_t)(wb + (long)(8 * q) * rowb + w_off), (lptr_t)(stage + q * 1024), 16, 0, 0);
-    const uint8_t *sb = sp + (long)c.kstep * 32 * srow + (long)ul * 8;
-    const uint32_t s_off = (uint32_t)((lane >> 1) * (int)srow + 4 * (lane & 1));
-    __builtin_amdgcn_global_load_lds((gptr_t)(sb + s_off), (lptr_t)(stage + MK_STAGE_W), 4, 0, 0);
-    c.j += MK_STREAM_WAVES;
-    c.kstep += MK_STREAM_WAVES;
-    if (c.kstep >= g.steps) {
-        c.kstep -= g.steps;
-        ++c.unit;
+        __builtin_amdgcn_global_load_lds((gptr_t)(c.wb + (long)(8 * q) * c.rowb + c.w_off), (lptr_t)(stage + q * 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((gptr_t)(c.sb + c.s_off), (lptr_t)(stage + MK_STAGE_W), 4, 0, 0);
+    c.j = uni(c.j + MK_STREAM_WAVES);
+    c.kstep = uni(c.kstep + MK_STREAM_WAVES);
+    if (c.kstep >= c.steps) {
+        c.kstep = uni(c.kstep - c.steps);
+        c.unit = uni(c.unit + 1);
+        if (c.j < c.n) cursor_locate(c, p, lane);
+    } else {
+        c.wb = uni(c.wb + (long)(32 * MK_STREAM_WAVES) * c.rowb);
+        c.sb = uni(c.sb + (long)(32 * MK_STREAM_WAVES) * c.srow);
     }
 }
 
@@ -296,18 +317,10 @@ struct Ring {
     uint32_t base;                        // LDS byte offset of the wave's ring
     int stages, head, tail, inflight;     // head: next slot to consume; tail: next slot to fill
 };
-// wave-uniform bookkeeping is pinned to scalar registers
-__device__ __forceinline__ int uni(int v) { return __builtin_amdgcn_readfirstlane(v); }
-__device__ __forceinline__ void pin(Cursor &c) {
-    c.layer = uni(c.layer); c.ph = uni(c.ph); c.j = uni(c.j); c.n = uni(c.n); c.unit = uni(c.unit); c.kstep = uni(c.kstep);
-}
 __device__ __forceinline__ void ring_fill(Ring &r, Cursor &c, CParams &p, uint8_t *lds, int w, int wave, int lane) {
     while (r.inflight < r.stages) {
-        const bool more = cursor_settle(c, p, w, wave);
-        pin(c);
-        if (!more) break;
+        if (c.j >= c.n && !cursor_settle(c, p, w, wave, lane)) break;
         cursor_issue(c, p, lds + r.base + r.tail * MK_STAGE, lane);
-        pin(c);
         r.tail = uni((r.tail + 1 == r.stages) ? 0 : r.tail + 1);
         r.inflight = uni(r.inflight + 1);
     }
@@ -435,11 +448,21 @@ __device__ __forceinline__ void load_x(CParams &p, CLayer &L, int ph, uint8_t *x
     const bool norm = (ph == MK_QKV || ph == MK_W13);
     float rstd = 0.f;
     if (norm) {
-        // lane m of every wave forms the row's 1/rms from the per-unit sums of squares
+        // lane 16q + m adds every fourth unit's sum of squares of row m (loads issued together), the four
+        // quarters are added across the wave, and lane m ends up with the row's 1/rms
         const float *ss = p.ssq + (long)(ph == MK_QKV ? 1 : 0) * (p.dim / 256) * M;
+        const int units = p.dim / 256, mm = lane & 15, qq = lane >> 4;
+        float v[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const int u = qq + 4 * i;
+            v[i] = (mm < M && u < units) ? ld_f32(ss + (long)u * M + mm) : 0.f;
+        }
         float tot = 0.f;
-        if (lane < M)
-            for (int u = 0; u < p.dim / 256; ++u) tot += ld_f32(ss + (long)u * M + lane);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) tot += v[i];
+        tot += __shfl_xor(tot, 16, 64);
+        tot += __shfl_xor(tot, 32, 64);
         const float r = 1.0f / sqrtf(tot / (float)p.dim + p.eps);
         rstd = __shfl(r, m, 64);
     }
@@ -799,8 +822,7 @@ __device__ __forceinline__ void stream_role(CParams &p, uint8_t *lds, int w, int
     asm volatile("" : "+v"(C.magic_hi), "+v"(C.magic_lo));
     Cursor cur{};
     Ring ring{};
-    cursor_enter(cur, p, w, wave);
-    pin(cur);
+    cursor_enter(cur, p, w, wave, lane0);
     ring.base = (uint32_t)(wave * (p.stages * MK_STAGE));
     ring.stages = p.stages;
     ring_fill(ring, cur, p, lds, w, wave, lane0);
@@ -982,7 +1004,7 @@ size_t align_up(size_t v, size_t a) { return (v + a - 1) / a * a; }
 int mega_plan(MegaPlan &pl, int n_layers, int M, int dim, int H, int Hkv, int ffn, int P, int Smax, int G, const char *who) {
     SMH_REQUIRE(M >= 1 && M <= MK_MAX_M, "%s: M=%d outside [1,%d]", who, M, MK_MAX_M);
     SMH_REQUIRE(H == Hkv, "%s: H=%d Hkv=%d (this kernel covers multi-head attention; grouped heads use the operator kernels)", who, H, Hkv);
-    SMH_REQUIRE(dim % 256 == 0 && ffn % 256 == 0 && (H * 128) % 256 == 0 && dim > 0 && ffn > 0,
+    SMH_REQUIRE(dim % 256 == 0 && ffn % 256 == 0 && (H * 128) % 256 == 0 && dim > 0 && dim <= 8192 && ffn > 0,
                 "%s: dim=%d ffn=%d H=%d (dim, ffn and 128*H must be multiples of 256)", who, dim, ffn, H);
     SMH_REQUIRE(n_layers >= 1 && P >= 0 && Smax >= 1 && G >= 1, "%s: n_layers=%d P=%d Smax=%d G=%d", who, n_layers, P, Smax, G);
     MegaParams &p = pl.p;

@@ -259,7 +259,8 @@ class Transformer(nn.Module):
         self._step_state = None       # int32 [2] on the device: (position, suffix index t)
         self._step_host = None
         self.fused = True             # fused decode-layer launches; False runs module by module
-        self.persistent = True        # decode steps of <= 16 branches as one persistent kernel (needs fused)
+        self.persistent = True        # decode steps of few branches as one persistent kernel (needs fused)
+        self.persistent_max_branches = 4   # above this the operator-by-operator launches are faster (the kernel itself takes up to 16)
         self._step_kernels = {}       # branches -> K.DecodeStepKernel
 
     # -- helpers -------------------------------------------------------------------------------
@@ -305,7 +306,7 @@ class Transformer(nn.Module):
         bsz, seqlen = tokens.shape
         M = bsz * seqlen
         p = self.params
-        if start_pos != 0 and seqlen == 1 and self.persistent:
+        if start_pos != 0 and seqlen == 1 and self.persistent and bsz <= self.persistent_max_branches:
             sk = self._step_kernel(bsz, tokens.device)
             if sk is not None:
                 pos_dev, t_dev = step_state
