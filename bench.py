@@ -29,6 +29,8 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 PROMPT_LEN = 512
 BATCHES = (1, 10, 100)
+# HBM bytes per q40_gemv_kernel launch at M=1 from rocprofv3 FETCH_SIZE + WRITE_SIZE (see profiles/), or None
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = None
 
 
 def q40_bytes(M, N, K):
@@ -76,36 +78,46 @@ def time_region(torch, fn, iters):
     return start.elapsed_time(end) / iters
 
 
-def gemv_roofline(torch, model, M, iters):
-    """All 224 Q4_0 matrices of one decode step, back to back, at batch M."""
-    from spec_mcts_amd import kernels as K
-    dev = torch.device("cuda:0")
-    lins = []
+def step_matmuls(model):
+    """The weight-streaming launches of one decode step as the model issues them: per layer the fused
+    wq|wk|wv, wo, the fused w1|w3 and w2 (128 launches for 32 layers)."""
+    out = []
     for layer in model.layers:
         a, f = layer.attention, layer.feed_forward
-        lins += [a.wq, a.wk, a.wv, a.wo, f.w1, f.w3, f.w2]
-    xs = {}
-    for lin in lins:
-        k_in = lin.shape[1]
-        if k_in not in xs:
-            xs[k_in] = torch.randn((M, k_in), device=dev).half()
-    outs = {lin.shape[0]: torch.empty((M, lin.shape[0]), device=dev, dtype=torch.float16) for lin in lins}
+        seg = lambda lin: (lin.w, lin.s, lin.shape[0])
+        out.append((a.wq.shape[1], [seg(a.wq), seg(a.wk), seg(a.wv)]))
+        out.append((a.wo.shape[1], [seg(a.wo)]))
+        out.append((f.w1.shape[1], [seg(f.w1), seg(f.w3)]))
+        out.append((f.w2.shape[1], [seg(f.w2)]))
+    return out
+
+
+def matmul_roofline(torch, model, M, iters):
+    """Only the Q4_0 matmul kernel (q40_gemv_kernel for M <= 16, q40_gemm_kernel above), launched once per
+    weight launch of a decode step at batch M, back to back in one HIP graph; timed with HIP events on the
+    stream the graph runs on.  Every launch reads different weights (3.4 GB per pass, the Infinity Cache
+    holds 256 MB)."""
+    from spec_mcts_amd import kernels as K
+    dev = torch.device("cuda:0")
+    launches = step_matmuls(model)
+    xs = {k: torch.randn((M, k), device=dev).half() for k in {k for k, _ in launches}}
 
     def run():
-        for lin in lins:
-            K.matmul_q40(xs[lin.shape[1]], lin.w, lin.s, (lin.shape[1], lin.shape[0]), out=outs[lin.shape[0]])
+        for k_in, segs in launches:
+            K.matmul_q40_partial(xs[k_in], segs)
 
-    # capture the sequence in a graph so that the timed region holds kernels, not Python
     run()
     torch.cuda.synchronize()
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         run()
     ms = time_region(torch, graph.replay, iters)
-    total_bytes = sum(q40_bytes(M, lin.shape[0], lin.shape[1]) for lin in lins)
-    n = len(lins)
-    return {"launches": n, "avg_us": ms * 1e3 / n, "bytes_per_launch": total_bytes / n,
-            "gbs": total_bytes / (ms * 1e-3) / 1e9}
+    total_bytes = sum(sum(q40_bytes(0, n, k_in) for _, _, n in segs) + 2 * M * k_in + 4 * M * sum(n for _, _, n in segs)
+                      for k_in, segs in launches)
+    flops = sum(2 * M * k_in * sum(n for _, _, n in segs) for k_in, segs in launches)
+    n = len(launches)
+    return {"launches": n, "avg_us": ms * 1e3 / n, "bytes_per_launch": total_bytes / n, "gbs": total_bytes / (ms * 1e-3) / 1e9,
+            "tflops": flops / (ms * 1e-3) / 1e12}
 
 
 def cpu_baseline(torch, args_kw, budget_s=20.0):
@@ -115,7 +127,7 @@ def cpu_baseline(torch, args_kw, budget_s=20.0):
     from oracle import q40_oracle as O
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
-    oargs = O.OracleArgs(**{**args_kw, "n_layers": 1, "max_batch_size": 10})
+    oargs = O.OracleArgs(**{**args_kw, "n_layers": 1, "max_batch_size": 100})
     sd = O.random_q40_state_dict(oargs, seed=7)
     model = O.OracleTransformer(oargs, sd, dense=False)     # dense=False: dequantise on every call, as the reference does
     P = 64                                                  # short prompt: the sample times the decode step, not prefill
@@ -123,7 +135,7 @@ def cpu_baseline(torch, args_kw, budget_s=20.0):
     model.forward(prompt, 0)
     res = {}
     t_start = time.perf_counter()
-    for B in (1, 10):
+    for B in (1, 10, 100):
         tok = torch.randint(0, oargs.vocab_size, (B, 1))
         times = []
         for i in range(3):
@@ -155,6 +167,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
+    ap.add_argument("--batches", default="", help="comma-separated subset of 1,10,100 to run (a partial run is not a valid result)")
+    ap.add_argument("--no-roofline", action="store_true", help="skip the matmul roofline legs (profiling runs)")
     ap.add_argument("--layers", type=int, default=32, help="fewer layers for a quick functional run (INVALID as a result)")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -172,8 +186,9 @@ def main():
     model = build_model(torch, args_kw, seed=3)
     prompt = torch.randint(0, 32016, (1, PROMPT_LEN), generator=torch.Generator().manual_seed(3)).cuda()
 
+    batches = tuple(int(x) for x in a.batches.split(",")) if a.batches else BATCHES
     by_batch = {}
-    for B in BATCHES:
+    for B in batches:
         dec = GraphDecoder(model, B, use_graph=not a.no_graph)
         dec.prefill(prompt)
         dec.capture()
@@ -183,7 +198,9 @@ def main():
         dec.decode(steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        by_batch[B] = {"tok_s": B * steps / dt, "ms_per_step": dt / steps * 1e3}
+        model.check_step_kernels()
+        by_batch[B] = {"tok_s": B * steps / dt, "ms_per_step": dt / steps * 1e3,
+                       "path": "persistent step kernel" if (model.persistent and B <= model.persistent_max_branches) else "operator kernels"}
         del dec
 
     # per-step algorithmic HBM bytes: Q4 linears + fp16 lm_head + shared prefix KV (once) + suffix KV (Q4 rows)
@@ -191,41 +208,50 @@ def main():
     head_bytes = 32016 * 4096 * 2
     prefix_bytes = 2 * PROMPT_LEN * 4096 * 2 * a.layers
     t_mid = warmup + steps // 2
-    for B in BATCHES:
+    for B in batches:
         step_bytes = lin_bytes + head_bytes + prefix_bytes + B * t_mid * a.layers * 2 * 32 * 68
         by_batch[B]["hbm_frac"] = step_bytes / (by_batch[B]["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
 
-    rf1 = gemv_roofline(torch, model, 1, 5)
-    rf10 = gemv_roofline(torch, model, 10, 5)
-    rf100 = gemv_roofline(torch, model, 100, 3)
-    flops100 = sum(2 * 100 * n * k for n, k in ((4096, 4096),) * 4 + ((11008, 4096),) * 2 + ((4096, 11008),)) * a.layers
-    gemm_tflops = flops100 / (rf100["avg_us"] * rf100["launches"] * 1e-6) / 1e12
-
+    head = by_batch.get(100) or by_batch[max(by_batch)]
+    head_b = 100 if 100 in by_batch else max(by_batch)
     result = {
         "metric": "Q4_0 7B decode tok/s at B=1/10/100; Q4_0 GEMV achieved HBM GB/s",
-        "value": by_batch[100]["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
-        "ms_per_step": by_batch[100]["ms_per_step"], "higher_is_better": True, "scaling": "weak",
+        "value": head["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
+        "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "codellama7b_arch_q40_decode_prompt512_shared_prefix", "branches": 100,
+        "config": {"workload": "codellama7b_arch_q40_decode_prompt512_shared_prefix", "branches": head_b,
                    "layers": a.layers, "graph": not a.no_graph},
-        "by_batch": {str(B): {k: round(v, 4) for k, v in d.items()} for B, d in by_batch.items()},
-        "roofline": {"kernel": "q40_gemv_kernel (M=1, the 224 Q4_0 matrices of one 7B decode step)", "bound": "hbm",
-                     "achieved": round(rf1["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                     "frac": round(rf1["gbs"] / HBM_PEAK_GBS, 4), "traffic": None,
-                     "avg_launch_us": round(rf1["avg_us"], 3), "bytes_per_launch": round(rf1["bytes_per_launch"])},
-        "rooflines_other": [
-            {"kernel": "q40_gemv_kernel (M=10)", "bound": "hbm", "achieved": round(rf10["gbs"], 1), "peak": HBM_PEAK_GBS,
-             "unit": "GB/s", "frac": round(rf10["gbs"] / HBM_PEAK_GBS, 4), "avg_launch_us": round(rf10["avg_us"], 3)},
-            {"kernel": "q40_gemm_kernel (M=100)", "bound": "mfma", "achieved": round(gemm_tflops, 1),
-             "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(gemm_tflops / MFMA_F16_PEAK_TFLOPS, 4),
-             "hbm_gbs": round(rf100["gbs"], 1), "avg_launch_us": round(rf100["avg_us"], 3)},
-        ],
+        "by_batch": {str(B): {k: (round(v, 4) if isinstance(v, float) else v) for k, v in d.items()} for B, d in by_batch.items()},
     }
+    if not a.no_roofline:
+        rf1 = matmul_roofline(torch, model, 1, 5)
+        rf10 = matmul_roofline(torch, model, 10, 5)
+        rf100 = matmul_roofline(torch, model, 100, 3)
+        result["roofline"] = {
+            "kernel": "q40_gemv_kernel at M=1: the 128 weight launches of one 7B decode step (wq|wk|wv, wo, w1|w3, w2 per layer)",
+            "bound": "hbm", "achieved": round(rf1["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+            "frac": round(rf1["gbs"] / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
+            "avg_launch_us": round(rf1["avg_us"], 3), "bytes_per_launch": round(rf1["bytes_per_launch"])}
+        result["rooflines_other"] = [
+            {"kernel": "q40_gemv_kernel at M=10", "bound": "hbm", "achieved": round(rf10["gbs"], 1), "peak": HBM_PEAK_GBS,
+             "unit": "GB/s", "frac": round(rf10["gbs"] / HBM_PEAK_GBS, 4), "avg_launch_us": round(rf10["avg_us"], 3)},
+            {"kernel": "q40_gemm_kernel at M=100", "bound": "mfma", "achieved": round(rf100["tflops"], 1),
+             "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(rf100["tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
+             "hbm_gbs": round(rf100["gbs"], 1), "avg_launch_us": round(rf100["avg_us"], 3)},
+        ]
+        if 1 in by_batch and by_batch[1]["path"].startswith("persistent"):
+            # the whole step is one launch: every weight, the prefix KV and the suffix KV once
+            b1 = lin_bytes + prefix_bytes + t_mid * a.layers * 2 * 32 * 68
+            result["rooflines_other"].append(
+                {"kernel": "decode_mega_kernel at M=1 (one launch per step; bound from the step time less lm_head/argmax is not separated)",
+                 "bound": "hbm", "achieved": round(b1 / (by_batch[1]["ms_per_step"] * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
+                 "unit": "GB/s", "frac": round(b1 / (by_batch[1]["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
     if not a.no_cpu_baseline:
         cpu, cores, raw = cpu_baseline(torch, args_kw)
-        result["cpu_baseline"] = {"value": round(cpu.get(1, 0.0), 4), "unit": "tok/s", "cores": cores, "kind": "port",
+        result["cpu_baseline"] = {"value": round(cpu.get(head_b, cpu.get(max(cpu), 0.0)), 4), "unit": "tok/s", "cores": cores, "kind": "port",
                                   "sample": "oracle CPU path (torch dequantise + F.linear, fp32 compute): one layer + lm_head, "
-                                            "median of 3 decode steps at B=1 (and B=10), 64-token prompt, layer time x n_layers",
+                                            "median of 3 decode steps at B=1, 10 and 100, 64-token prompt, layer time x n_layers; "
+                                            "value is the B=%d figure" % head_b,
                                   "by_batch": {str(B): round(v, 4) for B, v in cpu.items()}}
     print(json.dumps(result))
 
