@@ -29,8 +29,9 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 PROMPT_LEN = 512
 BATCHES = (1, 10, 100)
-# HBM bytes per q40_gemv_kernel launch at M=1 from rocprofv3 FETCH_SIZE + WRITE_SIZE (see profiles/), or None
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = None
+# HBM bytes per q40_gemv_kernel launch at M=1: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by a 1 GiB copy
+# (profiles/q40_gemv_m1_hbm_traffic.md has the commands and the factors: 2.0 for reads, 1.0 for writes)
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 32925390
 
 
 def q40_bytes(M, N, K):
@@ -169,6 +170,9 @@ def main():
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--batches", default="", help="comma-separated subset of 1,10,100 to run (a partial run is not a valid result)")
     ap.add_argument("--no-roofline", action="store_true", help="skip the matmul roofline legs (profiling runs)")
+    ap.add_argument("--roofline-only", type=int, default=0, metavar="M",
+                    help="profiling aid: run only the matmul roofline leg at batch M (eager launches, one pass) after a 1 GiB "
+                         "device copy that calibrates the profiler's byte counters, and print that leg's numbers")
     ap.add_argument("--layers", type=int, default=32, help="fewer layers for a quick functional run (INVALID as a result)")
     a = ap.parse_args()
     if a.gpus != 1:
@@ -186,6 +190,14 @@ def main():
     model = build_model(torch, args_kw, seed=3)
     prompt = torch.randint(0, 32016, (1, PROMPT_LEN), generator=torch.Generator().manual_seed(3)).cuda()
 
+    if a.roofline_only:
+        src = torch.empty(1 << 29, dtype=torch.float16, device="cuda:0").normal_()
+        dst = torch.empty_like(src)
+        dst.copy_(src)                                     # 1 GiB read + 1 GiB written by one elementwise kernel
+        torch.cuda.synchronize()
+        del src, dst
+        print(json.dumps(matmul_roofline(torch, model, a.roofline_only, 1)))
+        return
     batches = tuple(int(x) for x in a.batches.split(",")) if a.batches else BATCHES
     by_batch = {}
     for B in batches:

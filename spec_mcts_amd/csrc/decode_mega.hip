@@ -979,7 +979,10 @@ __device__ __forceinline__ void control_role(CParams &p, uint8_t *lds, int w, in
 __global__ __launch_bounds__(MK_THREADS) void decode_mega_kernel(const MegaParams *params) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     CParams &p = *reinterpret_cast<CParams *>(reinterpret_cast<uintptr_t>(params));
-    const int w = uni((int)blockIdx.x);
+    // workgroups are dealt round-robin to the 8 XCDs; consecutive LOGICAL workgroups (which stream adjacent
+    // column units and share the cache lines of their scales) are placed behind the same L2
+    int w = uni((int)blockIdx.x);
+    if ((p.G & 7) == 0) w = uni((w & 7) * (p.G >> 3) + (w >> 3));
     const int wave = uni((int)threadIdx.x >> 6);
     const int lane = threadIdx.x & 63;
     if (wave < MK_STREAM_WAVES) stream_role(p, lds, w, wave, lane);

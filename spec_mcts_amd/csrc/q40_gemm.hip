@@ -45,7 +45,10 @@ __global__ __launch_bounds__(GEMM_THREADS) void q40_gemm_kernel(MatmulParams p) 
     const int c = lane & 15;
     const int g = lane >> 4;
     int bid = blockIdx.x;
-    const int unit = bid % p.units;  bid /= p.units;
+    // slot -> unit: each XCD (blockIdx % 8) takes a contiguous run of column units, which share scale lines
+    const int slot = bid % p.units_pad;  bid /= p.units_pad;
+    const int unit = (slot & 7) * (p.units_pad >> 3) + (slot >> 3);
+    if (unit >= p.units) return;
     const int mb = bid % p.mblocks;
     const int slice = bid / p.mblocks;
     int sg = 0;
@@ -195,7 +198,7 @@ void gemm_fill_plan(MatmulParams &p) {
         col0 += p.seg[i].N;
     }
     p.units = unit0;
-    p.units_pad = unit0;
+    p.units_pad = (unit0 + 7) / 8 * 8;
     p.n_total = col0;
     p.mblocks = (p.M + GEMM_BM - 1) / GEMM_BM;
     const int steps = (p.K + 31) / 32;
@@ -216,7 +219,7 @@ void gemm_fill_plan(MatmulParams &p) {
 }
 
 int gemm_launch(const MatmulParams &p, hipStream_t stream) {
-    dim3 grid((unsigned)((long)p.units * p.mblocks * p.ksplit));
+    dim3 grid((unsigned)((long)p.units_pad * p.mblocks * p.ksplit));
     hipLaunchKernelGGL(q40_gemm_kernel, grid, dim3(GEMM_THREADS), GEMM_LDS, stream, p);
     return launch_status();
 }

@@ -22,8 +22,9 @@
 //     the product (partial_ops.hip: plain reduce, residual + RMSNorm, RoPE + KV append, SiLU*up).
 //   * up to three weights that share the input (wq|wk|wv, w1|w3) run as segments of one launch.
 //
-// blockIdx.x = slice * pairs_pad + pair with pairs_pad a multiple of 8: workgroups are dealt
-// round-robin to the 8 XCDs, so all K-slices of a column pair run behind the same L2.
+// blockIdx.x = slice * units_pad + slot with units_pad a multiple of 8: workgroups are dealt round-robin
+// to the 8 XCDs, so all K-slices of a column unit run behind the same L2, and slot -> unit gives every
+// XCD a contiguous run of units (they share the cache lines of the scales).
 #include <stdlib.h>
 
 #include "q40_matmul.hpp"
@@ -175,7 +176,11 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // WAVES rings, then reused as red[WAVES][M][256]
     constexpr int THREADS = WAVES * 64;
 
-    const int unit = blockIdx.x % p.units_pad;
+    // Workgroups are dealt round-robin to the 8 XCDs (8 L2s).  Neighbouring column units share the 128-byte
+    // lines of the scale rows, so each XCD takes a CONTIGUOUS run of units: a scale line is then fetched
+    // from HBM by one L2, not by eight.
+    const int slot = blockIdx.x % p.units_pad;
+    const int unit = (slot & 7) * (p.units_pad >> 3) + (slot >> 3);
     const int slice = blockIdx.x / p.units_pad;
     if (unit >= p.units) return;
     // which segment (weight) does this column pair belong to
