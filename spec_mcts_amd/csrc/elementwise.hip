@@ -65,14 +65,33 @@ __global__ __launch_bounds__(256) void silu_mul_kernel(const half_t *__restrict_
 __device__ __forceinline__ void argmax_merge(float &bv, int &bi, float v, int i) {
     if (v > bv || (v == bv && i < bi)) { bv = v; bi = i; }
 }
-__global__ __launch_bounds__(256) void argmax_kernel(const half_t *__restrict__ logits, int vocab, long ld,
-                                                     int64_t *__restrict__ out) {
-    __shared__ float s_v[4];
-    __shared__ int s_i[4];
+// one workgroup of 1024 threads per row; 128-bit loads, four in flight per thread, when the row allows them
+__global__ __launch_bounds__(1024) void argmax_kernel(const half_t *__restrict__ logits, int vocab, long ld,
+                                                      int64_t *__restrict__ out) {
+    __shared__ float s_v[16];
+    __shared__ int s_i[16];
     const half_t *row = logits + (long)blockIdx.x * ld;
     float bv = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = threadIdx.x; i < vocab; i += 256) argmax_merge(bv, bi, (float)row[i], i);
+    const bool wide = (ld % 8 == 0) && ((reinterpret_cast<uintptr_t>(logits) & 15) == 0);
+    const int chunks = wide ? vocab / 8 : 0;
+    for (int c0 = threadIdx.x; c0 < chunks; c0 += 4 * 1024) {
+        h8 v[4];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + 1024 * j;
+            if (c < chunks) v[j] = *reinterpret_cast<const h8 *>(row + 8 * c);
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const int c = c0 + 1024 * j;
+            if (c < chunks) {
+#pragma unroll
+                for (int e = 0; e < 8; ++e) argmax_merge(bv, bi, (float)v[j][e], 8 * c + e);
+            }
+        }
+    }
+    for (int i = 8 * chunks + threadIdx.x; i < vocab; i += 1024) argmax_merge(bv, bi, (float)row[i], i);
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         float ov = __shfl_xor(bv, o, 64);
@@ -82,7 +101,7 @@ __global__ __launch_bounds__(256) void argmax_kernel(const half_t *__restrict__ 
     if ((threadIdx.x & 63) == 0) { s_v[threadIdx.x >> 6] = bv; s_i[threadIdx.x >> 6] = bi; }
     __syncthreads();
     if (threadIdx.x == 0) {
-        for (int w = 1; w < 4; ++w) argmax_merge(bv, bi, s_v[w], s_i[w]);
+        for (int w = 1; w < 16; ++w) argmax_merge(bv, bi, s_v[w], s_i[w]);
         out[blockIdx.x] = (bi == 0x7fffffff) ? 0 : bi;
     }
 }
@@ -214,7 +233,7 @@ extern "C" int smh_argmax(const void *logits, int rows, int vocab, long ld, int6
     SMH_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "smh_argmax: rows=%d vocab=%d ld=%ld", rows, vocab, ld);
     if (rows == 0) return 0;
     SMH_REQUIRE(logits && out, "smh_argmax: null pointer");
-    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, out);
+    hipLaunchKernelGGL(argmax_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, out);
     return launch_status();
 }
 

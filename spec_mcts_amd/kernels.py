@@ -382,6 +382,37 @@ def prefill_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Ten
     return out
 
 
+
+def flash_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, B: int, L: int, H: int, D: int) -> torch.Tensor:
+    """Drop-in for triton_kernels.flash_attn (triton_kernels.py:621-647): one query per (branch, head) against
+    that branch's own L keys.  q [B,H,D], k/v [B,H,L,D] fp16 -> [B,H,D] fp16.  The keys are brought into the
+    token-major layout of the decode attention kernel ([B,L,H,D], one copy) and run as a suffix without prefix;
+    scores and the softmax state are fp32 (the reference keeps them in fp16)."""
+    _need_gpu(q, k, v)
+    assert q.shape == (B, H, D) and k.shape == (B, H, L, D) and v.shape == (B, H, L, D)
+    kt = k.transpose(1, 2).contiguous()
+    vt = v.transpose(1, 2).contiguous()
+    lens = torch.full((B,), L, dtype=torch.int32, device=q.device)
+    return shared_prefix_attn(q.contiguous(), None, None, 0, suffix_k=kt, suffix_v=vt, Smax=L, lens=lens, lens_stride=1,
+                              n_kv_heads=H)
+
+
+def page_flash_attn(p: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, P: int, B: int, L: int, H: int,
+                    D: int) -> torch.Tensor:
+    """Drop-in for triton_kernels.page_flash_attn (triton_kernels.py:764-789): branch b attends to the L pages
+    p[b, :] of the page pools k/v [H,P,D].  p [B,L] integer page ids, q [B,H,D] -> [B,H,D] fp16.  The pages of
+    each branch are gathered (one indexed copy) into the token-major suffix layout and attended to by the
+    decode attention kernel."""
+    _need_gpu(p, q, k, v)
+    assert p.shape == (B, L) and q.shape == (B, H, D) and k.shape == (H, P, D) and v.shape == (H, P, D)
+    idx = p.to(torch.int64)
+    kt = k.transpose(0, 1)[idx].contiguous()              # [B, L, H, D]
+    vt = v.transpose(0, 1)[idx].contiguous()
+    lens = torch.full((B,), L, dtype=torch.int32, device=q.device)
+    return shared_prefix_attn(q.contiguous(), None, None, 0, suffix_k=kt, suffix_v=vt, Smax=L, lens=lens, lens_stride=1,
+                              n_kv_heads=H)
+
+
 class DecodeStepKernel:
     """One decode step (embedding + every layer) of up to 16 branches as a single persistent kernel.
 

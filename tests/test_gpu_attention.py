@@ -125,3 +125,29 @@ def test_prefill_causal(S, H, Hkv):
     v = torch.randn((S, Hkv, 128), generator=g).to(torch.float16)
     got = K.prefill_attn(q.cuda(), k.cuda(), v.cuda())
     _check(got, O.causal_attention(q, k, v))
+
+
+def test_flash_attn_and_page_flash_attn_drop_ins():
+    """the reference's operator names (triton_kernels.py:621, :764) on top of the decode attention kernel, with
+    the shapes of its own checks (triton_kernels_bench.py:294-330: B=100, L=512, H=32, D=128, atol 1e-2)"""
+    from spec_mcts_amd import kernels as K
+    g = torch.Generator().manual_seed(1)
+    B, L, H, D = 100, 512, 32, 128
+    q = torch.randn((B, H, D), generator=g).half()
+    k = torch.randn((B, H, L, D), generator=g).half()
+    v = torch.randn((B, H, L, D), generator=g).half()
+    got = K.flash_attn(q.cuda(), k.cuda(), v.cuda(), B, L, H, D).cpu()
+    want = torch.nn.functional.scaled_dot_product_attention(q.float()[:, :, None], k.float(), v.float())[:, :, 0]
+    assert got.dtype == torch.float16 and torch.allclose(got.float(), want, rtol=1e-2, atol=2e-3)
+    # paged: a pool of P pages per head, every branch an arbitrary list of L pages (pages may repeat)
+    P, B2, L2 = 300, 27, 130
+    kp = torch.randn((H, P, D), generator=g).half()
+    vp = torch.randn((H, P, D), generator=g).half()
+    pager = torch.randint(0, P, (B2, L2), generator=g).to(torch.int16)
+    q2 = torch.randn((B2, H, D), generator=g).half()
+    got2 = K.page_flash_attn(pager.cuda(), q2.cuda(), kp.cuda(), vp.cuda(), P, B2, L2, H, D).cpu()
+    idx = pager.long()
+    kk = kp.float()[:, idx].permute(1, 0, 2, 3)           # [B, H, L, D]
+    vv = vp.float()[:, idx].permute(1, 0, 2, 3)
+    want2 = torch.nn.functional.scaled_dot_product_attention(q2.float()[:, :, None], kk, vv)[:, :, 0]
+    assert torch.allclose(got2.float(), want2, rtol=1e-2, atol=2e-3)
