@@ -252,7 +252,12 @@ class OracleTransformer:
                "feed_forward.w1", "feed_forward.w2", "feed_forward.w3")
 
     def __init__(self, args: OracleArgs, sd: Dict[str, torch.Tensor], dense: bool = True,
-                 quantize_kv: bool = True):
+                 quantize_kv: bool = True, per_branch_kv: bool = False):
+        # per_branch_kv=True restates hf_model_q40.Transformer instead (hf_model_q40.py:236-372): no shared
+        # prompt cache, EVERY position of every batch row lives in that row's Q4_0 cache, the rows of the
+        # tokens being processed are used exact (:313-314) and stored quantised (:322-343); a prefill takes
+        # B prompt rows and fills B caches.
+        self.per_branch_kv = per_branch_kv
         self.args = args
         self.sd = sd
         self.dense = dense
@@ -321,7 +326,19 @@ class OracleTransformer:
             xk = self._linear(p + "attention.wk", xn).view(B, S, Hkv, D)
             xv = self._linear(p + "attention.wv", xn).view(B, S, Hkv, D)
             xq, xk = apply_rotary_emb(xq, xk, freqs)
-            if start_pos == 0:
+            if self.per_branch_kv:
+                ck, cv = self.cache_k[i], self.cache_v[i]
+                sk = torch.cat((ck[:B, :start_pos], xk), dim=1)
+                sv = torch.cat((cv[:B, :start_pos], xv), dim=1)
+                ck[:B, start_pos:start_pos + S] = self._kv_roundtrip(xk)
+                cv[:B, start_pos:start_pos + S] = self._kv_roundtrip(xv)
+                if S == 1:
+                    none = torch.zeros((0, Hkv, D), dtype=DTYPE)
+                    attn = shared_prefix_attention(xq[:, 0], none, none, sk, sv, [start_pos + 1] * B)[:, None]
+                else:
+                    assert start_pos == 0, "multi-token calls are prefills"
+                    attn = torch.stack([causal_attention(xq[b], xk[b], xv[b]) for b in range(B)])
+            elif start_pos == 0:
                 # prefill: prompt KV taken from row 0 only, kept in fp16 (:324-329)
                 self.prompt_k[i] = xk[0].clone()
                 self.prompt_v[i] = xv[0].clone()
@@ -344,7 +361,7 @@ class OracleTransformer:
             g = self._linear(p + "feed_forward.w1", xn)
             u = self._linear(p + "feed_forward.w3", xn)
             h = h + self._linear(p + "feed_forward.w2", silu_mul(g, u))
-        if start_pos == 0:
+        if start_pos == 0 and not self.per_branch_kv:
             self.prompt_len = S
         h = rmsnorm(h, sd["norm.weight"], a.norm_eps)
         return (h.float() @ self._out_w.t()).to(DTYPE)

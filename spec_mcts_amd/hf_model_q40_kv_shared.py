@@ -259,6 +259,7 @@ class Transformer(nn.Module):
         self._step_state = None       # int32 [2] on the device: (position, suffix index t)
         self._step_host = None
         self.fused = True             # fused decode-layer launches; False runs module by module
+        self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
         self.persistent = True        # decode steps of few branches as one persistent kernel (needs fused)
         self.persistent_max_branches = 4   # above this the operator-by-operator launches are faster (the kernel itself takes up to 16)
         self._step_kernels = {}       # branches -> K.DecodeStepKernel
@@ -329,7 +330,14 @@ class Transformer(nn.Module):
                 outs = []
                 for b in range(bsz):
                     K.rope(xq[b], xk[b], cos, sin, 0)
-                    if b == 0:
+                    if self.per_branch_kv:
+                        # hf_model_q40.py:322-343: the rows of this call go into row b's cache as Q4_0
+                        assert seqlen <= p.max_seq_len
+                        for cache, cache_s, x in ((att.cache_k, att.cache_k_s, xk[b]), (att.cache_v, att.cache_v_s, xv[b])):
+                            w, sc = K.q_int40(x.reshape(-1), GROUP_SIZE)
+                            cache.view(p.max_batch_size, p.max_seq_len, Hkv, 64)[b, :seqlen] = w.view(seqlen, Hkv, 64)
+                            cache_s.view(p.max_batch_size, p.max_seq_len, Hkv, 2)[b, :seqlen] = sc.view(seqlen, Hkv, 2)
+                    elif b == 0:
                         att.cache_prompt_k[0, :seqlen] = xk[b]
                         att.cache_prompt_v[0, :seqlen] = xv[b]
                         att.cache_prompt_len = seqlen

@@ -34,14 +34,18 @@ def assign_q40(model: Transformer, model_dict: Dict[str, torch.Tensor], device) 
 
 
 def load_q40(model_file: Union[str, Dict[str, torch.Tensor]], params: Optional[ModelArgs] = None,
-             device: str = "cuda:0") -> Transformer:
-    """model_file: path of a converted checkpoint (torch.save of a flat dict) or the dict itself."""
+             device: str = "cuda:0", model_cls=None) -> Transformer:
+    """model_file: path of a converted checkpoint (torch.save of a flat dict) or the dict itself.
+    model_cls: the Transformer to build - hf_model_q40_kv_shared.Transformer (default) or
+    hf_model_q40.Transformer, with that module's ModelArgs."""
     if isinstance(model_file, str):
         model_dict = torch.load(model_file, map_location="cpu", mmap=True, weights_only=True)
     else:
         model_dict = model_file
     model_dict = remap_state_dict(model_dict)
-    model = Transformer(params if params is not None else ModelArgs())
+    if model_cls is None:
+        model_cls = Transformer
+    model = model_cls(params) if params is not None else (model_cls(ModelArgs()) if model_cls is Transformer else model_cls(__import__("spec_mcts_amd.hf_model_q40", fromlist=["ModelArgs"]).ModelArgs()))
     plain = {k: v for k, v in model_dict.items() if k.split(".")[-1] not in ("w", "s", "shape")}
     model.load_state_dict(plain, strict=False, assign=True)
     assign_q40(model, model_dict, device)

@@ -129,3 +129,37 @@ def test_fused_and_module_paths_agree():
     model.fused = True
     for x, y in zip(outs[True], outs[False]):
         assert torch.allclose(x.float(), y.float(), rtol=1e-2, atol=1e-2)
+
+
+def test_hf_model_q40_flavour_matches_oracle():
+    """hf_model_q40.Transformer: per-row Q4_0 cache for every position, B distinct prompt rows prefilled
+    together, fp32 logits; decode steps run the same kernels with an empty shared prefix"""
+    from spec_mcts_amd import hf_model_q40 as M
+    from spec_mcts_amd.load_q40 import load_q40
+    cfg = dict(dim=256, n_layers=2, n_heads=2, vocab_size=320, multiple_of=128, max_batch_size=4, max_seq_len=40)
+    oargs = O.OracleArgs(**cfg, max_prompt_seq_len=40)
+    sd = O.random_q40_state_dict(oargs, seed=37)
+    model = load_q40(dict(sd), M.ModelArgs(**cfg), device="cuda:0", model_cls=M.Transformer)
+    oracle = O.OracleTransformer(oargs, sd, dense=True, per_branch_kv=True)
+    g = torch.Generator().manual_seed(137)
+    prompt = torch.randint(0, cfg["vocab_size"], (3, 13), generator=g)           # three DIFFERENT rows
+    want = oracle.forward(prompt, 0)
+    got = model(prompt.cuda(), 0).cpu()
+    assert got.dtype == torch.float32 and got.shape == want.shape
+    assert torch.allclose(got, want.float(), rtol=2e-2, atol=2e-2)
+    for persistent in (True, False):              # the persistent step kernel, then the operator kernels
+        model.persistent = persistent
+        model.resetSeq()
+        oracle.reset()
+        oracle.forward(prompt, 0)
+        model(prompt.cuda(), 0)
+        for s in range(3):
+            tok = torch.randint(0, cfg["vocab_size"], (3, 1), generator=torch.Generator().manual_seed(200 + s))
+            want = oracle.forward(tok, 13 + s)
+            got = model(tok.cuda(), 13 + s).cpu()
+            assert torch.allclose(got, want.float(), rtol=2e-2, atol=2e-2), f"persistent={persistent} step {s}"
+    torch.cuda.synchronize()
+    model.check_step_kernels()
+    # greedy generation API of this flavour
+    res, lens = model.generate(prompt[:1].cuda(), 2, 5, temperature=0.0)
+    assert res.shape[0] == 2 and torch.equal(res[0], res[1])

@@ -178,3 +178,32 @@ def test_model_incremental_equals_full_recompute_without_kv_quant():
     inc = torch.stack(inc)
     assert torch.allclose(inc.float(), full[9:13].float(), atol=3e-2, rtol=3e-2)
     assert torch.equal(inc.argmax(-1), full[9:13].argmax(-1))
+
+
+def test_per_branch_flavour_reduces_to_shared_flavour_without_kv_quantisation():
+    """hf_model_q40's protocol (all positions in per-row caches) differs from the shared-prefix protocol only in
+    that the PROMPT rows are seen through Q4_0 by later steps: with KV quantisation switched off both
+    restatements must produce the same logits, prefill and decode, and with it on they must differ."""
+    args = O.OracleArgs(dim=256, n_layers=2, n_heads=2, vocab_size=320, multiple_of=128, max_batch_size=3, max_seq_len=12,
+                        max_prompt_seq_len=12)
+    sd = O.random_q40_state_dict(args, seed=11, std=0.05)
+    g = torch.Generator().manual_seed(12)
+    prompt = torch.randint(0, 320, (1, 7), generator=g)
+    toks = [torch.randint(0, 320, (3, 1), generator=g) for _ in range(3)]
+    outs = {}
+    for name, kw in (("shared", dict(quantize_kv=False)), ("rows", dict(quantize_kv=False, per_branch_kv=True)),
+                     ("rows_q", dict(quantize_kv=True, per_branch_kv=True))):
+        m = O.OracleTransformer(args, sd, dense=True, **kw)
+        if name == "shared":
+            res = [m.forward(prompt, 0)]
+            m.fork(0, 1, 2)
+        else:
+            res = [m.forward(prompt.expand(3, -1), 0)[:1]]
+        for s, t in enumerate(toks):
+            res.append(m.forward(t, 7 + s))
+        outs[name] = res
+    for a, b in zip(outs["shared"], outs["rows"]):
+        # same values up to the blocking of the host matmuls (one prompt row against three)
+        assert torch.allclose(a.float(), b.float(), rtol=0, atol=4e-3)
+    assert (outs["rows"][-1].float() - outs["rows_q"][-1].float()).abs().max() > 2e-2
+    assert torch.allclose(outs["rows"][-1].float(), outs["rows_q"][-1].float(), atol=0.5)
