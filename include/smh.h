@@ -163,6 +163,49 @@ int smh_shared_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int 
 int smh_prefill_attn(const void *q, const void *k, const void *v, void *out, int S, int H, int Hkv,
                      int D, smh_stream_t stream);
 
+/* ---- matmul with the following operator finished inside the same launch ---------------------------
+ * smh_q40_matmul_fused: the product of smh_q40_matmul_partial (same a / segments / partial buffer)
+ * followed, in the same launch for M <= 16 and as one more launch above, by the operator that
+ * consumes the linear in TransformerBlock.forward (hf_model_q40_kv_shared.py:456-467):
+ *   SMH_FIN_STORE            out[M, ldo] = fp16(sum) (+ residual)                       (LinearQ4_0, :228-236)
+ *   SMH_FIN_RESIDUAL_RMSNORM h_out = residual + fp16(sum); xn_out = RMSNorm(h_out) * norm_weight
+ *                            (the "h + wo(..)" / "h + w2(..)" of :463-466 and the norm of the next
+ *                            sub-block, :123-134).  One weight; h_out may be residual (in place).
+ *   SMH_FIN_SILU_MUL         out[M, ldo] = fp16(silu(fp16(sum_w1))) * fp16(sum_w3)      (:434)
+ *                            two weights of equal width: w1 (gate), w3 (up)
+ *   SMH_FIN_ROPE_APPEND      q, k, v = fp16(sum); apply_rotary_emb(q, k) (:173-203); Q4_0 append of k, v
+ *                            to row *t_dev of each branch's suffix cache (:365-371).  Three weights wq, wk,
+ *                            wv; arguments as smh_rope_append_kv.
+ * counters: 32 KiB of device memory zeroed once by the caller and owned by these calls afterwards
+ * (arrival counters that reset themselves + per-unit sums of squares).  Calls that share it must not
+ * overlap in time.  Same arithmetic and rounding points as smh_q40_matmul_partial + smh_partial_*.
+ */
+#define SMH_FIN_STORE 1
+#define SMH_FIN_RESIDUAL_RMSNORM 2
+#define SMH_FIN_SILU_MUL 3
+#define SMH_FIN_ROPE_APPEND 4
+#define SMH_FIN_COUNTER_BYTES 32768
+typedef struct smh_finish {
+    int mode;
+    void *counters;
+    void *out;
+    long ldo;
+    const void *residual;
+    long ldr;
+    void *h_out;
+    const void *norm_weight;
+    float eps;
+    void *xn_out;
+    int H, Hkv, Smax;
+    void *q, *k, *v;
+    const void *cos_tab, *sin_tab;
+    const int32_t *pos_dev, *t_dev;
+    void *cache_k, *cache_ks, *cache_v, *cache_vs;
+} smh_finish;
+int smh_q40_matmul_fused(const void *a, int M, int K, long lda, int nseg, const void *const *w,
+                         const void *const *s, const int *n, void *partial, size_t partial_bytes,
+                         const smh_finish *fin, smh_stream_t stream);
+
 /* ---- whole decode step ------------------------------------------------------------------------
  * smh_decode_step: one decode step (start_pos != 0) of Transformer.forward
  * (hf_model_q40_kv_shared.py:481-512) up to, not including, the final norm and lm_head, for

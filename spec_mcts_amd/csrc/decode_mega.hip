@@ -134,39 +134,6 @@ __device__ __forceinline__ int pick3(const int (&v)[3], int i) { return sel3(i, 
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
-// ---- coherent accessors ------------------------------------------------------------------------------
-__device__ __forceinline__ void st_u32(void *p, uint32_t v) {
-    __hip_atomic_store(reinterpret_cast<uint32_t *>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ uint32_t ld_u32(const void *p) {
-    return __hip_atomic_load(reinterpret_cast<const uint32_t *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ void st_u64(void *p, u32x2 v) {
-    __hip_atomic_store(reinterpret_cast<uint64_t *>(p), __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-__device__ __forceinline__ u32x2 ld_u64(const void *p) {
-    return __builtin_bit_cast(u32x2, __hip_atomic_load(reinterpret_cast<const uint64_t *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
-}
-__device__ __forceinline__ void st_f32(float *p, float v) { st_u32(p, __builtin_bit_cast(uint32_t, v)); }
-__device__ __forceinline__ float ld_f32(const float *p) { return __builtin_bit_cast(float, ld_u32(p)); }
-// (whole-vector bit casts only: __builtin_bit_cast applied to ONE ELEMENT of an ext_vector reads element 0)
-__device__ __forceinline__ void st_f4(float *p, f4 v) {
-    const u32x4 u = __builtin_bit_cast(u32x4, v);
-    st_u64(p, u32x2{u[0], u[1]});
-    st_u64(p + 2, u32x2{u[2], u[3]});
-}
-__device__ __forceinline__ f4 ld_f4(const float *p) {
-    const u32x2 a = ld_u64(p), b = ld_u64(p + 2);
-    return __builtin_bit_cast(f4, u32x4{a[0], a[1], b[0], b[1]});
-}
-__device__ __forceinline__ h4 ld_h4(const half_t *p) { return __builtin_bit_cast(h4, ld_u64(p)); }
-__device__ __forceinline__ void st_h4(half_t *p, h4 v) { st_u64(p, __builtin_bit_cast(u32x2, v)); }
-__device__ __forceinline__ void wait_vmem() {
-#ifdef SMH_MEGA_RELEASE_FENCE
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "agent");
-#endif
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-}
 // workgroup barrier that does not wait for the ring loads in flight (LDS traffic only)
 __device__ __forceinline__ void wg_sync() {
     asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");

@@ -294,7 +294,14 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         if (n_seg >= seg.N) continue;
         const int n = seg.col0 + n_seg;
         if (p.direct) p.c[(long)m * p.ldc + n] = matmul_epilogue(p, sum, m, n);
+        else if (p.fin.mode != 0) st_f32(slab + (long)m * p.n_total + n, sum);     // another workgroup of this launch reads it
         else slab[(long)m * p.n_total + n] = sum;
+    }
+    if (p.fin.mode != 0) {
+        uint32_t *s_flag = reinterpret_cast<uint32_t *>(lds);      // the sums in LDS have been consumed ...
+        __syncthreads();                                           // ... by every thread
+        matmul_finish<THREADS>(p.fin, p.partial, p.ksplit, p.M, p.n_total, unit, p.units, seg.col0 + col0,
+                               min(GEMV_COLS, seg.N - col0), sg, col0, s_flag);
     }
 }
 

@@ -10,6 +10,8 @@
 #define SMH_MAX_KSPLIT 16
 #define SMH_MAX_SEGMENTS 3
 
+#include "matmul_finish.hpp"
+
 namespace smh {
 
 struct MatmulSegment {
@@ -33,6 +35,7 @@ struct MatmulParams {
     int mblocks;             // GEMM: 128-row blocks
     int ksplit, steps_per_slice;
     int epilogue, direct;
+    MatmulFinish fin;        // fin.mode == 0: leave the slabs to another launch
 };
 
 __device__ __forceinline__ half_t matmul_epilogue(const MatmulParams &p, float acc, int m, int n) {

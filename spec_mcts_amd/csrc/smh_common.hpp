@@ -96,39 +96,39 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
-// ---- cross-workgroup hand-off of partial sums ----------------------------------------------------
-// Partial results written by one workgroup and read by another (possibly on a different XCD, i.e.
-// behind a different L2) travel as device-scope relaxed atomics: such stores write through to the
-// point of coherence and such loads never use a possibly stale cache line.  That makes full
-// device-scope fences unnecessary (they write back and invalidate the whole L2, which is ruinous
-// while other workgroups stream weights through it); all that is needed is that a workgroup's
-// stores have completed before its counter increment is issued.
-__device__ __forceinline__ void store_coherent(float *p, float v) {
-    __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+// ---- cross-workgroup hand-off inside one launch ------------------------------------------------------
+// Data written by one workgroup and read by another (possibly on a different XCD, i.e. behind a different
+// L2) travels as device-scope relaxed atomics: such stores write through to the point of coherence and
+// such loads never use a possibly stale cache line.  Full device-scope fences are avoided (they write back
+// and invalidate the whole L2, ruinous while other workgroups stream weights through it); all that is
+// needed is that a wave's stores have completed (wait_vmem) before it increments the counter that
+// announces them, and that a reader looks at the data only after it has seen the counter.
+__device__ __forceinline__ void st_u32(void *p, uint32_t v) {
+    __hip_atomic_store(reinterpret_cast<uint32_t *>(p), v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ float load_coherent(const float *p) {
-    return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ uint32_t ld_u32(const void *p) {
+    return __hip_atomic_load(reinterpret_cast<const uint32_t *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// wait until every memory operation this wave has issued is complete (stores acknowledged)
-__device__ __forceinline__ void wait_memory_ops() {
-    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+__device__ __forceinline__ void st_u64(void *p, u32x2 v) {
+    __hip_atomic_store(reinterpret_cast<uint64_t *>(p), __builtin_bit_cast(uint64_t, v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-// Counts arrivals of the workgroups that share `counter`; returns true in the last one (uniform over
-// the workgroup).  Call after store_coherent() of this workgroup's partials; in the last workgroup,
-// read the others' partials with load_coherent() and then reset the counter with arrive_reset().
-__device__ __forceinline__ bool arrive_is_last(uint32_t *counter, uint32_t expected, uint32_t *s_flag) {
-    wait_memory_ops();
-    __syncthreads();
-    if (threadIdx.x == 0) {
-        uint32_t prev = __hip_atomic_fetch_add(counter, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        *s_flag = (prev == expected - 1u) ? 1u : 0u;
-    }
-    __syncthreads();
-    return *s_flag != 0u;
+__device__ __forceinline__ u32x2 ld_u64(const void *p) {
+    return __builtin_bit_cast(u32x2, __hip_atomic_load(reinterpret_cast<const uint64_t *>(p), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
 }
-__device__ __forceinline__ void arrive_reset(uint32_t *counter) {
-    if (threadIdx.x == 0) __hip_atomic_store(counter, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+__device__ __forceinline__ void st_f32(float *p, float v) { st_u32(p, __builtin_bit_cast(uint32_t, v)); }
+__device__ __forceinline__ float ld_f32(const float *p) { return __builtin_bit_cast(float, ld_u32(p)); }
+// (whole-vector bit casts only: __builtin_bit_cast applied to ONE ELEMENT of an ext_vector reads element 0)
+__device__ __forceinline__ void st_f4(float *p, f4 v) {
+    const u32x4 u = __builtin_bit_cast(u32x4, v);
+    st_u64(p, u32x2{u[0], u[1]});
+    st_u64(p + 2, u32x2{u[2], u[3]});
 }
+__device__ __forceinline__ f4 ld_f4(const float *p) {
+    const u32x2 a = ld_u64(p), b = ld_u64(p + 2);
+    return __builtin_bit_cast(f4, u32x4{a[0], a[1], b[0], b[1]});
+}
+__device__ __forceinline__ h4 ld_h4(const half_t *p) { return __builtin_bit_cast(h4, ld_u64(p)); }
+__device__ __forceinline__ void st_h4(half_t *p, h4 v) { st_u64(p, __builtin_bit_cast(u32x2, v)); }
+__device__ __forceinline__ void wait_vmem() { asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); }
 
 }  // namespace smh

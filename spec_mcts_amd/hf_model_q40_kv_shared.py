@@ -259,6 +259,8 @@ class Transformer(nn.Module):
         self._step_state = None       # int32 [2] on the device: (position, suffix index t)
         self._step_host = None
         self.fused = True             # fused decode-layer launches; False runs module by module
+        self.finish_in_matmul = False # decode: finish the operator after each linear inside the matmul launch (6 launches per
+                                      # layer instead of 10; measured slower at B=10: the finisher's round trips are serial)
         self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
         self.persistent = True        # decode steps of few branches as one persistent kernel (needs fused)
         self.persistent_max_branches = 4   # above this the operator-by-operator launches are faster (the kernel itself takes up to 16)
@@ -316,6 +318,8 @@ class Transformer(nn.Module):
                 return self.output(hn.view(bsz, 1, p.dim)).to(DTYPE)
         h = self.tok_embeddings(tokens).to(DTYPE).reshape(M, p.dim)
         cos, sin = self._tables(h.device)
+        if start_pos != 0 and seqlen == 1 and self.finish_in_matmul and self._finish_shapes_ok():
+            return self._forward_decode_finished(h, cos, sin, step_state, bsz)
         pending = None                      # product of the previous layer's w2, not yet added to h
         for layer in self.layers:
             att, ff = layer.attention, layer.feed_forward
@@ -359,6 +363,36 @@ class Transformer(nn.Module):
             pending = K.matmul_q40_partial(act, [(ff.w2.w, ff.w2.s, ff.w2.shape[0])])
         _, hn = K.partial_rmsnorm(pending, h, self.norm.weight, self.norm.eps, want_h=False)
         return self.output(hn.view(bsz, seqlen, p.dim)).to(DTYPE)
+
+    def _finish_shapes_ok(self) -> bool:
+        """the in-launch finishers work on 256-column units: every linear's width must be a multiple of 256"""
+        att, ff = self.layers[0].attention, self.layers[0].feed_forward
+        widths = (self.params.dim, ff.w1.shape[0], att.n_local_heads * att.head_dim, att.n_local_kv_heads * att.head_dim)
+        return all(w % 256 == 0 for w in widths)
+
+    def _forward_decode_finished(self, h, cos, sin, step_state, bsz):
+        """One decode step with six launches per layer: wq|wk|wv (+RoPE, KV append), the two attention kernels,
+        wo (+residual, RMSNorm), w1|w3 (+SiLU*up), w2 (+residual, RMSNorm of the next sub-block); for more
+        than 16 rows each matmul is followed by its small finishing launch instead."""
+        p = self.params
+        pos_dev, t_dev = step_state
+        seg = lambda lin: (lin.w, lin.s, lin.shape[0])
+        xn = K.rmsnorm(h, self.layers[0].attention_norm.weight, self.layers[0].attention_norm.eps)
+        n_layers = len(self.layers)
+        for i, layer in enumerate(self.layers):
+            att, ff = layer.attention, layer.feed_forward
+            H, Hkv = att.n_local_heads, att.n_local_kv_heads
+            q, k, v = K.matmul_q40_rope_append_kv(xn, seg(att.wq), seg(att.wk), seg(att.wv), H, Hkv, cos, sin, pos_dev,
+                                                  att.cache_k, att.cache_k_s, att.cache_v, att.cache_v_s, p.max_seq_len, t_dev)
+            o = K.shared_prefix_attn(q, att.cache_prompt_k[0], att.cache_prompt_v[0], att.cache_prompt_len,
+                                     suffix_k=att.cache_k, suffix_v=att.cache_v, suffix_ks=att.cache_k_s,
+                                     suffix_vs=att.cache_v_s, Smax=p.max_seq_len, lens=t_dev, lens_stride=0,
+                                     cur_k=k, cur_v=v).view(bsz, H * att.head_dim)
+            h, xn = K.matmul_q40_residual_rmsnorm(o, seg(att.wo), h, layer.ffn_norm.weight, layer.ffn_norm.eps)
+            act = K.matmul_q40_silu_mul(xn, seg(ff.w1), seg(ff.w3))
+            nxt = self.layers[i + 1].attention_norm if i + 1 < n_layers else self.norm
+            h, xn = K.matmul_q40_residual_rmsnorm(act, seg(ff.w2), h, nxt.weight, nxt.eps)
+        return self.output(xn.view(bsz, 1, p.dim)).to(DTYPE)
 
     def _step_kernel(self, bsz: int, device):
         """The persistent decode kernel for `bsz` branches, or None when the model shape is outside it."""
