@@ -112,6 +112,8 @@ def matmul_roofline(torch, model, M, iters):
     graph = torch.cuda.CUDAGraph()
     with torch.cuda.graph(graph):
         run()
+    for _ in range(10):                  # clocks and caches settle before the timed replays
+        graph.replay()
     ms = time_region(torch, graph.replay, iters)
     total_bytes = sum(sum(q40_bytes(0, n, k_in) for _, _, n in segs) + 2 * M * k_in + 4 * M * sum(n for _, _, n in segs)
                       for k_in, segs in launches)
@@ -196,7 +198,7 @@ def main():
         dst.copy_(src)                                     # 1 GiB read + 1 GiB written by one elementwise kernel
         torch.cuda.synchronize()
         del src, dst
-        print(json.dumps(matmul_roofline(torch, model, a.roofline_only, 1)))
+        print(json.dumps(matmul_roofline(torch, model, a.roofline_only, 3)))
         return
     batches = tuple(int(x) for x in a.batches.split(",")) if a.batches else BATCHES
     by_batch = {}

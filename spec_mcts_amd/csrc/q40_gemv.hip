@@ -171,7 +171,9 @@ __device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K
 #undef SMH_GEMV_BYTE
 }
 
-template <int WAVES>
+// FINISH: the workgroup that completes a column unit also applies the operator that follows the linear
+// (matmul_finish.hpp); a separate instantiation, so that the plain kernel keeps its register budget
+template <int WAVES, bool FINISH>
 __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // WAVES rings, then reused as red[WAVES][M][256]
     constexpr int THREADS = WAVES * 64;
@@ -294,10 +296,10 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         if (n_seg >= seg.N) continue;
         const int n = seg.col0 + n_seg;
         if (p.direct) p.c[(long)m * p.ldc + n] = matmul_epilogue(p, sum, m, n);
-        else if (p.fin.mode != 0) st_f32(slab + (long)m * p.n_total + n, sum);     // another workgroup of this launch reads it
+        else if (FINISH) st_f32(slab + (long)m * p.n_total + n, sum);              // another workgroup of this launch reads it
         else slab[(long)m * p.n_total + n] = sum;
     }
-    if (p.fin.mode != 0) {
+    if constexpr (FINISH) {
         uint32_t *s_flag = reinterpret_cast<uint32_t *>(lds);      // the sums in LDS have been consumed ...
         __syncthreads();                                           // ... by every thread
         matmul_finish<THREADS>(p.fin, p.partial, p.ksplit, p.M, p.n_total, unit, p.units, seg.col0 + col0,
@@ -357,9 +359,10 @@ int gemv_launch(const MatmulParams &p, hipStream_t stream) {
     size_t lds = (size_t)waves * RING_BYTES;                       // rings, reused for the [waves][M][256] sums
     const size_t red = (size_t)waves * p.M * GEMV_COLS * sizeof(float);
     if (red > lds) lds = red;
-    if (waves == 2) hipLaunchKernelGGL(q40_gemv_kernel<2>, grid, dim3(128), lds, stream, p);
-    else if (waves == 8) hipLaunchKernelGGL(q40_gemv_kernel<8>, grid, dim3(512), lds, stream, p);
-    else hipLaunchKernelGGL(q40_gemv_kernel<4>, grid, dim3(256), lds, stream, p);
+    if (p.fin.mode != 0) hipLaunchKernelGGL((q40_gemv_kernel<4, true>), grid, dim3(256), lds, stream, p);
+    else if (waves == 2) hipLaunchKernelGGL((q40_gemv_kernel<2, false>), grid, dim3(128), lds, stream, p);
+    else if (waves == 8) hipLaunchKernelGGL((q40_gemv_kernel<8, false>), grid, dim3(512), lds, stream, p);
+    else hipLaunchKernelGGL((q40_gemv_kernel<4, false>), grid, dim3(256), lds, stream, p);
     return launch_status();
 }
 
