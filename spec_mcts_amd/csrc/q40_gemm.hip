@@ -1,18 +1,24 @@
 // Q4_0 dequant + matmul for large batches (decode at B = 100, prefill): c[M,N] = a[M,K] . deq(W)[K,N].
 //
-// A workgroup of 8 waves owns 128 rows of A, two adjacent 128-column blocks of the weight (one full
-// 128-byte line of packed nibbles per k) and a slice of K.  Everything a 32-row step needs - 4 KB of
-// nibbles, 256 B of scales, the 128 x 32 tile of A - goes global -> LDS by DMA (global_load_lds) into a
-// 4-stage ring shared by the workgroup, three steps ahead of the step being computed; one barrier per
-// step both publishes a stage and frees the oldest one.
-//   * wave w decodes ONE byte position of ONE block (block w/4, byte w%4 of every dword): perm pairs
-//     the byte of two consecutive rows, and-or drops the nibbles into fp16 mantissas, one packed op
-//     recovers the exact code and one packed multiply applies the scales - the value the reference's
-//     dequantiser produces, born in the B-operand layout of v_mfma_f32_16x16x32_f16, so dequantised
-//     weights never travel through LDS or HBM;
-//   * it multiplies its two B operands (high / low nibbles = columns c and c+64) with all (up to 8)
-//     16-row tiles of A, read from LDS with an XOR swizzle that keeps ds_read_b128 conflict-free;
-//   * the accumulators leave through LDS one row tile at a time, so global stores are 32-byte
+// A workgroup of 4 waves owns 128 rows of A, two adjacent 128-column blocks of the weight (one full
+// 128-byte line of packed nibbles per k) and a slice of K; two workgroups share a compute unit.
+// Everything a 32-row step needs - 4 KB of nibbles, 256 B of scales, the 128 x 32 tile of A - goes
+// global -> LDS by DMA (global_load_lds) into a 6-stage ring shared by the workgroup; one bare
+// s_barrier per step both publishes a stage and frees the oldest one.  (__syncthreads() would wait
+// for every outstanding DMA first, because they write LDS, and so empty the ring at every step.)
+//   * wave w decodes TWO byte positions of ONE block (block w/2, bytes 2(w%2) and 2(w%2)+1 of every
+//     dword): perm pairs the byte of two consecutive rows, and-or drops the nibbles into fp16
+//     mantissas, one packed op recovers the exact code and one packed multiply applies the scales -
+//     the value the reference's dequantiser produces, born in the B-operand layout of
+//     v_mfma_f32_16x16x32_f16, so dequantised weights never travel through LDS or HBM;
+//   * it multiplies its four B operands (2 byte positions x high / low nibbles = columns c and c+64)
+//     with all TILES 16-row tiles of A, read from LDS with an XOR swizzle that keeps ds_read_b128
+//     conflict-free: one read of the A tile feeds four MFMAs;
+//   * the step is software-pipelined inside the wave: while the matrix pipe works through step i,
+//     the vector ALU decodes the B operands of step i+1 (one basic block, no branches: the number of
+//     row tiles and the ragged-K handling are template parameters), and the DMA addresses are a
+//     scalar base per step plus lane offsets that never change, so issuing a stage costs no VALU work;
+//   * the accumulators leave through LDS one row tile at a time, so global stores are 64-byte
 //     contiguous per lane; K-slices are written as fp32 slabs and added by the consuming kernel.
 //
 // At M = 100 the work sits on the ridge of the roofline: 2*M*N*K flops against
@@ -22,21 +28,36 @@
 namespace smh {
 
 constexpr int GEMM_BM = 128;
-constexpr int GEMM_WAVES = 8;
+constexpr int GEMM_WAVES = 4;
 constexpr int GEMM_THREADS = GEMM_WAVES * 64;
-constexpr int GEMM_STAGES = 4;
+constexpr int GEMM_STAGES = 6;
 constexpr int GS_W = 32 * 128;                 // nibbles
 constexpr int GS_S = 32 * 8;                   // scales
 constexpr int GS_A = GEMM_BM * 64;             // A tile, 64 B per row, 16-byte chunks XOR-swizzled
-constexpr int GS_PAD = 256;                    // landing zone of the padding DMA (keeps 2 DMAs per wave per stage)
-constexpr int GS_BYTES = GS_W + GS_S + GS_A + GS_PAD;      // 12800
-constexpr int GEMM_LDS = GEMM_STAGES * GS_BYTES;           // 51200
+constexpr int GS_BYTES = GS_W + GS_S + GS_A;               // 12544
+constexpr int GEMM_LDS = GEMM_STAGES * GS_BYTES;           // 75264: two workgroups per compute unit
 constexpr int GEMM_COLS = 256;
 
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
-__global__ __launch_bounds__(GEMM_THREADS) void q40_gemm_kernel(MatmulParams p) {
+// Waits until at most `stages` younger stages (4 DMA instructions each) of this wave are still in flight.
+__device__ __forceinline__ void gemm_wait_dma(int stages) {
+    switch (stages) {
+        case 4: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+        case 3: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+        case 2: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+        case 1: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    }
+}
+
+// A bare workgroup barrier.  Every LDS read this wave has issued has returned (lgkmcnt), so after the
+// barrier no wave still reads the stage that is refilled next.
+__device__ __forceinline__ void gemm_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
+template <int TILES, bool RAGGED>
+__global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
     const int tid = threadIdx.x;
@@ -59,42 +80,54 @@ __global__ __launch_bounds__(GEMM_THREADS) void q40_gemm_kernel(MatmulParams p) 
     const int col0 = pair * GEMM_COLS;
     const bool two_blocks = col0 + 128 < seg.N;
     const int m0 = mb * GEMM_BM;
-    const int m_count = min(GEMM_BM, p.M - m0);
-    const int tiles = (m_count + 15) / 16;
-    const int blk = wave >> 2;                 // block of the pair this wave decodes
-    const uint32_t sel = 0x0c000c00u | (uint32_t)(wave & 3) | ((uint32_t)(4 + (wave & 3)) << 16);
+    const int blk = wave >> 1;                 // block of the pair this wave decodes
+    const int bp = wave & 1;                   // ... and its pair of byte positions
+    const uint32_t sel0 = 0x0c000c00u | (uint32_t)(2 * bp) | ((uint32_t)(4 + 2 * bp) << 16);
+    const uint32_t sel1 = sel0 + 0x00010001u;
 
-    const long w_row = seg.N / 2;
-    const long s_row = seg.N / 64;
-    // ---- this wave's two DMA instructions per stage ----
-    //  first : waves 0..3 -> 8 rows of nibbles each; wave 4 -> scales; waves 5..7 -> padding (scales again)
-    //  second: wave w -> rows 16w .. 16w+15 of the A tile
-    const uint8_t *w_lane = seg.w + (long)pair * 128 + 16 * (two_blocks ? (lane & 7) : (lane & 3));
-    const half_t *s_lane = seg.s + (long)pair * 4 + 2 * (two_blocks ? (lane & 1) : 0);
-    const int a_row = 16 * wave + (lane >> 2);                            // row of the tile this lane fetches
-    const int a_chunk = (lane & 3) ^ ((a_row >> 2) & 3);                  // logical 16-byte chunk stored in slot lane&3
-    const half_t *a_lane = p.a + (long)min(m0 + a_row, p.M - 1) * p.lda;
+    const long w_row = seg.N / 2;              // bytes per k of the nibbles
+    const long s_row = seg.N / 32;             // bytes per k of the scales
+    // ---- this wave's four DMA instructions per stage ----
+    //  rows 8w .. 8w+7 of the nibbles; their scales (lanes 0..15); rows 32w .. 32w+31 of the A tile.
+    //  Address = uniform base of the step (scalar arithmetic) + a lane offset fixed for the whole kernel.
+    const uint8_t *w_base = seg.w + (long)pair * 128;
+    const uint8_t *s_base = reinterpret_cast<const uint8_t *>(seg.s) + (long)pair * 8;
+    const uint8_t *a_base = reinterpret_cast<const uint8_t *>(p.a);
+    const int w_lrow = 8 * wave + (lane >> 3), w_lcol = 16 * (two_blocks ? (lane & 7) : (lane & 3));
+    const int s_lrow = 8 * wave + ((lane & 15) >> 1), s_lcol = 4 * (two_blocks ? (lane & 1) : 0);
+    const int a_chunk = (lane & 3) ^ ((lane >> 4) & 3);                   // logical 16-byte chunk stored in slot lane&3
+    const long a_r0 = (long)min(m0 + 32 * wave + (lane >> 2), p.M - 1) * p.lda * 2;
+    const long a_r1 = (long)min(m0 + 32 * wave + 16 + (lane >> 2), p.M - 1) * p.lda * 2;
+    const uint32_t w_voff = (uint32_t)(w_lrow * w_row + w_lcol);
+    const uint32_t s_voff = (uint32_t)(s_lrow * s_row + s_lcol);
+    const uint32_t a_voff0 = (uint32_t)(a_r0 + 16 * a_chunk), a_voff1 = (uint32_t)(a_r1 + 16 * a_chunk);
 
-    auto issue = [&](int step, int stage) {
-        uint8_t *st = lds + stage * GS_BYTES;
-        const int k0 = step * 32;
-        if (wave < 4) {
-            const int row = min(k0 + 8 * wave + (lane >> 3), p.K - 1);
-            __builtin_amdgcn_global_load_lds((gptr_t)(w_lane + (long)row * w_row), (lptr_t)(st + wave * 1024), 16, 0, 0);
+    auto issue = [&](int step, int slot_) {
+        uint8_t *st = lds + slot_ * GS_BYTES;
+        const long k0 = (long)step * 32;
+        if (!RAGGED) {
+            __builtin_amdgcn_global_load_lds((gptr_t)(w_base + k0 * w_row + w_voff), (lptr_t)(st + wave * 1024), 16, 0, 0);
+            if (lane < 16)
+                __builtin_amdgcn_global_load_lds((gptr_t)(s_base + k0 * s_row + s_voff), (lptr_t)(st + GS_W + wave * 64), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(a_base + k0 * 2 + a_voff0), (lptr_t)(st + GS_W + GS_S + wave * 2048), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(a_base + k0 * 2 + a_voff1), (lptr_t)(st + GS_W + GS_S + wave * 2048 + 1024), 16, 0, 0);
         } else {
-            const int row = min(k0 + (lane >> 1), p.K - 1);
-            uint8_t *dst = (wave == 4) ? st + GS_W : st + GS_W + GS_S + GS_A;
-            __builtin_amdgcn_global_load_lds((gptr_t)(s_lane + (long)row * s_row), (lptr_t)dst, 4, 0, 0);
+            // rows past K repeat row K-1 (their products are masked out below); the A columns stay inside the row
+            const long wr = min(k0 + w_lrow, (long)p.K - 1), sr = min(k0 + s_lrow, (long)p.K - 1);
+            const long ac = min(k0 + 8 * a_chunk, (long)p.K - 8) * 2;
+            __builtin_amdgcn_global_load_lds((gptr_t)(w_base + wr * w_row + w_lcol), (lptr_t)(st + wave * 1024), 16, 0, 0);
+            if (lane < 16)
+                __builtin_amdgcn_global_load_lds((gptr_t)(s_base + sr * s_row + s_lcol), (lptr_t)(st + GS_W + wave * 64), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(a_base + a_r0 + ac), (lptr_t)(st + GS_W + GS_S + wave * 2048), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(a_base + a_r1 + ac), (lptr_t)(st + GS_W + GS_S + wave * 2048 + 1024), 16, 0, 0);
         }
-        const int col = min(k0 + 8 * a_chunk, p.K - 8);
-        __builtin_amdgcn_global_load_lds((gptr_t)(a_lane + col), (lptr_t)(st + GS_W + GS_S + wave * 1024), 16, 0, 0);
     };
 
-    f4 acc[2][8];
+    f4 acc[4][TILES];
 #pragma unroll
-    for (int h = 0; h < 2; ++h)
+    for (int h = 0; h < 4; ++h)
 #pragma unroll
-        for (int t = 0; t < 8; ++t) acc[h][t] = f4{0.f, 0.f, 0.f, 0.f};
+        for (int t = 0; t < TILES; ++t) acc[h][t] = f4{0.f, 0.f, 0.f, 0.f};
 
     const int step0 = slice * p.steps_per_slice;
     const int step1 = min(step0 + p.steps_per_slice, (p.K + 31) / 32);
@@ -102,88 +135,128 @@ __global__ __launch_bounds__(GEMM_THREADS) void q40_gemm_kernel(MatmulParams p) 
     // workgroups that share a K-slice read the same A tiles; each starts at a different step of the
     // slice (and wraps) so that they do not all pull the same L2 lines at the same time
     const int rot = n_steps > 0 ? (unit * 5) % n_steps : 0;
-    auto step_of = [&](int i) { const int j = i + rot; return step0 + (j >= n_steps ? j - n_steps : j); };
+    int fetch = step0 + rot;                   // next step to fetch
+    auto fetch_next = [&](int slot_) {
+        issue(fetch, slot_);
+        fetch = fetch + 1 == step1 ? step0 : fetch + 1;
+    };
 #pragma unroll
     for (int i = 0; i < GEMM_STAGES - 1; ++i)
-        if (i < n_steps) issue(step_of(i), i);
+        if (i < n_steps) fetch_next(i);
 
-    for (int i = 0; i < n_steps; ++i) {
-        const int later = min(GEMM_STAGES - 2, n_steps - 1 - i);     // younger steps this wave has in flight
-        if (later >= 2) asm volatile("s_waitcnt vmcnt(4)" ::: "memory");
-        else if (later == 1) asm volatile("s_waitcnt vmcnt(2)" ::: "memory");
-        else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        __syncthreads();     // stage i is complete for everyone; everyone is done with stage i-1
-        if (i + GEMM_STAGES - 1 < n_steps) issue(step_of(i + GEMM_STAGES - 1), (i + GEMM_STAGES - 1) % GEMM_STAGES);
-
-        const uint8_t *st = lds + (i % GEMM_STAGES) * GS_BYTES;
-        const int k0 = step_of(i) * 32;
-        // ---- decode this wave's byte position: exact fp16 code * scale ----
-        uint32_t wv[8], sv[8];
+    // the eight dwords of this lane's column bytes and of their scales, for one step
+    auto load_ws = [&](const uint8_t *st, uint32_t (&wv)[8], uint32_t (&sv)[8]) {
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
             wv[r] = *reinterpret_cast<const uint32_t *>(st + (8 * g + r) * 128 + 64 * blk + 4 * c);
             sv[r] = *reinterpret_cast<const uint32_t *>(st + GS_W + (8 * g + r) * 8 + 4 * blk);
         }
-        u32x4 vh, vl;
+    };
+    // exact fp16 code * scale, as the four B operands (byte 2bp high / low, byte 2bp+1 high / low)
+    auto decode = [&](const uint32_t (&wv)[8], const uint32_t (&sv)[8], bool dead, h8 (&b)[4]) {
+        u32x4 v0h, v0l, v1h, v1l;
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            const uint32_t pr = __builtin_amdgcn_perm(wv[2 * j + 1], wv[2 * j], sel) ^ 0x00880088u;
-            vh[j] = as_u32(codes_high(pr) * as_h2(pack_lo16(sv[2 * j], sv[2 * j + 1])));
-            vl[j] = as_u32(codes_low(pr) * as_h2(pack_hi16(sv[2 * j], sv[2 * j + 1])));
+            const uint32_t pr0 = __builtin_amdgcn_perm(wv[2 * j + 1], wv[2 * j], sel0) ^ 0x00880088u;
+            const uint32_t pr1 = __builtin_amdgcn_perm(wv[2 * j + 1], wv[2 * j], sel1) ^ 0x00880088u;
+            const h2 s_hi = as_h2(pack_lo16(sv[2 * j], sv[2 * j + 1]));
+            const h2 s_lo = as_h2(pack_hi16(sv[2 * j], sv[2 * j + 1]));
+            v0h[j] = as_u32(codes_high(pr0) * s_hi);
+            v0l[j] = as_u32(codes_low(pr0) * s_lo);
+            v1h[j] = as_u32(codes_high(pr1) * s_hi);
+            v1l[j] = as_u32(codes_low(pr1) * s_lo);
         }
-        const h8 vb_h = __builtin_bit_cast(h8, vh), vb_l = __builtin_bit_cast(h8, vl);
-        const bool k_tail = k0 + 8 * g >= p.K;                       // only in the last step when K % 32 != 0
-        const uint8_t *at = st + GS_W + GS_S;
+        if (RAGGED && dead) v0h = v0l = v1h = v1l = u32x4{0u, 0u, 0u, 0u};     // k >= K: no contribution
+        b[0] = __builtin_bit_cast(h8, v0h);
+        b[1] = __builtin_bit_cast(h8, v0l);
+        b[2] = __builtin_bit_cast(h8, v1h);
+        b[3] = __builtin_bit_cast(h8, v1l);
+    };
+    auto k_dead = [&](int step) { return step * 32 + 8 * g >= p.K; };      // only in the last step when K % 32 != 0
+
+    if (n_steps > 0) {
+        h8 bq[4];
+        int cur = step0 + rot;                 // step being multiplied
+        {
+            gemm_wait_dma(min(GEMM_STAGES - 2, n_steps - 1));
+            gemm_barrier();
+            uint32_t wv[8], sv[8];
+            load_ws(lds, wv, sv);
+            decode(wv, sv, k_dead(cur), bq);
+        }
+        int stage = 0;                         // ring slot of step i
+        for (int i = 0; i < n_steps; ++i) {
+            // stage i+1 has landed for this wave (younger ones may still be in flight) ...
+            gemm_wait_dma(min(GEMM_STAGES - 3, max(n_steps - 2 - i, 0)));
+            // ... and for everyone; everyone is also done with stage i-1, whose slot is refilled now
+            gemm_barrier();
+            if (i + GEMM_STAGES - 1 < n_steps) fetch_next(stage == 0 ? GEMM_STAGES - 1 : stage - 1);
+
+            const uint8_t *st = lds + stage * GS_BYTES;
+            stage = stage == GEMM_STAGES - 1 ? 0 : stage + 1;
+            const int nxt = cur + 1 == step1 ? step0 : cur + 1;
+            cur = nxt;
+            // one basic block: the MFMAs of step i and the decode of step i+1 (past the last step the slot holds
+            // stale bytes, decoded and never used)
+            uint32_t wv[8], sv[8];
+            load_ws(lds + stage * GS_BYTES, wv, sv);
+            const uint8_t *at = st + GS_W + GS_S;
+            h8 av[TILES];
 #pragma unroll
-        for (int t = 0; t < 8; ++t) {
-            if (t < tiles) {
+            for (int t = 0; t < TILES; ++t) {
                 const int r = 16 * t + c;
-                h8 av = *reinterpret_cast<const h8 *>(at + r * 64 + ((g ^ ((r >> 2) & 3)) << 4));
-                if (k_tail) {
-#pragma unroll
-                    for (int e = 0; e < 8; ++e) av[e] = (half_t)0.f;
-                }
-                acc[0][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, vb_h, acc[0][t], 0, 0, 0);
-                acc[1][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av, vb_l, acc[1][t], 0, 0, 0);
+                av[t] = *reinterpret_cast<const h8 *>(at + r * 64 + ((g ^ ((r >> 2) & 3)) << 4));
             }
+            h8 bn[4];
+            decode(wv, sv, k_dead(nxt), bn);
+#pragma unroll
+            for (int t = 0; t < TILES; ++t) {
+#pragma unroll
+                for (int o = 0; o < 4; ++o) acc[o][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], bq[o], acc[o][t], 0, 0, 0);
+            }
+#pragma unroll
+            for (int o = 0; o < 4; ++o) bq[o] = bn[o];
         }
     }
 
     // ---- results leave one 16-row tile at a time through LDS: [16][256 + 4] floats ----
-    // accumulator element r of acc[h][t] is row 16t + 4g + r, column 128*blk + 64h + 4c + (wave & 3)
+    // accumulator element r of acc[o][t] is row 16t + 4g + r, column 128*blk + 64*(o&1) + 4c + 2*bp + (o>>1)
     constexpr int OP = GEMM_COLS + 4;
     float *otile = reinterpret_cast<float *>(lds);
     float *slab = p.partial + (long)slice * p.M * p.n_total;
-    const int o_row = tid >> 5;                 // 0..15
-    const int o_col = (tid & 31) * 8;           // 8 consecutive columns
+    const int o_row = tid >> 4;                 // 0..15
+    const int o_col = (tid & 15) * 16;          // 16 consecutive columns
 #pragma unroll
-    for (int t = 0; t < 8; ++t) {
-        if (t < tiles) {
-            __syncthreads();
+    for (int t = 0; t < TILES; ++t) {
+        __syncthreads();
 #pragma unroll
-            for (int h = 0; h < 2; ++h)
+        for (int o = 0; o < 4; ++o)
 #pragma unroll
-                for (int r = 0; r < 4; ++r) otile[(4 * g + r) * OP + 128 * blk + 64 * h + 4 * c + (wave & 3)] = acc[h][t][r];
-            __syncthreads();
-            const int m = m0 + 16 * t + o_row;
-            const int n_seg = col0 + o_col;
-            if (m < p.M && n_seg < seg.N) {
-                const f4 v0 = *reinterpret_cast<const f4 *>(otile + o_row * OP + o_col);
-                const f4 v1 = *reinterpret_cast<const f4 *>(otile + o_row * OP + o_col + 4);
-                const int n = seg.col0 + n_seg;
-                if (p.direct) {
+            for (int r = 0; r < 4; ++r)
+                otile[(4 * g + r) * OP + 128 * blk + 64 * (o & 1) + 4 * c + 2 * bp + (o >> 1)] = acc[o][t][r];
+        __syncthreads();
+        const int m = m0 + 16 * t + o_row;
+        const int n_seg = col0 + o_col;
+        if (m < p.M && n_seg < seg.N) {
+            const int n = seg.col0 + n_seg;
+            f4 v[4];
+#pragma unroll
+            for (int q = 0; q < 4; ++q) v[q] = *reinterpret_cast<const f4 *>(otile + o_row * OP + o_col + 4 * q);
+            if (p.direct) {
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
                     h8 o;
 #pragma unroll
                     for (int e = 0; e < 4; ++e) {
-                        o[e] = matmul_epilogue(p, v0[e], m, n + e);
-                        o[4 + e] = matmul_epilogue(p, v1[e], m, n + 4 + e);
+                        o[e] = matmul_epilogue(p, v[2 * q][e], m, n + 8 * q + e);
+                        o[4 + e] = matmul_epilogue(p, v[2 * q + 1][e], m, n + 8 * q + 4 + e);
                     }
-                    *reinterpret_cast<h8 *>(p.c + (long)m * p.ldc + n) = o;
-                } else {
-                    float *dst = slab + (long)m * p.n_total + n;
-                    *reinterpret_cast<f4 *>(dst) = v0;
-                    *reinterpret_cast<f4 *>(dst + 4) = v1;
+                    *reinterpret_cast<h8 *>(p.c + (long)m * p.ldc + n + 8 * q) = o;
                 }
+            } else {
+                float *dst = slab + (long)m * p.n_total + n;
+#pragma unroll
+                for (int q = 0; q < 4; ++q) *reinterpret_cast<f4 *>(dst + 4 * q) = v[q];
             }
         }
     }
@@ -218,9 +291,29 @@ void gemm_fill_plan(MatmulParams &p) {
     p.ksplit = (steps + p.steps_per_slice - 1) / p.steps_per_slice;
 }
 
+typedef void (*gemm_kernel_t)(MatmulParams);
+
 int gemm_launch(const MatmulParams &p, hipStream_t stream) {
+    // one instantiation per number of 16-row tiles (M <= 128) keeps the step free of branches; K % 32 != 0
+    // takes the masked variant with all 8 tiles
+    static const gemm_kernel_t exact[9] = {nullptr, q40_gemm_kernel<2, false>, q40_gemm_kernel<2, false>, q40_gemm_kernel<3, false>,
+                                           q40_gemm_kernel<4, false>, q40_gemm_kernel<5, false>, q40_gemm_kernel<6, false>,
+                                           q40_gemm_kernel<7, false>, q40_gemm_kernel<8, false>};
+    static const gemm_kernel_t ragged = q40_gemm_kernel<8, true>;
+    // more than 64 KB of dynamic LDS has to be allowed once per kernel (the attribute is not stream work,
+    // so a launch under graph capture is not affected)
+    static const hipError_t lds_ok = [] {
+        hipError_t e = hipFuncSetAttribute((const void *)ragged, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS);
+        for (int t = 2; t <= 8 && e == hipSuccess; ++t)
+            e = hipFuncSetAttribute((const void *)exact[t], hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS);
+        return e;
+    }();
+    if (lds_ok != hipSuccess) return (int)lds_ok;
+    if ((long)p.M * p.lda * 2 >= (1L << 32)) return (int)hipErrorInvalidValue;     // lane offsets of A are 32-bit
+    const int tiles = p.mblocks > 1 ? 8 : (p.M + 15) / 16;
+    const gemm_kernel_t kern = (p.K % 32 != 0) ? ragged : exact[tiles < 2 ? 2 : tiles];
     dim3 grid((unsigned)((long)p.units_pad * p.mblocks * p.ksplit));
-    hipLaunchKernelGGL(q40_gemm_kernel, grid, dim3(GEMM_THREADS), GEMM_LDS, stream, p);
+    hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), GEMM_LDS, stream, p);
     return launch_status();
 }
 
