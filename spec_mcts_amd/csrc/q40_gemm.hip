@@ -37,9 +37,24 @@ constexpr int GS_A = GEMM_BM * 64;             // A tile, 64 B per row, 16-byte 
 constexpr int GS_BYTES = GS_W + GS_S + GS_A;               // 12544
 constexpr int GEMM_LDS = GEMM_STAGES * GS_BYTES;           // 75264: two workgroups per compute unit
 constexpr int GEMM_COLS = 256;
+#ifndef GX_WAUX
+#define GX_WAUX 0
+#endif
 
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
+
+#ifdef GX_TRACE
+__device__ unsigned long long gx_trace[512][34][8];
+__device__ __forceinline__ unsigned long long gx_now() {
+    unsigned long long t;
+    asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
+    return t;
+}
+#define GXT(i, slot) do { if (lane == 0 && wave == GX_TRACE && blockIdx.x < 512 && (i) < 34) gx_trace[blockIdx.x][i][slot] = gx_now(); } while (0)
+#else
+#define GXT(i, slot) do { } while (0)
+#endif
 
 // Waits until at most `stages` younger stages (4 DMA instructions each) of this wave are still in flight.
 __device__ __forceinline__ void gemm_wait_dma(int stages) {
@@ -65,6 +80,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     const int lane = tid & 63;
     const int c = lane & 15;
     const int g = lane >> 4;
+    GXT(33, 1);
     int bid = blockIdx.x;
     // slot -> unit: each XCD (blockIdx % 8) takes a contiguous run of column units, which share scale lines
     const int slot = bid % p.units_pad;  bid /= p.units_pad;
@@ -106,7 +122,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
         uint8_t *st = lds + slot_ * GS_BYTES;
         const long k0 = (long)step * 32;
         if (!RAGGED) {
-            __builtin_amdgcn_global_load_lds((gptr_t)(w_base + k0 * w_row + w_voff), (lptr_t)(st + wave * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(w_base + k0 * w_row + w_voff), (lptr_t)(st + wave * 1024), 16, 0, GX_WAUX);
             if (lane < 16)
                 __builtin_amdgcn_global_load_lds((gptr_t)(s_base + k0 * s_row + s_voff), (lptr_t)(st + GS_W + wave * 64), 4, 0, 0);
             __builtin_amdgcn_global_load_lds((gptr_t)(a_base + k0 * 2 + a_voff0), (lptr_t)(st + GS_W + GS_S + wave * 2048), 16, 0, 0);
@@ -174,6 +190,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     };
     auto k_dead = [&](int step) { return step * 32 + 8 * g >= p.K; };      // only in the last step when K % 32 != 0
 
+    GXT(33, 2);
     if (n_steps > 0) {
         h8 bq[4];
         int cur = step0 + rot;                 // step being multiplied
@@ -185,12 +202,17 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             decode(wv, sv, k_dead(cur), bq);
         }
         int stage = 0;                         // ring slot of step i
+        GXT(33, 0);
         for (int i = 0; i < n_steps; ++i) {
+            if (i < 32) GXT(i, 0);
             // stage i+1 has landed for this wave (younger ones may still be in flight) ...
             gemm_wait_dma(min(GEMM_STAGES - 3, max(n_steps - 2 - i, 0)));
             // ... and for everyone; everyone is also done with stage i-1, whose slot is refilled now
+            if (i < 32) GXT(i, 1);
             gemm_barrier();
+            if (i < 32) GXT(i, 2);
             if (i + GEMM_STAGES - 1 < n_steps) fetch_next(stage == 0 ? GEMM_STAGES - 1 : stage - 1);
+            if (i < 32) GXT(i, 3);
 
             const uint8_t *st = lds + stage * GS_BYTES;
             stage = stage == GEMM_STAGES - 1 ? 0 : stage + 1;
@@ -216,50 +238,69 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             }
 #pragma unroll
             for (int o = 0; o < 4; ++o) bq[o] = bn[o];
+#ifdef GX_TRACE
+            asm volatile("" :: "v"(acc[0][0]), "v"(acc[3][TILES - 1]), "v"(bq[0]), "v"(bq[3]));
+            if (i < 32) { GXT(i, 4); GXT(i, 5); }
+#endif
         }
+        GXT(32, 0);
     }
 
-    // ---- results leave one 16-row tile at a time through LDS: [16][256 + 4] floats ----
-    // accumulator element r of acc[o][t] is row 16t + 4g + r, column 128*blk + 64*(o&1) + 4c + 2*bp + (o>>1)
+    // ---- results leave one 16-row tile at a time through LDS: [16][256 + 4] floats, two buffers in turn ----
+    // accumulator element r of acc[o][t] is row 16t + 4g + r, column 128*blk + 64*(o&1) + 4c + 2*bp + (o>>1).
+    // Bare barriers again: __syncthreads() would wait for the global stores of the previous tile to be
+    // acknowledged, one memory round trip per tile.  A buffer is rewritten two tiles later, after a barrier
+    // that every wave reaches only when its reads of that buffer have returned.
     constexpr int OP = GEMM_COLS + 4;
-    float *otile = reinterpret_cast<float *>(lds);
+    constexpr int OTILE_BYTES = 16 * OP * 4;
+    static_assert(2 * OTILE_BYTES <= GEMM_LDS, "two output tiles must fit in the ring");
     float *slab = p.partial + (long)slice * p.M * p.n_total;
     const int o_row = tid >> 4;                 // 0..15
-    const int o_col = (tid & 15) * 16;          // 16 consecutive columns
+    const int o_lane = tid & 15;                // store q of this lane: columns 64q + 4*o_lane .. (fp16: 128q + 8*o_lane ..),
+                                                // so that one store instruction writes whole contiguous rows
+    gemm_barrier();                             // every wave has left the main loop: the ring is free
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
-        __syncthreads();
+        float *otile = reinterpret_cast<float *>(lds + (t & 1) * OTILE_BYTES);
 #pragma unroll
         for (int o = 0; o < 4; ++o)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
                 otile[(4 * g + r) * OP + 128 * blk + 64 * (o & 1) + 4 * c + 2 * bp + (o >> 1)] = acc[o][t][r];
-        __syncthreads();
+        gemm_barrier();
         const int m = m0 + 16 * t + o_row;
-        const int n_seg = col0 + o_col;
-        if (m < p.M && n_seg < seg.N) {
-            const int n = seg.col0 + n_seg;
-            f4 v[4];
-#pragma unroll
-            for (int q = 0; q < 4; ++q) v[q] = *reinterpret_cast<const f4 *>(otile + o_row * OP + o_col + 4 * q);
+        if (m < p.M) {
             if (p.direct) {
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {
-                    h8 o;
+                    const int n_seg = col0 + 128 * q + 8 * o_lane;
+                    if (n_seg < seg.N) {
+                        const int n = seg.col0 + n_seg;
+                        const f4 v0 = *reinterpret_cast<const f4 *>(otile + o_row * OP + 128 * q + 8 * o_lane);
+                        const f4 v1 = *reinterpret_cast<const f4 *>(otile + o_row * OP + 128 * q + 8 * o_lane + 4);
+                        h8 o;
 #pragma unroll
-                    for (int e = 0; e < 4; ++e) {
-                        o[e] = matmul_epilogue(p, v[2 * q][e], m, n + 8 * q + e);
-                        o[4 + e] = matmul_epilogue(p, v[2 * q + 1][e], m, n + 8 * q + 4 + e);
+                        for (int e = 0; e < 4; ++e) {
+                            o[e] = matmul_epilogue(p, v0[e], m, n + e);
+                            o[4 + e] = matmul_epilogue(p, v1[e], m, n + 4 + e);
+                        }
+                        *reinterpret_cast<h8 *>(p.c + (long)m * p.ldc + n) = o;
                     }
-                    *reinterpret_cast<h8 *>(p.c + (long)m * p.ldc + n + 8 * q) = o;
                 }
             } else {
-                float *dst = slab + (long)m * p.n_total + n;
+                float *dst = slab + (long)m * p.n_total + seg.col0 + col0;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) *reinterpret_cast<f4 *>(dst + 4 * q) = v[q];
+                for (int q = 0; q < 4; ++q) {
+                    const int cq = 64 * q + 4 * o_lane;
+                    if (col0 + cq < seg.N) *reinterpret_cast<f4 *>(dst + cq) = *reinterpret_cast<const f4 *>(otile + o_row * OP + cq);
+                }
             }
         }
     }
+#ifdef GX_TRACE
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    GXT(33, 3);
+#endif
 }
 
 void gemm_fill_plan(MatmulParams &p) {
@@ -318,3 +359,9 @@ int gemm_launch(const MatmulParams &p, hipStream_t stream) {
 }
 
 }  // namespace smh
+
+#ifdef GX_TRACE
+extern "C" int smhdbg_gemm_trace(void *dst, size_t bytes) {
+    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(smh::gx_trace), bytes < sizeof(smh::gx_trace) ? bytes : sizeof(smh::gx_trace));
+}
+#endif
