@@ -23,6 +23,8 @@
 //
 // At M = 100 the work sits on the ridge of the roofline: 2*M*N*K flops against
 // N*K*0.53125 + 2*M*(K+N) bytes.
+#include <type_traits>
+
 #include "q40_matmul.hpp"
 
 namespace smh {
@@ -31,15 +33,14 @@ constexpr int GEMM_BM = 128;
 constexpr int GEMM_WAVES = 4;
 constexpr int GEMM_THREADS = GEMM_WAVES * 64;
 constexpr int GEMM_STAGES = 6;
-constexpr int GS_W = 32 * 128;                 // nibbles
+constexpr int GS_WBLOCK = 8 * 128 + 64;        // the 8 rows one wave fetches, padded by 16 banks: the four row groups a
+                                               // ds_read_b32 touches (lanes 16g..16g+15 read row 8g+r) then sit in different banks
+constexpr int GS_W = 4 * GS_WBLOCK;            // nibbles
 constexpr int GS_S = 32 * 8;                   // scales
 constexpr int GS_A = GEMM_BM * 64;             // A tile, 64 B per row, 16-byte chunks XOR-swizzled
-constexpr int GS_BYTES = GS_W + GS_S + GS_A;               // 12544
-constexpr int GEMM_LDS = GEMM_STAGES * GS_BYTES;           // 75264: two workgroups per compute unit
+constexpr int GS_BYTES = GS_W + GS_S + GS_A;               // 12800
+constexpr int GEMM_LDS = GEMM_STAGES * GS_BYTES;           // 76800: two workgroups per compute unit
 constexpr int GEMM_COLS = 256;
-#ifndef GX_WAUX
-#define GX_WAUX 0
-#endif
 
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
@@ -59,6 +60,7 @@ __device__ __forceinline__ unsigned long long gx_now() {
 // Waits until at most `stages` younger stages (4 DMA instructions each) of this wave are still in flight.
 __device__ __forceinline__ void gemm_wait_dma(int stages) {
     switch (stages) {
+        case 5: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
         case 4: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
         case 3: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
         case 2: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
@@ -122,7 +124,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
         uint8_t *st = lds + slot_ * GS_BYTES;
         const long k0 = (long)step * 32;
         if (!RAGGED) {
-            __builtin_amdgcn_global_load_lds((gptr_t)(w_base + k0 * w_row + w_voff), (lptr_t)(st + wave * 1024), 16, 0, GX_WAUX);
+            __builtin_amdgcn_global_load_lds((gptr_t)(w_base + k0 * w_row + w_voff), (lptr_t)(st + wave * GS_WBLOCK), 16, 0, 0);
             if (lane < 16)
                 __builtin_amdgcn_global_load_lds((gptr_t)(s_base + k0 * s_row + s_voff), (lptr_t)(st + GS_W + wave * 64), 4, 0, 0);
             __builtin_amdgcn_global_load_lds((gptr_t)(a_base + k0 * 2 + a_voff0), (lptr_t)(st + GS_W + GS_S + wave * 2048), 16, 0, 0);
@@ -131,7 +133,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             // rows past K repeat row K-1 (their products are masked out below); the A columns stay inside the row
             const long wr = min(k0 + w_lrow, (long)p.K - 1), sr = min(k0 + s_lrow, (long)p.K - 1);
             const long ac = min(k0 + 8 * a_chunk, (long)p.K - 8) * 2;
-            __builtin_amdgcn_global_load_lds((gptr_t)(w_base + wr * w_row + w_lcol), (lptr_t)(st + wave * 1024), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(w_base + wr * w_row + w_lcol), (lptr_t)(st + wave * GS_WBLOCK), 16, 0, 0);
             if (lane < 16)
                 __builtin_amdgcn_global_load_lds((gptr_t)(s_base + sr * s_row + s_lcol), (lptr_t)(st + GS_W + wave * 64), 4, 0, 0);
             __builtin_amdgcn_global_load_lds((gptr_t)(a_base + a_r0 + ac), (lptr_t)(st + GS_W + GS_S + wave * 2048), 16, 0, 0);
@@ -164,7 +166,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     auto load_ws = [&](const uint8_t *st, uint32_t (&wv)[8], uint32_t (&sv)[8]) {
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
-            wv[r] = *reinterpret_cast<const uint32_t *>(st + (8 * g + r) * 128 + 64 * blk + 4 * c);
+            wv[r] = *reinterpret_cast<const uint32_t *>(st + g * GS_WBLOCK + r * 128 + 64 * blk + 4 * c);
             sv[r] = *reinterpret_cast<const uint32_t *>(st + GS_W + (8 * g + r) * 8 + 4 * blk);
         }
     };
@@ -191,9 +193,28 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     auto k_dead = [&](int step) { return step * 32 + 8 * g >= p.K; };      // only in the last step when K % 32 != 0
 
     GXT(33, 2);
+    // While the matrix pipe multiplies step i (A tile read from stage i, B operands decoded one iteration
+    // earlier), the wave reads the nibbles of step i+1 from LDS and decodes them.  After the barrier of
+    // iteration i every wave has finished iteration i-1, so the slot of stage i-1 is refilled with step i+5.
+    auto load_a = [&](const uint8_t *st, h8 (&av)[TILES]) {
+        const uint8_t *at = st + GS_W + GS_S;
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            const int r = 16 * t + c;
+            av[t] = *reinterpret_cast<const h8 *>(at + r * 64 + ((g ^ ((r >> 2) & 3)) << 4));
+        }
+    };
+    auto multiply = [&](const h8 (&av)[TILES], const h8 (&b)[4]) {
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+#pragma unroll
+            for (int o = 0; o < 4; ++o) acc[o][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], b[o], acc[o][t], 0, 0, 0);
+        }
+    };
     if (n_steps > 0) {
         h8 bq[4];
         int cur = step0 + rot;                 // step being multiplied
+        int slot = 0;                          // its ring slot
         {
             gemm_wait_dma(min(GEMM_STAGES - 2, n_steps - 1));
             gemm_barrier();
@@ -201,48 +222,43 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             load_ws(lds, wv, sv);
             decode(wv, sv, k_dead(cur), bq);
         }
-        int stage = 0;                         // ring slot of step i
         GXT(33, 0);
-        for (int i = 0; i < n_steps; ++i) {
+        // one iteration: multiply step i with bq while the B operands of step i+1 are decoded; REFILL is a
+        // compile-time flag so that the body of the main loop is one basic block with its DMA inside
+        auto iterate = [&](int i, auto refill) {
             if (i < 32) GXT(i, 0);
-            // stage i+1 has landed for this wave (younger ones may still be in flight) ...
-            gemm_wait_dma(min(GEMM_STAGES - 3, max(n_steps - 2 - i, 0)));
-            // ... and for everyone; everyone is also done with stage i-1, whose slot is refilled now
+            // stage i+1 has landed for this wave (the three younger ones may still be in flight) ...
+            if (refill.value) gemm_wait_dma(GEMM_STAGES - 3);
+            else gemm_wait_dma(min(GEMM_STAGES - 3, max(n_steps - 2 - i, 0)));
             if (i < 32) GXT(i, 1);
-            gemm_barrier();
+            gemm_barrier();                    // ... and for everyone; everyone is done with stage i-1
             if (i < 32) GXT(i, 2);
-            if (i + GEMM_STAGES - 1 < n_steps) fetch_next(stage == 0 ? GEMM_STAGES - 1 : stage - 1);
+            if (refill.value) fetch_next(slot == 0 ? GEMM_STAGES - 1 : slot - 1);
             if (i < 32) GXT(i, 3);
-
-            const uint8_t *st = lds + stage * GS_BYTES;
-            stage = stage == GEMM_STAGES - 1 ? 0 : stage + 1;
-            const int nxt = cur + 1 == step1 ? step0 : cur + 1;
-            cur = nxt;
-            // one basic block: the MFMAs of step i and the decode of step i+1 (past the last step the slot holds
-            // stale bytes, decoded and never used)
+            const uint8_t *st = lds + slot * GS_BYTES;
+            slot = slot == GEMM_STAGES - 1 ? 0 : slot + 1;
+            cur = cur + 1 == step1 ? step0 : cur + 1;
+            // past the last step the next slot holds stale bytes: read, decoded and never used
             uint32_t wv[8], sv[8];
-            load_ws(lds + stage * GS_BYTES, wv, sv);
-            const uint8_t *at = st + GS_W + GS_S;
-            h8 av[TILES];
-#pragma unroll
-            for (int t = 0; t < TILES; ++t) {
-                const int r = 16 * t + c;
-                av[t] = *reinterpret_cast<const h8 *>(at + r * 64 + ((g ^ ((r >> 2) & 3)) << 4));
-            }
-            h8 bn[4];
-            decode(wv, sv, k_dead(nxt), bn);
-#pragma unroll
-            for (int t = 0; t < TILES; ++t) {
-#pragma unroll
-                for (int o = 0; o < 4; ++o) acc[o][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], bq[o], acc[o][t], 0, 0, 0);
-            }
+            h8 av[TILES], bn[4];
+            load_a(st, av);
+            load_ws(lds + slot * GS_BYTES, wv, sv);
+            multiply(av, bq);
+            decode(wv, sv, k_dead(cur), bn);
 #pragma unroll
             for (int o = 0; o < 4; ++o) bq[o] = bn[o];
 #ifdef GX_TRACE
             asm volatile("" :: "v"(acc[0][0]), "v"(acc[3][TILES - 1]), "v"(bq[0]), "v"(bq[3]));
             if (i < 32) { GXT(i, 4); GXT(i, 5); }
 #endif
-        }
+        };
+        typedef std::integral_constant<bool, true> yes;
+        typedef std::integral_constant<bool, false> no;
+        int i = 0;
+#pragma unroll 1
+        for (; i + GEMM_STAGES - 1 < n_steps; ++i) iterate(i, yes{});
+#pragma unroll 1
+        for (; i < n_steps; ++i) iterate(i, no{});
         GXT(32, 0);
     }
 
