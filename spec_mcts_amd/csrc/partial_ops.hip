@@ -1,7 +1,7 @@
 // Consumers of the Q4_0 matmul's K-slice slabs.
 //
-// The matmul kernels leave `ksplit` fp32 slabs partial[s][m][n]; every kernel here first forms
-// acc = sum_s partial[s][m][n] (slice order, so the result does not depend on scheduling), rounds
+// The matmul kernels leave `ksplit` slabs partial[s][m][n] (fp32 up to 16 rows, fp16 above: slab_is_half);
+// every kernel here first forms acc = sum_s partial[s][m][n] in fp32 (slice order, so the result does not depend on scheduling), rounds
 // it ONCE to fp16 - the value the reference's matmul_q40 returns - and then applies the operator
 // that follows the linear in the model:
 //   partial_reduce_kernel      c = fp16(acc) (+ fp16 residual add)
@@ -15,34 +15,56 @@
 
 namespace smh {
 
-__device__ __forceinline__ float slab_sum(const float *p, long slab_stride, int ksplit) {
+// Element `idx` of every slab, added in slice order in fp32.  `half`: the slabs hold fp16 (slab_is_half).
+__device__ __forceinline__ float slab_sum(const void *partial, long idx, long slab_stride, int ksplit, bool half) {
     float v[SMH_MAX_KSPLIT];
+    if (half) {
+        const half_t *p = reinterpret_cast<const half_t *>(partial) + idx;
 #pragma unroll
-    for (int s = 0; s < SMH_MAX_KSPLIT; ++s) v[s] = (s < ksplit) ? p[s * slab_stride] : 0.f;
+        for (int s = 0; s < SMH_MAX_KSPLIT; ++s) v[s] = (s < ksplit) ? (float)p[s * slab_stride] : 0.f;
+    } else {
+        const float *p = reinterpret_cast<const float *>(partial) + idx;
+#pragma unroll
+        for (int s = 0; s < SMH_MAX_KSPLIT; ++s) v[s] = (s < ksplit) ? p[s * slab_stride] : 0.f;
+    }
     float tot = 0.f;
 #pragma unroll
     for (int s = 0; s < SMH_MAX_KSPLIT; ++s) tot += v[s];
     return tot;
 }
-__device__ __forceinline__ f4 slab_sum4(const float *p, long slab_stride, int ksplit) {
-    f4 v[SMH_MAX_KSPLIT];
-#pragma unroll
-    for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
-        v[s] = (s < ksplit) ? *reinterpret_cast<const f4 *>(p + s * slab_stride) : f4{0.f, 0.f, 0.f, 0.f};
+// Four consecutive elements (idx % 4 == 0).
+__device__ __forceinline__ f4 slab_sum4(const void *partial, long idx, long slab_stride, int ksplit, bool half) {
     f4 tot = {0.f, 0.f, 0.f, 0.f};
+    if (half) {
+        const half_t *p = reinterpret_cast<const half_t *>(partial) + idx;
+        h4 v[SMH_MAX_KSPLIT];
 #pragma unroll
-    for (int s = 0; s < SMH_MAX_KSPLIT; ++s) tot += v[s];
+        for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
+            v[s] = (s < ksplit) ? *reinterpret_cast<const h4 *>(p + s * slab_stride) : h4{(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
+#pragma unroll
+        for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
+#pragma unroll
+            for (int j = 0; j < 4; ++j) tot[j] += (float)v[s][j];
+    } else {
+        const float *p = reinterpret_cast<const float *>(partial) + idx;
+        f4 v[SMH_MAX_KSPLIT];
+#pragma unroll
+        for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
+            v[s] = (s < ksplit) ? *reinterpret_cast<const f4 *>(p + s * slab_stride) : f4{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < SMH_MAX_KSPLIT; ++s) tot += v[s];
+    }
     return tot;
 }
 
 // ---- plain reduce (+ residual) ------------------------------------------------------------------
-__global__ __launch_bounds__(256) void partial_reduce_kernel(const float *__restrict__ partial, int ksplit, int M, int n_total,
+__global__ __launch_bounds__(256) void partial_reduce_kernel(const void *__restrict__ partial, int ksplit, int M, int n_total,
                                                              int col0, int N, half_t *__restrict__ c, long ldc, int epilogue,
                                                              const half_t *__restrict__ resid, long ldr) {
     const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= (long)M * N) return;
     const int m = (int)(i / N), n = (int)(i % N);          // N % 4 == 0: the 4 columns share a row
-    const f4 acc = slab_sum4(partial + (long)m * n_total + col0 + n, (long)M * n_total, ksplit);
+    const f4 acc = slab_sum4(partial, (long)m * n_total + col0 + n, (long)M * n_total, ksplit, slab_is_half(M));
     h4 out;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -55,7 +77,7 @@ __global__ __launch_bounds__(256) void partial_reduce_kernel(const float *__rest
 
 // ---- residual add + RMSNorm ---------------------------------------------------------------------
 // one workgroup of 1024 threads per row; h_out = h_in + fp16(acc) (fp16 add), xn = fp16(fp16(h*r)*w)
-__global__ __launch_bounds__(1024) void partial_rmsnorm_kernel(const float *__restrict__ partial, int ksplit, int M, int N,
+__global__ __launch_bounds__(1024) void partial_rmsnorm_kernel(const void *__restrict__ partial, int ksplit, int M, int N,
                                                                const half_t *__restrict__ h_in, const half_t *__restrict__ wt,
                                                                float eps, half_t *__restrict__ h_out, half_t *__restrict__ xn_out) {
     __shared__ float s_part[16];
@@ -71,7 +93,7 @@ __global__ __launch_bounds__(1024) void partial_rmsnorm_kernel(const float *__re
         if (n < N) {
             h4 v;
             if (partial != nullptr) {
-                const f4 acc = slab_sum4(partial + (long)m * N + n, slab, ksplit);
+                const f4 acc = slab_sum4(partial, (long)m * N + n, slab, ksplit, slab_is_half(M));
 #pragma unroll
                 for (int j = 0; j < 4; ++j) v[j] = (half_t)acc[j];
                 if (h_in != nullptr) {
@@ -113,14 +135,14 @@ __global__ __launch_bounds__(1024) void partial_rmsnorm_kernel(const float *__re
 
 // ---- SwiGLU gate ------------------------------------------------------------------------------------
 // slabs hold [gate | up] (2 * n_half columns)
-__global__ __launch_bounds__(256) void partial_silu_mul_kernel(const float *__restrict__ partial, int ksplit, int M, int n_half,
+__global__ __launch_bounds__(256) void partial_silu_mul_kernel(const void *__restrict__ partial, int ksplit, int M, int n_half,
                                                                half_t *__restrict__ out) {
     const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= (long)M * n_half) return;
     const int m = (int)(i / n_half), n = (int)(i % n_half);
     const long slab = (long)M * 2 * n_half;
-    const f4 ga = slab_sum4(partial + (long)m * 2 * n_half + n, slab, ksplit);
-    const f4 ua = slab_sum4(partial + (long)m * 2 * n_half + n_half + n, slab, ksplit);
+    const f4 ga = slab_sum4(partial, (long)m * 2 * n_half + n, slab, ksplit, slab_is_half(M));
+    const f4 ua = slab_sum4(partial, (long)m * 2 * n_half + n_half + n, slab, ksplit, slab_is_half(M));
     h4 o;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -133,7 +155,7 @@ __global__ __launch_bounds__(256) void partial_silu_mul_kernel(const float *__re
 
 // one wave per (branch, head); heads 0..H-1 queries, H..H+Hkv-1 keys, H+Hkv.. values.
 // slab columns: [q (H*128) | k (Hkv*128) | v (Hkv*128)]
-__global__ __launch_bounds__(256) void partial_rope_append_kernel(const float *__restrict__ partial, int ksplit, int B, int H, int Hkv,
+__global__ __launch_bounds__(256) void partial_rope_append_kernel(const void *__restrict__ partial, int ksplit, int B, int H, int Hkv,
                                                                   half_t *__restrict__ q, half_t *__restrict__ k, half_t *__restrict__ v,
                                                                   const half_t *__restrict__ cos_tab, const half_t *__restrict__ sin_tab,
                                                                   const int32_t *__restrict__ pos_dev,
@@ -147,10 +169,10 @@ __global__ __launch_bounds__(256) void partial_rope_append_kernel(const float *_
     const int b = (int)(item / heads);
     const int h = (int)(item % heads);
     const int n_total = heads * 128;
-    const float *src = partial + (long)b * n_total + (long)h * 128;
+    const long src = (long)b * n_total + (long)h * 128;
     const long slab = (long)B * n_total;
-    half_t x1 = (half_t)slab_sum(src + lane, slab, ksplit);
-    half_t x2 = (half_t)slab_sum(src + lane + 64, slab, ksplit);
+    half_t x1 = (half_t)slab_sum(partial, src + lane, slab, ksplit, slab_is_half(B));
+    half_t x2 = (half_t)slab_sum(partial, src + lane + 64, slab, ksplit, slab_is_half(B));
     const int t = (t_dev != nullptr) ? *t_dev : -1;
     if (h >= H + Hkv) {                                      // value head: store, append
         const int hk = h - H - Hkv;
@@ -202,6 +224,7 @@ static int fill_params(MatmulParams &p, const void *a, int M, int K, long lda, i
         p.seg[i].N = n[i];
     }
     if (M <= SMH_GEMV_MAX_M) gemv_fill_plan(p); else gemm_fill_plan(p);
+    p.slab_half = slab_is_half(M);
     return 0;
 }
 
@@ -312,7 +335,7 @@ extern "C" int smh_q40_matmul_fused(const void *a, int M, int K, long lda, int n
     }
 }
 
-static int reduce_launch(const float *partial, int ksplit, int M, int n_total, int col0, int N, void *c, long ldc,
+static int reduce_launch(const void *partial, int ksplit, int M, int n_total, int col0, int N, void *c, long ldc,
                          int epilogue, const void *residual, long ldr, hipStream_t stream) {
     long quads = ((long)M * N + 3) / 4;
     hipLaunchKernelGGL(partial_reduce_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, stream,
@@ -329,7 +352,7 @@ extern "C" int smh_partial_reduce(const void *partial, int ksplit, int M, int n_
     if (M == 0) return 0;
     SMH_REQUIRE(partial && c && ldc >= N && ldc % 4 == 0, "smh_partial_reduce: bad output");
     SMH_REQUIRE(epilogue != SMH_EPI_RESIDUAL || (residual && ldr >= N), "smh_partial_reduce: residual missing");
-    return reduce_launch((const float *)partial, ksplit, M, n_total, col0, N, c, ldc, epilogue, residual, ldr, (hipStream_t)stream);
+    return reduce_launch(partial, ksplit, M, n_total, col0, N, c, ldc, epilogue, residual, ldr, (hipStream_t)stream);
 }
 
 static int matmul_fp16(const void *a, int M, int K, long lda, const void *b_w, const void *b_s, int N, void *c, long ldc,
@@ -384,7 +407,7 @@ extern "C" int smh_partial_rmsnorm(const void *partial, int ksplit, int M, int N
     SMH_REQUIRE(partial != nullptr || h_in != nullptr, "smh_partial_rmsnorm: no input");
     if (M == 0) return 0;
     SMH_REQUIRE(weight && xn_out, "smh_partial_rmsnorm: null pointer");
-    hipLaunchKernelGGL(partial_rmsnorm_kernel, dim3(M), dim3(1024), 0, (hipStream_t)stream, (const float *)partial, ksplit, M, N,
+    hipLaunchKernelGGL(partial_rmsnorm_kernel, dim3(M), dim3(1024), 0, (hipStream_t)stream, partial, ksplit, M, N,
                        (const half_t *)h_in, (const half_t *)weight, eps, (half_t *)h_out, (half_t *)xn_out);
     return launch_status();
 }
@@ -396,7 +419,7 @@ extern "C" int smh_partial_silu_mul(const void *partial, int ksplit, int M, int 
     SMH_REQUIRE(partial && out, "smh_partial_silu_mul: null pointer");
     long quads = (long)M * n_half / 4;
     hipLaunchKernelGGL(partial_silu_mul_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
-                       (const float *)partial, ksplit, M, n_half, (half_t *)out);
+                       partial, ksplit, M, n_half, (half_t *)out);
     return launch_status();
 }
 
@@ -412,7 +435,7 @@ extern "C" int smh_partial_rope_append_kv(const void *partial, int ksplit, int B
     SMH_REQUIRE(!cache_k || (cache_ks && cache_v && cache_vs && t_dev && Smax > 0), "smh_partial_rope_append_kv: cache arguments incomplete");
     long items = (long)B * (H + 2 * Hkv);
     hipLaunchKernelGGL(partial_rope_append_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
-                       (const float *)partial, ksplit, B, H, Hkv, (half_t *)q, (half_t *)k, (half_t *)v,
+                       partial, ksplit, B, H, Hkv, (half_t *)q, (half_t *)k, (half_t *)v,
                        (const half_t *)cos_tab, (const half_t *)sin_tab, pos_dev, (uint8_t *)cache_k, (half_t *)cache_ks,
                        (uint8_t *)cache_v, (half_t *)cache_vs, Smax, t_dev);
     return launch_status();

@@ -19,7 +19,7 @@
 //     row tiles and the ragged-K handling are template parameters), and the DMA addresses are a
 //     scalar base per step plus lane offsets that never change, so issuing a stage costs no VALU work;
 //   * the accumulators leave through LDS one row tile at a time, so global stores are 64-byte
-//     contiguous per lane; K-slices are written as fp32 slabs and added by the consuming kernel.
+//     contiguous per lane; K-slices are written as slabs (fp16 above 16 rows) and added by the consuming kernel.
 //
 // At M = 100 the work sits on the ridge of the roofline: 2*M*N*K flops against
 // N*K*0.53125 + 2*M*(K+N) bytes.
@@ -301,6 +301,20 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
                             o[4 + e] = matmul_epilogue(p, v1[e], m, n + 4 + e);
                         }
                         *reinterpret_cast<h8 *>(p.c + (long)m * p.ldc + n) = o;
+                    }
+                }
+            } else if (p.slab_half) {
+                half_t *dst = reinterpret_cast<half_t *>(p.partial) + ((long)slice * p.M + m) * p.n_total + seg.col0 + col0;
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const int cq = 128 * q + 8 * o_lane;
+                    if (col0 + cq < seg.N) {
+                        const f4 v0 = *reinterpret_cast<const f4 *>(otile + o_row * OP + cq);
+                        const f4 v1 = *reinterpret_cast<const f4 *>(otile + o_row * OP + cq + 4);
+                        h8 o;
+#pragma unroll
+                        for (int e = 0; e < 4; ++e) { o[e] = (half_t)v0[e]; o[4 + e] = (half_t)v1[e]; }
+                        *reinterpret_cast<h8 *>(dst + cq) = o;
                     }
                 }
             } else {
