@@ -32,6 +32,28 @@ __device__ __forceinline__ float slab_sum(const void *partial, long idx, long sl
     for (int s = 0; s < SMH_MAX_KSPLIT; ++s) tot += v[s];
     return tot;
 }
+// Two consecutive elements (idx % 2 == 0).
+__device__ __forceinline__ f2 slab_sum2(const void *partial, long idx, long slab_stride, int ksplit, bool half) {
+    f2 tot = {0.f, 0.f};
+    if (half) {
+        const half_t *p = reinterpret_cast<const half_t *>(partial) + idx;
+        h2 v[SMH_MAX_KSPLIT];
+#pragma unroll
+        for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
+            v[s] = (s < ksplit) ? *reinterpret_cast<const h2 *>(p + s * slab_stride) : h2{(half_t)0.f, (half_t)0.f};
+#pragma unroll
+        for (int s = 0; s < SMH_MAX_KSPLIT; ++s) { tot[0] += (float)v[s][0]; tot[1] += (float)v[s][1]; }
+    } else {
+        const float *p = reinterpret_cast<const float *>(partial) + idx;
+        f2 v[SMH_MAX_KSPLIT];
+#pragma unroll
+        for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
+            v[s] = (s < ksplit) ? *reinterpret_cast<const f2 *>(p + s * slab_stride) : f2{0.f, 0.f};
+#pragma unroll
+        for (int s = 0; s < SMH_MAX_KSPLIT; ++s) tot += v[s];
+    }
+    return tot;
+}
 // Four consecutive elements (idx % 4 == 0).
 __device__ __forceinline__ f4 slab_sum4(const void *partial, long idx, long slab_stride, int ksplit, bool half) {
     f4 tot = {0.f, 0.f, 0.f, 0.f};
@@ -162,17 +184,25 @@ __global__ __launch_bounds__(256) void partial_rope_append_kernel(const void *__
                                                                   uint8_t *__restrict__ cache_k, half_t *__restrict__ cache_ks,
                                                                   uint8_t *__restrict__ cache_v, half_t *__restrict__ cache_vs,
                                                                   int Smax, const int32_t *__restrict__ t_dev) {
+    __shared__ float s_row[4][128];
     const int lane = threadIdx.x & 63;
-    const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int wave = threadIdx.x >> 6;
+    const long item = (long)blockIdx.x * 4 + wave;
     const int heads = H + 2 * Hkv;
-    if (item >= (long)B * heads) return;
-    const int b = (int)(item / heads);
-    const int h = (int)(item % heads);
+    const bool live = item < (long)B * heads;
+    const int b = live ? (int)(item / heads) : 0;
+    const int h = live ? (int)(item % heads) : 0;
     const int n_total = heads * 128;
-    const long src = (long)b * n_total + (long)h * 128;
-    const long slab = (long)B * n_total;
-    half_t x1 = (half_t)slab_sum(partial, src + lane, slab, ksplit, slab_is_half(B));
-    half_t x2 = (half_t)slab_sum(partial, src + lane + 64, slab, ksplit, slab_is_half(B));
+    // the slabs are read two adjacent columns per lane; the rotation pairs column i with i + 64, so the sums
+    // change lanes through LDS
+    if (live) {
+        const f2 sum = slab_sum2(partial, (long)b * n_total + (long)h * 128 + 2 * lane, (long)B * n_total, ksplit, slab_is_half(B));
+        *reinterpret_cast<f2 *>(&s_row[wave][2 * lane]) = sum;
+    }
+    __syncthreads();
+    if (!live) return;
+    half_t x1 = (half_t)s_row[wave][lane];
+    half_t x2 = (half_t)s_row[wave][lane + 64];
     const int t = (t_dev != nullptr) ? *t_dev : -1;
     if (h >= H + Hkv) {                                      // value head: store, append
         const int hk = h - H - Hkv;
