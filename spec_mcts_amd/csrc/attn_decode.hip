@@ -184,34 +184,76 @@ __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
 #pragma unroll
         for (int j = 0; j < 8; ++j) st.o[j] = 0.f;
 
-        // ---- this branch's suffix: group g takes rows g, g+4, ... ----
-        for (int t = g; t < len; t += 4) {
-            const long row = (row0 + t) * p.Hkv + hk;
-            RowRegs kr, vr;
-            if (p.suffix_format == SMH_KV_FP16) {
-                kr = row_from_fp16((const half_t *)p.suffix_k + row * ATT_D, c);
-                vr = row_from_fp16((const half_t *)p.suffix_v + row * ATT_D, c);
-            } else {
-                const uint32_t kb = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_k + row * 64 + 4 * c);
-                const uint32_t vb = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_v + row * 64 + 4 * c);
-                const uint32_t ksc = *reinterpret_cast<const uint32_t *>(p.suffix_ks + row * 2);
-                const uint32_t vsc = *reinterpret_cast<const uint32_t *>(p.suffix_vs + row * 2);
-                kr = row_from_q40(kb, ksc);
-                vr = row_from_q40(vb, vsc);
+        // Every load below is issued before its first use, a batch at a time: a wave has few rows to visit
+        // (tens, a quarter each per group), so its time is the number of memory round trips it makes in a row.
+        // ---- loads for the end of the pass: the new token's exact K/V, the first two prefix partials ----
+        const int qrow = b * p.n_rep + rep;
+        const bool has_cur = p.cur_k != nullptr && g == 0;
+        RowRegs cur_kr = qr, cur_vr = qr;
+        if (has_cur) {
+            const long off = ((long)b * p.Hkv + hk) * ATT_D;
+            cur_kr = row_from_fp16(p.cur_k + off, c);
+            cur_vr = row_from_fp16(p.cur_v + off, c);
+        }
+        constexpr int PRE = 2;
+        f4 pre_lo[PRE], pre_hi[PRE];
+        float pre_m[PRE], pre_l[PRE];
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            const int sp = g + 4 * i;
+            if (sp < p.splits) {
+                const long base = ((long)sp * p.Hkv + hk) * p.Bq + qrow;
+                pre_lo[i] = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 4 * c);
+                pre_hi[i] = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 64 + 4 * c);
+                pre_m[i] = p.part_ml[base * 2];
+                pre_l[i] = p.part_ml[base * 2 + 1];
             }
-            soft_add_row(st, row_dot(kr, qr) * p.scale_log2, vr);
+        }
+        // ---- this branch's suffix: group g takes rows g, g+4, ... in batches ----
+        if (p.suffix_format == SMH_KV_FP16) {
+            constexpr int U = 4;
+            for (int t0 = g; t0 < len; t0 += 4 * U) {
+                RowRegs kr[U], vr[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const long row = (row0 + min(t0 + 4 * u, len - 1)) * p.Hkv + hk;
+                    kr[u] = row_from_fp16((const half_t *)p.suffix_k + row * ATT_D, c);
+                    vr[u] = row_from_fp16((const half_t *)p.suffix_v + row * ATT_D, c);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (t0 + 4 * u < len) soft_add_row(st, row_dot(kr[u], qr) * p.scale_log2, vr[u]);
+            }
+        } else {
+            constexpr int U = 8;
+            for (int t0 = g; t0 < len; t0 += 4 * U) {
+                uint32_t kb[U], vb[U], ksc[U], vsc[U];
+#pragma unroll
+                for (int u = 0; u < U; ++u) {
+                    const long row = (row0 + min(t0 + 4 * u, len - 1)) * p.Hkv + hk;
+                    kb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_k + row * 64 + 4 * c);
+                    vb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_v + row * 64 + 4 * c);
+                    ksc[u] = *reinterpret_cast<const uint32_t *>(p.suffix_ks + row * 2);
+                    vsc[u] = *reinterpret_cast<const uint32_t *>(p.suffix_vs + row * 2);
+                }
+#pragma unroll
+                for (int u = 0; u < U; ++u)
+                    if (t0 + 4 * u < len)
+                        soft_add_row(st, row_dot(row_from_q40(kb[u], ksc[u]), qr) * p.scale_log2, row_from_q40(vb[u], vsc[u]));
+            }
         }
         // ---- the new token's exact K/V (group 0 only) ----
-        if (p.cur_k != nullptr && g == 0) {
-            const long off = ((long)b * p.Hkv + hk) * ATT_D;
-            const RowRegs kr = row_from_fp16(p.cur_k + off, c);
-            const RowRegs vr = row_from_fp16(p.cur_v + off, c);
-            soft_add_row(st, row_dot(kr, qr) * p.scale_log2, vr);
-        }
+        if (has_cur) soft_add_row(st, row_dot(cur_kr, qr) * p.scale_log2, cur_vr);
         // ---- prefix partials: group g folds in splits g, g+4, ... ----
-        const int qrow = b * p.n_rep + rep;
-        for (int s = g; s < p.splits; s += 4) {
-            const long base = ((long)s * p.Hkv + hk) * p.Bq + qrow;
+#pragma unroll
+        for (int i = 0; i < PRE; ++i) {
+            if (g + 4 * i < p.splits) {
+                const float o2[8] = {pre_lo[i][0], pre_lo[i][2], pre_lo[i][1], pre_lo[i][3], pre_hi[i][0], pre_hi[i][2], pre_hi[i][1], pre_hi[i][3]};
+                soft_merge(st, pre_m[i], pre_l[i], o2);
+            }
+        }
+        for (int sp = g + 4 * PRE; sp < p.splits; sp += 4) {
+            const long base = ((long)sp * p.Hkv + hk) * p.Bq + qrow;
             const f4 lo = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 4 * c);
             const f4 hi = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 64 + 4 * c);
             const float o2[8] = {lo[0], lo[2], lo[1], lo[3], hi[0], hi[2], hi[1], hi[3]};

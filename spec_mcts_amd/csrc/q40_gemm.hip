@@ -88,6 +88,10 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     const int slot = bid % p.units_pad;  bid /= p.units_pad;
     const int unit = (slot & 7) * (p.units_pad >> 3) + (slot >> 3);
     if (unit >= p.units) return;
+#ifdef GX_TRACE
+    asm volatile("" :: "s"(unit));
+    GXT(33, 4);
+#endif
     const int mb = bid % p.mblocks;
     const int slice = bid / p.mblocks;
     int sg = 0;
@@ -119,6 +123,10 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     const uint32_t w_voff = (uint32_t)(w_lrow * w_row + w_lcol);
     const uint32_t s_voff = (uint32_t)(s_lrow * s_row + s_lcol);
     const uint32_t a_voff0 = (uint32_t)(a_r0 + 16 * a_chunk), a_voff1 = (uint32_t)(a_r1 + 16 * a_chunk);
+#ifdef GX_TRACE
+    asm volatile("" :: "v"(w_voff), "v"(s_voff), "v"(a_voff0), "v"(a_voff1), "s"(w_base), "s"(s_base));
+    GXT(33, 5);
+#endif
 
     auto issue = [&](int step, int slot_) {
         uint8_t *st = lds + slot_ * GS_BYTES;
