@@ -355,11 +355,13 @@ void gemm_fill_plan(MatmulParams &p) {
     p.mblocks = (p.M + GEMM_BM - 1) / GEMM_BM;
     const int steps = (p.K + 31) / 32;
     const long tiles = (long)p.units * p.mblocks;
-    // one round of workgroups (2 per CU); fewer slices for bigger M, whose slabs are bigger (at M = 100 up to
-    // 16 slices: matrices with few column units need them to fill the GPU, and the slab traffic costs less
-    // than idle compute units)
+    // One round of workgroups.  One workgroup per compute unit when the column units divide the GPU well
+    // (at least 200 of the 256 units busy): a second co-resident workgroup buys little there and doubles the
+    // slabs the next kernel has to read.  Otherwise two per compute unit.  (At M = 100 matrices with few column
+    // units still take up to 16 slices: idle compute units cost more than the slab traffic.)
     static const int capacity = env_int("SMH_GEMM_WGS", 512);
-    int ks = (int)(capacity / tiles);
+    int ks = (int)(capacity / 2 / tiles);
+    if (ks < 1 || tiles * ks < 200) ks = (int)(capacity / tiles);
     static const int cap_num = env_int("SMH_GEMM_KSCAP", 1600);
     int cap = cap_num / (p.M > 0 ? p.M : 1);
     if (cap > SMH_MAX_KSPLIT) cap = SMH_MAX_KSPLIT;
