@@ -108,7 +108,13 @@ __global__ __launch_bounds__(1024) void partial_rmsnorm_kernel(const void *__res
     float ss = 0.f;
     // each thread owns columns 4t, 4t+1, 4t+2, 4t+3 (+ 4096 per pass); values kept for the second pass
     constexpr int MAXPASS = 4;      // N <= 16384
-    h4 hv[MAXPASS];
+    h4 hv[MAXPASS], wv[MAXPASS];
+    // the norm weights are not needed before the second pass: fetched now, they arrive with the slabs
+#pragma unroll
+    for (int ps = 0; ps < MAXPASS; ++ps) {
+        const int n = (ps * 1024 + threadIdx.x) * 4;
+        if (n < N) wv[ps] = *reinterpret_cast<const h4 *>(wt + n);
+    }
 #pragma unroll
     for (int ps = 0; ps < MAXPASS; ++ps) {
         const int n = (ps * 1024 + threadIdx.x) * 4;
@@ -143,7 +149,7 @@ __global__ __launch_bounds__(1024) void partial_rmsnorm_kernel(const void *__res
     for (int ps = 0; ps < MAXPASS; ++ps) {
         const int n = (ps * 1024 + threadIdx.x) * 4;
         if (n < N) {
-            const h4 w = *reinterpret_cast<const h4 *>(wt + n);
+            const h4 w = wv[ps];
             h4 o;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -195,6 +201,10 @@ __global__ __launch_bounds__(256) void partial_rope_append_kernel(const void *__
     const int n_total = heads * 128;
     // the slabs are read two adjacent columns per lane; the rotation pairs column i with i + 64, so the sums
     // change lanes through LDS
+    // the position and the rotation factors travel while the slabs are read
+    const int t = (t_dev != nullptr) ? *t_dev : -1;
+    const int pos = *pos_dev;
+    const half_t cos_l = cos_tab[(long)pos * 64 + lane], sin_l = sin_tab[(long)pos * 64 + lane];
     if (live) {
         const f2 sum = slab_sum2(partial, (long)b * n_total + (long)h * 128 + 2 * lane, (long)B * n_total, ksplit, slab_is_half(B));
         *reinterpret_cast<f2 *>(&s_row[wave][2 * lane]) = sum;
@@ -203,7 +213,6 @@ __global__ __launch_bounds__(256) void partial_rope_append_kernel(const void *__
     if (!live) return;
     half_t x1 = (half_t)s_row[wave][lane];
     half_t x2 = (half_t)s_row[wave][lane + 64];
-    const int t = (t_dev != nullptr) ? *t_dev : -1;
     if (h >= H + Hkv) {                                      // value head: store, append
         const int hk = h - H - Hkv;
         half_t *pv = v + ((long)b * Hkv + hk) * 128;
@@ -215,8 +224,7 @@ __global__ __launch_bounds__(256) void partial_rope_append_kernel(const void *__
         }
         return;
     }
-    const int pos = *pos_dev;
-    rope_pair2(x1, x2, cos_tab[(long)pos * 64 + lane], sin_tab[(long)pos * 64 + lane]);
+    rope_pair2(x1, x2, cos_l, sin_l);
     if (h < H) {
         half_t *pq = q + ((long)b * H + h) * 128;
         pq[lane] = x1;

@@ -45,17 +45,6 @@ constexpr int GEMM_COLS = 256;
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
-#ifdef GX_TRACE
-__device__ unsigned long long gx_trace[512][34][8];
-__device__ __forceinline__ unsigned long long gx_now() {
-    unsigned long long t;
-    asm volatile("s_memtime %0\n\ts_waitcnt lgkmcnt(0)" : "=s"(t) :: "memory");
-    return t;
-}
-#define GXT(i, slot) do { if (lane == 0 && wave == GX_TRACE && blockIdx.x < 512 && (i) < 34) gx_trace[blockIdx.x][i][slot] = gx_now(); } while (0)
-#else
-#define GXT(i, slot) do { } while (0)
-#endif
 
 // Waits until at most `stages` younger stages (4 DMA instructions each) of this wave are still in flight.
 __device__ __forceinline__ void gemm_wait_dma(int stages) {
@@ -82,16 +71,11 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     const int lane = tid & 63;
     const int c = lane & 15;
     const int g = lane >> 4;
-    GXT(33, 1);
     int bid = blockIdx.x;
     // slot -> unit: each XCD (blockIdx % 8) takes a contiguous run of column units, which share scale lines
     const int slot = bid % p.units_pad;  bid /= p.units_pad;
     const int unit = (slot & 7) * (p.units_pad >> 3) + (slot >> 3);
     if (unit >= p.units) return;
-#ifdef GX_TRACE
-    asm volatile("" :: "s"(unit));
-    GXT(33, 4);
-#endif
     const int mb = bid % p.mblocks;
     const int slice = bid / p.mblocks;
     int sg = 0;
@@ -123,10 +107,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     const uint32_t w_voff = (uint32_t)(w_lrow * w_row + w_lcol);
     const uint32_t s_voff = (uint32_t)(s_lrow * s_row + s_lcol);
     const uint32_t a_voff0 = (uint32_t)(a_r0 + 16 * a_chunk), a_voff1 = (uint32_t)(a_r1 + 16 * a_chunk);
-#ifdef GX_TRACE
-    asm volatile("" :: "v"(w_voff), "v"(s_voff), "v"(a_voff0), "v"(a_voff1), "s"(w_base), "s"(s_base));
-    GXT(33, 5);
-#endif
 
     auto issue = [&](int step, int slot_) {
         uint8_t *st = lds + slot_ * GS_BYTES;
@@ -199,8 +179,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
         b[3] = __builtin_bit_cast(h8, v1l);
     };
     auto k_dead = [&](int step) { return step * 32 + 8 * g >= p.K; };      // only in the last step when K % 32 != 0
-
-    GXT(33, 2);
     // While the matrix pipe multiplies step i (A tile read from stage i, B operands decoded one iteration
     // earlier), the wave reads the nibbles of step i+1 from LDS and decodes them.  After the barrier of
     // iteration i every wave has finished iteration i-1, so the slot of stage i-1 is refilled with step i+5.
@@ -230,19 +208,14 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             load_ws(lds, wv, sv);
             decode(wv, sv, k_dead(cur), bq);
         }
-        GXT(33, 0);
         // one iteration: multiply step i with bq while the B operands of step i+1 are decoded; REFILL is a
         // compile-time flag so that the body of the main loop is one basic block with its DMA inside
         auto iterate = [&](int i, auto refill) {
-            if (i < 32) GXT(i, 0);
             // stage i+1 has landed for this wave (the three younger ones may still be in flight) ...
             if (refill.value) gemm_wait_dma(GEMM_STAGES - 3);
             else gemm_wait_dma(min(GEMM_STAGES - 3, max(n_steps - 2 - i, 0)));
-            if (i < 32) GXT(i, 1);
             gemm_barrier();                    // ... and for everyone; everyone is done with stage i-1
-            if (i < 32) GXT(i, 2);
             if (refill.value) fetch_next(slot == 0 ? GEMM_STAGES - 1 : slot - 1);
-            if (i < 32) GXT(i, 3);
             const uint8_t *st = lds + slot * GS_BYTES;
             slot = slot == GEMM_STAGES - 1 ? 0 : slot + 1;
             cur = cur + 1 == step1 ? step0 : cur + 1;
@@ -255,10 +228,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             decode(wv, sv, k_dead(cur), bn);
 #pragma unroll
             for (int o = 0; o < 4; ++o) bq[o] = bn[o];
-#ifdef GX_TRACE
-            asm volatile("" :: "v"(acc[0][0]), "v"(acc[3][TILES - 1]), "v"(bq[0]), "v"(bq[3]));
-            if (i < 32) { GXT(i, 4); GXT(i, 5); }
-#endif
         };
         typedef std::integral_constant<bool, true> yes;
         typedef std::integral_constant<bool, false> no;
@@ -267,7 +236,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
         for (; i + GEMM_STAGES - 1 < n_steps; ++i) iterate(i, yes{});
 #pragma unroll 1
         for (; i < n_steps; ++i) iterate(i, no{});
-        GXT(32, 0);
     }
 
     // ---- results leave one 16-row tile at a time through LDS: [16][256 + 4] floats, two buffers in turn ----
@@ -335,10 +303,6 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             }
         }
     }
-#ifdef GX_TRACE
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    GXT(33, 3);
-#endif
 }
 
 void gemm_fill_plan(MatmulParams &p) {
@@ -400,8 +364,3 @@ int gemm_launch(const MatmulParams &p, hipStream_t stream) {
 
 }  // namespace smh
 
-#ifdef GX_TRACE
-extern "C" int smhdbg_gemm_trace(void *dst, size_t bytes) {
-    return (int)hipMemcpyFromSymbol(dst, HIP_SYMBOL(smh::gx_trace), bytes < sizeof(smh::gx_trace) ? bytes : sizeof(smh::gx_trace));
-}
-#endif
