@@ -59,7 +59,7 @@ int smh_q40_quantize(const void *in, void *w, void *s, long groups, smh_stream_t
  * Requires N % 128 == 0, K % 8 == 0, lda % 8 == 0, ldc % 4 == 0 and 16-byte aligned a.
  * smh_q40_matmul picks the GEMV kernel (M <= SMH_GEMV_MAX_M) or the LDS/MFMA GEMM.
  * workspace: smh_q40_matmul_workspace_bytes() bytes of scratch (no initialisation needed) that
- * holds the fp32 K-slice slabs between the producing kernel and the reduce kernel; calls that
+ * holds the K-slice slabs between the producing kernel and the reduce kernel; calls that
  * overlap on different streams need separate workspaces. */
 #define SMH_GEMV_MAX_M 16
 size_t smh_q40_matmul_workspace_bytes(int max_m, int max_n);
@@ -74,10 +74,14 @@ int smh_q40_matmul(const void *a, int M, int K, long lda, const void *b_w, const
                    void *workspace, size_t workspace_bytes, smh_stream_t stream);
 
 /* ---- fused decode-layer operators ------------------------------------------------------------
- * The matmul kernels cut K into `ksplit` slices and leave one fp32 slab per slice,
+ * The matmul kernels cut K into `ksplit` slices and leave one slab per slice,
  * partial[ksplit][M][n_total]; the operator that FOLLOWS the linear in the model adds the slabs
- * (in slice order), rounds once to fp16 - the value matmul_q40 returns - and carries on, so no
+ * (in fp32, in slice order), rounds once to fp16 - the value matmul_q40 returns - and carries on, so no
  * kernel waits for another workgroup and a decode layer needs 4 weight-streaming launches.
+ * The slabs are opaque to the caller: they hold fp32 when M <= SMH_GEMV_MAX_M and fp16 above (at those
+ * batch sizes slab traffic would otherwise exceed the weight traffic); producer and consumer derive the
+ * type from M (B for the rope operator), so the consumer must be given the M the producer was given.
+ * Sizes below are upper bounds in bytes for either type.
  * Up to 3 weights that share the input (wq|wk|wv of Attention.forward,
  * hf_model_q40_kv_shared.py:313; w1|w3 of FeedForward.forward, :434) run as segments of one
  * launch; their outputs are concatenated along the columns (n_total = sum of n[i]).
