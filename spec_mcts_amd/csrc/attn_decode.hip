@@ -17,6 +17,7 @@
 // Algorithmic HBM traffic: prefix 2*P*Hkv*D*2 B once + per branch its suffix rows
 // (512 B fp16 or 136 B Q4_0 per row and kv head) + q/out.
 #include "attn_rows.hpp"
+#include "rope_kv.hpp"
 
 namespace smh {
 
@@ -25,6 +26,7 @@ constexpr int ATT_TW_MAX = 128;            // prefix rows per workgroup
 constexpr int ATT_KPITCH = 136;            // halves per LDS row of K (272 B: 16 rows hit distinct banks)
 constexpr int ATT_VPITCH = ATT_TW_MAX + 8; // halves per LDS row of V^T
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr int ATT_FUSED_MAX_Q = 128;       // queries per kv head (branches x query heads per kv head) of the fused variant
 
 struct AttnParams {
     const half_t *q;
@@ -42,20 +44,75 @@ struct AttnParams {
     int suffix_format, lens_stride;
     int causal;                      // prefill mode: branch b attends to suffix rows 0..b
     float scale_log2;                // log2(e) / sqrt(D)
+    // FUSED kernels: q, the new token's k and v come straight from the fp32 K-slice slabs of the wq|wk|wv product
+    // ([qkv_ks][B][(H + 2 Hkv) * 128]); RoPE, the fp16 rounding points and the Q4_0 append of k, v are those of
+    // partial_rope_append_kernel (q / cur_k / cur_v above are not read)
+    const float *qkv;
+    int qkv_ks;
+    const half_t *cos_tab, *sin_tab;
+    const int32_t *pos_dev;
+    uint8_t *app_k, *app_v;          // the branches' suffix caches (row *app_t of every branch is written); may be null
+    half_t *app_ks, *app_vs;
+    const int32_t *app_t;
+    int app_smax;
 };
+
+// column `col` of branch b in the fused q|k|v product: the slabs added in slice order, rounded once to fp16
+__device__ __forceinline__ half_t qkv_value(const AttnParams &p, int b, int col) {
+    const int cols = (p.H + 2 * p.Hkv) * ATT_D;
+    const float *src = p.qkv + (long)b * cols + col;
+    const long slab = (long)p.B * cols;
+    float v[16];
+#pragma unroll
+    for (int s_ = 0; s_ < 16; ++s_) v[s_] = (s_ < p.qkv_ks) ? src[s_ * slab] : 0.f;
+    float tot = 0.f;
+#pragma unroll
+    for (int s_ = 0; s_ < 16; ++s_) tot += v[s_];
+    return (half_t)tot;
+}
+// four consecutive columns (col % 4 == 0)
+__device__ __forceinline__ h4 qkv_value4(const AttnParams &p, int b, int col) {
+    const int cols = (p.H + 2 * p.Hkv) * ATT_D;
+    const float *src = p.qkv + (long)b * cols + col;
+    const long slab = (long)p.B * cols;
+    f4 v[16];
+#pragma unroll
+    for (int s_ = 0; s_ < 16; ++s_) v[s_] = (s_ < p.qkv_ks) ? *reinterpret_cast<const f4 *>(src + s_ * slab) : f4{0.f, 0.f, 0.f, 0.f};
+    f4 tot = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+    for (int s_ = 0; s_ < 16; ++s_) tot += v[s_];
+    return h4{(half_t)tot[0], (half_t)tot[1], (half_t)tot[2], (half_t)tot[3]};
+}
 
 // position of prefix row t (0..tw-1) inside an LDS row of V^T: within each block of 32 rows the
 // order is chosen so that the 8 probabilities a lane holds after two S^T tiles (rows 4g+r of tile 2j
 // and of tile 2j+1) are 8 consecutive halves.
+// dims 4cc..4cc+3 (lo) and 64+4cc.. (hi) of the rotated query of head h, branch b: the rotation pairs d and d + 64
+// sit in the same lane
+__device__ __forceinline__ void qkv_query(const AttnParams &p, int b, int h, int pos, int cc, h4 &lo, h4 &hi) {
+    lo = qkv_value4(p, b, h * ATT_D + 4 * cc);
+    hi = qkv_value4(p, b, h * ATT_D + 64 + 4 * cc);
+    const h4 cs = *reinterpret_cast<const h4 *>(p.cos_tab + (long)pos * 64 + 4 * cc);
+    const h4 sn = *reinterpret_cast<const h4 *>(p.sin_tab + (long)pos * 64 + 4 * cc);
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        half_t x1 = lo[j], x2 = hi[j];
+        rope_pair2(x1, x2, cs[j], sn[j]);
+        lo[j] = x1; hi[j] = x2;
+    }
+}
+
 __device__ __forceinline__ int vt_pos(int t) {
     const int blk = t & ~31, w = t & 31;
     const int j2 = w >> 4, g = (w >> 2) & 3, r = w & 3;
     return blk + 8 * g + 4 * j2 + r;
 }
 
+template <bool FUSED>
 __global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
     __shared__ __attribute__((aligned(16))) half_t ks[ATT_TW_MAX][ATT_KPITCH];
     __shared__ __attribute__((aligned(16))) half_t vt[ATT_D][ATT_VPITCH];
+    __shared__ __attribute__((aligned(16))) half_t qs[FUSED ? ATT_FUSED_MAX_Q : 1][ATT_D + 8];      // FUSED: the rotated queries of this kv head
 
     const int split = blockIdx.x;
     const int hk = blockIdx.y;
@@ -64,6 +121,36 @@ __global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
     const int t0 = split * p.tw;
     const int cnt = min(p.tw, p.P - t0);
     const int tw32 = (cnt + 31) & ~31;          // rows actually touched by the matrix ops
+
+    // the B operand of S^T = K . Q^T for query tile qt: dims 32*k4 + 8g .. +7 of query row c
+    const int q_tiles = (p.Bq + 15) / 16;
+    auto load_q = [&](int qt, h8 (&qb)[4]) {
+        const int qr = min(qt * 16 + c, p.Bq - 1);
+        if (!FUSED) {
+            const int b = qr / p.n_rep, r_ = qr % p.n_rep;
+            const half_t *qp = p.q + ((long)b * p.H + hk * p.n_rep + r_) * ATT_D + 8 * g;
+#pragma unroll
+            for (int k4 = 0; k4 < 4; ++k4) qb[k4] = *reinterpret_cast<const h8 *>(qp + 32 * k4);
+        } else {
+#pragma unroll
+            for (int k4 = 0; k4 < 4; ++k4) qb[k4] = *reinterpret_cast<const h8 *>(&qs[qr][32 * k4 + 8 * g]);
+        }
+    };
+    if (FUSED) {
+        // all 256 threads build the rotated queries of this kv head from the slabs, 8 dims each, while
+        // the loads of K and V below are in flight; the barrier after the staging publishes them
+        const int cc = tid & 15;
+        const int pos = *p.pos_dev;
+        for (int qr = tid >> 4; qr < p.Bq; qr += 16) {
+            h4 lo, hi;
+            qkv_query(p, qr / p.n_rep, hk * p.n_rep + qr % p.n_rep, pos, cc, lo, hi);
+            *reinterpret_cast<h4 *>(&qs[qr][4 * cc]) = lo;
+            *reinterpret_cast<h4 *>(&qs[qr][64 + 4 * cc]) = hi;
+        }
+    }
+    // un-fused: the first tile's query is requested before the prefix slice is staged
+    h8 qb_first[4];
+    if (!FUSED && wave < q_tiles) load_q(wave, qb_first);
 
     // ---- stage K (row-major) and V (transposed) ----
     for (int idx = tid; idx < tw32 * 16; idx += 256) {
@@ -82,16 +169,15 @@ __global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
     }
     __syncthreads();
 
-    const int q_tiles = (p.Bq + 15) / 16;
     const int t_tiles = tw32 / 16;
     for (int qt = wave; qt < q_tiles; qt += 4) {
-        const int qr = min(qt * 16 + c, p.Bq - 1);
-        const int b = qr / p.n_rep, r_ = qr % p.n_rep;
-        const half_t *qp = p.q + ((long)b * p.H + hk * p.n_rep + r_) * ATT_D + 8 * g;
         h8 qb[4];
+        if (!FUSED && qt == wave) {
 #pragma unroll
-        for (int k4 = 0; k4 < 4; ++k4) qb[k4] = *reinterpret_cast<const h8 *>(qp + 32 * k4);
-
+            for (int k4 = 0; k4 < 4; ++k4) qb[k4] = qb_first[k4];
+        } else {
+            load_q(qt, qb);
+        }
         // S^T tiles: element r of st[j] is row t = 16j + 4g + r, column (query) c
         f4 st[ATT_TW_MAX / 16];
         float mx = -INFINITY;
@@ -164,20 +250,55 @@ __global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
     }
 }
 
+template <bool FUSED>
 __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
+    __shared__ __attribute__((aligned(16))) half_t s_kv[FUSED ? 4 : 1][2][ATT_D];     // FUSED: this wave's new k and v rows
     const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
-    const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    const int wave = threadIdx.x >> 6;
+    const long item = (long)blockIdx.x * 4 + wave;
     if (item >= (long)p.B * p.Hkv) return;
     const int b = (int)(item / p.Hkv);
     const int hk = (int)(item % p.Hkv);
+    // FUSED: query of head h in the row layout (dims 4c..4c+3 and 64+4c..)
+    auto fused_q = [&](int h, int pos_) {
+        h4 lo, hi;
+        qkv_query(p, b, h, pos_, c, lo, hi);
+        RowRegs qr;
+        qr.a02 = h2{lo[0], lo[2]}; qr.a13 = h2{lo[1], lo[3]};
+        qr.b02 = h2{hi[0], hi[2]}; qr.b13 = h2{hi[1], hi[3]};
+        return qr;
+    };
+    RowRegs q_first;
+    int pos = 0;
+    if (FUSED) {
+        // Everything that does not depend on another load is requested first: the position, the slabs of the new
+        // token's k and v (lane owns the pair (lane, lane + 64)) and of the first query.  k is rotated, both rows
+        // are appended to the branch's suffix cache as Q4_0 and left in LDS as exact fp16 for the pass below.
+        pos = *p.pos_dev;
+        const int t = p.app_k != nullptr ? *p.app_t : -1;
+        const int kcol = (p.H + hk) * ATT_D, vcol = (p.H + p.Hkv + hk) * ATT_D;
+        half_t k1 = qkv_value(p, b, kcol + lane), k2 = qkv_value(p, b, kcol + lane + 64);
+        const half_t v1 = qkv_value(p, b, vcol + lane), v2 = qkv_value(p, b, vcol + lane + 64);
+        q_first = fused_q(hk * p.n_rep, pos);
+        rope_pair2(k1, k2, p.cos_tab[(long)pos * 64 + lane], p.sin_tab[(long)pos * 64 + lane]);
+        if (t >= 0 && t < p.app_smax) {
+            const long row = ((long)b * p.app_smax + t) * p.Hkv + hk;
+            kv_store_row2(k1, k2, p.app_k + row * 64, p.app_ks + row * 2, lane);
+            kv_store_row2(v1, v2, p.app_v + row * 64, p.app_vs + row * 2, lane);
+        }
+        s_kv[wave][0][lane] = k1; s_kv[wave][0][lane + 64] = k2;
+        s_kv[wave][1][lane] = v1; s_kv[wave][1][lane + 64] = v2;
+        // same wave writes and reads: LDS operations of a wave complete in order
+    }
     int len = 0;
     if (p.suffix_format != SMH_KV_NONE) len = p.causal ? b + 1 : p.lens[(long)b * p.lens_stride];
     const long row0 = (long)b * p.suffix_batch_stride_rows;     // first suffix row of this branch
 
     for (int rep = 0; rep < p.n_rep; ++rep) {
         const int h = hk * p.n_rep + rep;
-        const half_t *qp = p.q + ((long)b * p.H + h) * ATT_D;
-        const RowRegs qr = row_from_fp16(qp, c);
+        RowRegs qr;
+        if (!FUSED) qr = row_from_fp16(p.q + ((long)b * p.H + h) * ATT_D, c);
+        else qr = rep == 0 ? q_first : fused_q(h, pos);
         SoftState st;
         st.m = -INFINITY;
         st.l = 0.f;
@@ -188,12 +309,17 @@ __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
         // (tens, a quarter each per group), so its time is the number of memory round trips it makes in a row.
         // ---- loads for the end of the pass: the new token's exact K/V, the first two prefix partials ----
         const int qrow = b * p.n_rep + rep;
-        const bool has_cur = p.cur_k != nullptr && g == 0;
+        const bool has_cur = (FUSED || p.cur_k != nullptr) && g == 0;
         RowRegs cur_kr = qr, cur_vr = qr;
         if (has_cur) {
-            const long off = ((long)b * p.Hkv + hk) * ATT_D;
-            cur_kr = row_from_fp16(p.cur_k + off, c);
-            cur_vr = row_from_fp16(p.cur_v + off, c);
+            if (FUSED) {
+                cur_kr = row_from_fp16(&s_kv[wave][0][0], c);
+                cur_vr = row_from_fp16(&s_kv[wave][1][0], c);
+            } else {
+                const long off = ((long)b * p.Hkv + hk) * ATT_D;
+                cur_kr = row_from_fp16(p.cur_k + off, c);
+                cur_vr = row_from_fp16(p.cur_v + off, c);
+            }
         }
         constexpr int PRE = 2;
         f4 pre_lo[PRE], pre_hi[PRE];
@@ -315,7 +441,7 @@ extern "C" int smh_shared_prefix_attn(const void *q, void *out, int B, int H, in
         SMH_REQUIRE(suffix_format != SMH_KV_Q40 || (suffix_ks && suffix_vs), "smh_shared_prefix_attn: null suffix scales");
     }
     SMH_REQUIRE((cur_k == nullptr) == (cur_v == nullptr), "smh_shared_prefix_attn: cur_k/cur_v must both be given or both be null");
-    AttnParams p;
+    AttnParams p{};
     p.q = (const half_t *)q; p.out = (half_t *)out;
     p.prefix_k = (const half_t *)prefix_k; p.prefix_v = (const half_t *)prefix_v;
     p.suffix_k = suffix_k; p.suffix_v = suffix_v;
@@ -334,9 +460,54 @@ extern "C" int smh_shared_prefix_attn(const void *q, void *out, int B, int H, in
     p.part_o = (float *)workspace;
     p.part_ml = p.part_o + n_part * ATT_D;
     if (p.splits > 0)
-        hipLaunchKernelGGL(attn_prefix_kernel, dim3(p.splits, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(attn_prefix_kernel<false>, dim3(p.splits, Hkv), dim3(256), 0, (hipStream_t)stream, p);
     long items = (long)B * Hkv;
-    hipLaunchKernelGGL(attn_suffix_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL(attn_suffix_kernel<false>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
+    return launch_status();
+}
+
+// The same attention fed by the un-reduced wq|wk|wv product: no q / k / v tensors and no separate RoPE launch.
+extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, void *out, int B, int H, int Hkv, int D,
+                                          const void *cos_tab, const void *sin_tab, const int32_t *pos_dev,
+                                          const void *prefix_k, const void *prefix_v, int P,
+                                          void *cache_k, void *cache_ks, void *cache_v, void *cache_vs, int Smax,
+                                          const int32_t *t_dev, void *workspace, size_t workspace_bytes, smh_stream_t stream) {
+    using namespace smh;
+    const char *who = "smh_shared_prefix_attn_qkv";
+    SMH_REQUIRE(D == ATT_D, "%s: head dim %d (only 128)", who, D);
+    SMH_REQUIRE(B >= 0 && B <= 16 && H > 0 && Hkv > 0 && H % Hkv == 0 && P >= 0, "%s: B=%d (at most 16) H=%d Hkv=%d P=%d", who, B, H, Hkv, P);
+    SMH_REQUIRE(ksplit >= 1 && ksplit <= 16, "%s: ksplit=%d", who, ksplit);
+    SMH_REQUIRE(B * (H / Hkv) <= ATT_FUSED_MAX_Q, "%s: %d queries per kv head (at most %d)", who, B * (H / Hkv), ATT_FUSED_MAX_Q);
+    if (B == 0) return 0;
+    SMH_REQUIRE(qkv_partial && out && cos_tab && sin_tab && pos_dev, "%s: null pointer", who);
+    SMH_REQUIRE(P == 0 || (prefix_k && prefix_v), "%s: null prefix", who);
+    SMH_REQUIRE(cache_k && cache_ks && cache_v && cache_vs && t_dev && Smax > 0, "%s: the suffix cache and its row counter are required", who);
+    AttnParams p{};
+    p.out = (half_t *)out;
+    p.prefix_k = (const half_t *)prefix_k; p.prefix_v = (const half_t *)prefix_v;
+    p.suffix_k = cache_k; p.suffix_v = cache_v;
+    p.suffix_ks = (const half_t *)cache_ks; p.suffix_vs = (const half_t *)cache_vs;
+    p.lens = t_dev; p.lens_stride = 0;
+    p.suffix_batch_stride_rows = Smax;
+    p.B = B; p.H = H; p.Hkv = Hkv; p.n_rep = H / Hkv; p.Bq = B * p.n_rep;
+    p.P = P; p.suffix_format = SMH_KV_Q40; p.causal = 0;
+    p.scale_log2 = LOG2E / sqrtf((float)D);
+    p.tw = attn_plan_tw(P, Hkv);
+    p.splits = P > 0 ? (P + p.tw - 1) / p.tw : 0;
+    p.qkv = (const float *)qkv_partial; p.qkv_ks = ksplit;
+    p.cos_tab = (const half_t *)cos_tab; p.sin_tab = (const half_t *)sin_tab; p.pos_dev = pos_dev;
+    p.app_k = (uint8_t *)cache_k; p.app_v = (uint8_t *)cache_v;
+    p.app_ks = (half_t *)cache_ks; p.app_vs = (half_t *)cache_vs;
+    p.app_t = t_dev; p.app_smax = Smax;
+    size_t n_part = (size_t)p.splits * Hkv * p.Bq;
+    SMH_REQUIRE(p.splits == 0 || (workspace && workspace_bytes >= n_part * (ATT_D + 2) * sizeof(float)),
+                "%s: workspace %zu < %zu bytes", who, workspace_bytes, n_part * (ATT_D + 2) * sizeof(float));
+    p.part_o = (float *)workspace;
+    p.part_ml = p.part_o + n_part * ATT_D;
+    if (p.splits > 0)
+        hipLaunchKernelGGL(attn_prefix_kernel<true>, dim3(p.splits, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+    long items = (long)B * Hkv;
+    hipLaunchKernelGGL(attn_suffix_kernel<true>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
 }
 
@@ -358,6 +529,6 @@ extern "C" int smh_prefill_attn(const void *q, const void *k, const void *v, voi
     p.suffix_format = SMH_KV_FP16; p.causal = 1;
     p.scale_log2 = LOG2E / sqrtf((float)D);
     long items = (long)S * Hkv;
-    hipLaunchKernelGGL(attn_suffix_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL(attn_suffix_kernel<false>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
 }

@@ -263,6 +263,7 @@ class Transformer(nn.Module):
                                       # layer instead of 10; measured slower at B=10: the finisher's round trips are serial)
         self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
         self.persistent = True        # decode steps of few branches as one persistent kernel (needs fused)
+        self.attn_from_qkv = False         # up to 16 branches the attention kernels can read the wq|wk|wv product themselves (one launch fewer; measured neutral)
         self.persistent_max_branches = 1   # from 2 branches on the operator-by-operator launches are faster (the kernel itself takes up to 16)
         self._step_kernels = {}       # branches -> K.DecodeStepKernel
 
@@ -350,12 +351,18 @@ class Transformer(nn.Module):
             else:
                 assert seqlen == 1, "decode steps take one token per branch"
                 pos_dev, t_dev = step_state
-                q, k, v = K.partial_rope_append_kv(qkv, H, Hkv, D, cos, sin, pos_dev, att.cache_k, att.cache_k_s,
-                                                   att.cache_v, att.cache_v_s, p.max_seq_len, t_dev)
-                o = K.shared_prefix_attn(q, att.cache_prompt_k[0], att.cache_prompt_v[0], att.cache_prompt_len,
-                                         suffix_k=att.cache_k, suffix_v=att.cache_v, suffix_ks=att.cache_k_s,
-                                         suffix_vs=att.cache_v_s, Smax=p.max_seq_len, lens=t_dev, lens_stride=0,
-                                         cur_k=k, cur_v=v).view(M, H * D)
+                if self.attn_from_qkv and M <= K.SMH_GEMV_MAX_M and M * (H // Hkv) <= 128 and not self.per_branch_kv:
+                    # RoPE and the KV append happen inside the attention kernels (one launch fewer)
+                    o = K.shared_prefix_attn_qkv(qkv, H, Hkv, D, cos, sin, pos_dev, att.cache_prompt_k[0], att.cache_prompt_v[0],
+                                                 att.cache_prompt_len, att.cache_k, att.cache_k_s, att.cache_v, att.cache_v_s,
+                                                 p.max_seq_len, t_dev).view(M, H * D)
+                else:
+                    q, k, v = K.partial_rope_append_kv(qkv, H, Hkv, D, cos, sin, pos_dev, att.cache_k, att.cache_k_s,
+                                                       att.cache_v, att.cache_v_s, p.max_seq_len, t_dev)
+                    o = K.shared_prefix_attn(q, att.cache_prompt_k[0], att.cache_prompt_v[0], att.cache_prompt_len,
+                                             suffix_k=att.cache_k, suffix_v=att.cache_v, suffix_ks=att.cache_k_s,
+                                             suffix_vs=att.cache_v_s, Smax=p.max_seq_len, lens=t_dev, lens_stride=0,
+                                             cur_k=k, cur_v=v).view(M, H * D)
             po = K.matmul_q40_partial(o, [(att.wo.w, att.wo.s, att.wo.shape[0])])
             h, xn = K.partial_rmsnorm(po, h, layer.ffn_norm.weight, layer.ffn_norm.eps)
             gu = K.matmul_q40_partial(xn, [(ff.w1.w, ff.w1.s, ff.w1.shape[0]), (ff.w3.w, ff.w3.s, ff.w3.shape[0])])

@@ -15,7 +15,7 @@ from typing import Dict, Optional, Sequence, Tuple
 import torch
 
 from . import _lib
-from ._lib import SMH_EPI_NONE, SMH_EPI_RESIDUAL, SMH_KV_FP16, SMH_KV_NONE, SMH_KV_Q40, check
+from ._lib import SMH_EPI_NONE, SMH_EPI_RESIDUAL, SMH_GEMV_MAX_M, SMH_KV_FP16, SMH_KV_NONE, SMH_KV_Q40, check
 from .quant import GROUP_SIZE, quantize_q40_torch
 
 DTYPE_torch = torch.float16
@@ -366,6 +366,30 @@ def shared_prefix_attn(q: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix
                                      fmt, _ptr(suffix_k), _ptr(suffix_v), _ptr(suffix_ks), _ptr(suffix_vs), int(Smax),
                                      _ptr(lens), int(lens_stride), _ptr(cur_k), _ptr(cur_v),
                                      ws.data_ptr(), ws.numel(), _stream()), "smh_shared_prefix_attn")
+    return out
+
+
+def shared_prefix_attn_qkv(p: PartialProduct, H: int, Hkv: int, D: int, cos: torch.Tensor, sin: torch.Tensor,
+                           pos_dev: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix_v: Optional[torch.Tensor], P: int,
+                           cache_k: torch.Tensor, cache_ks: torch.Tensor, cache_v: torch.Tensor, cache_vs: torch.Tensor,
+                           Smax: int, t_dev: torch.Tensor) -> torch.Tensor:
+    """partial_rope_append_kv + shared_prefix_attn without the RoPE launch and without q/k/v tensors, for up to
+    16 branches: the q|k|v product `p` goes straight into the attention kernels.  Returns out [B,H,D]."""
+    lib = _lib.load()
+    B = p.M
+    assert B <= SMH_GEMV_MAX_M and p.n_total == (H + 2 * Hkv) * D and p.buf.dtype == torch.float32
+    _need_gpu(p.buf, cache_k, cache_v, cache_ks, cache_vs, t_dev, pos_dev)
+    if prefix_k is not None:
+        assert prefix_k.is_contiguous() and prefix_v.is_contiguous() and prefix_k.dtype == torch.float16 and P <= prefix_k.shape[-3]
+    else:
+        assert P == 0
+    assert cache_k.dtype == torch.int8 and cache_ks.dtype == torch.float16 and t_dev.dtype == torch.int32
+    out = torch.empty((B, H, D), dtype=torch.float16, device=p.buf.device)
+    ws = attn_workspace(p.buf.device, B, H, P)
+    check(lib.smh_shared_prefix_attn_qkv(p.buf.data_ptr(), p.ksplit, out.data_ptr(), B, H, Hkv, D, cos.data_ptr(), sin.data_ptr(),
+                                         pos_dev.data_ptr(), _ptr(prefix_k), _ptr(prefix_v), int(P),
+                                         cache_k.data_ptr(), cache_ks.data_ptr(), cache_v.data_ptr(), cache_vs.data_ptr(), int(Smax),
+                                         t_dev.data_ptr(), ws.data_ptr(), ws.numel(), _stream()), "smh_shared_prefix_attn_qkv")
     return out
 
 

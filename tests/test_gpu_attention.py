@@ -151,3 +151,45 @@ def test_flash_attn_and_page_flash_attn_drop_ins():
     vv = vp.float()[:, idx].permute(1, 0, 2, 3)
     want2 = torch.nn.functional.scaled_dot_product_attention(q2.float()[:, :, None], kk, vv)[:, :, 0]
     assert torch.allclose(got2.float(), want2, rtol=1e-2, atol=2e-3)
+
+
+@pytest.mark.parametrize("B,H,Hkv,P,t", [(1, 4, 4, 40, 0), (3, 4, 4, 40, 5), (16, 8, 2, 100, 9), (5, 8, 8, 0, 3)])
+def test_attention_fed_by_the_qkv_product_matches_the_three_launch_sequence(B, H, Hkv, P, t):
+    """smh_shared_prefix_attn_qkv (RoPE + KV append inside the attention kernels) against
+    smh_partial_rope_append_kv + smh_shared_prefix_attn on the same slabs: same rounding points, so the
+    outputs and the appended cache rows must be bit-identical."""
+    from spec_mcts_amd import kernels as K
+    dev = "cuda:0"
+    D, Smax, dim = 128, 16, 512
+    g = torch.Generator(device="cpu").manual_seed(900 + B + t)
+    x = (torch.randn((B, dim), generator=g) * 0.5).half().to(dev)
+    ws = []
+    for n in (H * D, Hkv * D, Hkv * D):
+        w = torch.randint(-128, 128, (dim * n // 2,), generator=g, dtype=torch.int16).to(torch.int8).to(dev)
+        s = (torch.rand((dim * n // 64,), generator=g) * 0.02 + 0.005).half().to(dev)
+        ws.append((w, s, n))
+    qkv = K.matmul_q40_partial(x, ws)
+    ang = torch.rand((64, 64), generator=g) * 6.28
+    cos, sin = torch.cos(ang).half().to(dev), torch.sin(ang).half().to(dev)
+    pos_dev = torch.tensor([P + t], dtype=torch.int32, device=dev) % 64
+    t_dev = torch.tensor([t], dtype=torch.int32, device=dev)
+    pk = (torch.randn((max(P, 1), Hkv, D), generator=g) * 0.5).half().to(dev)
+    pv = (torch.randn((max(P, 1), Hkv, D), generator=g) * 0.5).half().to(dev)
+    caches = []
+    for _ in range(2):
+        ck = torch.randint(-128, 128, (B, Smax, Hkv, 64), generator=torch.Generator().manual_seed(7), dtype=torch.int16).to(torch.int8).to(dev)
+        cv = torch.randint(-128, 128, (B, Smax, Hkv, 64), generator=torch.Generator().manual_seed(8), dtype=torch.int16).to(torch.int8).to(dev)
+        cks = (torch.rand((B, Smax, Hkv, 2), generator=torch.Generator().manual_seed(9)) * 0.1 + 0.01).half().to(dev)
+        cvs = (torch.rand((B, Smax, Hkv, 2), generator=torch.Generator().manual_seed(10)) * 0.1 + 0.01).half().to(dev)
+        caches.append((ck, cks, cv, cvs))
+    ck, cks, cv, cvs = caches[0]
+    q, k, v = K.partial_rope_append_kv(qkv, H, Hkv, D, cos, sin, pos_dev, ck, cks, cv, cvs, Smax, t_dev)
+    want = K.shared_prefix_attn(q, pk if P else None, pv if P else None, P, suffix_k=ck, suffix_v=cv, suffix_ks=cks, suffix_vs=cvs,
+                                Smax=Smax, lens=t_dev, lens_stride=0, cur_k=k, cur_v=v, n_kv_heads=Hkv)
+    ck2, cks2, cv2, cvs2 = caches[1]
+    got = K.shared_prefix_attn_qkv(qkv, H, Hkv, D, cos, sin, pos_dev, pk if P else None, pv if P else None, P,
+                                   ck2, cks2, cv2, cvs2, Smax, t_dev)
+    torch.cuda.synchronize()
+    assert torch.equal(got, want)
+    for a, b_ in zip(caches[0], caches[1]):
+        assert torch.equal(a, b_), "appended cache rows differ"
