@@ -167,19 +167,28 @@ int smh_shared_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int 
 int smh_prefill_attn(const void *q, const void *k, const void *v, void *out, int S, int H, int Hkv,
                      int D, smh_stream_t stream);
 
-/* smh_shared_prefix_attn_qkv: smh_partial_rope_append_kv + smh_shared_prefix_attn in two launches instead of
- * three, for up to 16 branches: the attention kernels take q and the new token's k, v straight from the slabs
- * of the wq|wk|wv product (smh_q40_matmul_partial with the three weights as segments; B <= 16, so fp32 slabs),
+/* smh_shared_prefix_attn_qkv: smh_partial_rope_append_kv + smh_shared_prefix_attn without the RoPE launch, for up
+ * to 16 branches: the attention kernels take q and the new token's k, v straight from the slabs of the
+ * wq|wk|wv product (smh_q40_matmul_partial with the three weights as segments; B <= 16, so fp32 slabs),
  * apply apply_rotary_emb (hf_model_q40_kv_shared.py:173-203) at position *pos_dev, append Q4_0(k), Q4_0(v)
  * to row *t_dev of every branch's suffix cache (:365-371) and attend over prefix (P rows) || suffix rows
- * 0 .. *t_dev - 1 of the branch (the Q4_0 cache) || the new token (exact fp16).  Same rounding points as the
- * three-launch sequence: results are bit-identical to it.  q, k, v are not materialised.
- * B * (H / Hkv) <= 128. */
+ * 0 .. *t_dev - 1 of the branch (the Q4_0 cache) || the new token (exact fp16).  q, k, v are not
+ * materialised.  B * (H / Hkv) <= 128.
+ *   single_launch == 0: two launches (prefix slices, then suffix + merge), same rounding points and summation
+ *                       order as the three-launch sequence: results are bit-identical to it;
+ *                       workspace as for smh_shared_prefix_attn.
+ *   single_launch != 0: ONE launch: prefix slices and the branches' suffixes run side by side, the workgroup
+ *                       that arrives last at a head's counter merges the partials in a fixed order.
+ *                       workspace: smh_attn_qkv_workspace_bytes(B, H, P) bytes whose first 4096 bytes (the
+ *                       counters) are zero before the first call; the calls leave them zero.  Calls that
+ *                       overlap in time need separate workspaces. */
+size_t smh_attn_qkv_workspace_bytes(int B, int H, int P);
 int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, void *out, int B, int H, int Hkv, int D,
                                const void *cos_tab, const void *sin_tab, const int32_t *pos_dev,
                                const void *prefix_k, const void *prefix_v, int P,
                                void *cache_k, void *cache_ks, void *cache_v, void *cache_vs, int Smax,
-                               const int32_t *t_dev, void *workspace, size_t workspace_bytes, smh_stream_t stream);
+                               const int32_t *t_dev, int single_launch, void *workspace, size_t workspace_bytes,
+                               smh_stream_t stream);
 
 /* ---- matmul with the following operator finished inside the same launch ---------------------------
  * smh_q40_matmul_fused: the product of smh_q40_matmul_partial (same a / segments / partial buffer)

@@ -56,8 +56,9 @@ SIGNATURES = {
     "smh_shared_prefix_attn": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, c_int, _P, _P, _P, _P, c_int,
                                        _P, c_int, _P, _P, _P, c_size_t, _P]),
     "smh_prefill_attn": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
+    "smh_attn_qkv_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "smh_shared_prefix_attn_qkv": (c_int, [_P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_int,
-                                           _P, _P, _P, _P, c_int, _P, _P, c_size_t, _P]),
+                                           _P, _P, _P, _P, c_int, _P, c_int, _P, c_size_t, _P]),
     "smh_decode_step_workspace_bytes": (c_size_t, [c_int] * 8),
     "smh_q40_matmul_fused": (c_int, [_P, c_int, c_int, c_long, c_int, _P, _P, _P, _P, c_size_t, _P, _P]),
     "smh_decode_prepare": (c_int, [_P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, _P, _P, _P, _P, _P, _P,

@@ -24,8 +24,8 @@ namespace smh {
 constexpr int ATT_D = 128;
 constexpr int ATT_TW_MAX = 128;            // prefix rows per workgroup
 constexpr int ATT_KPITCH = 136;            // halves per LDS row of K (272 B: 16 rows hit distinct banks)
-constexpr int ATT_VPITCH = ATT_TW_MAX + 8; // halves per LDS row of V^T
 constexpr float LOG2E = 1.4426950408889634f;
+constexpr int ATT_ONE_TW = 64;             // prefix rows per workgroup of the one-launch kernel: two workgroups fit a compute unit
 constexpr int ATT_FUSED_MAX_Q = 128;       // queries per kv head (branches x query heads per kv head) of the fused variant
 
 struct AttnParams {
@@ -55,6 +55,7 @@ struct AttnParams {
     half_t *app_ks, *app_vs;
     const int32_t *app_t;
     int app_smax;
+    uint32_t *counters;              // one-launch variant: arrivals per kv head (zero between launches)
 };
 
 // column `col` of branch b in the fused q|k|v product: the slabs added in slice order, rounded once to fp16
@@ -108,14 +109,14 @@ __device__ __forceinline__ int vt_pos(int t) {
     return blk + 8 * g + 4 * j2 + r;
 }
 
-template <bool FUSED>
-__global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
-    __shared__ __attribute__((aligned(16))) half_t ks[ATT_TW_MAX][ATT_KPITCH];
-    __shared__ __attribute__((aligned(16))) half_t vt[ATT_D][ATT_VPITCH];
+// COHERENT: the partials are read by another workgroup of the same launch (device-scope stores)
+// TWM: most prefix rows a workgroup takes (p.tw <= TWM), which sizes its LDS
+template <bool FUSED, bool COHERENT, int TWM>
+__device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split, int hk) {
+    __shared__ __attribute__((aligned(16))) half_t ks[TWM][ATT_KPITCH];
+    __shared__ __attribute__((aligned(16))) half_t vt[ATT_D][TWM + 8];
     __shared__ __attribute__((aligned(16))) half_t qs[FUSED ? ATT_FUSED_MAX_Q : 1][ATT_D + 8];      // FUSED: the rotated queries of this kv head
 
-    const int split = blockIdx.x;
-    const int hk = blockIdx.y;
     const int tid = threadIdx.x;
     const int wave = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
     const int t0 = split * p.tw;
@@ -179,10 +180,10 @@ __global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
             load_q(qt, qb);
         }
         // S^T tiles: element r of st[j] is row t = 16j + 4g + r, column (query) c
-        f4 st[ATT_TW_MAX / 16];
+        f4 st[TWM / 16];
         float mx = -INFINITY;
 #pragma unroll
-        for (int j = 0; j < ATT_TW_MAX / 16; ++j) {
+        for (int j = 0; j < TWM / 16; ++j) {
             st[j] = f4{0.f, 0.f, 0.f, 0.f};
             if (j < t_tiles) {
 #pragma unroll
@@ -203,7 +204,7 @@ __global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
         mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
         float sum = 0.f;
 #pragma unroll
-        for (int j = 0; j < ATT_TW_MAX / 16; ++j) {
+        for (int j = 0; j < TWM / 16; ++j) {
             if (j < t_tiles) {
 #pragma unroll
                 for (int r = 0; r < 4; ++r) {
@@ -221,7 +222,7 @@ __global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
 #pragma unroll
         for (int dt = 0; dt < 8; ++dt) ot[dt] = f4{0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int jj = 0; jj < ATT_TW_MAX / 32; ++jj) {
+        for (int jj = 0; jj < TWM / 32; ++jj) {
             if (2 * jj < t_tiles) {
                 h8 pb;
 #pragma unroll
@@ -241,24 +242,30 @@ __global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
             const long base = ((long)split * p.Hkv + hk) * p.Bq + qrow;
             float *po = p.part_o + base * ATT_D;
 #pragma unroll
-            for (int dt = 0; dt < 8; ++dt) *reinterpret_cast<f4 *>(po + 16 * dt + 4 * g) = ot[dt];
+            for (int dt = 0; dt < 8; ++dt) {
+                if (COHERENT) st_f4(po + 16 * dt + 4 * g, ot[dt]);
+                else *reinterpret_cast<f4 *>(po + 16 * dt + 4 * g) = ot[dt];
+            }
             if (g == 0) {
-                p.part_ml[base * 2] = mx;
-                p.part_ml[base * 2 + 1] = sum;
+                if (COHERENT) { st_f32(p.part_ml + base * 2, mx); st_f32(p.part_ml + base * 2 + 1, sum); }
+                else { p.part_ml[base * 2] = mx; p.part_ml[base * 2 + 1] = sum; }
             }
         }
     }
 }
 
 template <bool FUSED>
-__global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
+__global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
+    attn_prefix_body<FUSED, false, ATT_TW_MAX>(p, blockIdx.x, blockIdx.y);
+}
+
+// One wave per (branch b, kv head hk).  PARTIAL: the pass over the suffix and the new token leaves an un-normalised
+// partial (split index p.splits) for the workgroup that merges, instead of folding in the prefix partials itself.
+template <bool FUSED, bool PARTIAL>
+__device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int hk) {
     __shared__ __attribute__((aligned(16))) half_t s_kv[FUSED ? 4 : 1][2][ATT_D];     // FUSED: this wave's new k and v rows
     const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
     const int wave = threadIdx.x >> 6;
-    const long item = (long)blockIdx.x * 4 + wave;
-    if (item >= (long)p.B * p.Hkv) return;
-    const int b = (int)(item / p.Hkv);
-    const int hk = (int)(item % p.Hkv);
     // FUSED: query of head h in the row layout (dims 4c..4c+3 and 64+4c..)
     auto fused_q = [&](int h, int pos_) {
         h4 lo, hi;
@@ -327,7 +334,7 @@ __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
 #pragma unroll
         for (int i = 0; i < PRE; ++i) {
             const int sp = g + 4 * i;
-            if (sp < p.splits) {
+            if (!PARTIAL && sp < p.splits) {
                 const long base = ((long)sp * p.Hkv + hk) * p.Bq + qrow;
                 pre_lo[i] = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 4 * c);
                 pre_hi[i] = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 64 + 4 * c);
@@ -373,12 +380,12 @@ __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
         // ---- prefix partials: group g folds in splits g, g+4, ... ----
 #pragma unroll
         for (int i = 0; i < PRE; ++i) {
-            if (g + 4 * i < p.splits) {
+            if (!PARTIAL && g + 4 * i < p.splits) {
                 const float o2[8] = {pre_lo[i][0], pre_lo[i][2], pre_lo[i][1], pre_lo[i][3], pre_hi[i][0], pre_hi[i][2], pre_hi[i][1], pre_hi[i][3]};
                 soft_merge(st, pre_m[i], pre_l[i], o2);
             }
         }
-        for (int sp = g + 4 * PRE; sp < p.splits; sp += 4) {
+        for (int sp = g + 4 * PRE; !PARTIAL && sp < p.splits; sp += 4) {
             const long base = ((long)sp * p.Hkv + hk) * p.Bq + qrow;
             const f4 lo = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 4 * c);
             const f4 hi = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 64 + 4 * c);
@@ -395,7 +402,12 @@ __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
             for (int j = 0; j < 8; ++j) o2[j] = __shfl_xor(st.o[j], sh, 64);
             soft_merge(st, m2, l2, o2);
         }
-        if (g == 0) {
+        if (g == 0 && PARTIAL) {
+            const long base = ((long)p.splits * p.Hkv + hk) * p.Bq + qrow;
+            st_f4(p.part_o + base * ATT_D + 4 * c, f4{st.o[0], st.o[2], st.o[1], st.o[3]});
+            st_f4(p.part_o + base * ATT_D + 64 + 4 * c, f4{st.o[4], st.o[6], st.o[5], st.o[7]});
+            if (c == 0) { st_f32(p.part_ml + base * 2, st.m); st_f32(p.part_ml + base * 2 + 1, st.l); }
+        } else if (g == 0) {
             const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
             half_t *op = p.out + ((long)b * p.H + h) * ATT_D;
             h4 lo = {(half_t)(st.o[0] * inv), (half_t)(st.o[2] * inv), (half_t)(st.o[1] * inv), (half_t)(st.o[3] * inv)};
@@ -403,6 +415,85 @@ __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
             *reinterpret_cast<h4 *>(op + 4 * c) = lo;
             *reinterpret_cast<h4 *>(op + 64 + 4 * c) = hi;
         }
+    }
+}
+
+template <bool FUSED>
+__global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
+    const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
+    if (item >= (long)p.B * p.Hkv) return;
+    attn_suffix_body<FUSED, false>(p, (int)(item / p.Hkv), (int)(item % p.Hkv));
+}
+
+// ---- the whole decode attention in ONE launch (fed by the wq|wk|wv slabs) -------------------------------------
+// grid (splits + ceil(B / 4), kv heads): workgroups x < splits take a slice of the prefix, the others four
+// branches' suffix + new token each (one wave per branch).  Every workgroup leaves partials with device-scope
+// stores and counts itself in on the head's counter; the one that arrives last merges the head's partials in
+// split order (so the result does not depend on which workgroup that is), normalises and writes the output.
+// Nobody waits for anybody.
+__global__ __launch_bounds__(256) void attn_one_kernel(AttnParams p) {
+    __shared__ uint32_t s_last;
+    const int hk = blockIdx.y;
+    const int tid = threadIdx.x;
+    const int sfx_groups = (p.B + 3) / 4;
+    if ((int)blockIdx.x < p.splits) {
+        attn_prefix_body<true, true, ATT_ONE_TW>(p, blockIdx.x, hk);
+    } else {
+        const int b = 4 * ((int)blockIdx.x - p.splits) + (tid >> 6);
+        if (b < p.B) attn_suffix_body<true, true>(p, b, hk);
+    }
+    wait_vmem();                               // this wave's partials have reached memory ...
+    __syncthreads();                           // ... and those of the whole workgroup
+    if (tid == 0) {
+        const uint32_t expected = (uint32_t)(p.splits + sfx_groups);
+        const uint32_t prev = __hip_atomic_fetch_add(p.counters + hk, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        const bool last = prev == expected - 1u;
+        if (last) st_u32(p.counters + hk, 0u);  // ready for the next launch
+        s_last = last ? 1u : 0u;
+    }
+    __syncthreads();
+    if (s_last == 0u) return;
+
+    // ---- merge: 16 lanes per query (dims 4cc.. and 64+4cc..), 16 queries at a time ----
+    const int cc = tid & 15;
+    const int n_part = p.splits + 1;
+    for (int qrow = tid >> 4; qrow < p.Bq; qrow += 16) {
+        float m = -INFINITY, l = 0.f;
+        float o[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) o[j] = 0.f;
+        for (int s0 = 0; s0 < n_part; s0 += 4) {
+            f4 lo[4], hi[4];
+            float pm[4], pl[4];
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (s0 + u < n_part) {
+                    const long base = ((long)(s0 + u) * p.Hkv + hk) * p.Bq + qrow;
+                    lo[u] = ld_f4(p.part_o + base * ATT_D + 4 * cc);
+                    hi[u] = ld_f4(p.part_o + base * ATT_D + 64 + 4 * cc);
+                    pm[u] = ld_f32(p.part_ml + base * 2);
+                    pl[u] = ld_f32(p.part_ml + base * 2 + 1);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+                if (s0 + u < n_part) {
+                    const float m_new = fmaxf(m, pm[u]);
+                    if (m_new != -INFINITY) {
+                        const float c1 = exp2f(m - m_new), c2 = exp2f(pm[u] - m_new);
+                        m = m_new;
+                        l = l * c1 + pl[u] * c2;
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) { o[j] = o[j] * c1 + lo[u][j] * c2; o[4 + j] = o[4 + j] * c1 + hi[u][j] * c2; }
+                    }
+                }
+            }
+        }
+        const float inv = l > 0.f ? 1.0f / l : 0.f;
+        const int b = qrow / p.n_rep, h = hk * p.n_rep + qrow % p.n_rep;
+        half_t *op = p.out + ((long)b * p.H + h) * ATT_D;
+        *reinterpret_cast<h4 *>(op + 4 * cc) = h4{(half_t)(o[0] * inv), (half_t)(o[1] * inv), (half_t)(o[2] * inv), (half_t)(o[3] * inv)};
+        *reinterpret_cast<h4 *>(op + 64 + 4 * cc) = h4{(half_t)(o[4] * inv), (half_t)(o[5] * inv), (half_t)(o[6] * inv), (half_t)(o[7] * inv)};
     }
 }
 
@@ -467,11 +558,20 @@ extern "C" int smh_shared_prefix_attn(const void *q, void *out, int B, int H, in
 }
 
 // The same attention fed by the un-reduced wq|wk|wv product: no q / k / v tensors and no separate RoPE launch.
+constexpr size_t ATT_COUNTER_BYTES = 4096;     // one-launch variant: arrival counters at the start of the workspace
+
+extern "C" size_t smh_attn_qkv_workspace_bytes(int B, int H, int P) {
+    if (B <= 0 || H <= 0) return ATT_COUNTER_BYTES + 256;
+    size_t splits = (size_t)(P > 0 ? (P + 31) / 32 : 0) + 1;      // worst case: 32 rows per workgroup; + the suffix partial
+    return ATT_COUNTER_BYTES + splits * (size_t)B * (size_t)H * (smh::ATT_D + 2) * sizeof(float) + 256;
+}
+
 extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, void *out, int B, int H, int Hkv, int D,
                                           const void *cos_tab, const void *sin_tab, const int32_t *pos_dev,
                                           const void *prefix_k, const void *prefix_v, int P,
                                           void *cache_k, void *cache_ks, void *cache_v, void *cache_vs, int Smax,
-                                          const int32_t *t_dev, void *workspace, size_t workspace_bytes, smh_stream_t stream) {
+                                          const int32_t *t_dev, int single_launch, void *workspace, size_t workspace_bytes,
+                                          smh_stream_t stream) {
     using namespace smh;
     const char *who = "smh_shared_prefix_attn_qkv";
     SMH_REQUIRE(D == ATT_D, "%s: head dim %d (only 128)", who, D);
@@ -499,6 +599,22 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
     p.app_k = (uint8_t *)cache_k; p.app_v = (uint8_t *)cache_v;
     p.app_ks = (half_t *)cache_ks; p.app_vs = (half_t *)cache_vs;
     p.app_t = t_dev; p.app_smax = Smax;
+    if (single_launch) {
+        if (p.tw > ATT_ONE_TW) {
+            p.tw = ATT_ONE_TW;
+            p.splits = P > 0 ? (P + p.tw - 1) / p.tw : 0;
+        }
+        // workspace = [arrival counters | partials of splits + 1 passes]
+        SMH_REQUIRE(Hkv * sizeof(uint32_t) <= ATT_COUNTER_BYTES, "%s: %d kv heads", who, Hkv);
+        size_t n_part = (size_t)(p.splits + 1) * Hkv * p.Bq;
+        size_t need = ATT_COUNTER_BYTES + n_part * (ATT_D + 2) * sizeof(float);
+        SMH_REQUIRE(workspace && workspace_bytes >= need, "%s: workspace %zu < %zu bytes", who, workspace_bytes, need);
+        p.counters = (uint32_t *)workspace;
+        p.part_o = (float *)((char *)workspace + ATT_COUNTER_BYTES);
+        p.part_ml = p.part_o + n_part * ATT_D;
+        hipLaunchKernelGGL(attn_one_kernel, dim3(p.splits + (B + 3) / 4, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+        return launch_status();
+    }
     size_t n_part = (size_t)p.splits * Hkv * p.Bq;
     SMH_REQUIRE(p.splits == 0 || (workspace && workspace_bytes >= n_part * (ATT_D + 2) * sizeof(float)),
                 "%s: workspace %zu < %zu bytes", who, workspace_bytes, n_part * (ATT_D + 2) * sizeof(float));

@@ -263,7 +263,7 @@ class Transformer(nn.Module):
                                       # layer instead of 10; measured slower at B=10: the finisher's round trips are serial)
         self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
         self.persistent = True        # decode steps of few branches as one persistent kernel (needs fused)
-        self.attn_from_qkv = False         # up to 16 branches the attention kernels can read the wq|wk|wv product themselves (one launch fewer; measured neutral)
+        self.attn_from_qkv = True          # up to 16 branches the attention takes the wq|wk|wv product itself, in one launch
         self.persistent_max_branches = 1   # from 2 branches on the operator-by-operator launches are faster (the kernel itself takes up to 16)
         self._step_kernels = {}       # branches -> K.DecodeStepKernel
 

@@ -61,6 +61,18 @@ def attn_workspace(device: torch.device, B: int, H: int, P: int) -> torch.Tensor
     return ws
 
 
+def attn_qkv_workspace(device: torch.device, B: int, H: int, P: int) -> torch.Tensor:
+    """Workspace of the one-launch attention: arrival counters (zero between calls) followed by the partials."""
+    lib = _lib.load()
+    need = lib.smh_attn_qkv_workspace_bytes(int(B), int(H), int(P))
+    key = ("attn_qkv", device.index if device.index is not None else torch.cuda.current_device())
+    ws = _workspaces.get(key)
+    if ws is None or ws.numel() < need:
+        ws = torch.zeros(need, dtype=torch.uint8, device=device)
+        _workspaces[key] = ws
+    return ws
+
+
 # ---------------------------------------------------------------------------------------------
 # Q4_0 matmul
 # ---------------------------------------------------------------------------------------------
@@ -372,9 +384,11 @@ def shared_prefix_attn(q: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix
 def shared_prefix_attn_qkv(p: PartialProduct, H: int, Hkv: int, D: int, cos: torch.Tensor, sin: torch.Tensor,
                            pos_dev: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix_v: Optional[torch.Tensor], P: int,
                            cache_k: torch.Tensor, cache_ks: torch.Tensor, cache_v: torch.Tensor, cache_vs: torch.Tensor,
-                           Smax: int, t_dev: torch.Tensor) -> torch.Tensor:
+                           Smax: int, t_dev: torch.Tensor, single_launch: bool = True) -> torch.Tensor:
     """partial_rope_append_kv + shared_prefix_attn without the RoPE launch and without q/k/v tensors, for up to
-    16 branches: the q|k|v product `p` goes straight into the attention kernels.  Returns out [B,H,D]."""
+    16 branches: the q|k|v product `p` goes straight into the attention kernels.  Returns out [B,H,D].
+    single_launch: everything in one launch (the workgroup that finishes last merges); otherwise two launches
+    whose result is bit-identical to the separate operators."""
     lib = _lib.load()
     B = p.M
     assert B <= SMH_GEMV_MAX_M and p.n_total == (H + 2 * Hkv) * D and p.buf.dtype == torch.float32
@@ -385,11 +399,12 @@ def shared_prefix_attn_qkv(p: PartialProduct, H: int, Hkv: int, D: int, cos: tor
         assert P == 0
     assert cache_k.dtype == torch.int8 and cache_ks.dtype == torch.float16 and t_dev.dtype == torch.int32
     out = torch.empty((B, H, D), dtype=torch.float16, device=p.buf.device)
-    ws = attn_workspace(p.buf.device, B, H, P)
+    ws = attn_qkv_workspace(p.buf.device, B, H, P) if single_launch else attn_workspace(p.buf.device, B, H, P)
     check(lib.smh_shared_prefix_attn_qkv(p.buf.data_ptr(), p.ksplit, out.data_ptr(), B, H, Hkv, D, cos.data_ptr(), sin.data_ptr(),
                                          pos_dev.data_ptr(), _ptr(prefix_k), _ptr(prefix_v), int(P),
                                          cache_k.data_ptr(), cache_ks.data_ptr(), cache_v.data_ptr(), cache_vs.data_ptr(), int(Smax),
-                                         t_dev.data_ptr(), ws.data_ptr(), ws.numel(), _stream()), "smh_shared_prefix_attn_qkv")
+                                         t_dev.data_ptr(), int(bool(single_launch)), ws.data_ptr(), ws.numel(), _stream()),
+          "smh_shared_prefix_attn_qkv")
     return out
 
 

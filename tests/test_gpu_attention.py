@@ -188,8 +188,19 @@ def test_attention_fed_by_the_qkv_product_matches_the_three_launch_sequence(B, H
                                 Smax=Smax, lens=t_dev, lens_stride=0, cur_k=k, cur_v=v, n_kv_heads=Hkv)
     ck2, cks2, cv2, cvs2 = caches[1]
     got = K.shared_prefix_attn_qkv(qkv, H, Hkv, D, cos, sin, pos_dev, pk if P else None, pv if P else None, P,
-                                   ck2, cks2, cv2, cvs2, Smax, t_dev)
+                                   ck2, cks2, cv2, cvs2, Smax, t_dev, single_launch=False)
     torch.cuda.synchronize()
     assert torch.equal(got, want)
     for a, b_ in zip(caches[0], caches[1]):
         assert torch.equal(a, b_), "appended cache rows differ"
+    # one launch: the partials are merged in another order, so equal up to fp32 summation order; three calls in a
+    # row check that the arrival counters are left ready for the next call
+    for rep in range(3):
+        ck3, cks3, cv3, cvs3 = (x.clone() for x in caches[0])
+        ck3[:, t], cks3[:, t], cv3[:, t], cvs3[:, t] = 0, 0, 0, 0
+        one = K.shared_prefix_attn_qkv(qkv, H, Hkv, D, cos, sin, pos_dev, pk if P else None, pv if P else None, P,
+                                       ck3, cks3, cv3, cvs3, Smax, t_dev, single_launch=True)
+        torch.cuda.synchronize()
+        assert torch.allclose(one.float(), want.float(), rtol=2e-3, atol=2e-3), f"call {rep}: {float((one.float() - want.float()).abs().max())}"
+        for a, b_ in zip(caches[0], (ck3, cks3, cv3, cvs3)):
+            assert torch.equal(a, b_), "appended cache rows differ"
