@@ -170,7 +170,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--no-persistent", action="store_true", help="small batches through the operator kernels too (comparison runs)")
+    ap.add_argument("--persistent", action="store_true", help="batches up to 4 through the persistent step kernel (comparison runs)")
     ap.add_argument("--batches", default="", help="comma-separated subset of 1,10,100 to run (a partial run is not a valid result)")
     ap.add_argument("--no-roofline", action="store_true", help="skip the matmul roofline legs (profiling runs)")
     ap.add_argument("--roofline-only", type=int, default=0, metavar="M",
@@ -191,8 +191,8 @@ def main():
                    rope_theta=1e6, max_batch_size=100, max_seq_len=128, max_prompt_seq_len=PROMPT_LEN)
     torch.manual_seed(3)
     model = build_model(torch, args_kw, seed=3)
-    if a.no_persistent:
-        model.persistent = False
+    if a.persistent:
+        model.persistent = True
     prompt = torch.randint(0, 32016, (1, PROMPT_LEN), generator=torch.Generator().manual_seed(3)).cuda()
 
     if a.roofline_only:

@@ -137,9 +137,36 @@ __device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split,
             for (int k4 = 0; k4 < 4; ++k4) qb[k4] = *reinterpret_cast<const h8 *>(&qs[qr][32 * k4 + 8 * g]);
         }
     };
-    if (FUSED) {
-        // all 256 threads build the rotated queries of this kv head from the slabs, 8 dims each, while
-        // the loads of K and V below are in flight; the barrier after the staging publishes them
+    // un-fused: the first tile's query is requested before the prefix slice is staged
+    h8 qb_first[4];
+    if (!FUSED && wave < q_tiles) load_q(wave, qb_first);
+
+    // ---- stage K (row-major) and V (transposed) ----
+    auto stage_store = [&](int idx, u32x4 kv, u32x4 vv) {
+        const int t = idx >> 4, ch = idx & 15;
+        *reinterpret_cast<u32x4 *>(&ks[t][ch * 8]) = kv;
+        const int pos = vt_pos(t);
+        const h8 vh = __builtin_bit_cast(h8, vv);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) vt[ch * 8 + j][pos] = vh[j];
+    };
+    auto stage_load = [&](int idx, u32x4 &kv, u32x4 &vv) {
+        const int t = idx >> 4, ch = idx & 15;
+        kv = u32x4{0, 0, 0, 0}; vv = u32x4{0, 0, 0, 0};
+        if (t < cnt) {
+            const long off = ((long)(t0 + t) * p.Hkv + hk) * ATT_D + ch * 8;
+            kv = *reinterpret_cast<const u32x4 *>(p.prefix_k + off);
+            vv = *reinterpret_cast<const u32x4 *>(p.prefix_v + off);
+        }
+    };
+    if (FUSED && TWM <= 64) {
+        // every load of the workgroup is requested before anything waits: the K / V slice into registers, then
+        // the slabs from which all 256 threads build the rotated queries of this kv head (8 dims each)
+        constexpr int PER = TWM * 16 / 256;
+        u32x4 kv[PER], vv[PER];
+#pragma unroll
+        for (int i = 0; i < PER; ++i)
+            if (tid + 256 * i < tw32 * 16) stage_load(tid + 256 * i, kv[i], vv[i]);
         const int cc = tid & 15;
         const int pos = *p.pos_dev;
         for (int qr = tid >> 4; qr < p.Bq; qr += 16) {
@@ -148,25 +175,25 @@ __device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split,
             *reinterpret_cast<h4 *>(&qs[qr][4 * cc]) = lo;
             *reinterpret_cast<h4 *>(&qs[qr][64 + 4 * cc]) = hi;
         }
-    }
-    // un-fused: the first tile's query is requested before the prefix slice is staged
-    h8 qb_first[4];
-    if (!FUSED && wave < q_tiles) load_q(wave, qb_first);
-
-    // ---- stage K (row-major) and V (transposed) ----
-    for (int idx = tid; idx < tw32 * 16; idx += 256) {
-        const int t = idx >> 4, ch = idx & 15;
-        u32x4 kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
-        if (t < cnt) {
-            const long off = ((long)(t0 + t) * p.Hkv + hk) * ATT_D + ch * 8;
-            kv = *reinterpret_cast<const u32x4 *>(p.prefix_k + off);
-            vv = *reinterpret_cast<const u32x4 *>(p.prefix_v + off);
-        }
-        *reinterpret_cast<u32x4 *>(&ks[t][ch * 8]) = kv;
-        const int pos = vt_pos(t);
-        const h8 vh = __builtin_bit_cast(h8, vv);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) vt[ch * 8 + j][pos] = vh[j];
+        for (int i = 0; i < PER; ++i)
+            if (tid + 256 * i < tw32 * 16) stage_store(tid + 256 * i, kv[i], vv[i]);
+    } else {
+        if (FUSED) {
+            const int cc = tid & 15;
+            const int pos = *p.pos_dev;
+            for (int qr = tid >> 4; qr < p.Bq; qr += 16) {
+                h4 lo, hi;
+                qkv_query(p, qr / p.n_rep, hk * p.n_rep + qr % p.n_rep, pos, cc, lo, hi);
+                *reinterpret_cast<h4 *>(&qs[qr][4 * cc]) = lo;
+                *reinterpret_cast<h4 *>(&qs[qr][64 + 4 * cc]) = hi;
+            }
+        }
+        for (int idx = tid; idx < tw32 * 16; idx += 256) {
+            u32x4 kv, vv;
+            stage_load(idx, kv, vv);
+            stage_store(idx, kv, vv);
+        }
     }
     __syncthreads();
 
@@ -275,9 +302,26 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
         qr.b02 = h2{hi[0], hi[2]}; qr.b13 = h2{hi[1], hi[3]};
         return qr;
     };
+    int len = 0;
+    if (p.suffix_format != SMH_KV_NONE) len = p.causal ? b + 1 : p.lens[(long)b * p.lens_stride];
+    const long row0 = (long)b * p.suffix_batch_stride_rows;     // first suffix row of this branch
+    // one batch of Q4_0 suffix rows: group g takes rows t0, t0 + 4, ... (rows past the end repeat the last one)
+    constexpr int UQ = 8;
+    auto load_q40_batch = [&](int t0, uint32_t (&kb)[UQ], uint32_t (&vb)[UQ], uint32_t (&ksc)[UQ], uint32_t (&vsc)[UQ]) {
+#pragma unroll
+        for (int u = 0; u < UQ; ++u) {
+            const long row = (row0 + min(t0 + 4 * u, len - 1)) * p.Hkv + hk;
+            kb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_k + row * 64 + 4 * c);
+            vb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_v + row * 64 + 4 * c);
+            ksc[u] = *reinterpret_cast<const uint32_t *>(p.suffix_ks + row * 2);
+            vsc[u] = *reinterpret_cast<const uint32_t *>(p.suffix_vs + row * 2);
+        }
+    };
+    uint32_t kb0[UQ], vb0[UQ], ksc0[UQ], vsc0[UQ];              // FUSED: the first batch, requested up front
     RowRegs q_first;
     int pos = 0;
     if (FUSED) {
+        if (p.suffix_format == SMH_KV_Q40 && g < len) load_q40_batch(g, kb0, vb0, ksc0, vsc0);
         // Everything that does not depend on another load is requested first: the position, the slabs of the new
         // token's k and v (lane owns the pair (lane, lane + 64)) and of the first query.  k is rotated, both rows
         // are appended to the branch's suffix cache as Q4_0 and left in LDS as exact fp16 for the pass below.
@@ -297,9 +341,6 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
         s_kv[wave][1][lane] = v1; s_kv[wave][1][lane + 64] = v2;
         // same wave writes and reads: LDS operations of a wave complete in order
     }
-    int len = 0;
-    if (p.suffix_format != SMH_KV_NONE) len = p.causal ? b + 1 : p.lens[(long)b * p.lens_stride];
-    const long row0 = (long)b * p.suffix_batch_stride_rows;     // first suffix row of this branch
 
     for (int rep = 0; rep < p.n_rep; ++rep) {
         const int h = hk * p.n_rep + rep;
@@ -358,16 +399,14 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
                     if (t0 + 4 * u < len) soft_add_row(st, row_dot(kr[u], qr) * p.scale_log2, vr[u]);
             }
         } else {
-            constexpr int U = 8;
+            constexpr int U = UQ;
             for (int t0 = g; t0 < len; t0 += 4 * U) {
                 uint32_t kb[U], vb[U], ksc[U], vsc[U];
+                if (FUSED && rep == 0 && t0 == g) {
 #pragma unroll
-                for (int u = 0; u < U; ++u) {
-                    const long row = (row0 + min(t0 + 4 * u, len - 1)) * p.Hkv + hk;
-                    kb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_k + row * 64 + 4 * c);
-                    vb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_v + row * 64 + 4 * c);
-                    ksc[u] = *reinterpret_cast<const uint32_t *>(p.suffix_ks + row * 2);
-                    vsc[u] = *reinterpret_cast<const uint32_t *>(p.suffix_vs + row * 2);
+                    for (int u = 0; u < U; ++u) { kb[u] = kb0[u]; vb[u] = vb0[u]; ksc[u] = ksc0[u]; vsc[u] = vsc0[u]; }
+                } else {
+                    load_q40_batch(t0, kb, vb, ksc, vsc);
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u)
@@ -431,7 +470,7 @@ __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
 // stores and counts itself in on the head's counter; the one that arrives last merges the head's partials in
 // split order (so the result does not depend on which workgroup that is), normalises and writes the output.
 // Nobody waits for anybody.
-__global__ __launch_bounds__(256) void attn_one_kernel(AttnParams p) {
+__global__ __launch_bounds__(256, 2) void attn_one_kernel(AttnParams p) {
     __shared__ uint32_t s_last;
     const int hk = blockIdx.y;
     const int tid = threadIdx.x;

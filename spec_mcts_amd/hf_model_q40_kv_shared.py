@@ -262,9 +262,9 @@ class Transformer(nn.Module):
         self.finish_in_matmul = False # decode: finish the operator after each linear inside the matmul launch (6 launches per
                                       # layer instead of 10; measured slower at B=10: the finisher's round trips are serial)
         self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
-        self.persistent = True        # decode steps of few branches as one persistent kernel (needs fused)
+        self.persistent = False       # True: decode steps of few branches as one persistent kernel (needs fused); the operator kernels are faster
         self.attn_from_qkv = True          # up to 16 branches the attention takes the wq|wk|wv product itself, in one launch
-        self.persistent_max_branches = 1   # from 2 branches on the operator-by-operator launches are faster (the kernel itself takes up to 16)
+        self.persistent_max_branches = 4   # with persistent = True: largest batch that uses the kernel (it takes up to 16)
         self._step_kernels = {}       # branches -> K.DecodeStepKernel
 
     # -- helpers -------------------------------------------------------------------------------

@@ -22,6 +22,7 @@ def _build(cfg, seed, std=0.05):
     oargs = O.OracleArgs(**cfg)
     sd = O.random_q40_state_dict(oargs, seed=seed, std=std)
     model = load_q40(dict(sd), ModelArgs(**cfg), device="cuda:0")
+    model.persistent = True
     model.persistent_max_branches = 16      # exercise the kernel over its whole range
     return oargs, sd, model
 
