@@ -31,7 +31,9 @@ PROMPT_LEN = 512
 BATCHES = (1, 10, 100)
 # HBM bytes per q40_gemv_kernel launch at M=1: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by a 1 GiB copy
 # (profiles/q40_gemv_m1_hbm_traffic.md has the commands and the factors: 2.0 for reads, 1.0 for writes)
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 32925390
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 32940444
+# the same for q40_gemm_kernel at M=100 (profiles/q40_gemm_m100_hbm_traffic.md): 43.95 MB read + 15.13 MB written
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 59075230
 
 
 def q40_bytes(M, N, K):
@@ -171,6 +173,7 @@ def main():
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
     ap.add_argument("--persistent", action="store_true", help="batches up to 4 through the persistent step kernel (comparison runs)")
+    ap.add_argument("--finish-in-matmul", action="store_true", help="operators after a linear finished inside the matmul launch (comparison runs)")
     ap.add_argument("--batches", default="", help="comma-separated subset of 1,10,100 to run (a partial run is not a valid result)")
     ap.add_argument("--no-roofline", action="store_true", help="skip the matmul roofline legs (profiling runs)")
     ap.add_argument("--roofline-only", type=int, default=0, metavar="M",
@@ -193,6 +196,8 @@ def main():
     model = build_model(torch, args_kw, seed=3)
     if a.persistent:
         model.persistent = True
+    if a.finish_in_matmul:
+        model.finish_in_matmul = True
     prompt = torch.randint(0, 32016, (1, PROMPT_LEN), generator=torch.Generator().manual_seed(3)).cuda()
 
     if a.roofline_only:
@@ -254,7 +259,7 @@ def main():
              "unit": "GB/s", "frac": round(rf10["gbs"] / HBM_PEAK_GBS, 4), "avg_launch_us": round(rf10["avg_us"], 3)},
             {"kernel": "q40_gemm_kernel at M=100", "bound": "mfma", "achieved": round(rf100["tflops"], 1),
              "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(rf100["tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
-             "hbm_gbs": round(rf100["gbs"], 1), "avg_launch_us": round(rf100["avg_us"], 3)},
+             "hbm_gbs": round(rf100["gbs"], 1), "avg_launch_us": round(rf100["avg_us"], 3), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH},
         ]
         if 1 in by_batch and by_batch[1]["path"].startswith("persistent"):
             # the whole step is one launch: every weight, the prefix KV and the suffix KV once
