@@ -1153,7 +1153,9 @@ extern "C" int smh_decode_status(const void *workspace, uint32_t *status3) {
     return 0;
 }
 
-// debugging aid (not part of the ABI): byte offsets of q, cur_k, cur_v, attn_out, act, slabs, ssq, att_part
+#ifdef SMH_MEGA_DEBUG
+// debugging aids of a -DSMH_MEGA_DEBUG build (not part of the ABI): byte offsets of q, cur_k, cur_v, attn_out, act,
+// slabs, ssq, att_part inside the workspace, and the cycle trace
 extern "C" int smhdbg_decode_offsets(int n_layers, int M, int dim, int H, int Hkv, int ffn, int P, int Smax, int G, size_t *out) {
     MegaPlan pl;
     if (mega_plan(pl, n_layers, M, dim, H, Hkv, ffn, P, Smax, G, "smhdbg_decode_offsets") != 0) return -1;
@@ -1163,7 +1165,6 @@ extern "C" int smhdbg_decode_offsets(int n_layers, int M, int dim, int H, int Hk
     return 0;
 }
 
-#ifdef SMH_MEGA_DEBUG
 extern "C" int smhdbg_read_trace(unsigned long long *out) {
     return (int)hipMemcpyFromSymbol(out, HIP_SYMBOL(smh_mega_trace), sizeof(unsigned long long) * 8 * 4096);
 }
