@@ -167,6 +167,19 @@ int smh_shared_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int 
 int smh_prefill_attn(const void *q, const void *k, const void *v, void *out, int S, int H, int Hkv,
                      int D, smh_stream_t stream);
 
+/* smh_shared_prefix_attn_one: smh_shared_prefix_attn (same arguments, same attention) in ONE launch instead of
+ * two: prefix slices and the branches' suffix passes run side by side and the workgroup that completes a
+ * tile of 16 queries merges its partials in a fixed order (deterministic; equal to the two-launch result up
+ * to fp32 summation order).  B * (H / Hkv) <= 128.  workspace: smh_attn_qkv_workspace_bytes(B, H, P) bytes whose
+ * first 4096 bytes (arrival counters) are zero before the first call; the calls leave them zero.  Calls that
+ * overlap in time need separate workspaces. */
+int smh_shared_prefix_attn_one(const void *q, void *out, int B, int H, int Hkv, int D,
+                               const void *prefix_k, const void *prefix_v, int P,
+                               int suffix_format, const void *suffix_k, const void *suffix_v,
+                               const void *suffix_ks, const void *suffix_vs, int Smax,
+                               const int32_t *lens, int lens_stride, const void *cur_k, const void *cur_v,
+                               void *workspace, size_t workspace_bytes, smh_stream_t stream);
+
 /* smh_shared_prefix_attn_qkv: smh_partial_rope_append_kv + smh_shared_prefix_attn without the RoPE launch, for up
  * to 16 branches: the attention kernels take q and the new token's k, v straight from the slabs of the
  * wq|wk|wv product (smh_q40_matmul_partial with the three weights as segments; B <= 16, so fp32 slabs),
@@ -178,7 +191,7 @@ int smh_prefill_attn(const void *q, const void *k, const void *v, void *out, int
  *                       order as the three-launch sequence: results are bit-identical to it;
  *                       workspace as for smh_shared_prefix_attn.
  *   single_launch != 0: ONE launch: prefix slices and the branches' suffixes run side by side, the workgroup
- *                       that arrives last at a head's counter merges the partials in a fixed order.
+ *                       that completes the count of a tile of 16 queries merges its partials in a fixed order.
  *                       workspace: smh_attn_qkv_workspace_bytes(B, H, P) bytes whose first 4096 bytes (the
  *                       counters) are zero before the first call; the calls leave them zero.  Calls that
  *                       overlap in time need separate workspaces. */

@@ -55,6 +55,8 @@ SIGNATURES = {
     "smh_attn_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "smh_shared_prefix_attn": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, c_int, _P, _P, _P, _P, c_int,
                                        _P, c_int, _P, _P, _P, c_size_t, _P]),
+    "smh_shared_prefix_attn_one": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, c_int, _P, _P, _P, _P, c_int,
+                                       _P, c_int, _P, _P, _P, c_size_t, _P]),
     "smh_prefill_attn": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     "smh_attn_qkv_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "smh_shared_prefix_attn_qkv": (c_int, [_P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_int,

@@ -464,39 +464,58 @@ __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
     attn_suffix_body<FUSED, false>(p, (int)(item / p.Hkv), (int)(item % p.Hkv));
 }
 
-// ---- the whole decode attention in ONE launch (fed by the wq|wk|wv slabs) -------------------------------------
+// ---- the whole decode attention in ONE launch -----------------------------------------------------------------
 // grid (splits + ceil(B / 4), kv heads): workgroups x < splits take a slice of the prefix, the others four
 // branches' suffix + new token each (one wave per branch).  Every workgroup leaves partials with device-scope
-// stores and counts itself in on the head's counter; the one that arrives last merges the head's partials in
-// split order (so the result does not depend on which workgroup that is), normalises and writes the output.
-// Nobody waits for anybody.
+// stores and counts itself in on the counters of the query tiles (16 queries of a kv head) it contributed to;
+// the workgroup that completes a tile's count merges that tile's partials in split order (so the result does
+// not depend on which workgroup that is), normalises and writes the output.  Nobody waits for anybody.
+// FUSED: q and the new token's k, v come from the wq|wk|wv slabs (up to 16 branches); otherwise from p.q, p.cur_k/v.
+constexpr int ATT_ONE_MAX_TILES = ATT_FUSED_MAX_Q / 16;
+
+template <bool FUSED>
 __global__ __launch_bounds__(256, 2) void attn_one_kernel(AttnParams p) {
-    __shared__ uint32_t s_last;
+    __shared__ uint32_t s_last[ATT_ONE_MAX_TILES];
     const int hk = blockIdx.y;
     const int tid = threadIdx.x;
-    const int sfx_groups = (p.B + 3) / 4;
+    const int q_tiles = (p.Bq + 15) / 16;
+    const int per_wg = 4 * p.n_rep;            // queries of one suffix workgroup (four branches)
+    int tile_lo = 0, tile_hi = q_tiles - 1;    // query tiles this workgroup contributed to
     if ((int)blockIdx.x < p.splits) {
-        attn_prefix_body<true, true, ATT_ONE_TW>(p, blockIdx.x, hk);
+        attn_prefix_body<FUSED, true, ATT_ONE_TW>(p, blockIdx.x, hk);
     } else {
-        const int b = 4 * ((int)blockIdx.x - p.splits) + (tid >> 6);
-        if (b < p.B) attn_suffix_body<true, true>(p, b, hk);
+        const int j = (int)blockIdx.x - p.splits;
+        const int b = 4 * j + (tid >> 6);
+        if (b < p.B) attn_suffix_body<FUSED, true>(p, b, hk);
+        tile_lo = (j * per_wg) / 16;
+        tile_hi = (min(p.Bq, (j + 1) * per_wg) - 1) / 16;
     }
     wait_vmem();                               // this wave's partials have reached memory ...
     __syncthreads();                           // ... and those of the whole workgroup
-    if (tid == 0) {
-        const uint32_t expected = (uint32_t)(p.splits + sfx_groups);
-        const uint32_t prev = __hip_atomic_fetch_add(p.counters + hk, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-        const bool last = prev == expected - 1u;
-        if (last) st_u32(p.counters + hk, 0u);  // ready for the next launch
-        s_last = last ? 1u : 0u;
+    if (tid < q_tiles) {
+        uint32_t last = 0u;
+        if (tid >= tile_lo && tid <= tile_hi) {
+            // arrivals a tile waits for: every prefix slice + the suffix workgroups whose queries fall into it
+            const int j_lo = (16 * tid) / per_wg, j_hi = (min(p.Bq, 16 * tid + 16) - 1) / per_wg;
+            const uint32_t expected = (uint32_t)(p.splits + j_hi - j_lo + 1);
+            uint32_t *cnt = p.counters + hk * q_tiles + tid;
+            const uint32_t prev = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            if (prev == expected - 1u) {
+                st_u32(cnt, 0u);               // ready for the next launch
+                last = 1u;
+            }
+        }
+        s_last[tid] = last;
     }
     __syncthreads();
-    if (s_last == 0u) return;
 
-    // ---- merge: 16 lanes per query (dims 4cc.. and 64+4cc..), 16 queries at a time ----
+    // ---- merge the completed tiles: 16 lanes per query (dims 4cc.. and 64+4cc..), 16 queries per tile ----
     const int cc = tid & 15;
     const int n_part = p.splits + 1;
-    for (int qrow = tid >> 4; qrow < p.Bq; qrow += 16) {
+    for (int qt = tile_lo; qt <= tile_hi; ++qt) {
+        if (s_last[qt] == 0u) continue;
+        const int qrow = 16 * qt + (tid >> 4);
+        if (qrow >= p.Bq) continue;
         float m = -INFINITY, l = 0.f;
         float o[8];
 #pragma unroll
@@ -551,26 +570,28 @@ extern "C" size_t smh_attn_workspace_bytes(int B, int H, int P) {
     return splits * (size_t)B * (size_t)H * (smh::ATT_D + 2) * sizeof(float) + 256;
 }
 
-extern "C" int smh_shared_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int D,
-                                      const void *prefix_k, const void *prefix_v, int P,
-                                      int suffix_format, const void *suffix_k, const void *suffix_v,
-                                      const void *suffix_ks, const void *suffix_vs, int Smax,
-                                      const int32_t *lens, int lens_stride, const void *cur_k, const void *cur_v,
-                                      void *workspace, size_t workspace_bytes, smh_stream_t stream) {
+constexpr size_t ATT_COUNTER_BYTES = 4096;     // one-launch variants: arrival counters at the start of the workspace
+
+static int shared_prefix_attn(const char *who, bool one, const void *q, void *out, int B, int H, int Hkv, int D,
+                              const void *prefix_k, const void *prefix_v, int P,
+                              int suffix_format, const void *suffix_k, const void *suffix_v,
+                              const void *suffix_ks, const void *suffix_vs, int Smax,
+                              const int32_t *lens, int lens_stride, const void *cur_k, const void *cur_v,
+                              void *workspace, size_t workspace_bytes, smh_stream_t stream) {
     using namespace smh;
-    SMH_REQUIRE(D == ATT_D, "smh_shared_prefix_attn: head dim %d (only 128)", D);
-    SMH_REQUIRE(B >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0 && P >= 0, "smh_shared_prefix_attn: B=%d H=%d Hkv=%d P=%d", B, H, Hkv, P);
+    SMH_REQUIRE(D == ATT_D, "%s: head dim %d (only 128)", who, D);
+    SMH_REQUIRE(B >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0 && P >= 0, "%s: B=%d H=%d Hkv=%d P=%d", who, B, H, Hkv, P);
     SMH_REQUIRE(suffix_format == SMH_KV_NONE || suffix_format == SMH_KV_FP16 || suffix_format == SMH_KV_Q40,
-                "smh_shared_prefix_attn: suffix_format=%d", suffix_format);
+                "%s: suffix_format=%d", who, suffix_format);
     if (B == 0) return 0;
-    SMH_REQUIRE(q && out, "smh_shared_prefix_attn: null q/out");
-    SMH_REQUIRE(P == 0 || (prefix_k && prefix_v), "smh_shared_prefix_attn: null prefix");
+    SMH_REQUIRE(q && out, "%s: null q/out", who);
+    SMH_REQUIRE(P == 0 || (prefix_k && prefix_v), "%s: null prefix", who);
     if (suffix_format != SMH_KV_NONE) {
         SMH_REQUIRE(suffix_k && suffix_v && lens && Smax > 0 && (lens_stride == 0 || lens_stride == 1),
-                    "smh_shared_prefix_attn: suffix arguments incomplete");
-        SMH_REQUIRE(suffix_format != SMH_KV_Q40 || (suffix_ks && suffix_vs), "smh_shared_prefix_attn: null suffix scales");
+                    "%s: suffix arguments incomplete", who);
+        SMH_REQUIRE(suffix_format != SMH_KV_Q40 || (suffix_ks && suffix_vs), "%s: null suffix scales", who);
     }
-    SMH_REQUIRE((cur_k == nullptr) == (cur_v == nullptr), "smh_shared_prefix_attn: cur_k/cur_v must both be given or both be null");
+    SMH_REQUIRE((cur_k == nullptr) == (cur_v == nullptr), "%s: cur_k/cur_v must both be given or both be null", who);
     AttnParams p{};
     p.q = (const half_t *)q; p.out = (half_t *)out;
     p.prefix_k = (const half_t *)prefix_k; p.prefix_v = (const half_t *)prefix_v;
@@ -583,10 +604,24 @@ extern "C" int smh_shared_prefix_attn(const void *q, void *out, int B, int H, in
     p.P = P; p.suffix_format = suffix_format; p.causal = 0;
     p.scale_log2 = LOG2E / sqrtf((float)D);
     p.tw = attn_plan_tw(P, Hkv);
+    if (one && p.tw > ATT_ONE_TW) p.tw = ATT_ONE_TW;
     p.splits = P > 0 ? (P + p.tw - 1) / p.tw : 0;
+    if (one) {
+        const int q_tiles = (p.Bq + 15) / 16;
+        SMH_REQUIRE(q_tiles <= ATT_ONE_MAX_TILES && (size_t)Hkv * q_tiles * sizeof(uint32_t) <= ATT_COUNTER_BYTES,
+                    "%s: %d queries per kv head (at most %d), %d kv heads", who, p.Bq, ATT_FUSED_MAX_Q, Hkv);
+        size_t n_part = (size_t)(p.splits + 1) * Hkv * p.Bq;
+        size_t need = ATT_COUNTER_BYTES + n_part * (ATT_D + 2) * sizeof(float);
+        SMH_REQUIRE(workspace && workspace_bytes >= need, "%s: workspace %zu < %zu bytes", who, workspace_bytes, need);
+        p.counters = (uint32_t *)workspace;
+        p.part_o = (float *)((char *)workspace + ATT_COUNTER_BYTES);
+        p.part_ml = p.part_o + n_part * ATT_D;
+        hipLaunchKernelGGL(attn_one_kernel<false>, dim3(p.splits + (B + 3) / 4, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+        return launch_status();
+    }
     size_t n_part = (size_t)p.splits * Hkv * p.Bq;
     SMH_REQUIRE(p.splits == 0 || (workspace && workspace_bytes >= n_part * (ATT_D + 2) * sizeof(float)),
-                "smh_shared_prefix_attn: workspace %zu < %zu bytes", workspace_bytes, n_part * (ATT_D + 2) * sizeof(float));
+                "%s: workspace %zu < %zu bytes", who, workspace_bytes, n_part * (ATT_D + 2) * sizeof(float));
     p.part_o = (float *)workspace;
     p.part_ml = p.part_o + n_part * ATT_D;
     if (p.splits > 0)
@@ -596,8 +631,26 @@ extern "C" int smh_shared_prefix_attn(const void *q, void *out, int B, int H, in
     return launch_status();
 }
 
-// The same attention fed by the un-reduced wq|wk|wv product: no q / k / v tensors and no separate RoPE launch.
-constexpr size_t ATT_COUNTER_BYTES = 4096;     // one-launch variant: arrival counters at the start of the workspace
+extern "C" int smh_shared_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int D,
+                                      const void *prefix_k, const void *prefix_v, int P,
+                                      int suffix_format, const void *suffix_k, const void *suffix_v,
+                                      const void *suffix_ks, const void *suffix_vs, int Smax,
+                                      const int32_t *lens, int lens_stride, const void *cur_k, const void *cur_v,
+                                      void *workspace, size_t workspace_bytes, smh_stream_t stream) {
+    return shared_prefix_attn("smh_shared_prefix_attn", false, q, out, B, H, Hkv, D, prefix_k, prefix_v, P, suffix_format, suffix_k,
+                              suffix_v, suffix_ks, suffix_vs, Smax, lens, lens_stride, cur_k, cur_v, workspace, workspace_bytes, stream);
+}
+
+extern "C" int smh_shared_prefix_attn_one(const void *q, void *out, int B, int H, int Hkv, int D,
+                                          const void *prefix_k, const void *prefix_v, int P,
+                                          int suffix_format, const void *suffix_k, const void *suffix_v,
+                                          const void *suffix_ks, const void *suffix_vs, int Smax,
+                                          const int32_t *lens, int lens_stride, const void *cur_k, const void *cur_v,
+                                          void *workspace, size_t workspace_bytes, smh_stream_t stream) {
+    return shared_prefix_attn("smh_shared_prefix_attn_one", true, q, out, B, H, Hkv, D, prefix_k, prefix_v, P, suffix_format, suffix_k,
+                              suffix_v, suffix_ks, suffix_vs, Smax, lens, lens_stride, cur_k, cur_v, workspace, workspace_bytes, stream);
+}
+
 
 extern "C" size_t smh_attn_qkv_workspace_bytes(int B, int H, int P) {
     if (B <= 0 || H <= 0) return ATT_COUNTER_BYTES + 256;
@@ -644,14 +697,14 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
             p.splits = P > 0 ? (P + p.tw - 1) / p.tw : 0;
         }
         // workspace = [arrival counters | partials of splits + 1 passes]
-        SMH_REQUIRE(Hkv * sizeof(uint32_t) <= ATT_COUNTER_BYTES, "%s: %d kv heads", who, Hkv);
+        SMH_REQUIRE((size_t)Hkv * ((p.Bq + 15) / 16) * sizeof(uint32_t) <= ATT_COUNTER_BYTES, "%s: %d kv heads x %d query tiles", who, Hkv, (p.Bq + 15) / 16);
         size_t n_part = (size_t)(p.splits + 1) * Hkv * p.Bq;
         size_t need = ATT_COUNTER_BYTES + n_part * (ATT_D + 2) * sizeof(float);
         SMH_REQUIRE(workspace && workspace_bytes >= need, "%s: workspace %zu < %zu bytes", who, workspace_bytes, need);
         p.counters = (uint32_t *)workspace;
         p.part_o = (float *)((char *)workspace + ATT_COUNTER_BYTES);
         p.part_ml = p.part_o + n_part * ATT_D;
-        hipLaunchKernelGGL(attn_one_kernel, dim3(p.splits + (B + 3) / 4, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(attn_one_kernel<true>, dim3(p.splits + (B + 3) / 4, Hkv), dim3(256), 0, (hipStream_t)stream, p);
         return launch_status();
     }
     size_t n_part = (size_t)p.splits * Hkv * p.Bq;

@@ -263,6 +263,7 @@ class Transformer(nn.Module):
                                       # layer instead of 10; measured slower at B=10: the finisher's round trips are serial)
         self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
         self.persistent = False       # True: decode steps of few branches as one persistent kernel (needs fused); the operator kernels are faster
+        self.attn_single_launch = True     # up to 16 branches: prefix slices, suffix passes and the merge in one launch (slower above)
         self.attn_from_qkv = True          # up to 16 branches the attention takes the wq|wk|wv product itself, in one launch
         self.persistent_max_branches = 4   # with persistent = True: largest batch that uses the kernel (it takes up to 16)
         self._step_kernels = {}       # branches -> K.DecodeStepKernel
@@ -362,7 +363,7 @@ class Transformer(nn.Module):
                     o = K.shared_prefix_attn(q, att.cache_prompt_k[0], att.cache_prompt_v[0], att.cache_prompt_len,
                                              suffix_k=att.cache_k, suffix_v=att.cache_v, suffix_ks=att.cache_k_s,
                                              suffix_vs=att.cache_v_s, Smax=p.max_seq_len, lens=t_dev, lens_stride=0,
-                                             cur_k=k, cur_v=v).view(M, H * D)
+                                             cur_k=k, cur_v=v, single_launch=self.attn_single_launch and M <= 16).view(M, H * D)
             po = K.matmul_q40_partial(o, [(att.wo.w, att.wo.s, att.wo.shape[0])])
             h, xn = K.partial_rmsnorm(po, h, layer.ffn_norm.weight, layer.ffn_norm.eps)
             gu = K.matmul_q40_partial(xn, [(ff.w1.w, ff.w1.s, ff.w1.shape[0]), (ff.w3.w, ff.w3.s, ff.w3.shape[0])])

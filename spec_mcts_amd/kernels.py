@@ -345,10 +345,12 @@ def shared_prefix_attn(q: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix
                        suffix_ks: Optional[torch.Tensor] = None, suffix_vs: Optional[torch.Tensor] = None,
                        Smax: int = 0, lens: Optional[torch.Tensor] = None, lens_stride: int = 1,
                        cur_k: Optional[torch.Tensor] = None, cur_v: Optional[torch.Tensor] = None,
-                       n_kv_heads: Optional[int] = None) -> torch.Tensor:
+                       n_kv_heads: Optional[int] = None, single_launch: bool = False) -> torch.Tensor:
     """out[b,h] = softmax(q[b,h] . K_b^T / sqrt(D)) . V_b with K_b = prefix[:P] (shared) ||
     suffix[b, :lens[b]] || cur_k[b].  The suffix is fp16 [B,Smax,Hkv,D] or Q4_0 (int8 rows +
-    fp16 scales, the model's cache layout); `lens` is int32 on the device."""
+    fp16 scales, the model's cache layout); `lens` is int32 on the device.
+    single_launch: one launch instead of two (at most 128 queries per kv head; same result up to fp32
+    summation order)."""
     lib = _lib.load()
     _need_gpu(q)
     assert q.is_contiguous() and q.dtype == torch.float16 and q.dim() == 3
@@ -373,11 +375,13 @@ def shared_prefix_attn(q: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix
     if cur_k is not None:
         assert cur_k.is_contiguous() and cur_v.is_contiguous() and cur_k.dtype == torch.float16
     out = torch.empty_like(q)
-    ws = attn_workspace(q.device, B, H, P)
-    check(lib.smh_shared_prefix_attn(q.data_ptr(), out.data_ptr(), B, H, Hkv, D, _ptr(prefix_k), _ptr(prefix_v), int(P),
-                                     fmt, _ptr(suffix_k), _ptr(suffix_v), _ptr(suffix_ks), _ptr(suffix_vs), int(Smax),
-                                     _ptr(lens), int(lens_stride), _ptr(cur_k), _ptr(cur_v),
-                                     ws.data_ptr(), ws.numel(), _stream()), "smh_shared_prefix_attn")
+    one = bool(single_launch) and B * (H // Hkv) <= 128
+    ws = attn_qkv_workspace(q.device, B, H, P) if one else attn_workspace(q.device, B, H, P)
+    fn = lib.smh_shared_prefix_attn_one if one else lib.smh_shared_prefix_attn
+    check(fn(q.data_ptr(), out.data_ptr(), B, H, Hkv, D, _ptr(prefix_k), _ptr(prefix_v), int(P),
+             fmt, _ptr(suffix_k), _ptr(suffix_v), _ptr(suffix_ks), _ptr(suffix_vs), int(Smax),
+             _ptr(lens), int(lens_stride), _ptr(cur_k), _ptr(cur_v),
+             ws.data_ptr(), ws.numel(), _stream()), "smh_shared_prefix_attn")
     return out
 
 

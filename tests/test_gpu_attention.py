@@ -204,3 +204,30 @@ def test_attention_fed_by_the_qkv_product_matches_the_three_launch_sequence(B, H
         assert torch.allclose(one.float(), want.float(), rtol=2e-3, atol=2e-3), f"call {rep}: {float((one.float() - want.float()).abs().max())}"
         for a, b_ in zip(caches[0], (ck3, cks3, cv3, cvs3)):
             assert torch.equal(a, b_), "appended cache rows differ"
+
+
+@pytest.mark.parametrize("B,H,Hkv,P,L", [(100, 4, 4, 150, 9), (33, 8, 2, 70, 4), (5, 4, 4, 0, 6), (128, 2, 2, 40, 0)])
+def test_one_launch_attention_matches_two_launches(B, H, Hkv, P, L):
+    """smh_shared_prefix_attn_one against smh_shared_prefix_attn on the same inputs (Q4_0 suffix, new token):
+    same partials, merged in another order; called three times to check the counters are left ready."""
+    from spec_mcts_amd import kernels as K
+    dev = "cuda:0"
+    D, Smax = 128, 16
+    g = torch.Generator().manual_seed(1200 + B)
+    q = (torch.randn((B, H, D), generator=g) * 0.7).half().to(dev)
+    pk = (torch.randn((max(P, 1), Hkv, D), generator=g) * 0.5).half().to(dev)
+    pv = (torch.randn((max(P, 1), Hkv, D), generator=g) * 0.5).half().to(dev)
+    ck = torch.randint(-128, 128, (B, Smax, Hkv, 64), generator=g, dtype=torch.int16).to(torch.int8).to(dev)
+    cv = torch.randint(-128, 128, (B, Smax, Hkv, 64), generator=g, dtype=torch.int16).to(torch.int8).to(dev)
+    cks = (torch.rand((B, Smax, Hkv, 2), generator=g) * 0.1 + 0.01).half().to(dev)
+    cvs = (torch.rand((B, Smax, Hkv, 2), generator=g) * 0.1 + 0.01).half().to(dev)
+    k = (torch.randn((B, Hkv, D), generator=g) * 0.5).half().to(dev)
+    v = (torch.randn((B, Hkv, D), generator=g) * 0.5).half().to(dev)
+    lens = torch.tensor([L], dtype=torch.int32, device=dev)
+    kw = dict(suffix_k=ck, suffix_v=cv, suffix_ks=cks, suffix_vs=cvs, Smax=Smax, lens=lens, lens_stride=0, cur_k=k, cur_v=v,
+              n_kv_heads=Hkv)
+    want = K.shared_prefix_attn(q, pk if P else None, pv if P else None, P, **kw)
+    for rep in range(3):
+        got = K.shared_prefix_attn(q, pk if P else None, pv if P else None, P, single_launch=True, **kw)
+        torch.cuda.synchronize()
+        assert torch.allclose(got.float(), want.float(), rtol=2e-3, atol=2e-3), f"call {rep}: {float((got.float() - want.float()).abs().max())}"
