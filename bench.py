@@ -87,7 +87,7 @@ def step_matmuls(model):
     out = []
     for layer in model.layers:
         a, f = layer.attention, layer.feed_forward
-        seg = lambda lin: (lin.w, lin.s, lin.shape[0])
+        seg = lambda lin: (lin.operand(model.tiled_weights), lin.shape[0])      # (what the model hands the kernel, columns)
         out.append((a.wq.shape[1], [seg(a.wq), seg(a.wk), seg(a.wv)]))
         out.append((a.wo.shape[1], [seg(a.wo)]))
         out.append((f.w1.shape[1], [seg(f.w1), seg(f.w3)]))
@@ -107,7 +107,7 @@ def matmul_roofline(torch, model, M, iters):
 
     def run():
         for k_in, segs in launches:
-            K.matmul_q40_partial(xs[k_in], segs)
+            K.matmul_q40_partial(xs[k_in], [op for op, _ in segs])
 
     run()
     torch.cuda.synchronize()
@@ -117,9 +117,9 @@ def matmul_roofline(torch, model, M, iters):
     for _ in range(10):                  # clocks and caches settle before the timed replays
         graph.replay()
     ms = time_region(torch, graph.replay, iters)
-    total_bytes = sum(sum(q40_bytes(0, n, k_in) for _, _, n in segs) + 2 * M * k_in + 4 * M * sum(n for _, _, n in segs)
+    total_bytes = sum(sum(q40_bytes(0, n, k_in) for _, n in segs) + 2 * M * k_in + 4 * M * sum(n for _, n in segs)
                       for k_in, segs in launches)
-    flops = sum(2 * M * k_in * sum(n for _, _, n in segs) for k_in, segs in launches)
+    flops = sum(2 * M * k_in * sum(n for _, n in segs) for k_in, segs in launches)
     n = len(launches)
     return {"launches": n, "avg_us": ms * 1e3 / n, "bytes_per_launch": total_bytes / n, "gbs": total_bytes / (ms * 1e-3) / 1e9,
             "tflops": flops / (ms * 1e-3) / 1e12}

@@ -102,6 +102,16 @@ int smh_q40_matmul_plan(int M, int K, int nseg, const int *n);
 int smh_q40_matmul_partial(const void *a, int M, int K, long lda, int nseg, const void *const *w,
                            const void *const *s, const int *n, void *partial, size_t partial_bytes,
                            smh_stream_t stream);
+/* Tiled weights.  The checkpoint layout written by fp16_to_int4.py:165-201 (bytes [K, N/2], scales [K, N/64])
+ * is what every entry point above takes.  smh_q40_tile rewrites one weight, once, into the order the matmul
+ * kernels consume it (256-column x 32-row tiles of 4352 contiguous bytes: nibbles in MFMA operand order, then the
+ * tile's scales); smh_q40_matmul_partial_tiled is smh_q40_matmul_partial on such weights and leaves bit-identical
+ * slabs - it replaces the same matmul_q40 (triton_kernels.py:471-500) calls, with fewer memory requests and fewer
+ * decode instructions per weight.  tiled buffers: smh_q40_tiled_bytes(K, N) bytes, 128-byte aligned. */
+size_t smh_q40_tiled_bytes(int K, int N);
+int smh_q40_tile(const void *w, const void *s, int K, int N, void *tiled, size_t tiled_bytes, smh_stream_t stream);
+int smh_q40_matmul_partial_tiled(const void *a, int M, int K, long lda, int nseg, const void *const *tiled,
+                                 const int *n, void *partial, size_t partial_bytes, smh_stream_t stream);
 int smh_partial_reduce(const void *partial, int ksplit, int M, int n_total, int col0, int N, void *c,
                        long ldc, int epilogue, const void *residual, long ldr, smh_stream_t stream);
 int smh_partial_rmsnorm(const void *partial, int ksplit, int M, int N, const void *h_in,

@@ -299,6 +299,23 @@ extern "C" int smh_q40_matmul_partial(const void *a, int M, int K, long lda, int
     return M <= SMH_GEMV_MAX_M ? gemv_launch(p, (hipStream_t)stream) : gemm_launch(p, (hipStream_t)stream);
 }
 
+extern "C" int smh_q40_matmul_partial_tiled(const void *a, int M, int K, long lda, int nseg, const void *const *tiled,
+                                            const int *n, void *partial, size_t partial_bytes, smh_stream_t stream) {
+    MatmulParams p;
+    int st = fill_params(p, a, M, K, lda, nseg, tiled, nullptr, n, "smh_q40_matmul_partial_tiled");
+    if (st) return st;
+    if (M == 0) return 0;
+    SMH_REQUIRE(a && tiled && partial, "smh_q40_matmul_partial_tiled: null pointer");
+    for (int i = 0; i < nseg; ++i)
+        SMH_REQUIRE(tiled[i] && ((uintptr_t)tiled[i] & 127) == 0, "smh_q40_matmul_partial_tiled: weight %d is null or not 128-byte aligned", i);
+    size_t need = (size_t)p.ksplit * M * p.n_total * sizeof(float);
+    SMH_REQUIRE(partial_bytes >= need, "smh_q40_matmul_partial_tiled: partial buffer %zu < %zu bytes", partial_bytes, need);
+    p.partial = (float *)partial;
+    p.direct = 0;
+    p.tiled = 1;
+    return M <= SMH_GEMV_MAX_M ? gemv_launch(p, (hipStream_t)stream) : gemm_launch(p, (hipStream_t)stream);
+}
+
 extern "C" int smh_q40_matmul_fused(const void *a, int M, int K, long lda, int nseg, const void *const *w,
                                     const void *const *s, const int *n, void *partial, size_t partial_bytes,
                                     const smh_finish *fin, smh_stream_t stream) {

@@ -3,7 +3,7 @@
 // Both kernels are pure streaming (HBM-bound): dequant reads 68 B and writes 256 B per row,
 // quantise reads 256 B and writes 68 B per row.  One lane owns 16 bytes of a row, so a row is
 // covered by 4 neighbouring lanes and every access is a 128-bit load/store.
-#include "smh_common.hpp"
+#include "q40_matmul.hpp"
 
 namespace smh {
 
@@ -100,7 +100,64 @@ __global__ __launch_bounds__(256) void q40_quantize_kernel(const u32x4 *__restri
     }
 }
 
+// One thread per output dword of the tiled layout (q40_matmul.hpp): 1024 nibble dwords + 64 scale dwords per tile.
+__global__ __launch_bounds__(256) void q40_tile_kernel(const uint8_t *__restrict__ w, const half_t *__restrict__ s,
+                                                       int K, int N, uint32_t *__restrict__ tiled, long tiles) {
+    const long idx = (long)blockIdx.x * 256 + threadIdx.x;
+    constexpr int DW = TILE_BYTES / 4;
+    if (idx >= tiles * DW) return;
+    const long tile = idx / DW;
+    const int d = (int)(idx - tile * DW);
+    const long steps = tiled_steps(K);
+    const int unit = (int)(tile / steps), step = (int)(tile - (long)unit * steps);
+    uint32_t out;
+    if (d < TILE_W_BYTES / 4) {
+        const int q = d >> 8, lane = (d >> 2) & 63, e = d & 3;         // piece, lane, dword of the lane's 16 bytes
+        const int g = lane >> 4, c = lane & 15, blk = q >> 1, B = 2 * (q & 1) + (e >> 1);
+        const long col = (long)unit * 128 + 64 * blk + 4 * c + B;       // byte column of the checkpoint row
+        const int r0 = 32 * step + 8 * g + ((e & 1) ? 2 : 0);           // x: rows 0,4,1,5; x2: rows 2,6,3,7
+        const int rows[4] = {r0, r0 + 4, r0 + 1, r0 + 5};
+        out = 0;
+#pragma unroll
+        for (int b = 0; b < 4; ++b) {
+            uint32_t byte = 0;                                           // code 0 | code 0 before the flip
+            if (rows[b] < K && col < N / 2) byte = w[(long)rows[b] * (N / 2) + col];
+            out |= (byte ^ 0x88u) << (8 * b);
+        }
+    } else {
+        const int e = d - TILE_W_BYTES / 4;                              // [g][group][i / 2]
+        const int g = e >> 4, grp = (e >> 2) & 3, i = 2 * (e & 3);
+        const long gcol = (long)unit * 4 + grp;
+        uint32_t v[2];
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int row = 32 * step + 8 * g + i + h;
+            v[h] = (row < K && gcol < N / 64) ? __builtin_bit_cast(uint16_t, s[(long)row * (N / 64) + gcol]) : 0u;
+        }
+        out = v[0] | (v[1] << 16);
+    }
+    tiled[idx] = out;
+}
+
 }  // namespace smh
+
+extern "C" size_t smh_q40_tiled_bytes(int K, int N) {
+    if (K <= 0 || N <= 0) return 0;
+    return (size_t)smh::tiled_units(N) * smh::tiled_steps(K) * smh::TILE_BYTES;
+}
+
+extern "C" int smh_q40_tile(const void *w, const void *s, int K, int N, void *tiled, size_t tiled_bytes, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(K > 0 && N > 0 && N % 128 == 0, "smh_q40_tile: K=%d N=%d (N must be a positive multiple of 128)", K, N);
+    SMH_REQUIRE(w && s && tiled, "smh_q40_tile: null pointer");
+    SMH_REQUIRE(tiled_bytes >= smh_q40_tiled_bytes(K, N), "smh_q40_tile: buffer %zu < %zu bytes", tiled_bytes, smh_q40_tiled_bytes(K, N));
+    SMH_REQUIRE(((uintptr_t)tiled & 127) == 0, "smh_q40_tile: the tiled buffer must be 128-byte aligned");
+    const long tiles = tiled_units(N) * tiled_steps(K);
+    const long threads = tiles * (TILE_BYTES / 4);
+    hipLaunchKernelGGL(q40_tile_kernel, dim3((unsigned)((threads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const uint8_t *)w, (const half_t *)s, K, N, (uint32_t *)tiled, tiles);
+    return launch_status();
+}
 
 extern "C" int smh_q40_dequant(const void *w, const void *s, void *out, long rows, smh_stream_t stream) {
     using namespace smh;

@@ -62,7 +62,10 @@ __device__ __forceinline__ void gemm_wait_dma(int stages) {
 // barrier no wave still reads the stage that is refilled next.
 __device__ __forceinline__ void gemm_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
 
-template <int TILES, bool RAGGED>
+// TILED: the weights are in the tiled layout (q40_matmul.hpp).  Wave w then moves and decodes piece w of a
+// tile (its two byte positions of its block, already paired by rows): one 16-byte LDS read instead of eight
+// dword reads, shifts instead of byte permutes, the scales already in operand order; rows past K hold zeros.
+template <int TILES, bool RAGGED, bool TILED>
 __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
 
@@ -96,7 +99,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     // ---- this wave's four DMA instructions per stage ----
     //  rows 8w .. 8w+7 of the nibbles; their scales (lanes 0..15); rows 32w .. 32w+31 of the A tile.
     //  Address = uniform base of the step (scalar arithmetic) + a lane offset fixed for the whole kernel.
-    const uint8_t *w_base = seg.w + (long)pair * 128;
+    const uint8_t *w_base = TILED ? seg.w + (long)pair * tiled_steps(p.K) * TILE_BYTES : seg.w + (long)pair * 128;
     const uint8_t *s_base = reinterpret_cast<const uint8_t *>(seg.s) + (long)pair * 8;
     const uint8_t *a_base = reinterpret_cast<const uint8_t *>(p.a);
     const int w_lrow = 8 * wave + (lane >> 3), w_lcol = 16 * (two_blocks ? (lane & 7) : (lane & 3));
@@ -111,7 +114,20 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     auto issue = [&](int step, int slot_) {
         uint8_t *st = lds + slot_ * GS_BYTES;
         const long k0 = (long)step * 32;
-        if (!RAGGED) {
+        if (TILED) {
+            const uint8_t *tile = w_base + (long)step * TILE_BYTES;
+            __builtin_amdgcn_global_load_lds((gptr_t)(tile + wave * 1024 + lane * 16), (lptr_t)(st + wave * 1024), 16, 0, 0);
+            if (lane < 16)
+                __builtin_amdgcn_global_load_lds((gptr_t)(tile + TILE_W_BYTES + (16 * wave + lane) * 4), (lptr_t)(st + GS_W + wave * 64), 4, 0, 0);
+            if (!RAGGED) {
+                __builtin_amdgcn_global_load_lds((gptr_t)(a_base + k0 * 2 + a_voff0), (lptr_t)(st + GS_W + GS_S + wave * 2048), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr_t)(a_base + k0 * 2 + a_voff1), (lptr_t)(st + GS_W + GS_S + wave * 2048 + 1024), 16, 0, 0);
+            } else {
+                const long ac = min(k0 + 8 * a_chunk, (long)p.K - 8) * 2;
+                __builtin_amdgcn_global_load_lds((gptr_t)(a_base + a_r0 + ac), (lptr_t)(st + GS_W + GS_S + wave * 2048), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr_t)(a_base + a_r1 + ac), (lptr_t)(st + GS_W + GS_S + wave * 2048 + 1024), 16, 0, 0);
+            }
+        } else if (!RAGGED) {
             __builtin_amdgcn_global_load_lds((gptr_t)(w_base + k0 * w_row + w_voff), (lptr_t)(st + wave * GS_WBLOCK), 16, 0, 0);
             if (lane < 16)
                 __builtin_amdgcn_global_load_lds((gptr_t)(s_base + k0 * s_row + s_voff), (lptr_t)(st + GS_W + wave * 64), 4, 0, 0);
@@ -152,6 +168,21 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
 
     // the eight dwords of this lane's column bytes and of their scales, for one step
     auto load_ws = [&](const uint8_t *st, uint32_t (&wv)[8], uint32_t (&sv)[8]) {
+        if (TILED) {
+            // wv[0..3] = (x, x2) of byte 2bp, (x, x2) of byte 2bp+1; sv[0..3] / sv[4..7] = the row pairs' scales of the
+            // block's first / second 64 columns
+            const u32x4 wq = *reinterpret_cast<const u32x4 *>(st + wave * 1024 + lane * 16);
+            const u32x4 sh = *reinterpret_cast<const u32x4 *>(st + GS_W + g * 64 + (2 * blk) * 16);
+            const u32x4 sl = *reinterpret_cast<const u32x4 *>(st + GS_W + g * 64 + (2 * blk + 1) * 16);
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                wv[r] = wq[r];
+                wv[4 + r] = 0;
+                sv[r] = sh[r];
+                sv[4 + r] = sl[r];
+            }
+            return;
+        }
 #pragma unroll
         for (int r = 0; r < 8; ++r) {
             wv[r] = *reinterpret_cast<const uint32_t *>(st + g * GS_WBLOCK + r * 128 + 64 * blk + 4 * c);
@@ -161,6 +192,23 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     // exact fp16 code * scale, as the four B operands (byte 2bp high / low, byte 2bp+1 high / low)
     auto decode = [&](const uint32_t (&wv)[8], const uint32_t (&sv)[8], bool dead, h8 (&b)[4]) {
         u32x4 v0h, v0l, v1h, v1l;
+        if (TILED) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t pr0 = j < 2 ? wv[j] : wv[j - 2] >> 8;           // rows (2j, 2j+1) of byte 2bp, codes + 8
+                const uint32_t pr1 = j < 2 ? wv[2 + j] : wv[j] >> 8;           // ... of byte 2bp+1
+                const h2 s_hi = as_h2(sv[j]), s_lo = as_h2(sv[4 + j]);
+                v0h[j] = as_u32(codes_high(pr0) * s_hi);
+                v0l[j] = as_u32(codes_low(pr0) * s_lo);
+                v1h[j] = as_u32(codes_high(pr1) * s_hi);
+                v1l[j] = as_u32(codes_low(pr1) * s_lo);
+            }
+            b[0] = __builtin_bit_cast(h8, v0h);
+            b[1] = __builtin_bit_cast(h8, v0l);
+            b[2] = __builtin_bit_cast(h8, v1h);
+            b[3] = __builtin_bit_cast(h8, v1l);
+            return;
+        }
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
             const uint32_t pr0 = __builtin_amdgcn_perm(wv[2 * j + 1], wv[2 * j], sel0) ^ 0x00880088u;
@@ -338,13 +386,15 @@ void gemm_fill_plan(MatmulParams &p) {
 
 typedef void (*gemm_kernel_t)(MatmulParams);
 
-int gemm_launch(const MatmulParams &p, hipStream_t stream) {
+template <bool TILED>
+static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
     // one instantiation per number of 16-row tiles (M <= 128) keeps the step free of branches; K % 32 != 0
     // takes the masked variant with all 8 tiles
-    static const gemm_kernel_t exact[9] = {nullptr, q40_gemm_kernel<2, false>, q40_gemm_kernel<2, false>, q40_gemm_kernel<3, false>,
-                                           q40_gemm_kernel<4, false>, q40_gemm_kernel<5, false>, q40_gemm_kernel<6, false>,
-                                           q40_gemm_kernel<7, false>, q40_gemm_kernel<8, false>};
-    static const gemm_kernel_t ragged = q40_gemm_kernel<8, true>;
+    static const gemm_kernel_t exact[9] = {nullptr, q40_gemm_kernel<2, false, TILED>, q40_gemm_kernel<2, false, TILED>,
+                                           q40_gemm_kernel<3, false, TILED>, q40_gemm_kernel<4, false, TILED>,
+                                           q40_gemm_kernel<5, false, TILED>, q40_gemm_kernel<6, false, TILED>,
+                                           q40_gemm_kernel<7, false, TILED>, q40_gemm_kernel<8, false, TILED>};
+    static const gemm_kernel_t ragged = q40_gemm_kernel<8, true, TILED>;
     // more than 64 KB of dynamic LDS has to be allowed once per kernel (the attribute is not stream work,
     // so a launch under graph capture is not affected)
     static const hipError_t lds_ok = [] {
@@ -360,6 +410,10 @@ int gemm_launch(const MatmulParams &p, hipStream_t stream) {
     dim3 grid((unsigned)((long)p.units_pad * p.mblocks * p.ksplit));
     hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), GEMM_LDS, stream, p);
     return launch_status();
+}
+
+int gemm_launch(const MatmulParams &p, hipStream_t stream) {
+    return p.tiled ? gemm_launch_layout<true>(p, stream) : gemm_launch_layout<false>(p, stream);
 }
 
 }  // namespace smh

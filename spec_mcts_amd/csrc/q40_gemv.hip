@@ -98,6 +98,25 @@ __device__ __forceinline__ void gemv_issue(const GemvLane &L, uint8_t *stage, in
     }
 }
 
+// Tiled weights: the step's tile is one contiguous run of TILE_BYTES; lane l moves bytes 16 l .. 16 l + 15 of
+// each 1 KB piece and dword l of the scales.  RAGGED only concerns the activations (rows of the tile past K
+// hold zeros): their columns are clamped to stay inside the row.
+template <bool RAGGED>
+__device__ __forceinline__ void gemv_issue_tiled(const GemvLane &L, uint8_t *stage, int step) {
+    const uint8_t *tile = L.w_base + (long)step * TILE_BYTES;
+#pragma unroll
+    for (int j = 0; j < 4; ++j)
+        __builtin_amdgcn_global_load_lds((gptr_t)(tile + j * 1024 + L.w_off), (lptr_t)(stage + j * 1024), 16, 0, 0);
+    __builtin_amdgcn_global_load_lds((gptr_t)(tile + TILE_W_BYTES + L.s_off), (lptr_t)(stage + STAGE_W_BYTES), 4, 0, 0);
+    const int k0 = step * 32;
+    if constexpr (!RAGGED) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(L.x_base + 2 * k0 + L.x_off), (lptr_t)(stage + STAGE_W_BYTES + STAGE_S_BYTES), 16, 0, 0);
+    } else {
+        const int col = min(k0 + 8 * (L.lane & 3), L.K - 8);
+        __builtin_amdgcn_global_load_lds((gptr_t)(L.x_base + (long)L.m_row + 2 * col), (lptr_t)(stage + STAGE_W_BYTES + STAGE_S_BYTES), 16, 0, 0);
+    }
+}
+
 // The two masks and the two fp16 magic numbers of the decoder, held in registers the compiler cannot
 // see through: (bits & mask) | magic then becomes ONE v_and_or_b32 (that instruction takes no
 // literal operands, so with visible constants the compiler emits an AND and an OR).
@@ -171,9 +190,50 @@ __device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K
 #undef SMH_GEMV_BYTE
 }
 
+// The same products from a tile (q40_matmul.hpp): the lane's 64 bytes are four linear 16-byte reads, the row
+// pairs come out of (x, x2, x >> 8, x2 >> 8) and the scales arrive in the register order of the A operands.
+// Same operands into the same MFMAs in the same order as gemv_consume: the results are bit-identical.
+template <bool RAGGED>
+__device__ __forceinline__ void gemv_consume_tiled(const uint8_t *stage, int k0, int K, int lane, const GemvConsts &C,
+                                                   f4 (&acc)[2][2][4], f4 (&corr)[4]) {
+    const int c = lane & 15, g = lane >> 4;
+    u32x4 wq[4];
+#pragma unroll
+    for (int q = 0; q < 4; ++q) wq[q] = *reinterpret_cast<const u32x4 *>(stage + q * 1024 + lane * 16);
+    h8 xv = *reinterpret_cast<const h8 *>(stage + STAGE_W_BYTES + STAGE_S_BYTES + c * 64 + 16 * g);
+    if constexpr (RAGGED) {
+        if (k0 + 8 * g >= K) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) xv[i] = (half_t)0.f;
+        }
+    }
+    h8 a[4];
+#pragma unroll
+    for (int grp = 0; grp < 4; ++grp) a[grp] = xv * *reinterpret_cast<const h8 *>(stage + STAGE_W_BYTES + g * 64 + grp * 16);
+    const h8 ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
+#pragma unroll
+    for (int bh = 0; bh < 4; ++bh) corr[bh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[bh], ones, corr[bh], 0, 0, 0);
+#pragma unroll
+    for (int q = 0; q < 4; ++q)
+#pragma unroll
+        for (int half = 0; half < 2; ++half) {
+            const int blk = q >> 1, B = 2 * (q & 1) + half;
+            const uint32_t pr[4] = {wq[q][2 * half], wq[q][2 * half + 1], wq[q][2 * half] >> 8, wq[q][2 * half + 1] >> 8};
+            u32x4 vh, vl;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                vh[j] = (pr[j] & C.mask_hi) | C.magic_hi;
+                vl[j] = (pr[j] & C.mask_lo) | C.magic_lo;
+            }
+            acc[blk][0][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * blk], __builtin_bit_cast(h8, vh), acc[blk][0][B], 0, 0, 0);
+            acc[blk][1][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * blk + 1], __builtin_bit_cast(h8, vl), acc[blk][1][B], 0, 0, 0);
+        }
+}
+
 // FINISH: the workgroup that completes a column unit also applies the operator that follows the linear
 // (matmul_finish.hpp); a separate instantiation, so that the plain kernel keeps its register budget
-template <int WAVES, bool FINISH>
+// TILED: the weights are in the tiled layout (smh_q40_tile)
+template <int WAVES, bool FINISH, bool TILED>
 __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // WAVES rings, then reused as red[WAVES][M][256]
     constexpr int THREADS = WAVES * 64;
@@ -215,6 +275,11 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     L.w_off = (uint32_t)((lane >> 3) * (seg.N / 2) + 16 * (two_blocks ? (lane & 7) : (lane & 3)));
     L.s_off = (uint32_t)((lane >> 1) * (seg.N / 32) + (two_blocks ? 4 * (lane & 1) : 0));
     L.x_off = (uint32_t)(L.m_row + 16 * (lane & 3));
+    if constexpr (TILED) {
+        L.w_base = seg.w + (long)pair * tiled_steps(p.K) * TILE_BYTES;     // this unit's tiles, step 0
+        L.w_off = (uint32_t)(16 * lane);
+        L.s_off = (uint32_t)(4 * lane);
+    }
     uint8_t *ring = lds + wave * RING_BYTES;
 
     GemvConsts C{0x00F000F0u, 0x000F000Fu, 0x54005400u, 0x64006400u};
@@ -238,8 +303,13 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     const int n_steps = first < step1 ? (step1 - first + WAVES - 1) / WAVES : 0;
     const int full_steps = p.K / 32;        // steps below this index have all their 32 rows
     auto issue = [&](uint8_t *stage, int step) {
-        if (step < full_steps) gemv_issue<false>(L, stage, step);
-        else gemv_issue<true>(L, stage, step);
+        if constexpr (TILED) {
+            if (step < full_steps) gemv_issue_tiled<false>(L, stage, step);
+            else gemv_issue_tiled<true>(L, stage, step);
+        } else {
+            if (step < full_steps) gemv_issue<false>(L, stage, step);
+            else gemv_issue<true>(L, stage, step);
+        }
     };
 #pragma unroll
     for (int i = 0; i < RING_STAGES; ++i)
@@ -253,7 +323,8 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         if (later >= 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
         else if (later == 1) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        gemv_consume<false>(ring + stage * STAGE_BYTES, 0, p.K, c, g, C, acc, corr);
+        if constexpr (TILED) gemv_consume_tiled<false>(ring + stage * STAGE_BYTES, 0, p.K, lane, C, acc, corr);
+        else gemv_consume<false>(ring + stage * STAGE_BYTES, 0, p.K, c, g, C, acc, corr);
         if (i + RING_STAGES < n_steps) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");        // this stage's LDS reads are done
             issue(ring + stage * STAGE_BYTES, first + (i + RING_STAGES) * WAVES);
@@ -262,7 +333,8 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     }
     if (n_full < n_steps) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        gemv_consume<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, c, g, C, acc, corr);
+        if constexpr (TILED) gemv_consume_tiled<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr);
+        else gemv_consume<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, c, g, C, acc, corr);
     }
     __syncthreads();                        // every wave is done with its ring: reuse LDS for the sums
 
@@ -359,10 +431,16 @@ int gemv_launch(const MatmulParams &p, hipStream_t stream) {
     size_t lds = (size_t)waves * RING_BYTES;                       // rings, reused for the [waves][M][256] sums
     const size_t red = (size_t)waves * p.M * GEMV_COLS * sizeof(float);
     if (red > lds) lds = red;
-    if (p.fin.mode != 0) hipLaunchKernelGGL((q40_gemv_kernel<4, true>), grid, dim3(256), lds, stream, p);
-    else if (waves == 2) hipLaunchKernelGGL((q40_gemv_kernel<2, false>), grid, dim3(128), lds, stream, p);
-    else if (waves == 8) hipLaunchKernelGGL((q40_gemv_kernel<8, false>), grid, dim3(512), lds, stream, p);
-    else hipLaunchKernelGGL((q40_gemv_kernel<4, false>), grid, dim3(256), lds, stream, p);
+    if (p.tiled) {
+        if (p.fin.mode != 0 || waves != 4) {
+            set_error("q40 gemv: tiled weights run with 4 waves and without a finishing operator");
+            return -1;
+        }
+        hipLaunchKernelGGL((q40_gemv_kernel<4, false, true>), grid, dim3(256), lds, stream, p);
+    } else if (p.fin.mode != 0) hipLaunchKernelGGL((q40_gemv_kernel<4, true, false>), grid, dim3(256), lds, stream, p);
+    else if (waves == 2) hipLaunchKernelGGL((q40_gemv_kernel<2, false, false>), grid, dim3(128), lds, stream, p);
+    else if (waves == 8) hipLaunchKernelGGL((q40_gemv_kernel<8, false, false>), grid, dim3(512), lds, stream, p);
+    else hipLaunchKernelGGL((q40_gemv_kernel<4, false, false>), grid, dim3(256), lds, stream, p);
     return launch_status();
 }
 

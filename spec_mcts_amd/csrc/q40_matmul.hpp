@@ -17,9 +17,30 @@
 
 namespace smh {
 
+// ---- tiled weight layout ---------------------------------------------------------------------------
+// The checkpoint layout (bytes [K, N/2], scales [K, N/64]) costs the matmul kernels one cache-line request
+// per k-row for the scales of a 256-column unit (8 bytes out of a 128-byte line) - as many requests as the
+// nibbles need - and byte permutes to bring 8 consecutive k of one column into a lane.  smh_q40_tile
+// rewrites a weight once into the order the kernels consume it:
+//   tiled[unit][step] = one contiguous tile of TILE_BYTES for 256 columns x 32 rows:
+//     TILE_W_BYTES of nibbles as [piece q = 0..3][lane = 16 g + c][4 dwords]: piece q = 2 blk + B / 2 holds,
+//       for byte column 64 blk + 4 c + B of the checkpoint row (B = 2 (q & 1) and 2 (q & 1) + 1) and rows
+//       r_i = 32 step + 8 g + i, the dwords x = bytes (r0, r4, r1, r5) and x2 = (r2, r6, r3, r7), every byte
+//       XORed with 0x88 (two's-complement nibble -> code + 8).  (x, x2, x >> 8, x2 >> 8) then carry the
+//       row pairs (0,1), (2,3), (4,5), (6,7) in bytes 0 and 2: the register layout of an MFMA B operand
+//       (lane = column, 8 consecutive k) is two shifts and eight AND-ORs away.
+//     TILE_S_BYTES of scales as [g][group = 0..3][i = 0..7] fp16: the 8 rows of k-octet g for each of the
+//       unit's four 64-column groups, i.e. the factors of one A operand in its register order.
+//   Columns past N and rows past K are filled with code 0 and scale 0 (they contribute exact zeros).
+constexpr int TILE_W_BYTES = 4096;
+constexpr int TILE_S_BYTES = 256;
+constexpr int TILE_BYTES = TILE_W_BYTES + TILE_S_BYTES;
+__host__ __device__ inline long tiled_units(int N) { return (N + 255) / 256; }
+__host__ __device__ inline long tiled_steps(int K) { return (K + 31) / 32; }
+
 struct MatmulSegment {
-    const uint8_t *w;    // packed nibbles [K, N/2]
-    const half_t *s;     // scales [K, N/64]
+    const uint8_t *w;    // packed nibbles [K, N/2]; tiled: the tiles of this weight
+    const half_t *s;     // scales [K, N/64]; tiled: unused
     int N;               // columns of this weight
     int col0;            // first output column
     int unit0;           // first work unit (column pair / column block) of this weight
@@ -39,6 +60,7 @@ struct MatmulParams {
     int ksplit, steps_per_slice;
     int epilogue, direct;
     int slab_half;           // slabs hold fp16 instead of fp32 (see slab_is_half)
+    int tiled;               // the segments' weights are in the tiled layout
     MatmulFinish fin;        // fin.mode == 0: leave the slabs to another launch
 };
 

@@ -99,6 +99,23 @@ class LinearQ4_0(torch.nn.Module):
         self.w = torch.zeros((int(in_features * out_features / group_size / 2), group_size), dtype=torch.int8, device="cpu")
         self.s = torch.zeros(int(in_features * out_features / group_size), dtype=DTYPE, device="cpu")
         self.shape = (out_features, in_features)
+        self._tiled = None
+        self._tiled_key = None
+
+    def operand(self, tiled: bool = True):
+        """What matmul_q40_partial takes for this weight: (w, s, N) in the checkpoint layout, or - the default
+        on the GPU - its tiled copy, made on first use (before any graph capture) and remade when `.w` / `.s`
+        are replaced; after changing them in place call `invalidate()`."""
+        if not tiled or not self.w.is_cuda:
+            return (self.w, self.s, self.shape[0])
+        key = (self.w.data_ptr(), self.s.data_ptr())
+        if self._tiled is None or self._tiled_key != key:
+            self._tiled = K.tile_q40(self.w, self.s, self.shape[1], self.shape[0])
+            self._tiled_key = key
+        return self._tiled
+
+    def invalidate(self):
+        self._tiled = None
 
     def forward(self, x, residual=None):
         shape = x.shape
@@ -263,6 +280,7 @@ class Transformer(nn.Module):
                                       # layer instead of 10; measured slower at B=10: the finisher's round trips are serial)
         self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
         self.persistent = False       # True: decode steps of few branches as one persistent kernel (needs fused); the operator kernels are faster
+        self.tiled_weights = True          # the fused path streams tiled copies of the weights (LinearQ4_0.operand)
         self.attn_single_launch = True     # up to 16 branches: prefix slices, suffix passes and the merge in one launch (slower above)
         self.attn_from_qkv = True          # up to 16 branches the attention takes the wq|wk|wv product itself, in one launch
         self.persistent_max_branches = 4   # with persistent = True: largest batch that uses the kernel (it takes up to 16)
@@ -327,8 +345,8 @@ class Transformer(nn.Module):
             att, ff = layer.attention, layer.feed_forward
             H, Hkv, D = att.n_local_heads, att.n_local_kv_heads, att.head_dim
             h, xn = K.partial_rmsnorm(pending, h, layer.attention_norm.weight, layer.attention_norm.eps)
-            qkv = K.matmul_q40_partial(xn, [(att.wq.w, att.wq.s, att.wq.shape[0]), (att.wk.w, att.wk.s, att.wk.shape[0]),
-                                            (att.wv.w, att.wv.s, att.wv.shape[0])])
+            tiled = self.tiled_weights
+            qkv = K.matmul_q40_partial(xn, [att.wq.operand(tiled), att.wk.operand(tiled), att.wv.operand(tiled)])
             if start_pos == 0:
                 xq = K.partial_reduce(qkv, 0, H * D).view(bsz, seqlen, H, D)
                 xk = K.partial_reduce(qkv, H * D, Hkv * D).view(bsz, seqlen, Hkv, D)
@@ -364,11 +382,11 @@ class Transformer(nn.Module):
                                              suffix_k=att.cache_k, suffix_v=att.cache_v, suffix_ks=att.cache_k_s,
                                              suffix_vs=att.cache_v_s, Smax=p.max_seq_len, lens=t_dev, lens_stride=0,
                                              cur_k=k, cur_v=v, single_launch=self.attn_single_launch and M <= 16).view(M, H * D)
-            po = K.matmul_q40_partial(o, [(att.wo.w, att.wo.s, att.wo.shape[0])])
+            po = K.matmul_q40_partial(o, [att.wo.operand(tiled)])
             h, xn = K.partial_rmsnorm(po, h, layer.ffn_norm.weight, layer.ffn_norm.eps)
-            gu = K.matmul_q40_partial(xn, [(ff.w1.w, ff.w1.s, ff.w1.shape[0]), (ff.w3.w, ff.w3.s, ff.w3.shape[0])])
+            gu = K.matmul_q40_partial(xn, [ff.w1.operand(tiled), ff.w3.operand(tiled)])
             act = K.partial_silu_mul(gu)
-            pending = K.matmul_q40_partial(act, [(ff.w2.w, ff.w2.s, ff.w2.shape[0])])
+            pending = K.matmul_q40_partial(act, [ff.w2.operand(tiled)])
         _, hn = K.partial_rmsnorm(pending, h, self.norm.weight, self.norm.eps, want_h=False)
         return self.output(hn.view(bsz, seqlen, p.dim)).to(DTYPE)
 

@@ -124,14 +124,50 @@ class PartialProduct:
         self.buf, self.ksplit, self.M, self.n_total = buf, ksplit, M, n_total
 
 
+class TiledQ40:
+    """A Q4_0 weight [K, N] rewritten into the matmul kernels' tile order (tile_q40)."""
+    __slots__ = ("buf", "K", "N")
+
+    def __init__(self, buf: torch.Tensor, K: int, N: int):
+        self.buf, self.K, self.N = buf, K, N
+
+
+def tile_q40(w: torch.Tensor, s: torch.Tensor, K: int, N: int) -> TiledQ40:
+    """Checkpoint layout (w int8 [K*N/128, 64], s fp16 [K*N/64]) -> tiled copy for matmul_q40_partial."""
+    lib = _lib.load()
+    _need_gpu(w, s)
+    assert w.is_contiguous() and s.is_contiguous() and w.dtype == torch.int8 and s.dtype == torch.float16
+    assert w.numel() == K * N // 2 and s.numel() == K * N // 64, "packed weight does not match [K, N]"
+    nbytes = int(lib.smh_q40_tiled_bytes(K, N))
+    buf = torch.empty(nbytes, dtype=torch.uint8, device=w.device)
+    check(lib.smh_q40_tile(w.data_ptr(), s.data_ptr(), K, N, buf.data_ptr(), nbytes, _stream()), "smh_q40_tile")
+    return TiledQ40(buf, K, N)
+
+
 def matmul_q40_partial(a: torch.Tensor, linears, out: Optional[torch.Tensor] = None) -> PartialProduct:
     """One launch for up to 3 Q4_0 weights that share the input a [M,K]; `linears` is a sequence of
-    (w, s, N).  Leaves the un-reduced product; the columns of the weights are concatenated."""
+    (w, s, N), or of TiledQ40 (same slabs, bit for bit).  Leaves the un-reduced product; the columns of the
+    weights are concatenated."""
     import ctypes
     lib = _lib.load()
     assert a.is_contiguous() and a.dtype == torch.float16 and a.dim() == 2 and a.data_ptr() % 16 == 0
     _need_gpu(a)
     M, Kd = a.shape
+    if isinstance(linears[0], TiledQ40):
+        assert all(isinstance(t, TiledQ40) and t.K == Kd for t in linears), "tiled and checkpoint-layout weights cannot share a launch"
+        ns = [t.N for t in linears]
+        ks = matmul_plan(M, Kd, ns)
+        n_total = sum(ns)
+        need = ks * M * n_total
+        if out is None:
+            out = torch.empty(need, dtype=torch.float32, device=a.device)
+        assert out.dtype == torch.float32 and out.numel() >= need and out.is_contiguous()
+        nseg = len(linears)
+        tp = (ctypes.c_void_p * nseg)(*[t.buf.data_ptr() for t in linears])
+        na = (ctypes.c_int * nseg)(*ns)
+        check(lib.smh_q40_matmul_partial_tiled(a.data_ptr(), M, Kd, Kd, nseg, tp, na, out.data_ptr(), out.numel() * 4, _stream()),
+              "smh_q40_matmul_partial_tiled")
+        return PartialProduct(out, ks, M, n_total)
     ns = [int(n) for (_, _, n) in linears]
     for (w, s, n) in linears:
         _need_gpu(w, s)

@@ -1,0 +1,79 @@
+"""Tiled weight layout (smh_q40_tile, smh_q40_matmul_partial_tiled): the tiles against an element-by-element
+numpy statement of the layout, and the products against the checkpoint-layout kernels (bit for bit) and the oracle."""
+import numpy as np
+import pytest
+import torch
+
+from oracle import q40_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+TILE_W, TILE_S = 4096, 256
+TILE = TILE_W + TILE_S
+
+
+def tiles_by_definition(w: np.ndarray, s: np.ndarray, K: int, N: int) -> np.ndarray:
+    """w uint8 [K, N/2], s uint16 [K, N/64] -> uint8 [units, steps, 4352].  Every checkpoint byte (k, byte column)
+    goes to: unit = column / 128, blk = column % 128 / 64, c = column % 64 / 4, B = column % 4, step = k / 32,
+    g = k % 32 / 8, i = k % 8; piece 2 blk + B / 2, lane 16 g + c, dword 2 (B % 2) + [i in 2,3,6,7], byte
+    (0, 2, 0, 2, 1, 3, 1, 3)[i]; value XOR 0x88.  Scale (k, group G): unit G / 4, offset 4096 + 16 (4 g + G % 4) + 2 i."""
+    units, steps = (N + 255) // 256, (K + 31) // 32
+    out = np.zeros((units, steps, TILE), dtype=np.uint8)
+    out[:, :, :TILE_W] = 0x88
+    k, col = np.meshgrid(np.arange(K), np.arange(N // 2), indexing="ij")
+    unit, blk, c, B = col // 128, col % 128 // 64, col % 64 // 4, col % 4
+    step, g, i = k // 32, k % 32 // 8, k % 8
+    dword = 2 * (B % 2) + np.isin(i, (2, 3, 6, 7)).astype(np.int64)
+    byte = np.array([0, 2, 0, 2, 1, 3, 1, 3])[i]
+    off = (2 * blk + B // 2) * 1024 + (16 * g + c) * 16 + dword * 4 + byte
+    out[unit, step, off] = w ^ 0x88
+    k, G = np.meshgrid(np.arange(K), np.arange(N // 64), indexing="ij")
+    off = TILE_W + 16 * (4 * (k % 32 // 8) + G % 4) + 2 * (k % 8)
+    s8 = s.view(np.uint8).reshape(K, N // 64, 2)
+    out[G // 4, k // 32, off] = s8[:, :, 0]
+    out[G // 4, k // 32, off + 1] = s8[:, :, 1]
+    return out
+
+
+def _weight(K, N, seed):
+    g = torch.Generator().manual_seed(seed)
+    v = (torch.randn((N, K), generator=g) * 0.02).half()
+    w, s, _ = O.quantize_weight(v)
+    return w, s
+
+
+@pytest.mark.parametrize("K,N", [(32, 128), (64, 256), (40, 384), (256, 640), (4096, 512)])
+def test_tiles_match_the_layout_definition(K, N):
+    from spec_mcts_amd import kernels as Kn
+    w, s = _weight(K, N, 900 + K + N)
+    t = Kn.tile_q40(w.cuda(), s.cuda(), K, N)
+    got = t.buf.cpu().numpy().reshape((N + 255) // 256, (K + 31) // 32, TILE)
+    want = tiles_by_definition(w.numpy().view(np.uint8).reshape(K, N // 2), s.numpy().view(np.uint16).reshape(K, N // 64), K, N)
+    assert np.array_equal(got, want)
+
+
+@pytest.mark.parametrize("M", [1, 3, 10, 16, 17, 100, 130])
+@pytest.mark.parametrize("K,ns", [(64, [128]), (40, [384]), (4096, [4096]), (1000, [256, 128, 128]), (4096, [1024, 256, 256]),
+                                  (11008, [4096]), (4096, [11008, 11008])])
+def test_tiled_products_equal_checkpoint_layout_products(M, K, ns):
+    """same operands into the same MFMAs in the same order: the slabs are bit-identical"""
+    from spec_mcts_amd import kernels as Kn
+    ws = [_weight(K, n, 910 + i + K) for i, n in enumerate(ns)]
+    a = (torch.randn((M, K), generator=torch.Generator().manual_seed(920 + M)) * 0.5).half().cuda()
+    lin = [(w.cuda(), s.cuda(), n) for (w, s), n in zip(ws, ns)]
+    tiled = [Kn.tile_q40(w, s, K, n) for (w, s, n) in lin]
+    p0 = Kn.matmul_q40_partial(a, lin)
+    p1 = Kn.matmul_q40_partial(a, tiled)
+    torch.cuda.synchronize()
+    assert p0.ksplit == p1.ksplit and p0.n_total == p1.n_total
+    n = p0.ksplit * M * p0.n_total
+    if M > 16:
+        n //= 2                  # above 16 rows the slabs hold fp16
+    assert torch.equal(p0.buf[:n].view(torch.int32), p1.buf[:n].view(torch.int32))
+    # and against the oracle's matmul (fp32 accumulation of the dequantised matrix)
+    got = Kn.partial_reduce(p1).cpu()
+    col = 0
+    for (w, s), nn in zip(ws, ns):
+        want = O.matmul_q40(a.cpu(), w, s, (K, nn))
+        assert torch.allclose(got[:, col:col + nn].float(), want.float(), rtol=1e-2, atol=2e-3)
+        col += nn
