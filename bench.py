@@ -31,9 +31,9 @@ PROMPT_LEN = 512
 BATCHES = (1, 10, 100)
 # HBM bytes per q40_gemv_kernel launch at M=1: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by a 1 GiB copy
 # (profiles/q40_gemv_m1_hbm_traffic.md has the commands and the factors: 2.0 for reads, 1.0 for writes)
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 32940444
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 27509321
 # the same for q40_gemm_kernel at M=100 (profiles/q40_gemm_m100_hbm_traffic.md): 43.95 MB read + 15.13 MB written
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 59075230
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 52357169
 
 
 def q40_bytes(M, N, K):
