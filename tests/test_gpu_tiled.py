@@ -77,3 +77,38 @@ def test_tiled_products_equal_checkpoint_layout_products(M, K, ns):
         want = O.matmul_q40(a.cpu(), w, s, (K, nn))
         assert torch.allclose(got[:, col:col + nn].float(), want.float(), rtol=1e-2, atol=2e-3)
         col += nn
+
+
+def test_model_logits_do_not_depend_on_the_weight_layout():
+    """the fused forward on tiled copies against the same forward on the checkpoint tensors: equal bit for bit,
+    at prefill (GEMM), at decode (GEMV) and again after a weight has been replaced"""
+    from spec_mcts_amd import ModelArgs
+    from spec_mcts_amd.load_q40 import load_q40
+    cfg = dict(dim=512, n_layers=2, n_heads=4, n_kv_heads=2, vocab_size=384, multiple_of=128, max_batch_size=4,
+               max_seq_len=16, max_prompt_seq_len=48)
+    oargs = O.OracleArgs(**cfg)
+    sd = O.random_q40_state_dict(oargs, seed=941)
+    model = load_q40(dict(sd), ModelArgs(**cfg), device="cuda:0")
+    prompt = torch.randint(0, cfg["vocab_size"], (1, 37), generator=torch.Generator().manual_seed(942)).cuda()
+    tok = torch.randint(0, cfg["vocab_size"], (3, 1), generator=torch.Generator().manual_seed(943)).cuda()
+
+    def run():
+        model.resetSeq()
+        return [model(prompt, 0).clone(), model(tok, 37).clone(), model(tok, 38).clone()]
+
+    assert model.tiled_weights
+    a = run()
+    model.tiled_weights = False
+    b = run()
+    for x, y in zip(a, b):
+        assert torch.equal(x, y)
+    # a replaced weight is re-tiled on the next use
+    lin = model.layers[1].feed_forward.w2
+    lin.w = lin.w.roll(1, 0).contiguous()
+    lin.s = lin.s.roll(3).contiguous()
+    c = run()
+    model.tiled_weights = True
+    d = run()
+    assert not torch.equal(c[1], b[1])
+    for x, y in zip(c, d):
+        assert torch.equal(x, y)
