@@ -125,6 +125,43 @@ def matmul_roofline(torch, model, M, iters):
             "tflops": flops / (ms * 1e-3) / 1e12}
 
 
+def attention_roofline(torch, iters=5, copies=3):
+    """The shared-prefix decode attention alone on the reference's tree-attention shape: 64 branches, 32 heads,
+    head_dim 128, one 1024-token fp16 prefix shared by all branches, ragged suffixes of 0..256 rows per branch held
+    as the model stores them (Q4_0 rows + scales), seed 2.  Algorithmic bytes: the prefix once, every valid suffix
+    row once, q and out.  `copies` distinct caches alternate so that the suffix does not stay in the Infinity Cache."""
+    from spec_mcts_amd import kernels as K
+    dev = torch.device("cuda:0")
+    B, H, D, P, S = 64, 32, 128, 1024, 256
+    g = torch.Generator().manual_seed(2)
+    lens = torch.randint(0, S + 1, (B,), generator=g, dtype=torch.int32)
+    q = torch.randn((B, H, D), generator=g).half().to(dev)
+    sets = []
+    for _ in range(copies):
+        pk, pv = torch.randn((P, H, D), device=dev).half(), torch.randn((P, H, D), device=dev).half()
+        sk = torch.randint(-128, 128, (B, S, H, 64), device=dev, dtype=torch.int16).to(torch.int8)
+        sv = torch.randint(-128, 128, (B, S, H, 64), device=dev, dtype=torch.int16).to(torch.int8)
+        sks, svs = (torch.rand((B, S, H, 2), device=dev) * 0.1).half(), (torch.rand((B, S, H, 2), device=dev) * 0.1).half()
+        sets.append((pk, pv, sk, sv, sks, svs))
+    lens_d = lens.to(dev)
+
+    def run():
+        for pk, pv, sk, sv, sks, svs in sets:
+            K.shared_prefix_attn(q, pk, pv, P, suffix_k=sk, suffix_v=sv, suffix_ks=sks, suffix_vs=svs, Smax=S, lens=lens_d, lens_stride=1)
+
+    run()
+    torch.cuda.synchronize()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph):
+        run()
+    for _ in range(5):
+        graph.replay()
+    ms = time_region(torch, graph.replay, iters) / copies
+    rows = int(lens.sum())
+    nbytes = 2 * P * H * D * 2 + rows * H * 2 * (64 + 4) + 2 * B * H * D * 2
+    return {"us": ms * 1e3, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9, "suffix_rows": rows}
+
+
 def cpu_baseline(torch, args_kw, budget_s=20.0):
     """The reference's CPU PyTorch path on ONE transformer layer (dequantise + F.linear for each of
     the 7 linears, explicit softmax attention over prompt + suffix), scaled by n_layers, plus the
@@ -261,6 +298,12 @@ def main():
              "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(rf100["tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
              "hbm_gbs": round(rf100["gbs"], 1), "avg_launch_us": round(rf100["avg_us"], 3), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH},
         ]
+        att = attention_roofline(torch)
+        result["rooflines_other"].append(
+            {"kernel": "attn_prefix_kernel + attn_suffix_kernel: 64 branches x 32 heads, shared 1024-token fp16 prefix, ragged Q4_0 "
+                       "suffixes of 0..256 rows (the two launches of one call)",
+             "bound": "hbm", "achieved": round(att["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+             "frac": round(att["gbs"] / HBM_PEAK_GBS, 4), "avg_call_us": round(att["us"], 2), "bytes_per_call": att["bytes"]})
         if 1 in by_batch and by_batch[1]["path"].startswith("persistent"):
             # the whole step is one launch: every weight, the prefix KV and the suffix KV once
             b1 = lin_bytes + prefix_bytes + t_mid * a.layers * 2 * 32 * 68

@@ -286,6 +286,148 @@ __global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
     attn_prefix_body<FUSED, false, ATT_TW_MAX>(p, blockIdx.x, blockIdx.y);
 }
 
+// ---- causal attention of a prefill on the matrix cores ----------------------------------------------------------
+// grid (ceil(S / 64), H): a workgroup owns 64 consecutive query positions of one head, wave w the 16 of them from
+// 64 qb + 16 w.  It walks the key tiles (PF_TW rows, staged once per workgroup: K row-major, V transposed, as in
+// attn_prefix_body) from position 0 to its diagonal with an online softmax: per tile S^T = K . Q^T and
+// O^T += V^T . P^T on the matrix cores (the B operand of the second product is the accumulator layout of the first),
+// running maximum / sum / O^T in registers, so nothing but the fp16 result is written.  The next tile's K / V rows
+// are in flight (registers) while the current one is multiplied.  q [S,H,128], k, v [S,Hkv,128], out [S,H,128].
+constexpr int PF_TW = 64;
+struct PrefillParams {
+    const half_t *q, *k, *v;
+    half_t *out;
+    int S, H, Hkv, n_rep;
+    float scale_log2;
+};
+
+__global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillParams p) {
+    __shared__ __attribute__((aligned(16))) half_t ks[PF_TW][ATT_KPITCH];
+    __shared__ __attribute__((aligned(16))) half_t vt[ATT_D][PF_TW + 8];
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6, lane = tid & 63, c = lane & 15, g = lane >> 4;
+    const int qb = gridDim.x - 1 - blockIdx.x, h = blockIdx.y, hk = h / p.n_rep;     // longest walks are dispatched first
+    const int q_lo = 64 * qb + 16 * wave;                  // this wave's first query position
+    const int my_q = q_lo + c;                             // this lane's query (column c of the tiles)
+    const int last_key = min(64 * qb + 63, p.S - 1);       // the workgroup's diagonal
+    const int n_tiles = last_key / PF_TW + 1;
+
+    // B operand of S^T = K . Q^T: dims 32 k4 + 8g .. +7 of query row c
+    h8 qbop[4];
+    {
+        const half_t *qp = p.q + ((long)min(my_q, p.S - 1) * p.H + h) * ATT_D + 8 * g;
+#pragma unroll
+        for (int k4 = 0; k4 < 4; ++k4) qbop[k4] = *reinterpret_cast<const h8 *>(qp + 32 * k4);
+    }
+    constexpr int PER = PF_TW * 16 / 256;                  // 16-byte pieces of K (and of V) per thread and tile
+    u32x4 kreg[PER], vreg[PER];
+    auto tile_load = [&](int kt) {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = tid + 256 * i, t = idx >> 4, ch = idx & 15;
+            const int row = kt * PF_TW + t;
+            kreg[i] = u32x4{0, 0, 0, 0}; vreg[i] = u32x4{0, 0, 0, 0};
+            if (row < p.S) {
+                const long off = ((long)row * p.Hkv + hk) * ATT_D + ch * 8;
+                kreg[i] = *reinterpret_cast<const u32x4 *>(p.k + off);
+                vreg[i] = *reinterpret_cast<const u32x4 *>(p.v + off);
+            }
+        }
+    };
+    auto tile_store = [&]() {
+#pragma unroll
+        for (int i = 0; i < PER; ++i) {
+            const int idx = tid + 256 * i, t = idx >> 4, ch = idx & 15;
+            *reinterpret_cast<u32x4 *>(&ks[t][ch * 8]) = kreg[i];
+            const int pos = vt_pos(t);
+            const h8 vh = __builtin_bit_cast(h8, vreg[i]);
+#pragma unroll
+            for (int j = 0; j < 8; ++j) vt[ch * 8 + j][pos] = vh[j];
+        }
+    };
+
+    float m_run = -INFINITY, l_run = 0.f;                  // of query c (the same in the four lane groups)
+    f4 ot[8];                                              // O^T: element r of ot[dt] is dim 16 dt + 4g + r of query c
+#pragma unroll
+    for (int dt = 0; dt < 8; ++dt) ot[dt] = f4{0.f, 0.f, 0.f, 0.f};
+
+    tile_load(0);
+    for (int kt = 0; kt < n_tiles; ++kt) {
+        __syncthreads();                                   // everyone is done with the previous tile
+        tile_store();
+        __syncthreads();
+        if (kt + 1 < n_tiles) tile_load(kt + 1);
+        const int k_lo = kt * PF_TW;
+        if (k_lo > q_lo + 15) continue;                    // every key of this tile lies after this wave's queries
+        // 16-row sub-tiles that hold a key <= the wave's last query
+        const int subs = min(PF_TW / 16, (q_lo + 15 - k_lo) / 16 + 1);
+        f4 st[PF_TW / 16];
+        float mx = -INFINITY;
+#pragma unroll
+        for (int j = 0; j < PF_TW / 16; ++j) {
+            st[j] = f4{0.f, 0.f, 0.f, 0.f};
+            if (j < subs) {
+#pragma unroll
+                for (int k4 = 0; k4 < 4; ++k4) {
+                    h8 ka = *reinterpret_cast<const h8 *>(&ks[16 * j + c][32 * k4 + 8 * g]);
+                    st[j] = __builtin_amdgcn_mfma_f32_16x16x32_f16(ka, qbop[k4], st[j], 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const int key = k_lo + 16 * j + 4 * g + r;
+                const float sv = (j < subs && key <= my_q && key < p.S) ? st[j][r] * p.scale_log2 : -INFINITY;
+                st[j][r] = sv;
+                mx = fmaxf(mx, sv);
+            }
+        }
+        mx = fmaxf(mx, __shfl_xor(mx, 16, 64));
+        mx = fmaxf(mx, __shfl_xor(mx, 32, 64));
+        const float m_new = fmaxf(m_run, mx);              // finite from the first tile on: key 0 precedes every query
+        const float alpha = exp2f(m_run - m_new);          // exp2(-inf) = 0 on the first tile
+        float sum = 0.f;
+#pragma unroll
+        for (int j = 0; j < PF_TW / 16; ++j)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) {
+                const float e = exp2f(st[j][r] - m_new);
+                st[j][r] = e;
+                sum += e;
+            }
+        sum += __shfl_xor(sum, 16, 64);
+        sum += __shfl_xor(sum, 32, 64);
+        l_run = l_run * alpha + sum;
+        m_run = m_new;
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) ot[dt] *= alpha;
+#pragma unroll
+        for (int jj = 0; jj < PF_TW / 32; ++jj) {
+            if (2 * jj < subs) {
+                h8 pb;
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    pb[r] = (half_t)st[2 * jj][r];
+                    pb[4 + r] = (half_t)st[2 * jj + 1][r];
+                }
+#pragma unroll
+                for (int dt = 0; dt < 8; ++dt) {
+                    h8 va = *reinterpret_cast<const h8 *>(&vt[16 * dt + c][32 * jj + 8 * g]);
+                    ot[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(va, pb, ot[dt], 0, 0, 0);
+                }
+            }
+        }
+    }
+    if (my_q < p.S) {
+        const float inv = l_run > 0.f ? 1.0f / l_run : 0.f;
+        half_t *op = p.out + ((long)my_q * p.H + h) * ATT_D;
+#pragma unroll
+        for (int dt = 0; dt < 8; ++dt) {
+            const h4 o = {(half_t)(ot[dt][0] * inv), (half_t)(ot[dt][1] * inv), (half_t)(ot[dt][2] * inv), (half_t)(ot[dt][3] * inv)};
+            *reinterpret_cast<h4 *>(op + 16 * dt + 4 * g) = o;
+        }
+    }
+}
+
 // One wave per (branch b, kv head hk).  PARTIAL: the pass over the suffix and the new token leaves an un-normalised
 // partial (split index p.splits) for the workgroup that merges, instead of folding in the prefix partials itself.
 template <bool FUSED, bool PARTIAL>
@@ -728,15 +870,10 @@ extern "C" int smh_prefill_attn(const void *q, const void *k, const void *v, voi
     SMH_REQUIRE(S >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0, "smh_prefill_attn: S=%d H=%d Hkv=%d", S, H, Hkv);
     if (S == 0) return 0;
     SMH_REQUIRE(q && k && v && out, "smh_prefill_attn: null pointer");
-    AttnParams p = {};
-    p.q = (const half_t *)q; p.out = (half_t *)out;
-    p.suffix_k = k; p.suffix_v = v;
-    p.suffix_batch_stride_rows = 0;
-    p.B = S; p.H = H; p.Hkv = Hkv; p.n_rep = H / Hkv; p.Bq = S * p.n_rep;
-    p.P = 0; p.splits = 0; p.tw = 32;
-    p.suffix_format = SMH_KV_FP16; p.causal = 1;
+    PrefillParams p;
+    p.q = (const half_t *)q; p.k = (const half_t *)k; p.v = (const half_t *)v; p.out = (half_t *)out;
+    p.S = S; p.H = H; p.Hkv = Hkv; p.n_rep = H / Hkv;
     p.scale_log2 = LOG2E / sqrtf((float)D);
-    long items = (long)S * Hkv;
-    hipLaunchKernelGGL(attn_suffix_kernel<false>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL(attn_prefill_kernel, dim3((unsigned)((S + 63) / 64), (unsigned)H), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
 }

@@ -116,7 +116,7 @@ def test_special_cases():
     assert torch.allclose(full.float(), moved.float(), atol=2e-3, rtol=1e-2)
 
 
-@pytest.mark.parametrize("S,H,Hkv", [(1, 2, 2), (19, 4, 2), (512, 32, 32)])
+@pytest.mark.parametrize("S,H,Hkv", [(1, 2, 2), (19, 4, 2), (63, 2, 1), (64, 2, 2), (65, 4, 1), (200, 8, 2), (512, 32, 32), (1100, 8, 1)])
 def test_prefill_causal(S, H, Hkv):
     from spec_mcts_amd import kernels as K
     g = _g(40 + S)
@@ -125,6 +125,28 @@ def test_prefill_causal(S, H, Hkv):
     v = torch.randn((S, Hkv, 128), generator=g).to(torch.float16)
     got = K.prefill_attn(q.cuda(), k.cuda(), v.cuda())
     _check(got, O.causal_attention(q, k, v))
+
+
+def test_prefill_causal_special_cases():
+    """what the mathematics fixes: position 0 sees only itself (out = v[0]); equal keys give the running mean of v;
+    one key that dominates every score makes every later position return that key's v"""
+    from spec_mcts_amd import kernels as K
+    S, H = 150, 2
+    g = _g(77)
+    q = torch.randn((S, H, 128), generator=g).half()
+    k = torch.randn((S, H, 128), generator=g).half()
+    v = torch.randn((S, H, 128), generator=g).half()
+    out = K.prefill_attn(q.cuda(), k.cuda(), v.cuda()).cpu()
+    assert torch.equal(out[0], v[0])
+    k_same = k[:1].expand(S, H, 128).contiguous()
+    out = K.prefill_attn(q.cuda(), k_same.cuda(), v.cuda()).cpu().float()
+    mean = v.float().cumsum(0) / torch.arange(1, S + 1).view(S, 1, 1)
+    assert torch.allclose(out, mean, atol=2e-3, rtol=1e-2)
+    k_dom = (torch.randn((S, H, 128), generator=g) * 0.01).half()
+    k_dom[70] = q[100] * 4                       # huge score for every query that resembles q[100]; use q = q[100] everywhere
+    q_all = q[100:101].expand(S, H, 128).contiguous()
+    out = K.prefill_attn(q_all.cuda(), k_dom.cuda(), v.cuda()).cpu().float()
+    assert torch.allclose(out[70:], v[70:71].float().expand(S - 70, H, 128), atol=2e-3, rtol=1e-2)
 
 
 def test_flash_attn_and_page_flash_attn_drop_ins():
