@@ -352,8 +352,10 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
                 for (int r = 0; r < 4; ++r) {
                     const int m = 4 * g + r;
                     const float off = h ? 1032.f : 72.f;
-                    if (m < p.M)
-                        red[(wave * p.M + m) * GEMV_COLS + 128 * d + 64 * h + 4 * c + b] = acc[d][h][b][r] - off * corr[2 * d + h][r];
+                    if (r < p.M) {                  // uniform: with fewer than 4 rows whole store instructions drop out
+                        if (m < p.M)
+                            red[(wave * p.M + m) * GEMV_COLS + 128 * d + 64 * h + 4 * c + b] = acc[d][h][b][r] - off * corr[2 * d + h][r];
+                    }
                 }
     __syncthreads();
 
