@@ -112,6 +112,13 @@ size_t smh_q40_tiled_bytes(int K, int N);
 int smh_q40_tile(const void *w, const void *s, int K, int N, void *tiled, size_t tiled_bytes, smh_stream_t stream);
 int smh_q40_matmul_partial_tiled(const void *a, int M, int K, long lda, int nseg, const void *const *tiled,
                                  const int *n, void *partial, size_t partial_bytes, smh_stream_t stream);
+/* smh_q40_matmul_partial_tiled_silu: w2(F.silu(w1 x) * w3 x) of FeedForward.forward (hf_model_q40_kv_shared.py:434) without
+ * the launch between the two matmuls, for M <= 2 rows: the activations of the product are not read from memory but made by
+ * every workgroup for its own K-slice from the gate|up slabs (columns 0..K-1 gate, K..2K-1 up, as smh_partial_silu_mul takes
+ * them), with the same roundings; the slabs it leaves equal those of smh_partial_silu_mul + smh_q40_matmul_partial_tiled. */
+int smh_q40_matmul_partial_tiled_silu(const void *gate_up_partial, int gate_up_ksplit, int M, int K, int nseg,
+                                      const void *const *tiled, const int *n, void *partial, size_t partial_bytes,
+                                      smh_stream_t stream);
 int smh_partial_reduce(const void *partial, int ksplit, int M, int n_total, int col0, int N, void *c,
                        long ldc, int epilogue, const void *residual, long ldr, smh_stream_t stream);
 int smh_partial_rmsnorm(const void *partial, int ksplit, int M, int N, const void *h_in,

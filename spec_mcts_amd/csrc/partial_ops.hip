@@ -12,72 +12,9 @@
 // for another workgroup.
 #include "q40_matmul.hpp"
 #include "rope_kv.hpp"
+#include "slab_sum.hpp"
 
 namespace smh {
-
-// Element `idx` of every slab, added in slice order in fp32.  `half`: the slabs hold fp16 (slab_is_half).
-__device__ __forceinline__ float slab_sum(const void *partial, long idx, long slab_stride, int ksplit, bool half) {
-    float v[SMH_MAX_KSPLIT];
-    if (half) {
-        const half_t *p = reinterpret_cast<const half_t *>(partial) + idx;
-#pragma unroll
-        for (int s = 0; s < SMH_MAX_KSPLIT; ++s) v[s] = (s < ksplit) ? (float)p[s * slab_stride] : 0.f;
-    } else {
-        const float *p = reinterpret_cast<const float *>(partial) + idx;
-#pragma unroll
-        for (int s = 0; s < SMH_MAX_KSPLIT; ++s) v[s] = (s < ksplit) ? p[s * slab_stride] : 0.f;
-    }
-    float tot = 0.f;
-#pragma unroll
-    for (int s = 0; s < SMH_MAX_KSPLIT; ++s) tot += v[s];
-    return tot;
-}
-// Two consecutive elements (idx % 2 == 0).
-__device__ __forceinline__ f2 slab_sum2(const void *partial, long idx, long slab_stride, int ksplit, bool half) {
-    f2 tot = {0.f, 0.f};
-    if (half) {
-        const half_t *p = reinterpret_cast<const half_t *>(partial) + idx;
-        h2 v[SMH_MAX_KSPLIT];
-#pragma unroll
-        for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
-            v[s] = (s < ksplit) ? *reinterpret_cast<const h2 *>(p + s * slab_stride) : h2{(half_t)0.f, (half_t)0.f};
-#pragma unroll
-        for (int s = 0; s < SMH_MAX_KSPLIT; ++s) { tot[0] += (float)v[s][0]; tot[1] += (float)v[s][1]; }
-    } else {
-        const float *p = reinterpret_cast<const float *>(partial) + idx;
-        f2 v[SMH_MAX_KSPLIT];
-#pragma unroll
-        for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
-            v[s] = (s < ksplit) ? *reinterpret_cast<const f2 *>(p + s * slab_stride) : f2{0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < SMH_MAX_KSPLIT; ++s) tot += v[s];
-    }
-    return tot;
-}
-// Four consecutive elements (idx % 4 == 0).
-__device__ __forceinline__ f4 slab_sum4(const void *partial, long idx, long slab_stride, int ksplit, bool half) {
-    f4 tot = {0.f, 0.f, 0.f, 0.f};
-    if (half) {
-        const half_t *p = reinterpret_cast<const half_t *>(partial) + idx;
-        h4 v[SMH_MAX_KSPLIT];
-#pragma unroll
-        for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
-            v[s] = (s < ksplit) ? *reinterpret_cast<const h4 *>(p + s * slab_stride) : h4{(half_t)0.f, (half_t)0.f, (half_t)0.f, (half_t)0.f};
-#pragma unroll
-        for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
-#pragma unroll
-            for (int j = 0; j < 4; ++j) tot[j] += (float)v[s][j];
-    } else {
-        const float *p = reinterpret_cast<const float *>(partial) + idx;
-        f4 v[SMH_MAX_KSPLIT];
-#pragma unroll
-        for (int s = 0; s < SMH_MAX_KSPLIT; ++s)
-            v[s] = (s < ksplit) ? *reinterpret_cast<const f4 *>(p + s * slab_stride) : f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-        for (int s = 0; s < SMH_MAX_KSPLIT; ++s) tot += v[s];
-    }
-    return tot;
-}
 
 // ---- plain reduce (+ residual) ------------------------------------------------------------------
 __global__ __launch_bounds__(256) void partial_reduce_kernel(const void *__restrict__ partial, int ksplit, int M, int n_total,
@@ -314,6 +251,30 @@ extern "C" int smh_q40_matmul_partial_tiled(const void *a, int M, int K, long ld
     p.direct = 0;
     p.tiled = 1;
     return M <= SMH_GEMV_MAX_M ? gemv_launch(p, (hipStream_t)stream) : gemm_launch(p, (hipStream_t)stream);
+}
+
+extern "C" int smh_q40_matmul_partial_tiled_silu(const void *gate_up_partial, int gate_up_ksplit, int M, int K, int nseg,
+                                                 const void *const *tiled, const int *n, void *partial, size_t partial_bytes,
+                                                 smh_stream_t stream) {
+    MatmulParams p;
+    int st = fill_params(p, nullptr, M, K, (K + 7) / 8 * 8, nseg, tiled, nullptr, n, "smh_q40_matmul_partial_tiled_silu");
+    if (st) return st;
+    if (M == 0) return 0;
+    SMH_REQUIRE(M <= SMH_SILU_IN_MAX_M, "smh_q40_matmul_partial_tiled_silu: M=%d (at most %d rows; use smh_partial_silu_mul above)", M, SMH_SILU_IN_MAX_M);
+    SMH_REQUIRE(K % 32 == 0, "smh_q40_matmul_partial_tiled_silu: K=%d must be a multiple of 32", K);
+    SMH_REQUIRE(gate_up_partial && tiled && partial, "smh_q40_matmul_partial_tiled_silu: null pointer");
+    SMH_REQUIRE(gate_up_ksplit >= 1 && gate_up_ksplit <= SMH_MAX_KSPLIT, "smh_q40_matmul_partial_tiled_silu: ksplit=%d", gate_up_ksplit);
+    for (int i = 0; i < nseg; ++i)
+        SMH_REQUIRE(tiled[i] && ((uintptr_t)tiled[i] & 127) == 0, "smh_q40_matmul_partial_tiled_silu: weight %d is null or not 128-byte aligned", i);
+    size_t need = (size_t)p.ksplit * M * p.n_total * sizeof(float);
+    SMH_REQUIRE(partial_bytes >= need, "smh_q40_matmul_partial_tiled_silu: partial buffer %zu < %zu bytes", partial_bytes, need);
+    SMH_REQUIRE(partial != gate_up_partial, "smh_q40_matmul_partial_tiled_silu: the product cannot overwrite the slabs it is made from");
+    p.partial = (float *)partial;
+    p.direct = 0;
+    p.tiled = 1;
+    p.gu_partial = (const float *)gate_up_partial;
+    p.gu_ksplit = gate_up_ksplit;
+    return gemv_launch(p, (hipStream_t)stream);
 }
 
 extern "C" int smh_q40_matmul_fused(const void *a, int M, int K, long lda, int nseg, const void *const *w,

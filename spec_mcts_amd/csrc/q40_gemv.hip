@@ -28,6 +28,7 @@
 #include <stdlib.h>
 
 #include "q40_matmul.hpp"
+#include "slab_sum.hpp"
 
 namespace smh {
 
@@ -101,13 +102,14 @@ __device__ __forceinline__ void gemv_issue(const GemvLane &L, uint8_t *stage, in
 // Tiled weights: the step's tile is one contiguous run of TILE_BYTES; lane l moves bytes 16 l .. 16 l + 15 of
 // each 1 KB piece and dword l of the scales.  RAGGED only concerns the activations (rows of the tile past K
 // hold zeros): their columns are clamped to stay inside the row.
-template <bool RAGGED>
+template <bool RAGGED, bool WITH_A>
 __device__ __forceinline__ void gemv_issue_tiled(const GemvLane &L, uint8_t *stage, int step) {
     const uint8_t *tile = L.w_base + (long)step * TILE_BYTES;
 #pragma unroll
     for (int j = 0; j < 4; ++j)
         __builtin_amdgcn_global_load_lds((gptr_t)(tile + j * 1024 + L.w_off), (lptr_t)(stage + j * 1024), 16, 0, 0);
     __builtin_amdgcn_global_load_lds((gptr_t)(tile + TILE_W_BYTES + L.s_off), (lptr_t)(stage + STAGE_W_BYTES), 4, 0, 0);
+    if constexpr (!WITH_A) return;
     const int k0 = step * 32;
     if constexpr (!RAGGED) {
         __builtin_amdgcn_global_load_lds((gptr_t)(L.x_base + 2 * k0 + L.x_off), (lptr_t)(stage + STAGE_W_BYTES + STAGE_S_BYTES), 16, 0, 0);
@@ -193,14 +195,15 @@ __device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K
 // The same products from a tile (q40_matmul.hpp): the lane's 64 bytes are four linear 16-byte reads, the row
 // pairs come out of (x, x2, x >> 8, x2 >> 8) and the scales arrive in the register order of the A operands.
 // Same operands into the same MFMAs in the same order as gemv_consume: the results are bit-identical.
+// `xrow`: the 8 activations k0 + 8g .. of this lane's batch row when they do not come from the stage (nullptr otherwise)
 template <bool RAGGED>
 __device__ __forceinline__ void gemv_consume_tiled(const uint8_t *stage, int k0, int K, int lane, const GemvConsts &C,
-                                                   f4 (&acc)[2][2][4], f4 (&corr)[4]) {
+                                                   f4 (&acc)[2][2][4], f4 (&corr)[4], const half_t *xrow = nullptr) {
     const int c = lane & 15, g = lane >> 4;
     u32x4 wq[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) wq[q] = *reinterpret_cast<const u32x4 *>(stage + q * 1024 + lane * 16);
-    h8 xv = *reinterpret_cast<const h8 *>(stage + STAGE_W_BYTES + STAGE_S_BYTES + c * 64 + 16 * g);
+    h8 xv = xrow ? *reinterpret_cast<const h8 *>(xrow) : *reinterpret_cast<const h8 *>(stage + STAGE_W_BYTES + STAGE_S_BYTES + c * 64 + 16 * g);
     if constexpr (RAGGED) {
         if (k0 + 8 * g >= K) {
 #pragma unroll
@@ -232,11 +235,15 @@ __device__ __forceinline__ void gemv_consume_tiled(const uint8_t *stage, int k0,
 
 // FINISH: the workgroup that completes a column unit also applies the operator that follows the linear
 // (matmul_finish.hpp); a separate instantiation, so that the plain kernel keeps its register budget
-// TILED: the weights are in the tiled layout (smh_q40_tile)
-template <int WAVES, bool FINISH, bool TILED>
+// LAYOUT 0: checkpoint layout; 1: tiled weights (smh_q40_tile); 2: tiled weights and activations made from the
+// gate|up slabs by the workgroup itself (p.gu_partial): SiLU(gate) * up needs no launch of its own
+template <int WAVES, bool FINISH, int LAYOUT>
 __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // WAVES rings, then reused as red[WAVES][M][256]
     constexpr int THREADS = WAVES * 64;
+    constexpr bool TILED = LAYOUT != 0;
+    constexpr bool SILU_IN = LAYOUT == 2;
+    constexpr int PER_STAGE = SILU_IN ? 5 : 6;                      // vector-memory instructions per stage
 
     // Workgroups are dealt round-robin to the 8 XCDs (8 L2s).  Neighbouring column units share the 128-byte
     // lines of the scale rows, so each XCD takes a CONTIGUOUS run of units: a scale line is then fetched
@@ -304,26 +311,71 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     const int full_steps = p.K / 32;        // steps below this index have all their 32 rows
     auto issue = [&](uint8_t *stage, int step) {
         if constexpr (TILED) {
-            if (step < full_steps) gemv_issue_tiled<false>(L, stage, step);
-            else gemv_issue_tiled<true>(L, stage, step);
+            if (step < full_steps) gemv_issue_tiled<false, !SILU_IN>(L, stage, step);
+            else gemv_issue_tiled<true, !SILU_IN>(L, stage, step);
         } else {
             if (step < full_steps) gemv_issue<false>(L, stage, step);
             else gemv_issue<true>(L, stage, step);
         }
     };
+    // SILU_IN: xs[M][slice rows] fp16 behind the rings.  The slab loads of this thread's share are requested first, the
+    // weight stages right behind them, so that both are in flight together.
+    half_t *xs = reinterpret_cast<half_t *>(lds + WAVES * RING_BYTES);
+    const int slice_k0 = step0 * 32, slice_rows = (step1 - step0) * 32;
+    if constexpr (SILU_IN) {
+        constexpr int MAXQ = SMH_SILU_IN_MAX_M * SMH_SILU_IN_MAX_K / 4 / THREADS;     // quads of columns per thread
+        f4 ga[MAXQ], ua[MAXQ];
+        const int quads = slice_rows / 4, total = p.M * quads;
+        const long gu_slab = (long)p.M * 2 * p.K;
 #pragma unroll
-    for (int i = 0; i < RING_STAGES; ++i)
-        if (i < n_steps) issue(ring + i * STAGE_BYTES, first + i * WAVES);
+        for (int i = 0; i < MAXQ; ++i) {
+            const int idx = tid + i * THREADS;
+            if (idx < total) {
+                const int m = idx / quads, k = slice_k0 + 4 * (idx % quads);
+                if (k < p.K) {
+                    ga[i] = slab_sum4(p.gu_partial, (long)m * 2 * p.K + k, gu_slab, p.gu_ksplit, false);
+                    ua[i] = slab_sum4(p.gu_partial, (long)m * 2 * p.K + p.K + k, gu_slab, p.gu_ksplit, false);
+                } else {
+                    ga[i] = f4{0.f, 0.f, 0.f, 0.f};
+                    ua[i] = f4{0.f, 0.f, 0.f, 0.f};
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < RING_STAGES; ++i)
+            if (i < n_steps) issue(ring + i * STAGE_BYTES, first + i * WAVES);
+#pragma unroll
+        for (int i = 0; i < MAXQ; ++i) {
+            const int idx = tid + i * THREADS;
+            if (idx < total) {
+                h4 o;
+#pragma unroll
+                for (int j = 0; j < 4; ++j) {                  // the roundings of partial_silu_mul_kernel
+                    const float gf = (float)(half_t)ga[i][j];
+                    const half_t sl = (half_t)(gf / (1.0f + expf(-gf)));
+                    o[j] = sl * (half_t)ua[i][j];
+                }
+                *reinterpret_cast<h4 *>(xs + (long)(idx / quads) * slice_rows + 4 * (idx % quads)) = o;
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // xs is complete; the DMA ring stays in flight
+    } else {
+#pragma unroll
+        for (int i = 0; i < RING_STAGES; ++i)
+            if (i < n_steps) issue(ring + i * STAGE_BYTES, first + i * WAVES);
+    }
+    const half_t *xlane = xs + (long)min(c, p.M - 1) * slice_rows + 8 * g;     // SILU_IN: this lane's row of xs, its k-octet
     // the one step that may lack rows is the last step of K, hence the last one of its wave; it is
     // peeled off so that the loop has a single decoder in it
     const int n_full = first < full_steps ? min(n_steps, (full_steps - first + WAVES - 1) / WAVES) : 0;
     int stage = 0;
     for (int i = 0; i < n_full; ++i) {
         const int later = min(RING_STAGES - 1, n_steps - 1 - i);     // steps issued after step i and still in flight
-        if (later >= 2) asm volatile("s_waitcnt vmcnt(12)" ::: "memory");
-        else if (later == 1) asm volatile("s_waitcnt vmcnt(6)" ::: "memory");
+        if (later >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PER_STAGE) : "memory");
+        else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_STAGE) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if constexpr (TILED) gemv_consume_tiled<false>(ring + stage * STAGE_BYTES, 0, p.K, lane, C, acc, corr);
+        if constexpr (SILU_IN) gemv_consume_tiled<false>(ring + stage * STAGE_BYTES, 0, p.K, lane, C, acc, corr, xlane + (first + i * WAVES - step0) * 32);
+        else if constexpr (TILED) gemv_consume_tiled<false>(ring + stage * STAGE_BYTES, 0, p.K, lane, C, acc, corr);
         else gemv_consume<false>(ring + stage * STAGE_BYTES, 0, p.K, c, g, C, acc, corr);
         if (i + RING_STAGES < n_steps) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");        // this stage's LDS reads are done
@@ -333,7 +385,8 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     }
     if (n_full < n_steps) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if constexpr (TILED) gemv_consume_tiled<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr);
+        if constexpr (SILU_IN) gemv_consume_tiled<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr, xlane + (first + n_full * WAVES - step0) * 32);
+        else if constexpr (TILED) gemv_consume_tiled<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr);
         else gemv_consume<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, c, g, C, acc, corr);
     }
     __syncthreads();                        // every wave is done with its ring: reuse LDS for the sums
@@ -438,11 +491,25 @@ int gemv_launch(const MatmulParams &p, hipStream_t stream) {
             set_error("q40 gemv: tiled weights run with 4 waves and without a finishing operator");
             return -1;
         }
-        hipLaunchKernelGGL((q40_gemv_kernel<4, false, true>), grid, dim3(256), lds, stream, p);
-    } else if (p.fin.mode != 0) hipLaunchKernelGGL((q40_gemv_kernel<4, true, false>), grid, dim3(256), lds, stream, p);
-    else if (waves == 2) hipLaunchKernelGGL((q40_gemv_kernel<2, false, false>), grid, dim3(128), lds, stream, p);
-    else if (waves == 8) hipLaunchKernelGGL((q40_gemv_kernel<8, false, false>), grid, dim3(512), lds, stream, p);
-    else hipLaunchKernelGGL((q40_gemv_kernel<4, false, false>), grid, dim3(256), lds, stream, p);
+        if (p.gu_partial != nullptr) {
+            if (p.M > SMH_SILU_IN_MAX_M || p.steps_per_slice * 32 > SMH_SILU_IN_MAX_K) {
+                set_error("q40 gemv: activations from the gate|up slabs need M <= %d and K-slices of at most %d rows", SMH_SILU_IN_MAX_M,
+                          SMH_SILU_IN_MAX_K);
+                return -1;
+            }
+            lds += (size_t)p.M * p.steps_per_slice * 32 * sizeof(half_t);          // xs behind the rings
+            // more than 64 KB of dynamic LDS has to be allowed once (not stream work: fine under graph capture)
+            static const hipError_t lds_ok = hipFuncSetAttribute((const void *)q40_gemv_kernel<4, false, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                                 4 * RING_BYTES + SMH_SILU_IN_MAX_M * SMH_SILU_IN_MAX_K * (int)sizeof(half_t));
+            if (lds_ok != hipSuccess) return (int)lds_ok;
+            hipLaunchKernelGGL((q40_gemv_kernel<4, false, 2>), grid, dim3(256), lds, stream, p);
+        } else {
+            hipLaunchKernelGGL((q40_gemv_kernel<4, false, 1>), grid, dim3(256), lds, stream, p);
+        }
+    } else if (p.fin.mode != 0) hipLaunchKernelGGL((q40_gemv_kernel<4, true, 0>), grid, dim3(256), lds, stream, p);
+    else if (waves == 2) hipLaunchKernelGGL((q40_gemv_kernel<2, false, 0>), grid, dim3(128), lds, stream, p);
+    else if (waves == 8) hipLaunchKernelGGL((q40_gemv_kernel<8, false, 0>), grid, dim3(512), lds, stream, p);
+    else hipLaunchKernelGGL((q40_gemv_kernel<4, false, 0>), grid, dim3(256), lds, stream, p);
     return launch_status();
 }
 

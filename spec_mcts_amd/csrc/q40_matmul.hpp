@@ -12,6 +12,8 @@
 
 #define SMH_MAX_KSPLIT 16
 #define SMH_MAX_SEGMENTS 3
+#define SMH_SILU_IN_MAX_M 2
+#define SMH_SILU_IN_MAX_K 2048      /* rows of a K-slice whose activations fit the workgroup's LDS */
 
 #include "matmul_finish.hpp"
 
@@ -61,6 +63,11 @@ struct MatmulParams {
     int epilogue, direct;
     int slab_half;           // slabs hold fp16 instead of fp32 (see slab_is_half)
     int tiled;               // the segments' weights are in the tiled layout
+    // GEMV, at most SMH_SILU_IN_MAX_M rows: the activations are not read from `a` but made by every workgroup for
+    // its own K-slice from the slabs of the gate|up product, a[m][k] = silu(gate[m][k]) * up[m][k] (gate = columns
+    // 0..K-1, up = columns K..2K-1 of the slabs), with the roundings of partial_silu_mul_kernel
+    const float *gu_partial;
+    int gu_ksplit;
     MatmulFinish fin;        // fin.mode == 0: leave the slabs to another launch
 };
 

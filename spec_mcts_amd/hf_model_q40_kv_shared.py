@@ -280,6 +280,7 @@ class Transformer(nn.Module):
                                       # layer instead of 10; measured slower at B=10: the finisher's round trips are serial)
         self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
         self.persistent = False       # True: decode steps of few branches as one persistent kernel (needs fused); the operator kernels are faster
+        self.silu_in_matmul = True         # up to 2 rows: w2's launch makes its own SiLU(gate)*up activations
         self.tiled_weights = True          # the fused path streams tiled copies of the weights (LinearQ4_0.operand)
         self.attn_single_launch = True     # up to 16 branches: prefix slices, suffix passes and the merge in one launch (slower above)
         self.attn_from_qkv = True          # up to 16 branches the attention takes the wq|wk|wv product itself, in one launch
@@ -385,8 +386,11 @@ class Transformer(nn.Module):
             po = K.matmul_q40_partial(o, [att.wo.operand(tiled)])
             h, xn = K.partial_rmsnorm(po, h, layer.ffn_norm.weight, layer.ffn_norm.eps)
             gu = K.matmul_q40_partial(xn, [ff.w1.operand(tiled), ff.w3.operand(tiled)])
-            act = K.partial_silu_mul(gu)
-            pending = K.matmul_q40_partial(act, [ff.w2.operand(tiled)])
+            if tiled and self.silu_in_matmul and M <= K.SILU_IN_MAX_M and ff.w2.shape[1] % 32 == 0 and ff.w2.w.is_cuda:
+                pending = K.matmul_q40_partial_silu(gu, [ff.w2.operand(True)])      # SiLU(gate)*up made inside w2's launch
+            else:
+                act = K.partial_silu_mul(gu)
+                pending = K.matmul_q40_partial(act, [ff.w2.operand(tiled)])
         _, hn = K.partial_rmsnorm(pending, h, self.norm.weight, self.norm.eps, want_h=False)
         return self.output(hn.view(bsz, seqlen, p.dim)).to(DTYPE)
 

@@ -188,6 +188,32 @@ def matmul_q40_partial(a: torch.Tensor, linears, out: Optional[torch.Tensor] = N
     return PartialProduct(out, ks, M, n_total)
 
 
+SILU_IN_MAX_M = 2
+
+
+def matmul_q40_partial_silu(gu: PartialProduct, linears, out: Optional[torch.Tensor] = None) -> PartialProduct:
+    """matmul_q40_partial(partial_silu_mul(gu), linears) in one launch for at most SILU_IN_MAX_M rows and tiled
+    weights: every workgroup makes the activations of its own K-slice from the gate|up slabs.  Same slabs, bit for bit."""
+    import ctypes
+    lib = _lib.load()
+    M, Kd = gu.M, gu.n_total // 2
+    assert M <= SILU_IN_MAX_M and gu.buf.dtype == torch.float32
+    assert all(isinstance(t, TiledQ40) and t.K == Kd for t in linears), "tiled weights with K = half the gate|up columns"
+    ns = [t.N for t in linears]
+    ks = matmul_plan(M, Kd, ns)
+    n_total = sum(ns)
+    need = ks * M * n_total
+    if out is None:
+        out = torch.empty(need, dtype=torch.float32, device=gu.buf.device)
+    assert out.dtype == torch.float32 and out.numel() >= need and out.is_contiguous() and out.data_ptr() != gu.buf.data_ptr()
+    nseg = len(linears)
+    tp = (ctypes.c_void_p * nseg)(*[t.buf.data_ptr() for t in linears])
+    na = (ctypes.c_int * nseg)(*ns)
+    check(lib.smh_q40_matmul_partial_tiled_silu(gu.buf.data_ptr(), gu.ksplit, M, Kd, nseg, tp, na, out.data_ptr(), out.numel() * 4,
+                                                _stream()), "smh_q40_matmul_partial_tiled_silu")
+    return PartialProduct(out, ks, M, n_total)
+
+
 def partial_reduce(p: PartialProduct, col0: int = 0, N: Optional[int] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     lib = _lib.load()
     N = p.n_total - col0 if N is None else N

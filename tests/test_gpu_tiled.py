@@ -112,3 +112,22 @@ def test_model_logits_do_not_depend_on_the_weight_layout():
     assert not torch.equal(c[1], b[1])
     for x, y in zip(c, d):
         assert torch.equal(x, y)
+
+
+@pytest.mark.parametrize("M", [1, 2])
+@pytest.mark.parametrize("K,n1,n2", [(11008, 4096, 4096), (256, 128, 512), (2048, 384, 256), (28672, 8192, 1024)])
+def test_w2_that_makes_its_own_silu_activations(M, K, n1, n2):
+    """smh_q40_matmul_partial_tiled_silu against smh_partial_silu_mul + smh_q40_matmul_partial_tiled: bit-identical slabs
+    (K = FFN width, n1 = model width feeding w1|w3, n2 = columns of w2)"""
+    from spec_mcts_amd import kernels as Kn
+    w1, w3, w2 = _weight(n1, K, 950 + K), _weight(n1, K, 951 + K), _weight(K, n2, 952 + K)
+    x = (torch.randn((M, n1), generator=torch.Generator().manual_seed(953 + M)) * 0.7).half().cuda()
+    t1, t3 = Kn.tile_q40(w1[0].cuda(), w1[1].cuda(), n1, K), Kn.tile_q40(w3[0].cuda(), w3[1].cuda(), n1, K)
+    t2 = Kn.tile_q40(w2[0].cuda(), w2[1].cuda(), K, n2)
+    gu = Kn.matmul_q40_partial(x, [t1, t3])
+    want = Kn.matmul_q40_partial(Kn.partial_silu_mul(gu), [t2])
+    got = Kn.matmul_q40_partial_silu(gu, [t2])
+    torch.cuda.synchronize()
+    n = want.ksplit * M * want.n_total
+    assert got.ksplit == want.ksplit
+    assert torch.equal(got.buf[:n].view(torch.int32), want.buf[:n].view(torch.int32))
