@@ -196,14 +196,16 @@ __device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K
 // pairs come out of (x, x2, x >> 8, x2 >> 8) and the scales arrive in the register order of the A operands.
 // Same operands into the same MFMAs in the same order as gemv_consume: the results are bit-identical.
 // `xrow`: the 8 activations k0 + 8g .. of this lane's batch row when they do not come from the stage (nullptr otherwise)
-template <bool RAGGED>
+template <bool RAGGED, bool XROW = false>
 __device__ __forceinline__ void gemv_consume_tiled(const uint8_t *stage, int k0, int K, int lane, const GemvConsts &C,
                                                    f4 (&acc)[2][2][4], f4 (&corr)[4], const half_t *xrow = nullptr) {
     const int c = lane & 15, g = lane >> 4;
     u32x4 wq[4];
 #pragma unroll
     for (int q = 0; q < 4; ++q) wq[q] = *reinterpret_cast<const u32x4 *>(stage + q * 1024 + lane * 16);
-    h8 xv = xrow ? *reinterpret_cast<const h8 *>(xrow) : *reinterpret_cast<const h8 *>(stage + STAGE_W_BYTES + STAGE_S_BYTES + c * 64 + 16 * g);
+    h8 xv;
+    if constexpr (XROW) xv = *reinterpret_cast<const h8 *>(xrow);      // (no select between two pointers: this stays an LDS read)
+    else xv = *reinterpret_cast<const h8 *>(stage + STAGE_W_BYTES + STAGE_S_BYTES + c * 64 + 16 * g);
     if constexpr (RAGGED) {
         if (k0 + 8 * g >= K) {
 #pragma unroll
@@ -374,7 +376,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         if (later >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PER_STAGE) : "memory");
         else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_STAGE) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if constexpr (SILU_IN) gemv_consume_tiled<false>(ring + stage * STAGE_BYTES, 0, p.K, lane, C, acc, corr, xlane + (first + i * WAVES - step0) * 32);
+        if constexpr (SILU_IN) gemv_consume_tiled<false, true>(ring + stage * STAGE_BYTES, 0, p.K, lane, C, acc, corr, xlane + (first + i * WAVES - step0) * 32);
         else if constexpr (TILED) gemv_consume_tiled<false>(ring + stage * STAGE_BYTES, 0, p.K, lane, C, acc, corr);
         else gemv_consume<false>(ring + stage * STAGE_BYTES, 0, p.K, c, g, C, acc, corr);
         if (i + RING_STAGES < n_steps) {
@@ -385,7 +387,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     }
     if (n_full < n_steps) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if constexpr (SILU_IN) gemv_consume_tiled<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr, xlane + (first + n_full * WAVES - step0) * 32);
+        if constexpr (SILU_IN) gemv_consume_tiled<true, true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr, xlane + (first + n_full * WAVES - step0) * 32);
         else if constexpr (TILED) gemv_consume_tiled<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr);
         else gemv_consume<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, c, g, C, acc, corr);
     }
@@ -400,21 +402,33 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
-            for (int b = 0; b < 4; ++b)
-#pragma unroll
-                for (int r = 0; r < 4; ++r) {
-                    const int m = 4 * g + r;
-                    const float off = h ? 1032.f : 72.f;
-                    if (r < p.M) {                  // uniform: with fewer than 4 rows whole store instructions drop out
-                        if (m < p.M)
-                            red[(wave * p.M + m) * GEMV_COLS + 128 * d + 64 * h + 4 * c + b] = acc[d][h][b][r] - off * corr[2 * d + h][r];
+            for (int r = 0; r < 4; ++r) {
+                const int m = 4 * g + r;
+                const float off = h ? 1032.f : 72.f;
+                if (r < p.M) {                      // uniform: with fewer than 4 rows whole store instructions drop out
+                    if (m < p.M) {                  // the four columns 4c .. 4c+3 of (block d, half h) as one 16-byte store
+                        const float cr = off * corr[2 * d + h][r];
+                        *reinterpret_cast<f4 *>(&red[(wave * p.M + m) * GEMV_COLS + 128 * d + 64 * h + 4 * c]) =
+                            f4{acc[d][h][0][r] - cr, acc[d][h][1][r] - cr, acc[d][h][2][r] - cr, acc[d][h][3][r] - cr};
                     }
                 }
+            }
     __syncthreads();
 
-    // thread -> outputs idx = tid, tid + THREADS, ... with idx = m * 256 + local column
     const int outputs = p.M * GEMV_COLS;
     float *slab = p.partial + (long)slice * p.M * p.n_total;
+    if (!FINISH && !p.direct) {
+        // slabs: four consecutive columns per thread (segment widths are multiples of 128, so a quad is inside or outside)
+        for (int q = tid; q < outputs / 4; q += THREADS) {
+            f4 sum = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+            for (int wv_ = 0; wv_ < WAVES; ++wv_) sum += *reinterpret_cast<const f4 *>(red + wv_ * outputs + 4 * q);
+            const int m = q >> 6, n_seg = col0 + 4 * (q & 63);
+            if (n_seg < seg.N) *reinterpret_cast<f4 *>(slab + (long)m * p.n_total + seg.col0 + n_seg) = sum;
+        }
+        return;
+    }
+    // thread -> outputs idx = tid, tid + THREADS, ... with idx = m * 256 + local column
     for (int idx = tid; idx < outputs; idx += THREADS) {
         float sum = 0.f;
 #pragma unroll
