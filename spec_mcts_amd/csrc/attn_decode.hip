@@ -142,31 +142,31 @@ __device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split,
     if (!FUSED && wave < q_tiles) load_q(wave, qb_first);
 
     // ---- stage K (row-major) and V (transposed) ----
-    auto stage_store = [&](int idx, u32x4 kv, u32x4 vv) {
-        const int t = idx >> 4, ch = idx & 15;
-        *reinterpret_cast<u32x4 *>(&ks[t][ch * 8]) = kv;
-        const int pos = vt_pos(t);
-        const h8 vh = __builtin_bit_cast(h8, vv);
+    // A thread moves piece ch (8 dims) of FOUR consecutive rows 4 kg .. 4 kg + 3: their V values sit side by side in a
+    // row of vt (vt_pos), so V goes out as 8-byte stores instead of 2-byte ones.
+    const int ch = tid & 15;
+    auto stage_load4 = [&](int kg, u32x4 (&kv)[4], u32x4 (&vv)[4]) {
 #pragma unroll
-        for (int j = 0; j < 8; ++j) vt[ch * 8 + j][pos] = vh[j];
-    };
-    auto stage_load = [&](int idx, u32x4 &kv, u32x4 &vv) {
-        const int t = idx >> 4, ch = idx & 15;
-        kv = u32x4{0, 0, 0, 0}; vv = u32x4{0, 0, 0, 0};
-        if (t < cnt) {
-            const long off = ((long)(t0 + t) * p.Hkv + hk) * ATT_D + ch * 8;
-            kv = *reinterpret_cast<const u32x4 *>(p.prefix_k + off);
-            vv = *reinterpret_cast<const u32x4 *>(p.prefix_v + off);
+        for (int e = 0; e < 4; ++e) {
+            const int t = 4 * kg + e;
+            kv[e] = u32x4{0, 0, 0, 0}; vv[e] = u32x4{0, 0, 0, 0};
+            if (t < cnt) {
+                const long off = ((long)(t0 + t) * p.Hkv + hk) * ATT_D + ch * 8;
+                kv[e] = *reinterpret_cast<const u32x4 *>(p.prefix_k + off);
+                vv[e] = *reinterpret_cast<const u32x4 *>(p.prefix_v + off);
+            }
         }
     };
-    if (FUSED && TWM <= 64) {
-        // every load of the workgroup is requested before anything waits: the K / V slice into registers, then
-        // the slabs from which all 256 threads build the rotated queries of this kv head (8 dims each)
-        constexpr int PER = TWM * 16 / 256;
-        u32x4 kv[PER], vv[PER];
+    auto stage_store4 = [&](int kg, const u32x4 (&kv)[4], const u32x4 (&vv)[4]) {
 #pragma unroll
-        for (int i = 0; i < PER; ++i)
-            if (tid + 256 * i < tw32 * 16) stage_load(tid + 256 * i, kv[i], vv[i]);
+        for (int e = 0; e < 4; ++e) *reinterpret_cast<u32x4 *>(&ks[4 * kg + e][ch * 8]) = kv[e];
+        const int pos = vt_pos(4 * kg);
+        const h8 v0 = __builtin_bit_cast(h8, vv[0]), v1 = __builtin_bit_cast(h8, vv[1]);
+        const h8 v2 = __builtin_bit_cast(h8, vv[2]), v3 = __builtin_bit_cast(h8, vv[3]);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) *reinterpret_cast<h4 *>(&vt[ch * 8 + j][pos]) = h4{v0[j], v1[j], v2[j], v3[j]};
+    };
+    auto build_queries = [&]() {
         const int cc = tid & 15;
         const int pos = *p.pos_dev;
         for (int qr = tid >> 4; qr < p.Bq; qr += 16) {
@@ -175,24 +175,22 @@ __device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split,
             *reinterpret_cast<h4 *>(&qs[qr][4 * cc]) = lo;
             *reinterpret_cast<h4 *>(&qs[qr][64 + 4 * cc]) = hi;
         }
-#pragma unroll
-        for (int i = 0; i < PER; ++i)
-            if (tid + 256 * i < tw32 * 16) stage_store(tid + 256 * i, kv[i], vv[i]);
+    };
+    if (FUSED && TWM <= 64) {
+        // every load of the workgroup is requested before anything waits: the K / V slice into registers, then
+        // the slabs from which all 256 threads build the rotated queries of this kv head (8 dims each)
+        static_assert(!FUSED || TWM > 64 || TWM == 64, "one group of four rows per thread");
+        u32x4 kv[4], vv[4];
+        const int kg = tid >> 4;
+        if (4 * kg < tw32) stage_load4(kg, kv, vv);
+        build_queries();
+        if (4 * kg < tw32) stage_store4(kg, kv, vv);
     } else {
-        if (FUSED) {
-            const int cc = tid & 15;
-            const int pos = *p.pos_dev;
-            for (int qr = tid >> 4; qr < p.Bq; qr += 16) {
-                h4 lo, hi;
-                qkv_query(p, qr / p.n_rep, hk * p.n_rep + qr % p.n_rep, pos, cc, lo, hi);
-                *reinterpret_cast<h4 *>(&qs[qr][4 * cc]) = lo;
-                *reinterpret_cast<h4 *>(&qs[qr][64 + 4 * cc]) = hi;
-            }
-        }
-        for (int idx = tid; idx < tw32 * 16; idx += 256) {
-            u32x4 kv, vv;
-            stage_load(idx, kv, vv);
-            stage_store(idx, kv, vv);
+        if (FUSED) build_queries();
+        for (int kg = tid >> 4; 4 * kg < tw32; kg += 16) {
+            u32x4 kv[4], vv[4];
+            stage_load4(kg, kv, vv);
+            stage_store4(kg, kv, vv);
         }
     }
     __syncthreads();
@@ -321,10 +319,12 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillParams p) {
     }
     constexpr int PER = PF_TW * 16 / 256;                  // 16-byte pieces of K (and of V) per thread and tile
     u32x4 kreg[PER], vreg[PER];
+    // a thread moves piece ch (8 dims) of FOUR consecutive keys, so that V goes to its transposed tile as 8-byte stores
+    static_assert(PER == 4, "four keys per thread");
     auto tile_load = [&](int kt) {
 #pragma unroll
         for (int i = 0; i < PER; ++i) {
-            const int idx = tid + 256 * i, t = idx >> 4, ch = idx & 15;
+            const int t = 4 * (tid >> 4) + i, ch = tid & 15;
             const int row = kt * PF_TW + t;
             kreg[i] = u32x4{0, 0, 0, 0}; vreg[i] = u32x4{0, 0, 0, 0};
             if (row < p.S) {
@@ -335,15 +335,14 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillParams p) {
         }
     };
     auto tile_store = [&]() {
+        const int t0 = 4 * (tid >> 4), ch = tid & 15;
 #pragma unroll
-        for (int i = 0; i < PER; ++i) {
-            const int idx = tid + 256 * i, t = idx >> 4, ch = idx & 15;
-            *reinterpret_cast<u32x4 *>(&ks[t][ch * 8]) = kreg[i];
-            const int pos = vt_pos(t);
-            const h8 vh = __builtin_bit_cast(h8, vreg[i]);
+        for (int i = 0; i < PER; ++i) *reinterpret_cast<u32x4 *>(&ks[t0 + i][ch * 8]) = kreg[i];
+        const int pos = vt_pos(t0);                            // keys t0 .. t0+3 sit side by side in a row of vt
+        const h8 v0 = __builtin_bit_cast(h8, vreg[0]), v1 = __builtin_bit_cast(h8, vreg[1]);
+        const h8 v2 = __builtin_bit_cast(h8, vreg[2]), v3 = __builtin_bit_cast(h8, vreg[3]);
 #pragma unroll
-            for (int j = 0; j < 8; ++j) vt[ch * 8 + j][pos] = vh[j];
-        }
+        for (int j = 0; j < 8; ++j) *reinterpret_cast<h4 *>(&vt[ch * 8 + j][pos]) = h4{v0[j], v1[j], v2[j], v3[j]};
     };
 
     float m_run = -INFINITY, l_run = 0.f;                  // of query c (the same in the four lane groups)
