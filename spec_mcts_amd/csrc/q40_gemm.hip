@@ -302,11 +302,12 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
 #pragma unroll
     for (int t = 0; t < TILES; ++t) {
         float *otile = reinterpret_cast<float *>(lds + (t & 1) * OTILE_BYTES);
+        // operands o and o + 2 are neighbouring columns: one 8-byte LDS store for the pair
 #pragma unroll
-        for (int o = 0; o < 4; ++o)
+        for (int o = 0; o < 2; ++o)
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                otile[(4 * g + r) * OP + 128 * blk + 64 * (o & 1) + 4 * c + 2 * bp + (o >> 1)] = acc[o][t][r];
+                *reinterpret_cast<f2 *>(&otile[(4 * g + r) * OP + 128 * blk + 64 * o + 4 * c + 2 * bp]) = f2{acc[o][t][r], acc[o + 2][t][r]};
         gemm_barrier();
         const int m = m0 + 16 * t + o_row;
         if (m < p.M) {
