@@ -149,6 +149,13 @@ int smh_rmsnorm(const void *x, const void *weight, void *out, int rows, int dim,
                 smh_stream_t stream);
 int smh_silu_mul(const void *g, const void *u, void *out, long n, smh_stream_t stream);
 int smh_argmax(const void *logits, int rows, int vocab, long ld, int64_t *out, smh_stream_t stream);
+/* smh_sample_topk: the sampling step of Transformer.generate (hf_model_q40_kv_shared.py:580-589: logits / temperature,
+ * torch.topk, F.softmax, torch.multinomial, gather) for fp16 logits [rows, vocab] in one launch: x = fp16(logit /
+ * temperature), the top_k largest x (equal values: lowest index first), p = fp16(softmax over them), one candidate per
+ * row drawn by inverse CDF over the candidates in descending order with uniform[row] in [0, 1) - the caller's random
+ * numbers take the place of torch.multinomial's generator.  1 <= top_k <= 1024, temperature > 0. */
+int smh_sample_topk(const void *logits, int rows, int vocab, long ld, float temperature, int top_k,
+                    const float *uniform, int64_t *out, smh_stream_t stream);
 int smh_rope_append_kv(void *q, void *k, const void *v, int B, int H, int Hkv, int D,
                        const void *cos_tab, const void *sin_tab, const int32_t *pos_dev,
                        void *cache_k, void *cache_ks, void *cache_v, void *cache_vs,

@@ -25,6 +25,9 @@ live in tests/test_oracle_*.py):
   OracleTransformer              composition only; cross-checked by (i) dense-weight F.linear model,
                                  (ii) prefill-vs-incremental equality with KV quantisation off,
                                  (iii) identical branches give identical tokens.
+  topk_probs / sample_topk       candidate values against torch.topk, probabilities against F.softmax of those values,
+                                 k = 1 is the argmax, k = vocab with a huge temperature is uniform; the draw against a
+                                 brute-force scan in float64 and, over many uniform numbers, its frequencies against p.
 No function here is "parity unpinned".
 """
 from __future__ import annotations
@@ -160,6 +163,29 @@ def apply_rotary_emb(q: torch.Tensor, k: torch.Tensor, freqs_cis: torch.Tensor):
     q_embed = (q * cos) + (rotate_half(q) * sin)
     k_embed = (k * cos) + (rotate_half(k) * sin)
     return q_embed, k_embed
+
+
+def topk_probs(logits: torch.Tensor, temperature: float, top_k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The candidates of the reference's sampling step (hf_model_q40_kv_shared.py:580-586): `logits / temperature` on
+    the fp16 tensor, `torch.topk`, `F.softmax` (fp16 in, fp16 out).  Returns (p [rows, k] fp16, idx [rows, k]) in
+    descending order of value; equal values are ordered by index (torch.topk leaves that order open)."""
+    x = logits / temperature                                   # fp16 tensor / python float: fp16 result
+    k = min(top_k, x.shape[-1])
+    order = torch.argsort(x.float(), dim=-1, descending=True, stable=True)[:, :k]
+    v = torch.gather(x, 1, order)
+    return F.softmax(v, dim=-1), order
+
+
+def sample_topk(logits: torch.Tensor, temperature: float, top_k: int, u: torch.Tensor) -> torch.Tensor:
+    """One draw per row from topk_probs by inverse CDF with the given uniform numbers u [rows] in [0, 1): the first
+    candidate (descending order) whose cumulative probability exceeds u * total.  Stands in for `torch.multinomial`
+    (:588), whose generator cannot be reproduced: same distribution, the caller's randomness."""
+    p, order = topk_probs(logits, temperature, top_k)
+    cdf = p.float().cumsum(-1)
+    target = u.float().unsqueeze(1) * cdf[:, -1:]
+    hit = cdf > target
+    j = torch.where(hit.any(-1), hit.float().argmax(-1), torch.full((p.shape[0],), p.shape[1] - 1))
+    return order.gather(1, j.unsqueeze(1))[:, 0]
 
 
 def silu_mul(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:

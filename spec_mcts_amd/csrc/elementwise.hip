@@ -228,6 +228,161 @@ extern "C" int smh_silu_mul(const void *g, const void *u, void *out, long n, smh
     return launch_status();
 }
 
+namespace smh {
+
+// ---- temperature / top-k sampling -----------------------------------------------------------------------------
+// One 1024-thread workgroup per row.  x = fp16(logit / temperature) (the reference divides fp16 tensors); the k largest
+// x, equal values taken lowest index first, are found with a two-pass radix select on an order-preserving 16-bit key
+// (256-bin histograms in LDS), gathered, ordered by (x descending, index ascending) with a rank sort, turned into
+// probabilities p = fp16(softmax) as F.softmax on an fp16 tensor returns them, and one candidate is drawn by inverse
+// CDF with the caller's uniform number.
+constexpr int SAMPLE_MAX_K = 1024;
+
+__device__ __forceinline__ uint32_t sample_key(half_t x) {
+    const uint32_t b = __builtin_bit_cast(uint16_t, x);
+    return (b & 0x8000u) ? (~b & 0xFFFFu) : (b | 0x8000u);       // larger value <=> larger key
+}
+__device__ __forceinline__ half_t sample_unkey(uint32_t k) {
+    const uint16_t b = (uint16_t)((k & 0x8000u) ? (k & 0x7FFFu) : (~k & 0xFFFFu));
+    return __builtin_bit_cast(half_t, b);
+}
+
+// bins[t] <- sum of bins[t..255]; then the bin where the count from the top reaches `want` and the count above it
+__device__ __forceinline__ void sample_pick_bin(int *bins, int want, int *out_bin, int *out_above) {
+    const int t = threadIdx.x;
+    for (int off = 1; off < 256; off <<= 1) {
+        int v = 0;
+        if (t < 256 && t + off < 256) v = bins[t + off];
+        __syncthreads();
+        if (t < 256) bins[t] += v;
+        __syncthreads();
+    }
+    if (t < 256) {
+        const int above = t == 255 ? 0 : bins[t + 1];
+        if (bins[t] >= want && above < want) { *out_bin = t; *out_above = above; }
+    }
+    __syncthreads();
+}
+
+__global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restrict__ logits, int vocab, long ld, float temperature,
+                                                           int top_k, const float *__restrict__ uniform, int64_t *__restrict__ out) {
+    __shared__ int bins[256];
+    __shared__ int s_bin, s_above, s_count;
+    __shared__ int scan[1024];
+    __shared__ uint32_t c_key[SAMPLE_MAX_K];
+    __shared__ int c_idx[SAMPLE_MAX_K];
+    __shared__ uint32_t o_key[SAMPLE_MAX_K];
+    __shared__ int o_idx[SAMPLE_MAX_K];
+    __shared__ float cdf[SAMPLE_MAX_K];
+    const int tid = threadIdx.x;
+    const half_t *row = logits + (long)blockIdx.x * ld;
+    const int k = min(top_k, vocab);
+    auto key_at = [&](int i) { return sample_key((half_t)((float)row[i] / temperature)); };
+
+    // ---- the k-th largest key: high byte, then low byte ----
+    if (tid < 256) bins[tid] = 0;
+    if (tid == 0) s_count = 0;
+    __syncthreads();
+    for (int i = tid; i < vocab; i += 1024) atomicAdd(&bins[key_at(i) >> 8], 1);
+    __syncthreads();
+    sample_pick_bin(bins, k, &s_bin, &s_above);
+    const int b1 = s_bin, above1 = s_above;
+    __syncthreads();
+    if (tid < 256) bins[tid] = 0;
+    __syncthreads();
+    for (int i = tid; i < vocab; i += 1024) {
+        const uint32_t key = key_at(i);
+        if ((int)(key >> 8) == b1) atomicAdd(&bins[key & 255], 1);
+    }
+    __syncthreads();
+    sample_pick_bin(bins, k - above1, &s_bin, &s_above);
+    const uint32_t kth = ((uint32_t)b1 << 8) | (uint32_t)s_bin;      // key of the k-th largest value
+    const int ties_wanted = k - (above1 + s_above);                    // how many of the values equal to it are in
+    __syncthreads();
+
+    // ---- gather: everything above the k-th key, and of the ties the lowest indices (contiguous chunk per thread,
+    //      exclusive scan of the per-thread tie counts gives each tie its rank by index) ----
+    const int chunk = (vocab + 1023) / 1024;
+    const int lo = tid * chunk, hi = min(vocab, lo + chunk);
+    int my_ties = 0;
+    for (int i = lo; i < hi; ++i) my_ties += key_at(i) == kth;
+    scan[tid] = my_ties;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        const int v = tid >= off ? scan[tid - off] : 0;
+        __syncthreads();
+        scan[tid] += v;
+        __syncthreads();
+    }
+    int tie_rank = scan[tid] - my_ties;                                // ties at lower indices
+    for (int i = lo; i < hi; ++i) {
+        const uint32_t key = key_at(i);
+        bool take = key > kth;
+        if (key == kth) { take = tie_rank < ties_wanted; ++tie_rank; }
+        if (take) {
+            const int slot = atomicAdd(&s_count, 1);
+            c_key[slot] = key;
+            c_idx[slot] = i;
+        }
+    }
+    __syncthreads();
+
+    // ---- order the k candidates: rank = number of candidates that come before ----
+    if (tid < k) {
+        const uint32_t mk = c_key[tid];
+        const int mi = c_idx[tid];
+        int rank = 0;
+        for (int j = 0; j < k; ++j) rank += (c_key[j] > mk) || (c_key[j] == mk && c_idx[j] < mi);
+        o_key[rank] = mk;
+        o_idx[rank] = mi;
+    }
+    __syncthreads();
+
+    // ---- p = fp16(softmax), inverse CDF ----
+    const float xmax = (float)sample_unkey(o_key[0]);
+    const float e = tid < k ? expf((float)sample_unkey(o_key[tid]) - xmax) : 0.f;
+    cdf[tid] = e;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        const float v = tid >= off ? cdf[tid - off] : 0.f;
+        __syncthreads();
+        cdf[tid] += v;
+        __syncthreads();
+    }
+    const float total = cdf[k - 1];
+    __syncthreads();
+    const float pr = tid < k ? (float)(half_t)(e / total) : 0.f;
+    cdf[tid] = pr;
+    __syncthreads();
+    for (int off = 1; off < 1024; off <<= 1) {
+        const float v = tid >= off ? cdf[tid - off] : 0.f;
+        __syncthreads();
+        cdf[tid] += v;
+        __syncthreads();
+    }
+    const float target = uniform[blockIdx.x] * cdf[k - 1];
+    if (tid < k) {
+        const float before = tid == 0 ? 0.f : cdf[tid - 1];
+        // first candidate whose cumulative probability exceeds the target (the last one if rounding leaves none)
+        if ((before <= target && target < cdf[tid]) || (tid == k - 1 && target >= cdf[tid])) out[blockIdx.x] = o_idx[tid];
+    }
+}
+
+}  // namespace smh
+
+extern "C" int smh_sample_topk(const void *logits, int rows, int vocab, long ld, float temperature, int top_k,
+                               const float *uniform, int64_t *out, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "smh_sample_topk: rows=%d vocab=%d ld=%ld", rows, vocab, ld);
+    SMH_REQUIRE(top_k >= 1 && top_k <= SAMPLE_MAX_K, "smh_sample_topk: top_k=%d outside [1,%d]", top_k, SAMPLE_MAX_K);
+    SMH_REQUIRE(temperature > 0.f, "smh_sample_topk: temperature=%g must be positive (greedy decoding is smh_argmax)", (double)temperature);
+    if (rows == 0) return 0;
+    SMH_REQUIRE(logits && uniform && out, "smh_sample_topk: null pointer");
+    hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, temperature,
+                       top_k, uniform, out);
+    return launch_status();
+}
+
 extern "C" int smh_argmax(const void *logits, int rows, int vocab, long ld, int64_t *out, smh_stream_t stream) {
     using namespace smh;
     SMH_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "smh_argmax: rows=%d vocab=%d ld=%ld", rows, vocab, ld);

@@ -280,6 +280,7 @@ class Transformer(nn.Module):
                                       # layer instead of 10; measured slower at B=10: the finisher's round trips are serial)
         self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
         self.persistent = False       # True: decode steps of few branches as one persistent kernel (needs fused); the operator kernels are faster
+        self.fused_sampler = True          # generate(): temperature / top-k / draw as one kernel instead of five torch ops
         self.silu_in_matmul = True         # up to 2 rows: w2's launch makes its own SiLU(gate)*up activations
         self.tiled_weights = True          # the fused path streams tiled copies of the weights (LinearQ4_0.operand)
         self.attn_single_launch = True     # up to 16 branches: prefix slices, suffix passes and the merge in one launch (slower above)
@@ -517,6 +518,9 @@ class Transformer(nn.Module):
                 logits = logits[:, -1, :]
             if temperature == 0.0:
                 idx_next = K.argmax(logits.contiguous())[:, None]
+            elif self.fused_sampler and logits.dtype == torch.float16 and top_k <= 1024:
+                # division, top-k, softmax and the draw in one launch; torch.rand supplies the randomness
+                idx_next = K.sample_topk(logits.contiguous(), temperature, top_k)[:, None]
             else:
                 logits = logits / temperature
                 v, top_k_idx = torch.topk(logits, top_k)

@@ -358,6 +358,23 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def sample_topk(logits: torch.Tensor, temperature: float, top_k: int, uniform: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per row of fp16 logits [rows, vocab]: top-k of logits / temperature, softmax, one draw (the sampling
+    lines of the reference's generate).  `uniform`: fp32 [rows] in [0, 1), default torch.rand on the logits' device."""
+    lib = _lib.load()
+    _need_gpu(logits)
+    assert logits.dim() == 2 and logits.dtype == torch.float16 and logits.stride(1) == 1
+    rows, vocab = logits.shape
+    if uniform is None:
+        uniform = torch.rand(rows, device=logits.device, dtype=torch.float32)
+    _need_gpu(uniform)
+    assert uniform.dtype == torch.float32 and uniform.numel() == rows and uniform.is_contiguous()
+    out = torch.empty(rows, device=logits.device, dtype=torch.int64)
+    check(lib.smh_sample_topk(logits.data_ptr(), rows, vocab, logits.stride(0), float(temperature), int(min(top_k, vocab)),
+                              uniform.data_ptr(), out.data_ptr(), _stream()), "smh_sample_topk")
+    return out
+
+
 def rope(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, pos0: int) -> None:
     """In-place rotate-half RoPE of q [S,H,128] and k [S,Hkv,128]; token s is at position pos0+s."""
     lib = _lib.load()

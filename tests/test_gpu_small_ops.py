@@ -107,3 +107,49 @@ def test_kv_fork_copies_rows():
     want_c[3:5] = want_c[1]; want_s[3:5] = want_s[1]
     assert torch.equal(cd.cpu().view(Bmax, -1), want_c)
     assert torch.equal(sd_.cpu().view(Bmax, -1).view(torch.int16), want_s.view(torch.int16))
+
+
+@pytest.mark.parametrize("rows,vocab,k,temperature", [(100, 32016, 32, 0.8), (3, 320, 5, 1.0), (7, 1000, 1, 1.3), (4, 50, 50, 2.0),
+                                                      (5, 4096, 1000, 0.6), (2, 70000, 64, 1.0)])
+def test_sample_topk_matches_the_oracle(rows, vocab, k, temperature):
+    """same candidates, same fp16 probabilities, same draw for the same uniform numbers; where u * total falls within
+    fp32 rounding of a boundary of the cumulative probabilities either neighbour is accepted"""
+    from spec_mcts_amd import kernels as K
+    g = torch.Generator().manual_seed(500 + vocab + k)
+    logits = (torch.randn((rows, vocab), generator=g) * 2.5).half()
+    p, idx = O.topk_probs(logits, temperature, k)
+    cdf = p.float().cumsum(-1)
+    for trial in range(4):
+        u = torch.rand(rows, generator=g)
+        want = O.sample_topk(logits, temperature, k, u)
+        got = K.sample_topk(logits.cuda(), temperature, k, u.cuda()).cpu()
+        for r in range(rows):
+            if int(got[r]) == int(want[r]):
+                continue
+            pos = (idx[r] == int(got[r])).nonzero()
+            assert len(pos) == 1, f"row {r}: token {int(got[r])} is not a candidate"
+            j = int(pos[0])
+            target = float(u[r]) * float(cdf[r, -1])
+            edges = [float(cdf[r, j - 1]) if j else 0.0, float(cdf[r, j])]
+            assert min(abs(e - target) for e in edges) < 1e-5, f"row {r}: drew candidate {j}, target {target}, interval {edges}"
+
+
+def test_sample_topk_ties_take_the_lowest_indices_and_frequencies_follow_p():
+    from spec_mcts_amd import kernels as K
+    # ties: a row of few distinct values; the candidates must be those of the stable order
+    logits = torch.tensor([[1.0, 3.0, 2.0, 3.0, 2.0, 2.0, 0.5, 3.0]], dtype=torch.float16).repeat(64, 1)
+    p, idx = O.topk_probs(logits, 1.0, 5)                       # 3.0 at 1, 3, 7, then 2.0 at 2, 4 (not 5)
+    assert idx[0].tolist() == [1, 3, 7, 2, 4]
+    u = torch.linspace(0.0, 0.999, 64)
+    got = K.sample_topk(logits.cuda(), 1.0, 5, u.cuda()).cpu()
+    assert set(got.tolist()) <= {1, 3, 7, 2, 4} and 5 not in got.tolist()
+    assert torch.equal(got, O.sample_topk(logits, 1.0, 5, u)) or (got != O.sample_topk(logits, 1.0, 5, u)).sum() <= 2
+    # frequencies
+    g = torch.Generator().manual_seed(9)
+    row = (torch.randn((1, 2000), generator=g) * 2).half()
+    n = 20000
+    p, idx = O.topk_probs(row, 0.9, 8)
+    draws = K.sample_topk(row.expand(n, -1).contiguous().cuda(), 0.9, 8, torch.rand(n, generator=g).cuda()).cpu()
+    for j in range(8):
+        freq = float((draws == idx[0, j]).float().mean()); pj = float(p[0, j])
+        assert abs(freq - pj) < 4 * (pj * (1 - pj) / n) ** 0.5 + 1e-3

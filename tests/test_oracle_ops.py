@@ -207,3 +207,45 @@ def test_per_branch_flavour_reduces_to_shared_flavour_without_kv_quantisation():
         assert torch.allclose(a.float(), b.float(), rtol=0, atol=4e-3)
     assert (outs["rows"][-1].float() - outs["rows_q"][-1].float()).abs().max() > 2e-2
     assert torch.allclose(outs["rows"][-1].float(), outs["rows_q"][-1].float(), atol=0.5)
+
+
+def test_sampler_candidates_and_draw():
+    """topk_probs against torch.topk + F.softmax; sample_topk against a brute-force float64 scan and, over many
+    uniform numbers, against the probabilities themselves"""
+    import torch.nn.functional as F
+    g = torch.Generator().manual_seed(77)
+    logits = (torch.randn((6, 500), generator=g) * 3).half()
+    for temperature, k in ((1.0, 32), (0.7, 5), (2.5, 500)):
+        p, idx = O.topk_probs(logits, temperature, k)
+        v_ref, _ = torch.topk(logits / temperature, k)
+        assert torch.equal(torch.gather(logits / temperature, 1, idx), v_ref)          # same values in the same order
+        assert torch.equal(p, F.softmax(v_ref, dim=-1))
+    # k = 1 is the argmax whatever u is
+    u = torch.rand(6, generator=g)
+    assert torch.equal(O.sample_topk(logits, 1.0, 1, u), logits.float().argmax(-1))
+    # huge temperature, all candidates: uniform probabilities
+    p, _ = O.topk_probs(logits, 1e4, 500)
+    assert torch.allclose(p.float(), torch.full_like(p, 1 / 500).float(), rtol=2e-2)
+    # the draw: brute force in float64
+    p, idx = O.topk_probs(logits, 0.9, 20)
+    for trial in range(50):
+        u = torch.rand(6, generator=g)
+        got = O.sample_topk(logits, 0.9, 20, u)
+        for r in range(6):
+            cum, pick = 0.0, 19
+            tot = float(p[r].double().sum())
+            for j in range(20):
+                cum += float(p[r, j])
+                if cum > float(u[r]) * tot + 1e-9:
+                    pick = j
+                    break
+            near = abs(cum - float(u[r]) * tot) < 1e-5          # a boundary within fp32 rounding of the target
+            assert int(got[r]) == int(idx[r, pick]) or near
+    # frequencies over many draws follow p (row 0, 5 candidates)
+    p, idx = O.topk_probs(logits[:1], 1.0, 5)
+    n = 20000
+    u = torch.rand(n, generator=g)
+    draws = O.sample_topk(logits[:1].expand(n, -1).contiguous(), 1.0, 5, u)
+    for j in range(5):
+        freq = float((draws == idx[0, j]).float().mean())
+        assert abs(freq - float(p[0, j])) < 4 * (float(p[0, j]) * (1 - float(p[0, j])) / n) ** 0.5 + 1e-3
