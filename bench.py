@@ -29,6 +29,14 @@ HBM_PEAK_GBS = 8000.0
 MFMA_F16_PEAK_TFLOPS = 2500.0
 PROMPT_LEN = 512
 BATCHES = (1, 10, 100)
+# architectures of the reference's checkpoints (params.json of CodeLlama-7b and -70b); "70b" is the one-GPU 70B
+# workload: 2048-token prompt shared by the branches, 64 tokens decoded per branch
+ARCHS = {
+    "7b": dict(dim=4096, n_layers=32, n_heads=32, n_kv_heads=None, vocab_size=32016, multiple_of=256, ffn_dim_multiplier=None,
+               prompt=PROMPT_LEN, max_seq_len=128),
+    "70b": dict(dim=8192, n_layers=80, n_heads=64, n_kv_heads=8, vocab_size=32016, multiple_of=4096, ffn_dim_multiplier=1.3,
+                prompt=2048, max_seq_len=64),
+}
 # HBM bytes per q40_gemv_kernel launch at M=1: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by a 1 GiB copy
 # (profiles/q40_gemv_m1_hbm_traffic.md has the commands and the factors: 2.0 for reads, 1.0 for writes)
 GEMV_TRAFFIC_BYTES_PER_LAUNCH = 27509321
@@ -216,8 +224,14 @@ def main():
     ap.add_argument("--roofline-only", type=int, default=0, metavar="M",
                     help="profiling aid: run only the matmul roofline leg at batch M (eager launches, one pass) after a 1 GiB "
                          "device copy that calibrates the profiler's byte counters, and print that leg's numbers")
-    ap.add_argument("--layers", type=int, default=32, help="fewer layers for a quick functional run (INVALID as a result)")
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers for a quick functional run (INVALID as a result)")
+    ap.add_argument("--arch", choices=sorted(ARCHS), default="7b",
+                    help="7b is the headline workload; 70b is the 80-layer GQA architecture with a 2048-token prompt (about 38 GB of Q4_0 "
+                         "weights, run with --steps + --warmup < 64)")
     a = ap.parse_args()
+    arch = dict(ARCHS[a.arch])
+    prompt_len, max_seq = arch.pop("prompt"), arch.pop("max_seq_len")
+    a.layers = a.layers or arch["n_layers"]
     if a.gpus != 1:
         sys.exit("bench.py: this build runs the Q4_0 decode path on ONE GPU; --gpus must be 1 "
                  "(branches would shard data-parallel across GPUs, which this run does not exercise)")
@@ -226,16 +240,16 @@ def main():
 
     assert torch.cuda.is_available(), "bench.py needs a GPU"
     steps, warmup = a.steps, a.warmup
-    assert steps + warmup + 1 <= 128, "configs[3] decodes at most 128 tokens per branch"
-    args_kw = dict(dim=4096, n_layers=a.layers, n_heads=32, vocab_size=32016, multiple_of=256, norm_eps=1e-5,
-                   rope_theta=1e6, max_batch_size=100, max_seq_len=128, max_prompt_seq_len=PROMPT_LEN)
+    assert steps + warmup + 1 <= max_seq, "this workload decodes at most %d tokens per branch" % max_seq
+    args_kw = dict(arch, n_layers=a.layers, norm_eps=1e-5, rope_theta=1e6, max_batch_size=100, max_seq_len=max_seq,
+                   max_prompt_seq_len=prompt_len)
     torch.manual_seed(3)
     model = build_model(torch, args_kw, seed=3)
     if a.persistent:
         model.persistent = True
     if a.finish_in_matmul:
         model.finish_in_matmul = True
-    prompt = torch.randint(0, 32016, (1, PROMPT_LEN), generator=torch.Generator().manual_seed(3)).cuda()
+    prompt = torch.randint(0, 32016, (1, prompt_len), generator=torch.Generator().manual_seed(3)).cuda()
 
     if a.roofline_only:
         src = torch.empty(1 << 29, dtype=torch.float16, device="cuda:0").normal_()
@@ -263,22 +277,25 @@ def main():
         del dec
 
     # per-step algorithmic HBM bytes: Q4 linears + fp16 lm_head + shared prefix KV (once) + suffix KV (Q4 rows)
-    lin_bytes = sum(q40_bytes(0, n, k) for n, k in ((4096, 4096),) * 4 + ((11008, 4096),) * 2 + ((4096, 11008),)) * a.layers
-    head_bytes = 32016 * 4096 * 2
-    prefix_bytes = 2 * PROMPT_LEN * 4096 * 2 * a.layers
+    lin_bytes = sum(q40_bytes(0, n, k_in) for k_in, segs in step_matmuls(model) for _, n in segs)
+    kv_heads = model.layers[0].attention.n_kv_heads
+    kv_dim = kv_heads * 128
+    head_bytes = 32016 * arch["dim"] * 2
+    prefix_bytes = 2 * prompt_len * kv_dim * 2 * a.layers
+    suffix_row_bytes = a.layers * 2 * kv_heads * 68          # K and V, 64 nibble bytes + 2 fp16 scales per head
     t_mid = warmup + steps // 2
     for B in batches:
-        step_bytes = lin_bytes + head_bytes + prefix_bytes + B * t_mid * a.layers * 2 * 32 * 68
+        step_bytes = lin_bytes + head_bytes + prefix_bytes + B * t_mid * suffix_row_bytes
         by_batch[B]["hbm_frac"] = step_bytes / (by_batch[B]["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS
 
     head = by_batch.get(100) or by_batch[max(by_batch)]
     head_b = 100 if 100 in by_batch else max(by_batch)
     result = {
-        "metric": "Q4_0 7B decode tok/s at B=1/10/100; Q4_0 GEMV achieved HBM GB/s",
+        "metric": "Q4_0 %s decode tok/s at B=1/10/100; Q4_0 GEMV achieved HBM GB/s" % a.arch.upper(),
         "value": head["tok_s"], "unit": "tok/s", "n_gpus": 1, "steps": steps, "warmup": warmup,
         "ms_per_step": head["ms_per_step"], "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "codellama7b_arch_q40_decode_prompt512_shared_prefix", "branches": head_b,
+        "config": {"workload": "codellama%s_arch_q40_decode_prompt%d_shared_prefix" % (a.arch, prompt_len), "branches": head_b,
                    "layers": a.layers, "graph": not a.no_graph},
         "by_batch": {str(B): {k: (round(v, 4) if isinstance(v, float) else v) for k, v in d.items()} for B, d in by_batch.items()},
     }
@@ -287,16 +304,17 @@ def main():
         rf10 = matmul_roofline(torch, model, 10, 5)
         rf100 = matmul_roofline(torch, model, 100, 3)
         result["roofline"] = {
-            "kernel": "q40_gemv_kernel at M=1: the 128 weight launches of one 7B decode step (wq|wk|wv, wo, w1|w3, w2 per layer)",
+            "kernel": "q40_gemv_kernel at M=1: the %d weight launches of one %s decode step (wq|wk|wv, wo, w1|w3, w2 per layer)"
+                      % (rf1["launches"], a.arch.upper()),
             "bound": "hbm", "achieved": round(rf1["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-            "frac": round(rf1["gbs"] / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH,
+            "frac": round(rf1["gbs"] / HBM_PEAK_GBS, 4), "traffic": GEMV_TRAFFIC_BYTES_PER_LAUNCH if a.arch == "7b" else None,
             "avg_launch_us": round(rf1["avg_us"], 3), "bytes_per_launch": round(rf1["bytes_per_launch"])}
         result["rooflines_other"] = [
             {"kernel": "q40_gemv_kernel at M=10", "bound": "hbm", "achieved": round(rf10["gbs"], 1), "peak": HBM_PEAK_GBS,
              "unit": "GB/s", "frac": round(rf10["gbs"] / HBM_PEAK_GBS, 4), "avg_launch_us": round(rf10["avg_us"], 3)},
             {"kernel": "q40_gemm_kernel at M=100", "bound": "mfma", "achieved": round(rf100["tflops"], 1),
              "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(rf100["tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
-             "hbm_gbs": round(rf100["gbs"], 1), "avg_launch_us": round(rf100["avg_us"], 3), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH},
+             "hbm_gbs": round(rf100["gbs"], 1), "avg_launch_us": round(rf100["avg_us"], 3), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH if a.arch == "7b" else None},
         ]
         att = attention_roofline(torch)
         result["rooflines_other"].append(
@@ -306,7 +324,7 @@ def main():
              "frac": round(att["gbs"] / HBM_PEAK_GBS, 4), "avg_call_us": round(att["us"], 2), "bytes_per_call": att["bytes"]})
         if 1 in by_batch and by_batch[1]["path"].startswith("persistent"):
             # the whole step is one launch: every weight, the prefix KV and the suffix KV once
-            b1 = lin_bytes + prefix_bytes + t_mid * a.layers * 2 * 32 * 68
+            b1 = lin_bytes + prefix_bytes + t_mid * suffix_row_bytes
             result["rooflines_other"].append(
                 {"kernel": "decode_mega_kernel at M=1 (one launch per step; bound from the step time less lm_head/argmax is not separated)",
                  "bound": "hbm", "achieved": round(b1 / (by_batch[1]["ms_per_step"] * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,

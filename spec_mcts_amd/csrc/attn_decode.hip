@@ -427,10 +427,13 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillParams p) {
     }
 }
 
-// One wave per (branch b, kv head hk).  PARTIAL: the pass over the suffix and the new token leaves an un-normalised
+// One wave per (branch b, query head h): the query heads of one kv head walk the same suffix rows in different
+// waves (the rows come from the cache after the first), so a wave's chain of memory round trips does not grow with
+// the number of query heads per kv head.  PARTIAL: the pass over the suffix and the new token leaves an un-normalised
 // partial (split index p.splits) for the workgroup that merges, instead of folding in the prefix partials itself.
 template <bool FUSED, bool PARTIAL>
-__device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int hk) {
+__device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int h) {
+    const int hk = h / p.n_rep;
     __shared__ __attribute__((aligned(16))) half_t s_kv[FUSED ? 4 : 1][2][ATT_D];     // FUSED: this wave's new k and v rows
     const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
     const int wave = threadIdx.x >> 6;
@@ -471,9 +474,9 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
         const int kcol = (p.H + hk) * ATT_D, vcol = (p.H + p.Hkv + hk) * ATT_D;
         half_t k1 = qkv_value(p, b, kcol + lane), k2 = qkv_value(p, b, kcol + lane + 64);
         const half_t v1 = qkv_value(p, b, vcol + lane), v2 = qkv_value(p, b, vcol + lane + 64);
-        q_first = fused_q(hk * p.n_rep, pos);
+        q_first = fused_q(h, pos);
         rope_pair2(k1, k2, p.cos_tab[(long)pos * 64 + lane], p.sin_tab[(long)pos * 64 + lane]);
-        if (t >= 0 && t < p.app_smax) {
+        if (h == hk * p.n_rep && t >= 0 && t < p.app_smax) {     // the first query head of a kv head appends the rows
             const long row = ((long)b * p.app_smax + t) * p.Hkv + hk;
             kv_store_row2(k1, k2, p.app_k + row * 64, p.app_ks + row * 2, lane);
             kv_store_row2(v1, v2, p.app_v + row * 64, p.app_vs + row * 2, lane);
@@ -483,11 +486,10 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
         // same wave writes and reads: LDS operations of a wave complete in order
     }
 
-    for (int rep = 0; rep < p.n_rep; ++rep) {
-        const int h = hk * p.n_rep + rep;
+    {
         RowRegs qr;
         if (!FUSED) qr = row_from_fp16(p.q + ((long)b * p.H + h) * ATT_D, c);
-        else qr = rep == 0 ? q_first : fused_q(h, pos);
+        else qr = q_first;
         SoftState st;
         st.m = -INFINITY;
         st.l = 0.f;
@@ -497,7 +499,7 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
         // Every load below is issued before its first use, a batch at a time: a wave has few rows to visit
         // (tens, a quarter each per group), so its time is the number of memory round trips it makes in a row.
         // ---- loads for the end of the pass: the new token's exact K/V, the first two prefix partials ----
-        const int qrow = b * p.n_rep + rep;
+        const int qrow = b * p.n_rep + (h - hk * p.n_rep);
         const bool has_cur = (FUSED || p.cur_k != nullptr) && g == 0;
         RowRegs cur_kr = qr, cur_vr = qr;
         if (has_cur) {
@@ -543,7 +545,7 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
             constexpr int U = UQ;
             for (int t0 = g; t0 < len; t0 += 4 * U) {
                 uint32_t kb[U], vb[U], ksc[U], vsc[U];
-                if (FUSED && rep == 0 && t0 == g) {
+                if (FUSED && t0 == g) {
 #pragma unroll
                     for (int u = 0; u < U; ++u) { kb[u] = kb0[u]; vb[u] = vb0[u]; ksc[u] = ksc0[u]; vsc[u] = vsc0[u]; }
                 } else {
@@ -601,13 +603,13 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
 template <bool FUSED>
 __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
     const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (item >= (long)p.B * p.Hkv) return;
-    attn_suffix_body<FUSED, false>(p, (int)(item / p.Hkv), (int)(item % p.Hkv));
+    if (item >= (long)p.B * p.H) return;
+    attn_suffix_body<FUSED, false>(p, (int)(item / p.H), (int)(item % p.H));
 }
 
 // ---- the whole decode attention in ONE launch -----------------------------------------------------------------
-// grid (splits + ceil(B / 4), kv heads): workgroups x < splits take a slice of the prefix, the others four
-// branches' suffix + new token each (one wave per branch).  Every workgroup leaves partials with device-scope
+// grid (splits + ceil(Bq / 4), kv heads): workgroups x < splits take a slice of the prefix, the others the suffix
+// + new token of four of the kv head's Bq = B x n_rep queries (one wave per query).  Every workgroup leaves partials with device-scope
 // stores and counts itself in on the counters of the query tiles (16 queries of a kv head) it contributed to;
 // the workgroup that completes a tile's count merges that tile's partials in split order (so the result does
 // not depend on which workgroup that is), normalises and writes the output.  Nobody waits for anybody.
@@ -620,16 +622,15 @@ __global__ __launch_bounds__(256, 2) void attn_one_kernel(AttnParams p) {
     const int hk = blockIdx.y;
     const int tid = threadIdx.x;
     const int q_tiles = (p.Bq + 15) / 16;
-    const int per_wg = 4 * p.n_rep;            // queries of one suffix workgroup (four branches)
+    constexpr int per_wg = 4;                  // queries of one suffix workgroup (one per wave)
     int tile_lo = 0, tile_hi = q_tiles - 1;    // query tiles this workgroup contributed to
     if ((int)blockIdx.x < p.splits) {
         attn_prefix_body<FUSED, true, ATT_ONE_TW>(p, blockIdx.x, hk);
     } else {
         const int j = (int)blockIdx.x - p.splits;
-        const int b = 4 * j + (tid >> 6);
-        if (b < p.B) attn_suffix_body<FUSED, true>(p, b, hk);
-        tile_lo = (j * per_wg) / 16;
-        tile_hi = (min(p.Bq, (j + 1) * per_wg) - 1) / 16;
+        const int qrow = 4 * j + (tid >> 6);   // query of this kv head: branch qrow / n_rep, its query head qrow % n_rep
+        if (qrow < p.Bq) attn_suffix_body<FUSED, true>(p, qrow / p.n_rep, hk * p.n_rep + qrow % p.n_rep);
+        tile_lo = tile_hi = (4 * j) / 16;      // four consecutive queries never straddle a tile of 16
     }
     wait_vmem();                               // this wave's partials have reached memory ...
     __syncthreads();                           // ... and those of the whole workgroup
@@ -650,24 +651,44 @@ __global__ __launch_bounds__(256, 2) void attn_one_kernel(AttnParams p) {
     }
     __syncthreads();
 
-    // ---- merge the completed tiles: 16 lanes per query (dims 4cc.. and 64+4cc..), 16 queries per tile ----
-    const int cc = tid & 15;
+    // ---- merge the completed tiles: 16 lanes per query (dims 4cc.. and 64+4cc..), 16 groups of 16 lanes ----
+    // A tile of nq queries (npow = nq rounded up to a power of two) gives each query sub = 16 / npow consecutive
+    // groups; group `si` of a query folds partials si, si + sub, ... (its loads go out together, four partials at
+    // a time).  The groups of a query are then folded within their wave by lane exchange and across waves through
+    // LDS.  The order depends only on the shape, not on which workgroup merges.
+    __shared__ float s_merge[4][16][10];
+    const int cc = tid & 15, gi = tid >> 4, wave = tid >> 6;
     const int n_part = p.splits + 1;
     for (int qt = tile_lo; qt <= tile_hi; ++qt) {
-        if (s_last[qt] == 0u) continue;
-        const int qrow = 16 * qt + (tid >> 4);
-        if (qrow >= p.Bq) continue;
+        if (s_last[qt] == 0u) continue;                       // (uniform over the workgroup)
+        const int nq = min(16, p.Bq - 16 * qt);
+        int npow = 1;
+        while (npow < nq) npow <<= 1;
+        const int sub = 16 / npow;
+        const int qi = gi / sub, si = gi & (sub - 1);
+        const int qrow = 16 * qt + qi;
+        const bool live = qi < nq;
         float m = -INFINITY, l = 0.f;
         float o[8];
 #pragma unroll
         for (int j = 0; j < 8; ++j) o[j] = 0.f;
-        for (int s0 = 0; s0 < n_part; s0 += 4) {
+        auto fold = [&](float pm, float pl, const float (&po)[8]) {
+            const float m_new = fmaxf(m, pm);
+            if (m_new != -INFINITY) {
+                const float c1 = exp2f(m - m_new), c2 = exp2f(pm - m_new);
+                m = m_new;
+                l = l * c1 + pl * c2;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) o[j] = o[j] * c1 + po[j] * c2;
+            }
+        };
+        for (int s0 = si; live && s0 < n_part; s0 += 4 * sub) {
             f4 lo[4], hi[4];
             float pm[4], pl[4];
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                if (s0 + u < n_part) {
-                    const long base = ((long)(s0 + u) * p.Hkv + hk) * p.Bq + qrow;
+                if (s0 + u * sub < n_part) {
+                    const long base = ((long)(s0 + u * sub) * p.Hkv + hk) * p.Bq + qrow;
                     lo[u] = ld_f4(p.part_o + base * ATT_D + 4 * cc);
                     hi[u] = ld_f4(p.part_o + base * ATT_D + 64 + 4 * cc);
                     pm[u] = ld_f32(p.part_ml + base * 2);
@@ -676,18 +697,38 @@ __global__ __launch_bounds__(256, 2) void attn_one_kernel(AttnParams p) {
             }
 #pragma unroll
             for (int u = 0; u < 4; ++u) {
-                if (s0 + u < n_part) {
-                    const float m_new = fmaxf(m, pm[u]);
-                    if (m_new != -INFINITY) {
-                        const float c1 = exp2f(m - m_new), c2 = exp2f(pm[u] - m_new);
-                        m = m_new;
-                        l = l * c1 + pl[u] * c2;
-#pragma unroll
-                        for (int j = 0; j < 4; ++j) { o[j] = o[j] * c1 + lo[u][j] * c2; o[4 + j] = o[4 + j] * c1 + hi[u][j] * c2; }
-                    }
+                if (s0 + u * sub < n_part) {
+                    const float po[8] = {lo[u][0], lo[u][1], lo[u][2], lo[u][3], hi[u][0], hi[u][1], hi[u][2], hi[u][3]};
+                    fold(pm[u], pl[u], po);
                 }
             }
         }
+        // groups of one wave (sub >= 2: neighbours, sub >= 4: all four); every lane of the wave takes part
+        for (int sh = 16; sh <= 32 && sh < 16 * sub; sh <<= 1) {
+            const float m2 = __shfl_xor(m, sh, 64), l2 = __shfl_xor(l, sh, 64);
+            float o2[8];
+#pragma unroll
+            for (int j = 0; j < 8; ++j) o2[j] = __shfl_xor(o[j], sh, 64);
+            fold(m2, l2, o2);
+        }
+        if (sub > 4) {                                        // a query spans sub / 4 waves (uniform over the workgroup)
+            if ((gi & 3) == 0) {
+                float *mine = s_merge[wave][cc];
+                mine[0] = m; mine[1] = l;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) mine[2 + j] = o[j];
+            }
+            __syncthreads();
+            if (si == 0 && live) {
+                for (int k = 1; k < sub / 4; ++k) {
+                    const float *other = s_merge[wave + k][cc];
+                    const float po[8] = {other[2], other[3], other[4], other[5], other[6], other[7], other[8], other[9]};
+                    fold(other[0], other[1], po);
+                }
+            }
+            __syncthreads();                                  // s_merge is free for the next tile
+        }
+        if (si != 0 || !live) continue;
         const float inv = l > 0.f ? 1.0f / l : 0.f;
         const int b = qrow / p.n_rep, h = hk * p.n_rep + qrow % p.n_rep;
         half_t *op = p.out + ((long)b * p.H + h) * ATT_D;
@@ -757,7 +798,7 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
         p.counters = (uint32_t *)workspace;
         p.part_o = (float *)((char *)workspace + ATT_COUNTER_BYTES);
         p.part_ml = p.part_o + n_part * ATT_D;
-        hipLaunchKernelGGL(attn_one_kernel<false>, dim3(p.splits + (B + 3) / 4, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(attn_one_kernel<false>, dim3(p.splits + (p.Bq + 3) / 4, Hkv), dim3(256), 0, (hipStream_t)stream, p);
         return launch_status();
     }
     size_t n_part = (size_t)p.splits * Hkv * p.Bq;
@@ -767,7 +808,7 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
     p.part_ml = p.part_o + n_part * ATT_D;
     if (p.splits > 0)
         hipLaunchKernelGGL(attn_prefix_kernel<false>, dim3(p.splits, Hkv), dim3(256), 0, (hipStream_t)stream, p);
-    long items = (long)B * Hkv;
+    long items = (long)B * H;
     hipLaunchKernelGGL(attn_suffix_kernel<false>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
 }
@@ -845,7 +886,7 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
         p.counters = (uint32_t *)workspace;
         p.part_o = (float *)((char *)workspace + ATT_COUNTER_BYTES);
         p.part_ml = p.part_o + n_part * ATT_D;
-        hipLaunchKernelGGL(attn_one_kernel<true>, dim3(p.splits + (B + 3) / 4, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(attn_one_kernel<true>, dim3(p.splits + (p.Bq + 3) / 4, Hkv), dim3(256), 0, (hipStream_t)stream, p);
         return launch_status();
     }
     size_t n_part = (size_t)p.splits * Hkv * p.Bq;
@@ -855,7 +896,7 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
     p.part_ml = p.part_o + n_part * ATT_D;
     if (p.splits > 0)
         hipLaunchKernelGGL(attn_prefix_kernel<true>, dim3(p.splits, Hkv), dim3(256), 0, (hipStream_t)stream, p);
-    long items = (long)B * Hkv;
+    long items = (long)B * H;
     hipLaunchKernelGGL(attn_suffix_kernel<true>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
 }

@@ -283,7 +283,8 @@ class Transformer(nn.Module):
         self.fused_sampler = True          # generate(): temperature / top-k / draw as one kernel instead of five torch ops
         self.silu_in_matmul = True         # up to 2 rows: w2's launch makes its own SiLU(gate)*up activations
         self.tiled_weights = True          # the fused path streams tiled copies of the weights (LinearQ4_0.operand)
-        self.attn_single_launch = True     # up to 16 branches: prefix slices, suffix passes and the merge in one launch (slower above)
+        self.attn_single_launch = True     # up to 16 queries per kv head: prefix slices, suffix passes and the merge in one launch
+                                           # (above, the one workgroup that merges a kv head's query tiles takes longer than a launch)
         self.attn_from_qkv = True          # up to 16 branches the attention takes the wq|wk|wv product itself, in one launch
         self.persistent_max_branches = 4   # with persistent = True: largest batch that uses the kernel (it takes up to 16)
         self._step_kernels = {}       # branches -> K.DecodeStepKernel
@@ -376,14 +377,16 @@ class Transformer(nn.Module):
                     # RoPE and the KV append happen inside the attention kernels (one launch fewer)
                     o = K.shared_prefix_attn_qkv(qkv, H, Hkv, D, cos, sin, pos_dev, att.cache_prompt_k[0], att.cache_prompt_v[0],
                                                  att.cache_prompt_len, att.cache_k, att.cache_k_s, att.cache_v, att.cache_v_s,
-                                                 p.max_seq_len, t_dev).view(M, H * D)
+                                                 p.max_seq_len, t_dev,
+                                                 single_launch=self.attn_single_launch and M * (H // Hkv) <= 16).view(M, H * D)
                 else:
                     q, k, v = K.partial_rope_append_kv(qkv, H, Hkv, D, cos, sin, pos_dev, att.cache_k, att.cache_k_s,
                                                        att.cache_v, att.cache_v_s, p.max_seq_len, t_dev)
                     o = K.shared_prefix_attn(q, att.cache_prompt_k[0], att.cache_prompt_v[0], att.cache_prompt_len,
                                              suffix_k=att.cache_k, suffix_v=att.cache_v, suffix_ks=att.cache_k_s,
                                              suffix_vs=att.cache_v_s, Smax=p.max_seq_len, lens=t_dev, lens_stride=0,
-                                             cur_k=k, cur_v=v, single_launch=self.attn_single_launch and M <= 16).view(M, H * D)
+                                             cur_k=k, cur_v=v,
+                                             single_launch=self.attn_single_launch and M * (H // Hkv) <= 16).view(M, H * D)
             po = K.matmul_q40_partial(o, [att.wo.operand(tiled)])
             h, xn = K.partial_rmsnorm(po, h, layer.ffn_norm.weight, layer.ffn_norm.eps)
             gu = K.matmul_q40_partial(xn, [ff.w1.operand(tiled), ff.w3.operand(tiled)])
