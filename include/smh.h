@@ -119,6 +119,20 @@ int smh_q40_matmul_partial_tiled(const void *a, int M, int K, long lda, int nseg
 int smh_q40_matmul_partial_tiled_silu(const void *gate_up_partial, int gate_up_ksplit, int M, int K, int nseg,
                                       const void *const *tiled, const int *n, void *partial, size_t partial_bytes,
                                       smh_stream_t stream);
+/* RMSNorm.forward (hf_model_q40_kv_shared.py:85-94) of the residual stream followed by a linear, for up to 16 rows, as two
+ * launches instead of three.  smh_partial_residual_sumsq is the first half of smh_partial_rmsnorm spread over 16
+ * workgroups a row: h_out = h_in + fp16(sum of the slabs) and sums[m][0..15], partial sums of squares of h_out's row m
+ * (fp32; added in index order they are smh_partial_rmsnorm's sum bit for bit).  smh_q40_matmul_partial_tiled_norm is
+ * smh_q40_matmul_partial_tiled on a = RMSNorm(h) * norm_weight, which every workgroup makes for its own K-slice from h,
+ * sums and norm_weight with smh_partial_rmsnorm's roundings; the slabs it leaves equal those of smh_partial_rmsnorm +
+ * smh_q40_matmul_partial_tiled.  M rows x the K-slice must fit the workgroup's LDS: smh_q40_norm_in_fits says (1 / 0)
+ * whether a shape does; where it does not, smh_partial_rmsnorm is the path. */
+int smh_partial_residual_sumsq(const void *partial, int ksplit, int M, int N, const void *h_in, void *h_out, void *sums,
+                               smh_stream_t stream);
+int smh_q40_norm_in_fits(int M, int K, int nseg, const int *n);
+int smh_q40_matmul_partial_tiled_norm(const void *h, long ldh, const void *sums, const void *norm_weight, float eps,
+                                      int M, int K, int nseg, const void *const *tiled, const int *n,
+                                      void *partial, size_t partial_bytes, smh_stream_t stream);
 int smh_partial_reduce(const void *partial, int ksplit, int M, int n_total, int col0, int N, void *c,
                        long ldc, int epilogue, const void *residual, long ldr, smh_stream_t stream);
 int smh_partial_rmsnorm(const void *partial, int ksplit, int M, int N, const void *h_in,

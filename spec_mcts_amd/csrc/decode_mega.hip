@@ -430,7 +430,7 @@ __device__ __forceinline__ void load_x(CParams &p, CLayer &L, int ph, uint8_t *x
         for (int i = 0; i < 8; ++i) tot += v[i];
         tot += __shfl_xor(tot, 16, 64);
         tot += __shfl_xor(tot, 32, 64);
-        const float r = 1.0f / sqrtf(tot / (float)p.dim + p.eps);
+        const float r = rms_factor(tot, p.dim, p.eps);
         rstd = __shfl(r, m, 64);
     }
     const half_t *src;
@@ -451,7 +451,7 @@ __device__ __forceinline__ void load_x(CParams &p, CLayer &L, int ph, uint8_t *x
             const h8 wv = *reinterpret_cast<const h8 *>(wn + k);
 #pragma unroll
             for (int i = 0; i < 8; ++i) {
-                const half_t nv = (half_t)((float)v[i] * rstd);
+                const half_t nv = scale_to_half(v[i], rstd);
                 v[i] = nv * wv[i];
             }
         }

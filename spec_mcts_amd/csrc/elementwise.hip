@@ -23,14 +23,14 @@ __global__ __launch_bounds__(256) void rmsnorm_kernel(const half_t *__restrict__
     if ((threadIdx.x & 63) == 0) s_part[threadIdx.x >> 6] = ss;
     __syncthreads();
     const float total = s_part[0] + s_part[1] + s_part[2] + s_part[3];
-    const float r = 1.0f / sqrtf(total / (float)dim + eps);
+    const float r = rms_factor(total, dim, eps);
     for (int i = threadIdx.x * 8; i < dim; i += 256 * 8) {
         h8 v = *reinterpret_cast<const h8 *>(xr + i);
         h8 w = *reinterpret_cast<const h8 *>(wt + i);
         h8 o;
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
-            half_t n = (half_t)((float)v[j] * r);
+            half_t n = scale_to_half(v[j], r);
             o[j] = n * w[j];
         }
         *reinterpret_cast<h8 *>(orow + i) = o;

@@ -195,14 +195,14 @@ __device__ __forceinline__ void matmul_finish(const MatmulFinish &f, const float
         float tot = 0.f;
         for (int u = lane; u < units; u += 64) tot += ld_f32(f.ssq + (long)u * M + m);
         tot = wave_sum(tot);
-        const float r = 1.0f / sqrtf(tot / (float)n_total + f.eps);
+        const float r = rms_factor(tot, n_total, f.eps);
         for (int c4 = 4 * lane; c4 < n_total; c4 += 256) {
             const h4 hv = ld_h4(f.h_out + (long)m * n_total + c4);
             const h4 w = *reinterpret_cast<const h4 *>(f.norm_w + c4);
             h4 o;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                const half_t nv = (half_t)((float)hv[j] * r);
+                const half_t nv = scale_to_half(hv[j], r);
                 o[j] = nv * w[j];
             }
             *reinterpret_cast<h4 *>(f.xn_out + (long)m * n_total + c4) = o;

@@ -72,7 +72,7 @@ __global__ __launch_bounds__(1024) void partial_rmsnorm_kernel(const void *__res
             hv[ps] = v;
             if (h_out != nullptr) *reinterpret_cast<h4 *>(h_out + (long)m * N + n) = v;
 #pragma unroll
-            for (int j = 0; j < 4; ++j) ss += (float)v[j] * (float)v[j];
+            for (int j = 0; j < 4; ++j) ss = sumsq_add(ss, (float)v[j]);
         }
     }
     ss = wave_sum(ss);
@@ -81,7 +81,7 @@ __global__ __launch_bounds__(1024) void partial_rmsnorm_kernel(const void *__res
     float total = 0.f;
 #pragma unroll
     for (int w = 0; w < 16; ++w) total += s_part[w];
-    const float r = 1.0f / sqrtf(total / (float)N + eps);
+    const float r = rms_factor(total, N, eps);
 #pragma unroll
     for (int ps = 0; ps < MAXPASS; ++ps) {
         const int n = (ps * 1024 + threadIdx.x) * 4;
@@ -90,12 +90,53 @@ __global__ __launch_bounds__(1024) void partial_rmsnorm_kernel(const void *__res
             h4 o;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                half_t nv = (half_t)((float)hv[ps][j] * r);
+                half_t nv = scale_to_half(hv[ps][j], r);
                 o[j] = nv * w[j];
             }
             *reinterpret_cast<h4 *>(xn_out + (long)m * N + n) = o;
         }
     }
+}
+
+// ---- residual add + sums of squares (the first half of partial_rmsnorm_kernel, spread over 16 workgroups a row) ----
+// grid (16, M), one wave each: wave w of a row is wave w of partial_rmsnorm_kernel's workgroup (same columns per
+// thread, same order of additions), so sums[m][0..15] added in index order give that kernel's sum of squares bit
+// for bit.  The consumer (the matmul that follows, q40_gemv_kernel LAYOUT 3) normalises its own K-slice.
+__global__ __launch_bounds__(64) void partial_residual_sumsq_kernel(const void *__restrict__ partial, int ksplit, int M, int N,
+                                                                    const half_t *__restrict__ h_in, half_t *__restrict__ h_out,
+                                                                    float *__restrict__ sums) {
+    const int m = blockIdx.y;
+    const int vt = blockIdx.x * 64 + threadIdx.x;      // thread index inside partial_rmsnorm_kernel's workgroup
+    const long slab = (long)M * N;
+    constexpr int MAXPASS = 4;      // N <= 16384
+    f4 acc[MAXPASS];
+    h4 res[MAXPASS];
+#pragma unroll
+    for (int ps = 0; ps < MAXPASS; ++ps) {
+        const int n = (ps * 1024 + vt) * 4;
+        if (n < N) {
+            acc[ps] = slab_sum4(partial, (long)m * N + n, slab, ksplit, slab_is_half(M));
+            if (h_in != nullptr) res[ps] = *reinterpret_cast<const h4 *>(h_in + (long)m * N + n);
+        }
+    }
+    float ss = 0.f;
+#pragma unroll
+    for (int ps = 0; ps < MAXPASS; ++ps) {
+        const int n = (ps * 1024 + vt) * 4;
+        if (n < N) {
+            h4 v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                v[j] = (half_t)acc[ps][j];
+                if (h_in != nullptr) v[j] = (half_t)((float)res[ps][j] + (float)v[j]);
+            }
+            *reinterpret_cast<h4 *>(h_out + (long)m * N + n) = v;
+#pragma unroll
+            for (int j = 0; j < 4; ++j) ss = sumsq_add(ss, (float)v[j]);
+        }
+    }
+    ss = wave_sum(ss);
+    if (threadIdx.x == 0) sums[(long)m * SMH_NORM_SUMS + blockIdx.x] = ss;
 }
 
 // ---- SwiGLU gate ------------------------------------------------------------------------------------
@@ -277,6 +318,40 @@ extern "C" int smh_q40_matmul_partial_tiled_silu(const void *gate_up_partial, in
     return gemv_launch(p, (hipStream_t)stream);
 }
 
+extern "C" int smh_q40_norm_in_fits(int M, int K, int nseg, const int *n) {
+    MatmulParams p;
+    if (M <= 0 || M > SMH_GEMV_MAX_M || K % 32 != 0) return 0;
+    int st = fill_params(p, nullptr, M, K, (K + 7) / 8 * 8, nseg, nullptr, nullptr, n, "smh_q40_norm_in_fits");
+    return st < 0 ? st : (gemv_norm_in_fits(p) ? 1 : 0);
+}
+
+extern "C" int smh_q40_matmul_partial_tiled_norm(const void *h, long ldh, const void *sums, const void *norm_weight, float eps,
+                                                 int M, int K, int nseg, const void *const *tiled, const int *n,
+                                                 void *partial, size_t partial_bytes, smh_stream_t stream) {
+    const char *who = "smh_q40_matmul_partial_tiled_norm";
+    MatmulParams p;
+    int st = fill_params(p, h, M, K, ldh, nseg, tiled, nullptr, n, who);
+    if (st) return st;
+    if (M == 0) return 0;
+    SMH_REQUIRE(M <= SMH_GEMV_MAX_M, "%s: M=%d (at most %d rows; use smh_partial_rmsnorm above)", who, M, SMH_GEMV_MAX_M);
+    SMH_REQUIRE(K % 32 == 0 && ldh % 8 == 0, "%s: K=%d must be a multiple of 32, ldh=%ld of 8", who, K, ldh);
+    SMH_REQUIRE(h && sums && norm_weight && tiled && partial, "%s: null pointer", who);
+    SMH_REQUIRE(((uintptr_t)h & 15) == 0 && ((uintptr_t)norm_weight & 15) == 0 && ((uintptr_t)sums & 15) == 0, "%s: h, norm_weight and sums must be 16-byte aligned", who);
+    for (int i = 0; i < nseg; ++i)
+        SMH_REQUIRE(tiled[i] && ((uintptr_t)tiled[i] & 127) == 0, "%s: weight %d is null or not 128-byte aligned", who, i);
+    SMH_REQUIRE(gemv_norm_in_fits(p), "%s: %d rows x K-slices of %d rows exceed %d bytes (ask smh_q40_norm_in_fits first)", who, M,
+                p.steps_per_slice * 32, SMH_NORM_IN_MAX_XS_BYTES);
+    size_t need = (size_t)p.ksplit * M * p.n_total * sizeof(float);
+    SMH_REQUIRE(partial_bytes >= need, "%s: partial buffer %zu < %zu bytes", who, partial_bytes, need);
+    p.partial = (float *)partial;
+    p.direct = 0;
+    p.tiled = 1;
+    p.norm_w = (const half_t *)norm_weight;
+    p.norm_ss = (const float *)sums;
+    p.norm_eps = eps;
+    return gemv_launch(p, (hipStream_t)stream);
+}
+
 extern "C" int smh_q40_matmul_fused(const void *a, int M, int K, long lda, int nseg, const void *const *w,
                                     const void *const *s, const int *n, void *partial, size_t partial_bytes,
                                     const smh_finish *fin, smh_stream_t stream) {
@@ -425,6 +500,17 @@ extern "C" int smh_partial_rmsnorm(const void *partial, int ksplit, int M, int N
     SMH_REQUIRE(weight && xn_out, "smh_partial_rmsnorm: null pointer");
     hipLaunchKernelGGL(partial_rmsnorm_kernel, dim3(M), dim3(1024), 0, (hipStream_t)stream, partial, ksplit, M, N,
                        (const half_t *)h_in, (const half_t *)weight, eps, (half_t *)h_out, (half_t *)xn_out);
+    return launch_status();
+}
+
+extern "C" int smh_partial_residual_sumsq(const void *partial, int ksplit, int M, int N, const void *h_in, void *h_out, void *sums,
+                                          smh_stream_t stream) {
+    SMH_REQUIRE(partial != nullptr && ksplit >= 1 && ksplit <= SMH_MAX_KSPLIT, "smh_partial_residual_sumsq: partial=%p ksplit=%d", partial, ksplit);
+    SMH_REQUIRE(M >= 0 && N > 0 && N % 4 == 0 && N <= 16384, "smh_partial_residual_sumsq: M=%d N=%d (N must be a multiple of 4, <= 16384)", M, N);
+    if (M == 0) return 0;
+    SMH_REQUIRE(h_out && sums, "smh_partial_residual_sumsq: null pointer");
+    hipLaunchKernelGGL(partial_residual_sumsq_kernel, dim3(SMH_NORM_SUMS, M), dim3(64), 0, (hipStream_t)stream, partial, ksplit, M, N,
+                       (const half_t *)h_in, (half_t *)h_out, (float *)sums);
     return launch_status();
 }
 

@@ -49,6 +49,9 @@ constexpr int STAGE_S_BYTES = 32 * 8;
 constexpr int STAGE_X_BYTES = 16 * 64;
 constexpr int STAGE_BYTES = STAGE_W_BYTES + STAGE_S_BYTES + STAGE_X_BYTES;   // 5376
 constexpr int RING_BYTES = RING_STAGES * STAGE_BYTES;                        // 16128 per wave
+// kernels that keep their activations in LDS outside the ring (LAYOUT 2 and 3) have no activation tile in a stage
+constexpr int STAGE_BYTES_NO_X = STAGE_W_BYTES + STAGE_S_BYTES;             // 4352
+constexpr int RING_BYTES_NO_X = RING_STAGES * STAGE_BYTES_NO_X;             // 13056 per wave
 
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
@@ -238,14 +241,20 @@ __device__ __forceinline__ void gemv_consume_tiled(const uint8_t *stage, int k0,
 // FINISH: the workgroup that completes a column unit also applies the operator that follows the linear
 // (matmul_finish.hpp); a separate instantiation, so that the plain kernel keeps its register budget
 // LAYOUT 0: checkpoint layout; 1: tiled weights (smh_q40_tile); 2: tiled weights and activations made from the
-// gate|up slabs by the workgroup itself (p.gu_partial): SiLU(gate) * up needs no launch of its own
+// gate|up slabs by the workgroup itself (p.gu_partial): SiLU(gate) * up needs no launch of its own; 3: tiled weights
+// and activations made from the residual stream by the workgroup itself (p.norm_w, p.norm_ss): RMSNorm needs only
+// the small launch that adds the slabs and leaves the sums of squares
 template <int WAVES, bool FINISH, int LAYOUT>
 __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // WAVES rings, then reused as red[WAVES][M][256]
     constexpr int THREADS = WAVES * 64;
     constexpr bool TILED = LAYOUT != 0;
     constexpr bool SILU_IN = LAYOUT == 2;
-    constexpr int PER_STAGE = SILU_IN ? 5 : 6;                      // vector-memory instructions per stage
+    constexpr bool NORM_IN = LAYOUT == 3;
+    constexpr bool X_IN_LDS = SILU_IN || NORM_IN;                   // activations: xs[M][slice rows] behind the rings
+    constexpr int PER_STAGE = X_IN_LDS ? 5 : 6;                     // vector-memory instructions per stage
+    constexpr int STAGE = X_IN_LDS ? STAGE_BYTES_NO_X : STAGE_BYTES;
+    constexpr int RING = RING_STAGES * STAGE;
 
     // Workgroups are dealt round-robin to the 8 XCDs (8 L2s).  Neighbouring column units share the 128-byte
     // lines of the scale rows, so each XCD takes a CONTIGUOUS run of units: a scale line is then fetched
@@ -289,7 +298,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         L.w_off = (uint32_t)(16 * lane);
         L.s_off = (uint32_t)(4 * lane);
     }
-    uint8_t *ring = lds + wave * RING_BYTES;
+    uint8_t *ring = lds + wave * RING;
 
     GemvConsts C{0x00F000F0u, 0x000F000Fu, 0x54005400u, 0x64006400u};
     asm volatile("" : "+s"(C.mask_hi), "+s"(C.mask_lo));
@@ -313,8 +322,8 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     const int full_steps = p.K / 32;        // steps below this index have all their 32 rows
     auto issue = [&](uint8_t *stage, int step) {
         if constexpr (TILED) {
-            if (step < full_steps) gemv_issue_tiled<false, !SILU_IN>(L, stage, step);
-            else gemv_issue_tiled<true, !SILU_IN>(L, stage, step);
+            if (step < full_steps) gemv_issue_tiled<false, !X_IN_LDS>(L, stage, step);
+            else gemv_issue_tiled<true, !X_IN_LDS>(L, stage, step);
         } else {
             if (step < full_steps) gemv_issue<false>(L, stage, step);
             else gemv_issue<true>(L, stage, step);
@@ -322,7 +331,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     };
     // SILU_IN: xs[M][slice rows] fp16 behind the rings.  The slab loads of this thread's share are requested first, the
     // weight stages right behind them, so that both are in flight together.
-    half_t *xs = reinterpret_cast<half_t *>(lds + WAVES * RING_BYTES);
+    half_t *xs = reinterpret_cast<half_t *>(lds + WAVES * RING);
     const int slice_k0 = step0 * 32, slice_rows = (step1 - step0) * 32;
     if constexpr (SILU_IN) {
         constexpr int MAXQ = SMH_SILU_IN_MAX_M * SMH_SILU_IN_MAX_K / 4 / THREADS;     // quads of columns per thread
@@ -345,7 +354,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         }
 #pragma unroll
         for (int i = 0; i < RING_STAGES; ++i)
-            if (i < n_steps) issue(ring + i * STAGE_BYTES, first + i * WAVES);
+            if (i < n_steps) issue(ring + i * STAGE, first + i * WAVES);
 #pragma unroll
         for (int i = 0; i < MAXQ; ++i) {
             const int idx = tid + i * THREADS;
@@ -361,12 +370,64 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // xs is complete; the DMA ring stays in flight
+    } else if constexpr (NORM_IN) {
+        // the loads of this thread's share of h (eight consecutive k of one row at a time), of the matching norm
+        // weights and, in the first threads, of a row's sums of squares go out first, the weight stages right
+        // behind them
+        constexpr int MAXO = (SMH_NORM_IN_MAX_XS_BYTES / 16 + THREADS - 1) / THREADS;     // k-octets per thread
+        float *s_r = reinterpret_cast<float *>(xs + (long)p.M * slice_rows);           // r[m], behind xs
+        h8 hv[MAXO], wv[MAXO];
+        const int octs = slice_rows / 8, total = p.M * octs;
+#pragma unroll
+        for (int i = 0; i < MAXO; ++i) {
+            const int idx = tid + i * THREADS;
+            if (idx < total) {
+                const int m = idx / octs, k = slice_k0 + 8 * (idx % octs);
+                if (k < p.K) {
+                    hv[i] = *reinterpret_cast<const h8 *>(p.a + (long)m * p.lda + k);
+                    wv[i] = *reinterpret_cast<const h8 *>(p.norm_w + k);
+                } else {
+                    hv[i] = h8{0, 0, 0, 0, 0, 0, 0, 0};
+                    wv[i] = hv[i];
+                }
+            }
+        }
+        f4 ssv[SMH_NORM_SUMS / 4];
+        if (tid < p.M) {
+#pragma unroll
+            for (int j = 0; j < SMH_NORM_SUMS / 4; ++j) ssv[j] = *reinterpret_cast<const f4 *>(p.norm_ss + (long)tid * SMH_NORM_SUMS + 4 * j);
+        }
+#pragma unroll
+        for (int i = 0; i < RING_STAGES; ++i)
+            if (i < n_steps) issue(ring + i * STAGE, first + i * WAVES);
+        if (tid < p.M) {
+            float sum = 0.f;
+#pragma unroll
+            for (int j = 0; j < SMH_NORM_SUMS; ++j) sum += ssv[j / 4][j % 4];
+            s_r[tid] = rms_factor(sum, p.K, p.norm_eps);
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // r[] is complete
+#pragma unroll
+        for (int i = 0; i < MAXO; ++i) {
+            const int idx = tid + i * THREADS;
+            if (idx < total) {
+                const float r = s_r[idx / octs];
+                h8 o;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {                  // the roundings of partial_rmsnorm_kernel
+                    const half_t nv = scale_to_half(hv[i][j], r);
+                    o[j] = nv * wv[i][j];
+                }
+                *reinterpret_cast<h8 *>(xs + (long)(idx / octs) * slice_rows + 8 * (idx % octs)) = o;
+            }
+        }
+        asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // xs is complete; the DMA ring stays in flight
     } else {
 #pragma unroll
         for (int i = 0; i < RING_STAGES; ++i)
-            if (i < n_steps) issue(ring + i * STAGE_BYTES, first + i * WAVES);
+            if (i < n_steps) issue(ring + i * STAGE, first + i * WAVES);
     }
-    const half_t *xlane = xs + (long)min(c, p.M - 1) * slice_rows + 8 * g;     // SILU_IN: this lane's row of xs, its k-octet
+    const half_t *xlane = xs + (long)min(c, p.M - 1) * slice_rows + 8 * g;     // X_IN_LDS: this lane's row of xs, its k-octet
     // the one step that may lack rows is the last step of K, hence the last one of its wave; it is
     // peeled off so that the loop has a single decoder in it
     const int n_full = first < full_steps ? min(n_steps, (full_steps - first + WAVES - 1) / WAVES) : 0;
@@ -376,20 +437,20 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         if (later >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PER_STAGE) : "memory");
         else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_STAGE) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if constexpr (SILU_IN) gemv_consume_tiled<false, true>(ring + stage * STAGE_BYTES, 0, p.K, lane, C, acc, corr, xlane + (first + i * WAVES - step0) * 32);
-        else if constexpr (TILED) gemv_consume_tiled<false>(ring + stage * STAGE_BYTES, 0, p.K, lane, C, acc, corr);
-        else gemv_consume<false>(ring + stage * STAGE_BYTES, 0, p.K, c, g, C, acc, corr);
+        if constexpr (X_IN_LDS) gemv_consume_tiled<false, true>(ring + stage * STAGE, 0, p.K, lane, C, acc, corr, xlane + (first + i * WAVES - step0) * 32);
+        else if constexpr (TILED) gemv_consume_tiled<false>(ring + stage * STAGE, 0, p.K, lane, C, acc, corr);
+        else gemv_consume<false>(ring + stage * STAGE, 0, p.K, c, g, C, acc, corr);
         if (i + RING_STAGES < n_steps) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");        // this stage's LDS reads are done
-            issue(ring + stage * STAGE_BYTES, first + (i + RING_STAGES) * WAVES);
+            issue(ring + stage * STAGE, first + (i + RING_STAGES) * WAVES);
         }
         stage = (stage + 1 == RING_STAGES) ? 0 : stage + 1;
     }
     if (n_full < n_steps) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if constexpr (SILU_IN) gemv_consume_tiled<true, true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr, xlane + (first + n_full * WAVES - step0) * 32);
-        else if constexpr (TILED) gemv_consume_tiled<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr);
-        else gemv_consume<true>(ring + stage * STAGE_BYTES, (first + n_full * WAVES) * 32, p.K, c, g, C, acc, corr);
+        if constexpr (X_IN_LDS) gemv_consume_tiled<true, true>(ring + stage * STAGE, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr, xlane + (first + n_full * WAVES - step0) * 32);
+        else if constexpr (TILED) gemv_consume_tiled<true>(ring + stage * STAGE, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr);
+        else gemv_consume<true>(ring + stage * STAGE, (first + n_full * WAVES) * 32, p.K, c, g, C, acc, corr);
     }
     __syncthreads();                        // every wave is done with its ring: reuse LDS for the sums
 
@@ -494,11 +555,17 @@ void gemv_fill_plan(MatmulParams &p) {
     gemv_plan(p.units, p.K, gemv_waves(p.M), &p.ksplit, &p.steps_per_slice);
 }
 
+bool gemv_norm_in_fits(const MatmulParams &p) {
+    return p.M <= SMH_GEMV_MAX_M && (size_t)p.M * p.steps_per_slice * 32 * sizeof(half_t) <= SMH_NORM_IN_MAX_XS_BYTES;
+}
+
 int gemv_launch(const MatmulParams &p, hipStream_t stream) {
     const int waves = gemv_waves(p.M);
     dim3 grid((unsigned)(p.units_pad * p.ksplit));
     size_t lds = (size_t)waves * RING_BYTES;                       // rings, reused for the [waves][M][256] sums
     const size_t red = (size_t)waves * p.M * GEMV_COLS * sizeof(float);
+    if (p.tiled && (p.gu_partial != nullptr || p.norm_w != nullptr))   // rings without activation tiles, xs (and r[]) behind them
+        lds = (size_t)waves * RING_BYTES_NO_X + (size_t)p.M * p.steps_per_slice * 32 * sizeof(half_t) + SMH_GEMV_MAX_M * sizeof(float);
     if (red > lds) lds = red;
     if (p.tiled) {
         if (p.fin.mode != 0 || waves != 4) {
@@ -511,12 +578,21 @@ int gemv_launch(const MatmulParams &p, hipStream_t stream) {
                           SMH_SILU_IN_MAX_K);
                 return -1;
             }
-            lds += (size_t)p.M * p.steps_per_slice * 32 * sizeof(half_t);          // xs behind the rings
             // more than 64 KB of dynamic LDS has to be allowed once (not stream work: fine under graph capture)
             static const hipError_t lds_ok = hipFuncSetAttribute((const void *)q40_gemv_kernel<4, false, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
-                                                                 4 * RING_BYTES + SMH_SILU_IN_MAX_M * SMH_SILU_IN_MAX_K * (int)sizeof(half_t));
+                                                                 80 * 1024);
             if (lds_ok != hipSuccess) return (int)lds_ok;
             hipLaunchKernelGGL((q40_gemv_kernel<4, false, 2>), grid, dim3(256), lds, stream, p);
+        } else if (p.norm_w != nullptr) {
+            if (!gemv_norm_in_fits(p)) {
+                set_error("q40 gemv: %d rows x K-slices of %d rows do not fit next to the weight rings (RMSNorm inside the matmul)", p.M,
+                          p.steps_per_slice * 32);
+                return -1;
+            }
+            static const hipError_t lds_ok = hipFuncSetAttribute((const void *)q40_gemv_kernel<4, false, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
+                                                                 80 * 1024);
+            if (lds_ok != hipSuccess) return (int)lds_ok;
+            hipLaunchKernelGGL((q40_gemv_kernel<4, false, 3>), grid, dim3(256), lds, stream, p);
         } else {
             hipLaunchKernelGGL((q40_gemv_kernel<4, false, 1>), grid, dim3(256), lds, stream, p);
         }

@@ -14,6 +14,8 @@
 #define SMH_MAX_SEGMENTS 3
 #define SMH_SILU_IN_MAX_M 2
 #define SMH_SILU_IN_MAX_K 2048      /* rows of a K-slice whose activations fit the workgroup's LDS */
+#define SMH_NORM_SUMS 16            /* partial sums of squares per row that smh_partial_residual_sumsq leaves */
+#define SMH_NORM_IN_MAX_XS_BYTES 28160   /* M x K-slice fp16 activations next to the weight rings, two workgroups per CU */
 
 #include "matmul_finish.hpp"
 
@@ -68,6 +70,12 @@ struct MatmulParams {
     // 0..K-1, up = columns K..2K-1 of the slabs), with the roundings of partial_silu_mul_kernel
     const float *gu_partial;
     int gu_ksplit;
+    // GEMV, norm_w != nullptr: `a` holds the un-normalised residual stream h; every workgroup makes its K-slice of
+    // RMSNorm(h) * norm_w itself, a[m][k] = fp16(fp16(h[m][k] * r[m]) * norm_w[k]) with r[m] = 1 / sqrt(sum / K + eps)
+    // and sum = norm_ss[m][0] + ... + norm_ss[m][SMH_NORM_SUMS - 1] added in that order (partial_rmsnorm_kernel's roundings)
+    const half_t *norm_w;
+    const float *norm_ss;
+    float norm_eps;
     MatmulFinish fin;        // fin.mode == 0: leave the slabs to another launch
 };
 
@@ -83,6 +91,7 @@ __host__ __device__ inline bool slab_is_half(int M) { return M > SMH_GEMV_MAX_M;
 int env_int(const char *name, int dflt);
 void gemv_fill_plan(MatmulParams &p);
 int gemv_launch(const MatmulParams &p, hipStream_t stream);
+bool gemv_norm_in_fits(const MatmulParams &p);     // after gemv_fill_plan: can RMSNorm be made inside the launch
 void gemm_fill_plan(MatmulParams &p);
 int gemm_launch(const MatmulParams &p, hipStream_t stream);
 

@@ -97,6 +97,25 @@ __device__ __forceinline__ float row16_sum(float v) {
     return v;
 }
 
+// ---- RMSNorm arithmetic shared by every kernel that normalises ---------------------------------------
+// Kernels that must agree bit for bit (the RMSNorm launch and the matmul that normalises its own activations) take
+// their roundings from here, so that none of them depends on what the compiler chooses to fuse in its context.
+__device__ __forceinline__ float sumsq_add(float ss, float x) { return __builtin_fmaf(x, x, ss); }
+// fp16(x * r) with the product rounded to fp32 first and to fp16 second, as x.float() * r followed by .half() rounds.
+// The empty asm keeps the compiler from merging the two into one mixed-precision multiply that converts on the fly,
+// whose results differ from the two roundings in rare last bits.
+__device__ __forceinline__ half_t scale_to_half(half_t x, float r) {
+    float f = (float)x * r;
+    asm("" : "+v"(f));
+    return (half_t)f;
+}
+__device__ __forceinline__ float rms_factor(float total, int n, float eps) {
+#pragma clang fp contract(off)
+    const float mean = total / (float)n;
+    const float shifted = mean + eps;
+    return 1.0f / sqrtf(shifted);
+}
+
 // ---- cross-workgroup hand-off inside one launch ------------------------------------------------------
 // Data written by one workgroup and read by another (possibly on a different XCD, i.e. behind a different
 // L2) travels as device-scope relaxed atomics: such stores write through to the point of coherence and

@@ -285,6 +285,9 @@ class Transformer(nn.Module):
         self.tiled_weights = True          # the fused path streams tiled copies of the weights (LinearQ4_0.operand)
         self.attn_single_launch = True     # up to 16 queries per kv head: prefix slices, suffix passes and the merge in one launch
                                            # (above, the one workgroup that merges a kv head's query tiles takes longer than a launch)
+        self.norm_in_matmul = True         # RMSNorm made by the matmul that consumes it (a shorter launch in between) ...
+        self.norm_in_max_rows = 2          # ... up to this many rows: at 10 rows the matmul's longer prologue costs more than it saves
+        self._norm_in_ok = {}
         self.attn_from_qkv = True          # up to 16 branches the attention takes the wq|wk|wv product itself, in one launch
         self.persistent_max_branches = 4   # with persistent = True: largest batch that uses the kernel (it takes up to 16)
         self._step_kernels = {}       # branches -> K.DecodeStepKernel
@@ -347,9 +350,15 @@ class Transformer(nn.Module):
         for layer in self.layers:
             att, ff = layer.attention, layer.feed_forward
             H, Hkv, D = att.n_local_heads, att.n_local_kv_heads, att.head_dim
-            h, xn = K.partial_rmsnorm(pending, h, layer.attention_norm.weight, layer.attention_norm.eps)
             tiled = self.tiled_weights
-            qkv = K.matmul_q40_partial(xn, [att.wq.operand(tiled), att.wk.operand(tiled), att.wv.operand(tiled)])
+            qkv_ops = [att.wq.operand(tiled), att.wk.operand(tiled), att.wv.operand(tiled)]
+            if pending is not None and self._norm_in(M, p.dim, qkv_ops):
+                # RMSNorm made inside the matmul: the launch before it only adds the slabs and leaves sums of squares
+                h, sums = K.partial_residual_sumsq(pending, h)
+                qkv = K.matmul_q40_partial_norm(h, sums, layer.attention_norm.weight, layer.attention_norm.eps, qkv_ops)
+            else:
+                h, xn = K.partial_rmsnorm(pending, h, layer.attention_norm.weight, layer.attention_norm.eps)
+                qkv = K.matmul_q40_partial(xn, qkv_ops)
             if start_pos == 0:
                 xq = K.partial_reduce(qkv, 0, H * D).view(bsz, seqlen, H, D)
                 xk = K.partial_reduce(qkv, H * D, Hkv * D).view(bsz, seqlen, Hkv, D)
@@ -388,8 +397,13 @@ class Transformer(nn.Module):
                                              cur_k=k, cur_v=v,
                                              single_launch=self.attn_single_launch and M * (H // Hkv) <= 16).view(M, H * D)
             po = K.matmul_q40_partial(o, [att.wo.operand(tiled)])
-            h, xn = K.partial_rmsnorm(po, h, layer.ffn_norm.weight, layer.ffn_norm.eps)
-            gu = K.matmul_q40_partial(xn, [ff.w1.operand(tiled), ff.w3.operand(tiled)])
+            gu_ops = [ff.w1.operand(tiled), ff.w3.operand(tiled)]
+            if self._norm_in(M, p.dim, gu_ops):
+                h, sums = K.partial_residual_sumsq(po, h)
+                gu = K.matmul_q40_partial_norm(h, sums, layer.ffn_norm.weight, layer.ffn_norm.eps, gu_ops)
+            else:
+                h, xn = K.partial_rmsnorm(po, h, layer.ffn_norm.weight, layer.ffn_norm.eps)
+                gu = K.matmul_q40_partial(xn, gu_ops)
             if tiled and self.silu_in_matmul and M <= K.SILU_IN_MAX_M and ff.w2.shape[1] % 32 == 0 and ff.w2.w.is_cuda:
                 pending = K.matmul_q40_partial_silu(gu, [ff.w2.operand(True)])      # SiLU(gate)*up made inside w2's launch
             else:
@@ -397,6 +411,18 @@ class Transformer(nn.Module):
                 pending = K.matmul_q40_partial(act, [ff.w2.operand(tiled)])
         _, hn = K.partial_rmsnorm(pending, h, self.norm.weight, self.norm.eps, want_h=False)
         return self.output(hn.view(bsz, seqlen, p.dim)).to(DTYPE)
+
+    def _norm_in(self, M: int, Kd: int, ops) -> bool:
+        """RMSNorm inside the matmul that follows it: tiled weights, few rows, and rows x K-slice small enough for the
+        kernel's LDS (asked of the library once per shape)."""
+        if not (self.norm_in_matmul and self.tiled_weights and M <= min(self.norm_in_max_rows, K.SMH_GEMV_MAX_M)
+                and isinstance(ops[0], K.TiledQ40)):
+            return False
+        key = (M, Kd, tuple(t.N for t in ops))
+        ok = self._norm_in_ok.get(key)
+        if ok is None:
+            ok = self._norm_in_ok[key] = K.norm_in_fits(M, Kd, list(key[2]))
+        return ok
 
     def _finish_shapes_ok(self) -> bool:
         """the in-launch finishers work on 256-column units: every linear's width must be a multiple of 256"""

@@ -214,6 +214,56 @@ def matmul_q40_partial_silu(gu: PartialProduct, linears, out: Optional[torch.Ten
     return PartialProduct(out, ks, M, n_total)
 
 
+def norm_in_fits(M: int, Kd: int, ns) -> bool:
+    """Can matmul_q40_partial_norm take this shape (M rows x its K-slice next to the weight rings)?"""
+    import ctypes
+    if M < 1 or M > SMH_GEMV_MAX_M or Kd % 32 != 0:
+        return False
+    na = (ctypes.c_int * len(ns))(*ns)
+    st = _lib.load().smh_q40_norm_in_fits(M, Kd, len(ns), na)
+    check(min(st, 0), "smh_q40_norm_in_fits")
+    return st == 1
+
+
+def partial_residual_sumsq(p: PartialProduct, h_in: Optional[torch.Tensor]):
+    """h = h_in + fp16(product), sums[m][0..15] = partial sums of squares of h's row m.  Returns (h, sums)."""
+    lib = _lib.load()
+    M, N = p.M, p.n_total
+    if h_in is not None:
+        assert h_in.shape == (M, N) and h_in.is_contiguous() and h_in.dtype == torch.float16
+    h = torch.empty((M, N), dtype=torch.float16, device=p.buf.device)
+    sums = torch.empty((M, 16), dtype=torch.float32, device=p.buf.device)
+    check(lib.smh_partial_residual_sumsq(p.buf.data_ptr(), p.ksplit, M, N, _ptr(h_in), h.data_ptr(), sums.data_ptr(), _stream()),
+          "smh_partial_residual_sumsq")
+    return h, sums
+
+
+def matmul_q40_partial_norm(h: torch.Tensor, sums: torch.Tensor, weight: torch.Tensor, eps: float, linears,
+                            out: Optional[torch.Tensor] = None) -> PartialProduct:
+    """matmul_q40_partial(RMSNorm(h) * weight, linears) in one launch for up to 16 rows and tiled weights, given the
+    sums of squares partial_residual_sumsq left: every workgroup normalises its own K-slice.  Same slabs, bit for bit,
+    as partial_rmsnorm + matmul_q40_partial."""
+    import ctypes
+    lib = _lib.load()
+    M, Kd = h.shape
+    assert h.dtype == torch.float16 and h.is_contiguous() and sums.shape == (M, 16) and sums.dtype == torch.float32
+    assert weight.numel() == Kd and weight.dtype == torch.float16
+    assert all(isinstance(t, TiledQ40) and t.K == Kd for t in linears), "tiled weights with K = the width of h"
+    ns = [t.N for t in linears]
+    ks = matmul_plan(M, Kd, ns)
+    n_total = sum(ns)
+    need = ks * M * n_total
+    if out is None:
+        out = torch.empty(need, dtype=torch.float32, device=h.device)
+    assert out.dtype == torch.float32 and out.numel() >= need and out.is_contiguous()
+    nseg = len(linears)
+    tp = (ctypes.c_void_p * nseg)(*[t.buf.data_ptr() for t in linears])
+    na = (ctypes.c_int * nseg)(*ns)
+    check(lib.smh_q40_matmul_partial_tiled_norm(h.data_ptr(), Kd, sums.data_ptr(), weight.data_ptr(), float(eps), M, Kd, nseg, tp, na,
+                                                out.data_ptr(), out.numel() * 4, _stream()), "smh_q40_matmul_partial_tiled_norm")
+    return PartialProduct(out, ks, M, n_total)
+
+
 def partial_reduce(p: PartialProduct, col0: int = 0, N: Optional[int] = None, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
     lib = _lib.load()
     N = p.n_total - col0 if N is None else N

@@ -131,3 +131,79 @@ def test_w2_that_makes_its_own_silu_activations(M, K, n1, n2):
     n = want.ksplit * M * want.n_total
     assert got.ksplit == want.ksplit
     assert torch.equal(got.buf[:n].view(torch.int32), want.buf[:n].view(torch.int32))
+
+
+@pytest.mark.parametrize("M", [1, 2, 7, 10, 16])
+@pytest.mark.parametrize("n0,K,ns", [(1024, 4096, (4096, 1024, 1024)), (256, 4096, (11008, 11008)), (384, 512, (384,)),
+                                     (512, 8192, (1024, 256)), (256, 1152, (128, 256))])
+def test_matmul_that_makes_its_own_rmsnorm(M, n0, K, ns):
+    """smh_partial_residual_sumsq + smh_q40_matmul_partial_tiled_norm against smh_partial_rmsnorm +
+    smh_q40_matmul_partial_tiled on the slabs of a first matmul (n0 -> K) and a residual: the same residual stream and
+    the same slabs, bit for bit, wherever the library says the shape fits."""
+    from spec_mcts_amd import kernels as Kn
+    g = torch.Generator().manual_seed(960 + M + K)
+    w0 = _weight(n0, K, 961 + K)
+    t0 = Kn.tile_q40(w0[0].cuda(), w0[1].cuda(), n0, K)
+    ops = []
+    for i, n in enumerate(ns):
+        w = _weight(K, n, 962 + K + i)
+        ops.append(Kn.tile_q40(w[0].cuda(), w[1].cuda(), K, n))
+    x = (torch.randn((M, n0), generator=g) * 0.8).half().cuda()
+    resid = torch.randn((M, K), generator=g).half().cuda()
+    norm_w = (1.0 + 0.2 * torch.randn(K, generator=g)).half().cuda()
+    eps = 1e-5
+    first = Kn.matmul_q40_partial(x, [t0])
+    h_want, xn = Kn.partial_rmsnorm(first, resid, norm_w, eps)
+    want = Kn.matmul_q40_partial(xn, ops)
+    if not Kn.norm_in_fits(M, K, list(ns)):
+        h, sums = Kn.partial_residual_sumsq(first, resid)
+        with pytest.raises(RuntimeError, match="K-slices"):
+            Kn.matmul_q40_partial_norm(h, sums, norm_w, eps, ops)
+        return
+    h, sums = Kn.partial_residual_sumsq(first, resid)
+    got = Kn.matmul_q40_partial_norm(h, sums, norm_w, eps, ops)
+    torch.cuda.synchronize()
+    assert torch.equal(h, h_want)
+    # the sums of squares, added in index order in fp32, against fp64 of the same row
+    ref = (h.double() ** 2).sum(1)
+    tot = sums.double().sum(1)
+    assert torch.allclose(tot, ref, rtol=1e-5)
+    n = want.ksplit * M * want.n_total
+    assert got.ksplit == want.ksplit
+    assert torch.equal(got.buf[:n].view(torch.int32), want.buf[:n].view(torch.int32))
+
+
+def test_rmsnorm_in_matmul_shape_limits():
+    """the 70B-architecture w1|w3 launch holds one row's K-slice (4096 of 8192) but not ten; M above 16 never fits"""
+    from spec_mcts_amd import kernels as Kn
+    assert Kn.norm_in_fits(1, 8192, [28672, 28672])
+    assert not Kn.norm_in_fits(10, 8192, [28672, 28672])
+    assert Kn.norm_in_fits(16, 4096, [11008, 11008])
+    assert not Kn.norm_in_fits(17, 4096, [4096])
+
+
+def test_model_logits_do_not_depend_on_where_rmsnorm_is_made():
+    """the fused forward with RMSNorm inside the matmuls against the same forward with partial_rmsnorm launches: equal bit
+    for bit at decode with 1, 3 and 4 branches"""
+    from spec_mcts_amd import ModelArgs
+    from spec_mcts_amd.load_q40 import load_q40
+    cfg = dict(dim=512, n_layers=3, n_heads=4, n_kv_heads=2, vocab_size=384, multiple_of=128, max_batch_size=4,
+               max_seq_len=16, max_prompt_seq_len=48)
+    oargs = O.OracleArgs(**cfg)
+    sd = O.random_q40_state_dict(oargs, seed=971)
+    model = load_q40(dict(sd), ModelArgs(**cfg), device="cuda:0")
+    prompt = torch.randint(0, cfg["vocab_size"], (1, 21), generator=torch.Generator().manual_seed(972)).cuda()
+    for B in (1, 3, 4):
+        tok = torch.randint(0, cfg["vocab_size"], (B, 1), generator=torch.Generator().manual_seed(973 + B)).cuda()
+
+        def run():
+            model.resetSeq()
+            return [model(prompt, 0).clone(), model(tok, 21).clone(), model(tok, 22).clone()]
+
+        model.norm_in_matmul, model.norm_in_max_rows = True, 16
+        a = run()
+        assert model._norm_in_ok and all(model._norm_in_ok.values())
+        model.norm_in_matmul = False
+        b = run()
+        for x, y in zip(a, b):
+            assert torch.equal(x, y)
