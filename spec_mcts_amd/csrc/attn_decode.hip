@@ -3,12 +3,13 @@
 //     || the new token's exact fp16 K/V ].
 //
 // Two kernels.
-//  1. attn_prefix_kernel, grid (splits, kv heads): a workgroup stages one slice of the prefix for one
-//     kv head in LDS ONCE (K row-major, V transposed) and every branch's query for that head is
-//     multiplied against it on the matrix cores: the B queries are the N dimension of
+//  1. attn_prefix_kernel, grid (splits, kv heads, query groups): a workgroup stages one slice of the
+//     prefix for one kv head in LDS ONCE (K row-major, V transposed) and the branches' queries for
+//     that head are multiplied against it on the matrix cores: the queries are the N dimension of
 //     S^T = K . Q^T and of O^T = V^T . P^T, so the prefix is read from HBM once per head instead of
-//     once per branch.  Each (slice, query) leaves an un-normalised partial (max, sum, o[128]).
-//  2. attn_suffix_kernel, one wave per (branch, kv head): streams the branch's own suffix rows
+//     once per branch (with many queries a slice's query tiles are dealt to a few workgroups, which
+//     re-read it from the cache).  Each (slice, query) leaves an un-normalised partial (max, sum, o[128]).
+//  2. attn_suffix_kernel, one wave per (branch, query head): streams the branch's own suffix rows
 //     (HBM-bound; Q4_0 rows are decoded in registers), keeps an online softmax per 16-lane group,
 //     folds in the prefix partials and the new token, normalises and writes fp16.
 // Scores and softmax are fp32 throughout (exp2 of log2(e)-scaled scores); probabilities are rounded
@@ -111,8 +112,9 @@ __device__ __forceinline__ int vt_pos(int t) {
 
 // COHERENT: the partials are read by another workgroup of the same launch (device-scope stores)
 // TWM: most prefix rows a workgroup takes (p.tw <= TWM), which sizes its LDS
+// qg, n_qg: this workgroup takes the query tiles of rounds qg, qg + n_qg, ... (a round = one tile per wave)
 template <bool FUSED, bool COHERENT, int TWM>
-__device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split, int hk) {
+__device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split, int hk, int qg = 0, int n_qg = 1) {
     __shared__ __attribute__((aligned(16))) half_t ks[TWM][ATT_KPITCH];
     __shared__ __attribute__((aligned(16))) half_t vt[ATT_D][TWM + 8];
     __shared__ __attribute__((aligned(16))) half_t qs[FUSED ? ATT_FUSED_MAX_Q : 1][ATT_D + 8];      // FUSED: the rotated queries of this kv head
@@ -139,7 +141,8 @@ __device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split,
     };
     // un-fused: the first tile's query is requested before the prefix slice is staged
     h8 qb_first[4];
-    if (!FUSED && wave < q_tiles) load_q(wave, qb_first);
+    const int qt_first = wave + 4 * qg;
+    if (!FUSED && qt_first < q_tiles) load_q(qt_first, qb_first);
 
     // ---- stage K (row-major) and V (transposed) ----
     // A thread moves piece ch (8 dims) of FOUR consecutive rows 4 kg .. 4 kg + 3: their V values sit side by side in a
@@ -196,9 +199,9 @@ __device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split,
     __syncthreads();
 
     const int t_tiles = tw32 / 16;
-    for (int qt = wave; qt < q_tiles; qt += 4) {
+    for (int qt = qt_first; qt < q_tiles; qt += 4 * n_qg) {
         h8 qb[4];
-        if (!FUSED && qt == wave) {
+        if (!FUSED && qt == qt_first) {
 #pragma unroll
             for (int k4 = 0; k4 < 4; ++k4) qb[k4] = qb_first[k4];
         } else {
@@ -281,7 +284,7 @@ __device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split,
 
 template <bool FUSED>
 __global__ __launch_bounds__(256) void attn_prefix_kernel(AttnParams p) {
-    attn_prefix_body<FUSED, false, ATT_TW_MAX>(p, blockIdx.x, blockIdx.y);
+    attn_prefix_body<FUSED, false, ATT_TW_MAX>(p, blockIdx.x, blockIdx.y, blockIdx.z, gridDim.z);
 }
 
 // ---- causal attention of a prefill on the matrix cores ----------------------------------------------------------
@@ -744,6 +747,22 @@ static int attn_plan_tw(int P, int Hkv) {
     return tw;
 }
 
+// Two launches: rows of the prefix per workgroup and the number of workgroups that share one slice's query tiles.
+// Every slice leaves a partial per query, so wide slices mean less partial traffic; the CUs are filled first by
+// dealing the rounds of query tiles (four tiles, one per wave) of a slice to several workgroups, which re-read the
+// slice from the cache but write nothing extra, and only then by narrower slices.
+static void attn_plan(int P, int Hkv, int Bq, int *tw_out, int *qgroups_out) {
+    const int rounds = ((Bq + 15) / 16 + 3) / 4;
+    int tw = ATT_TW_MAX, qg = 1;
+    while ((long)((P + tw - 1) / tw) * Hkv * qg < 256) {
+        if (qg < rounds) qg = min(rounds, 2 * qg);
+        else if (tw > 32) tw >>= 1;
+        else break;
+    }
+    *tw_out = tw;
+    *qgroups_out = qg;
+}
+
 }  // namespace smh
 
 extern "C" size_t smh_attn_workspace_bytes(int B, int H, int P) {
@@ -785,8 +804,9 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
     p.B = B; p.H = H; p.Hkv = Hkv; p.n_rep = H / Hkv; p.Bq = B * p.n_rep;
     p.P = P; p.suffix_format = suffix_format; p.causal = 0;
     p.scale_log2 = LOG2E / sqrtf((float)D);
-    p.tw = attn_plan_tw(P, Hkv);
-    if (one && p.tw > ATT_ONE_TW) p.tw = ATT_ONE_TW;
+    int qgroups = 1;
+    if (one) p.tw = min(attn_plan_tw(P, Hkv), ATT_ONE_TW);
+    else attn_plan(P, Hkv, p.Bq, &p.tw, &qgroups);
     p.splits = P > 0 ? (P + p.tw - 1) / p.tw : 0;
     if (one) {
         const int q_tiles = (p.Bq + 15) / 16;
@@ -807,7 +827,7 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
     p.part_o = (float *)workspace;
     p.part_ml = p.part_o + n_part * ATT_D;
     if (p.splits > 0)
-        hipLaunchKernelGGL(attn_prefix_kernel<false>, dim3(p.splits, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(attn_prefix_kernel<false>, dim3(p.splits, Hkv, qgroups), dim3(256), 0, (hipStream_t)stream, p);
     long items = (long)B * H;
     hipLaunchKernelGGL(attn_suffix_kernel<false>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
@@ -866,7 +886,9 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
     p.B = B; p.H = H; p.Hkv = Hkv; p.n_rep = H / Hkv; p.Bq = B * p.n_rep;
     p.P = P; p.suffix_format = SMH_KV_Q40; p.causal = 0;
     p.scale_log2 = LOG2E / sqrtf((float)D);
-    p.tw = attn_plan_tw(P, Hkv);
+    int qgroups = 1;
+    if (single_launch) p.tw = min(attn_plan_tw(P, Hkv), ATT_ONE_TW);
+    else attn_plan(P, Hkv, p.Bq, &p.tw, &qgroups);
     p.splits = P > 0 ? (P + p.tw - 1) / p.tw : 0;
     p.qkv = (const float *)qkv_partial; p.qkv_ks = ksplit;
     p.cos_tab = (const half_t *)cos_tab; p.sin_tab = (const half_t *)sin_tab; p.pos_dev = pos_dev;
@@ -874,10 +896,6 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
     p.app_ks = (half_t *)cache_ks; p.app_vs = (half_t *)cache_vs;
     p.app_t = t_dev; p.app_smax = Smax;
     if (single_launch) {
-        if (p.tw > ATT_ONE_TW) {
-            p.tw = ATT_ONE_TW;
-            p.splits = P > 0 ? (P + p.tw - 1) / p.tw : 0;
-        }
         // workspace = [arrival counters | partials of splits + 1 passes]
         SMH_REQUIRE((size_t)Hkv * ((p.Bq + 15) / 16) * sizeof(uint32_t) <= ATT_COUNTER_BYTES, "%s: %d kv heads x %d query tiles", who, Hkv, (p.Bq + 15) / 16);
         size_t n_part = (size_t)(p.splits + 1) * Hkv * p.Bq;
@@ -895,7 +913,7 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
     p.part_o = (float *)workspace;
     p.part_ml = p.part_o + n_part * ATT_D;
     if (p.splits > 0)
-        hipLaunchKernelGGL(attn_prefix_kernel<true>, dim3(p.splits, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(attn_prefix_kernel<true>, dim3(p.splits, Hkv, qgroups), dim3(256), 0, (hipStream_t)stream, p);
     long items = (long)B * H;
     hipLaunchKernelGGL(attn_suffix_kernel<true>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
