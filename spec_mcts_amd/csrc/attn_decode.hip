@@ -22,6 +22,8 @@
 
 namespace smh {
 
+int env_int(const char *name, int dflt);      // q40_gemv.hip
+
 constexpr int ATT_D = 128;
 constexpr int ATT_TW_MAX = 128;            // prefix rows per workgroup
 constexpr int ATT_KPITCH = 136;            // halves per LDS row of K (272 B: 16 rows hit distinct banks)
@@ -41,6 +43,7 @@ struct AttnParams {
     float *part_ml;          // [splits][Hkv][Bq][2]
     long suffix_batch_stride_rows;   // rows (tokens) between consecutive branches of the suffix
     int B, H, Hkv, n_rep, Bq;        // Bq = B * n_rep queries per kv head
+    int suffix_waves;                // one-launch kernel: waves that share one query's suffix rows (1, 2 or 4)
     int P, tw, splits;
     int suffix_format, lens_stride;
     int causal;                      // prefill mode: branch b attends to suffix rows 0..b
@@ -434,30 +437,27 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillParams p) {
 // waves (the rows come from the cache after the first), so a wave's chain of memory round trips does not grow with
 // the number of query heads per kv head.  PARTIAL: the pass over the suffix and the new token leaves an un-normalised
 // partial (split index p.splits) for the workgroup that merges, instead of folding in the prefix partials itself.
+// sub, nsub (PARTIAL only): nsub consecutive waves of the workgroup share the query; wave `sub` of them walks every
+// nsub-th group of four rows, so that a long suffix is a single batch of loads per wave instead of a chain of
+// batches; the waves' results are folded through LDS (every wave of the workgroup must then make this call; a wave
+// without a query of its own passes a valid (b, h) and live = false, and writes nothing).
 template <bool FUSED, bool PARTIAL>
-__device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int h) {
+__device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int h, int sub = 0, int nsub = 1, bool live = true) {
     const int hk = h / p.n_rep;
-    __shared__ __attribute__((aligned(16))) half_t s_kv[FUSED ? 4 : 1][2][ATT_D];     // FUSED: this wave's new k and v rows
+    __shared__ __attribute__((aligned(16))) half_t s_kv[FUSED ? 4 : 1][3][ATT_D];     // FUSED: this wave's new k and v rows, its query
+    __shared__ float s_fold[PARTIAL ? 4 : 1][16][10];                                   // PARTIAL: the waves' states (m, l, o[8])
     const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
     const int wave = threadIdx.x >> 6;
-    // FUSED: query of head h in the row layout (dims 4c..4c+3 and 64+4c..)
-    auto fused_q = [&](int h, int pos_) {
-        h4 lo, hi;
-        qkv_query(p, b, h, pos_, c, lo, hi);
-        RowRegs qr;
-        qr.a02 = h2{lo[0], lo[2]}; qr.a13 = h2{lo[1], lo[3]};
-        qr.b02 = h2{hi[0], hi[2]}; qr.b13 = h2{hi[1], hi[3]};
-        return qr;
-    };
     int len = 0;
     if (p.suffix_format != SMH_KV_NONE) len = p.causal ? b + 1 : p.lens[(long)b * p.lens_stride];
+    const int gg = g + 4 * sub, gstride = 4 * nsub;      // this group's first row and the distance to its next one
     const long row0 = (long)b * p.suffix_batch_stride_rows;     // first suffix row of this branch
     // one batch of Q4_0 suffix rows: group g takes rows t0, t0 + 4, ... (rows past the end repeat the last one)
     constexpr int UQ = 8;
     auto load_q40_batch = [&](int t0, uint32_t (&kb)[UQ], uint32_t (&vb)[UQ], uint32_t (&ksc)[UQ], uint32_t (&vsc)[UQ]) {
 #pragma unroll
         for (int u = 0; u < UQ; ++u) {
-            const long row = (row0 + min(t0 + 4 * u, len - 1)) * p.Hkv + hk;
+            const long row = (row0 + min(t0 + gstride * u, len - 1)) * p.Hkv + hk;
             kb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_k + row * 64 + 4 * c);
             vb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_v + row * 64 + 4 * c);
             ksc[u] = *reinterpret_cast<const uint32_t *>(p.suffix_ks + row * 2);
@@ -468,25 +468,40 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
     RowRegs q_first;
     int pos = 0;
     if (FUSED) {
-        if (p.suffix_format == SMH_KV_Q40 && g < len) load_q40_batch(g, kb0, vb0, ksc0, vsc0);
+        if (p.suffix_format == SMH_KV_Q40 && gg < len) load_q40_batch(gg, kb0, vb0, ksc0, vsc0);
         // Everything that does not depend on another load is requested first: the position, the slabs of the new
         // token's k and v (lane owns the pair (lane, lane + 64)) and of the first query.  k is rotated, both rows
         // are appended to the branch's suffix cache as Q4_0 and left in LDS as exact fp16 for the pass below.
+        // The query is read like k: lane owns the rotation pair (lane, lane + 64), 2 x ksplit loads of 4 bytes, and
+        // changes to the row layout through LDS.  (Read in the row layout - 8 dims a lane, 16-byte loads - its slabs
+        // alone take 128 registers, and the loads of q, k and v then go out one after the other, each a round trip.)
         pos = *p.pos_dev;
-        const int t = p.app_k != nullptr ? *p.app_t : -1;
-        const int kcol = (p.H + hk) * ATT_D, vcol = (p.H + p.Hkv + hk) * ATT_D;
-        half_t k1 = qkv_value(p, b, kcol + lane), k2 = qkv_value(p, b, kcol + lane + 64);
-        const half_t v1 = qkv_value(p, b, vcol + lane), v2 = qkv_value(p, b, vcol + lane + 64);
-        q_first = fused_q(h, pos);
-        rope_pair2(k1, k2, p.cos_tab[(long)pos * 64 + lane], p.sin_tab[(long)pos * 64 + lane]);
-        if (h == hk * p.n_rep && t >= 0 && t < p.app_smax) {     // the first query head of a kv head appends the rows
-            const long row = ((long)b * p.app_smax + t) * p.Hkv + hk;
-            kv_store_row2(k1, k2, p.app_k + row * 64, p.app_ks + row * 2, lane);
-            kv_store_row2(v1, v2, p.app_v + row * 64, p.app_vs + row * 2, lane);
+        half_t q1 = qkv_value(p, b, h * ATT_D + lane), q2 = qkv_value(p, b, h * ATT_D + lane + 64);
+        half_t k1 = q1, k2 = q1, v1 = q1, v2 = q1;
+        int t = -1;
+        if (sub == 0) {                                            // the wave that owns the new token
+            t = p.app_k != nullptr ? *p.app_t : -1;
+            const int kcol = (p.H + hk) * ATT_D, vcol = (p.H + p.Hkv + hk) * ATT_D;
+            k1 = qkv_value(p, b, kcol + lane); k2 = qkv_value(p, b, kcol + lane + 64);
+            v1 = qkv_value(p, b, vcol + lane); v2 = qkv_value(p, b, vcol + lane + 64);
         }
-        s_kv[wave][0][lane] = k1; s_kv[wave][0][lane + 64] = k2;
-        s_kv[wave][1][lane] = v1; s_kv[wave][1][lane + 64] = v2;
-        // same wave writes and reads: LDS operations of a wave complete in order
+        const half_t cos_l = p.cos_tab[(long)pos * 64 + lane], sin_l = p.sin_tab[(long)pos * 64 + lane];
+        rope_pair2(q1, q2, cos_l, sin_l);
+        s_kv[wave][2][lane] = q1; s_kv[wave][2][lane + 64] = q2;
+        asm volatile("" ::: "memory");                              // the reads below are of another type: keep them behind the writes
+        q_first = row_from_fp16(&s_kv[wave][2][0], c);             // same wave writes and reads: LDS operations complete in order
+        if (sub == 0) {
+            rope_pair2(k1, k2, cos_l, sin_l);
+            if (live && h == hk * p.n_rep && t >= 0 && t < p.app_smax) {     // the first query head of a kv head appends the rows
+                const long row = ((long)b * p.app_smax + t) * p.Hkv + hk;
+                kv_store_row2(k1, k2, p.app_k + row * 64, p.app_ks + row * 2, lane);
+                kv_store_row2(v1, v2, p.app_v + row * 64, p.app_vs + row * 2, lane);
+            }
+            s_kv[wave][0][lane] = k1; s_kv[wave][0][lane + 64] = k2;
+            s_kv[wave][1][lane] = v1; s_kv[wave][1][lane + 64] = v2;
+            asm volatile("" ::: "memory");
+            // same wave writes and reads: LDS operations of a wave complete in order
+        }
     }
 
     {
@@ -503,7 +518,7 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
         // (tens, a quarter each per group), so its time is the number of memory round trips it makes in a row.
         // ---- loads for the end of the pass: the new token's exact K/V, the first two prefix partials ----
         const int qrow = b * p.n_rep + (h - hk * p.n_rep);
-        const bool has_cur = (FUSED || p.cur_k != nullptr) && g == 0;
+        const bool has_cur = (FUSED || p.cur_k != nullptr) && g == 0 && sub == 0;
         RowRegs cur_kr = qr, cur_vr = qr;
         if (has_cur) {
             if (FUSED) {
@@ -532,23 +547,23 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
         // ---- this branch's suffix: group g takes rows g, g+4, ... in batches ----
         if (p.suffix_format == SMH_KV_FP16) {
             constexpr int U = 4;
-            for (int t0 = g; t0 < len; t0 += 4 * U) {
+            for (int t0 = gg; t0 < len; t0 += gstride * U) {
                 RowRegs kr[U], vr[U];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    const long row = (row0 + min(t0 + 4 * u, len - 1)) * p.Hkv + hk;
+                    const long row = (row0 + min(t0 + gstride * u, len - 1)) * p.Hkv + hk;
                     kr[u] = row_from_fp16((const half_t *)p.suffix_k + row * ATT_D, c);
                     vr[u] = row_from_fp16((const half_t *)p.suffix_v + row * ATT_D, c);
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u)
-                    if (t0 + 4 * u < len) soft_add_row(st, row_dot(kr[u], qr) * p.scale_log2, vr[u]);
+                    if (t0 + gstride * u < len) soft_add_row(st, row_dot(kr[u], qr) * p.scale_log2, vr[u]);
             }
         } else {
             constexpr int U = UQ;
-            for (int t0 = g; t0 < len; t0 += 4 * U) {
+            for (int t0 = gg; t0 < len; t0 += gstride * U) {
                 uint32_t kb[U], vb[U], ksc[U], vsc[U];
-                if (FUSED && t0 == g) {
+                if (FUSED && t0 == gg) {
 #pragma unroll
                     for (int u = 0; u < U; ++u) { kb[u] = kb0[u]; vb[u] = vb0[u]; ksc[u] = ksc0[u]; vsc[u] = vsc0[u]; }
                 } else {
@@ -556,7 +571,7 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u)
-                    if (t0 + 4 * u < len)
+                    if (t0 + gstride * u < len)
                         soft_add_row(st, row_dot(row_from_q40(kb[u], ksc[u]), qr) * p.scale_log2, row_from_q40(vb[u], vsc[u]));
             }
         }
@@ -587,7 +602,19 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
             for (int j = 0; j < 8; ++j) o2[j] = __shfl_xor(st.o[j], sh, 64);
             soft_merge(st, m2, l2, o2);
         }
+        if (PARTIAL && nsub > 1) {                     // (uniform over the workgroup)
+            if (g == 0) {
+                float *mine = s_fold[wave][c];
+                mine[0] = st.m; mine[1] = st.l;
+#pragma unroll
+                for (int j = 0; j < 8; ++j) mine[2 + j] = st.o[j];
+            }
+            __syncthreads();
+            if (g == 0 && sub == 0)
+                for (int k = 1; k < nsub; ++k) soft_merge(st, s_fold[wave + k][c][0], s_fold[wave + k][c][1], &s_fold[wave + k][c][2]);
+        }
         if (g == 0 && PARTIAL) {
+            if (sub != 0 || !live) return;
             const long base = ((long)p.splits * p.Hkv + hk) * p.Bq + qrow;
             st_f4(p.part_o + base * ATT_D + 4 * c, f4{st.o[0], st.o[2], st.o[1], st.o[3]});
             st_f4(p.part_o + base * ATT_D + 64 + 4 * c, f4{st.o[4], st.o[6], st.o[5], st.o[7]});
@@ -611,8 +638,9 @@ __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
 }
 
 // ---- the whole decode attention in ONE launch -----------------------------------------------------------------
-// grid (splits + ceil(Bq / 4), kv heads): workgroups x < splits take a slice of the prefix, the others the suffix
-// + new token of four of the kv head's Bq = B x n_rep queries (one wave per query).  Every workgroup leaves partials with device-scope
+// grid (splits + ceil(Bq / per_wg), kv heads): workgroups x < splits take a slice of the prefix, the others the suffix
+// + new token of per_wg = 1, 2 or 4 of the kv head's Bq = B x n_rep queries (4, 2 or 1 waves per query: with few
+// queries a query's rows are spread over the waves, which shortens the longest chain of loads in the launch).  Every workgroup leaves partials with device-scope
 // stores and counts itself in on the counters of the query tiles (16 queries of a kv head) it contributed to;
 // the workgroup that completes a tile's count merges that tile's partials in split order (so the result does
 // not depend on which workgroup that is), normalises and writes the output.  Nobody waits for anybody.
@@ -625,15 +653,16 @@ __global__ __launch_bounds__(256, 2) void attn_one_kernel(AttnParams p) {
     const int hk = blockIdx.y;
     const int tid = threadIdx.x;
     const int q_tiles = (p.Bq + 15) / 16;
-    constexpr int per_wg = 4;                  // queries of one suffix workgroup (one per wave)
+    const int per_wg = 4 / p.suffix_waves;     // queries of one suffix workgroup (suffix_waves = 1, 2 or 4 waves each)
     int tile_lo = 0, tile_hi = q_tiles - 1;    // query tiles this workgroup contributed to
     if ((int)blockIdx.x < p.splits) {
         attn_prefix_body<FUSED, true, ATT_ONE_TW>(p, blockIdx.x, hk);
     } else {
-        const int j = (int)blockIdx.x - p.splits;
-        const int qrow = 4 * j + (tid >> 6);   // query of this kv head: branch qrow / n_rep, its query head qrow % n_rep
-        if (qrow < p.Bq) attn_suffix_body<FUSED, true>(p, qrow / p.n_rep, hk * p.n_rep + qrow % p.n_rep);
-        tile_lo = tile_hi = (4 * j) / 16;      // four consecutive queries never straddle a tile of 16
+        const int j = (int)blockIdx.x - p.splits, wave_ = tid >> 6;
+        const int qrow = per_wg * j + wave_ / p.suffix_waves;     // query of this kv head: branch qrow / n_rep, its query head qrow % n_rep
+        const int qc = min(qrow, p.Bq - 1);
+        attn_suffix_body<FUSED, true>(p, qc / p.n_rep, hk * p.n_rep + qc % p.n_rep, wave_ % p.suffix_waves, p.suffix_waves, qrow < p.Bq);
+        tile_lo = tile_hi = (per_wg * j) / 16;  // a workgroup's 1, 2 or 4 consecutive queries never straddle a tile of 16
     }
     wait_vmem();                               // this wave's partials have reached memory ...
     __syncthreads();                           // ... and those of the whole workgroup
@@ -763,6 +792,15 @@ static void attn_plan(int P, int Hkv, int Bq, int *tw_out, int *qgroups_out) {
     *qgroups_out = qg;
 }
 
+// One-launch kernel: waves that share a query's suffix rows - as many as keep the launch within one round of
+// workgroups (two fit a compute unit).
+static int attn_plan_suffix_waves(int splits, int Bq, int Hkv) {
+    static const int most = env_int("SMH_ATTN_SUFFIX_WAVES", 4);
+    int nsub = most >= 4 ? 4 : (most >= 2 ? 2 : 1);
+    while (nsub > 1 && (long)(splits + (Bq + 4 / nsub - 1) / (4 / nsub)) * Hkv > 512) nsub >>= 1;
+    return nsub;
+}
+
 }  // namespace smh
 
 extern "C" size_t smh_attn_workspace_bytes(int B, int H, int P) {
@@ -809,6 +847,7 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
     else attn_plan(P, Hkv, p.Bq, &p.tw, &qgroups);
     p.splits = P > 0 ? (P + p.tw - 1) / p.tw : 0;
     if (one) {
+        p.suffix_waves = attn_plan_suffix_waves(p.splits, p.Bq, Hkv);
         const int q_tiles = (p.Bq + 15) / 16;
         SMH_REQUIRE(q_tiles <= ATT_ONE_MAX_TILES && (size_t)Hkv * q_tiles * sizeof(uint32_t) <= ATT_COUNTER_BYTES,
                     "%s: %d queries per kv head (at most %d), %d kv heads", who, p.Bq, ATT_FUSED_MAX_Q, Hkv);
@@ -818,7 +857,7 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
         p.counters = (uint32_t *)workspace;
         p.part_o = (float *)((char *)workspace + ATT_COUNTER_BYTES);
         p.part_ml = p.part_o + n_part * ATT_D;
-        hipLaunchKernelGGL(attn_one_kernel<false>, dim3(p.splits + (p.Bq + 3) / 4, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(attn_one_kernel<false>, dim3(p.splits + (p.Bq + 4 / p.suffix_waves - 1) / (4 / p.suffix_waves), Hkv), dim3(256), 0, (hipStream_t)stream, p);
         return launch_status();
     }
     size_t n_part = (size_t)p.splits * Hkv * p.Bq;
@@ -896,6 +935,7 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
     p.app_ks = (half_t *)cache_ks; p.app_vs = (half_t *)cache_vs;
     p.app_t = t_dev; p.app_smax = Smax;
     if (single_launch) {
+        p.suffix_waves = attn_plan_suffix_waves(p.splits, p.Bq, Hkv);
         // workspace = [arrival counters | partials of splits + 1 passes]
         SMH_REQUIRE((size_t)Hkv * ((p.Bq + 15) / 16) * sizeof(uint32_t) <= ATT_COUNTER_BYTES, "%s: %d kv heads x %d query tiles", who, Hkv, (p.Bq + 15) / 16);
         size_t n_part = (size_t)(p.splits + 1) * Hkv * p.Bq;
@@ -904,7 +944,7 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
         p.counters = (uint32_t *)workspace;
         p.part_o = (float *)((char *)workspace + ATT_COUNTER_BYTES);
         p.part_ml = p.part_o + n_part * ATT_D;
-        hipLaunchKernelGGL(attn_one_kernel<true>, dim3(p.splits + (p.Bq + 3) / 4, Hkv), dim3(256), 0, (hipStream_t)stream, p);
+        hipLaunchKernelGGL(attn_one_kernel<true>, dim3(p.splits + (p.Bq + 4 / p.suffix_waves - 1) / (4 / p.suffix_waves), Hkv), dim3(256), 0, (hipStream_t)stream, p);
         return launch_status();
     }
     size_t n_part = (size_t)p.splits * Hkv * p.Bq;
