@@ -75,6 +75,21 @@ __device__ __forceinline__ half_t qkv_value(const AttnParams &p, int b, int col)
     for (int s_ = 0; s_ < 16; ++s_) tot += v[s_];
     return (half_t)tot;
 }
+// the same in two steps, so that a caller can request several columns before it waits for any of them
+struct SlabColumn { float v[16]; };
+__device__ __forceinline__ void qkv_request(const AttnParams &p, int b, int col, SlabColumn &c) {
+    const int cols = (p.H + 2 * p.Hkv) * ATT_D;
+    const float *src = p.qkv + (long)b * cols + col;
+    const long slab = (long)p.B * cols;
+#pragma unroll
+    for (int s_ = 0; s_ < 16; ++s_) c.v[s_] = (s_ < p.qkv_ks) ? src[s_ * slab] : 0.f;
+}
+__device__ __forceinline__ half_t qkv_sum(const SlabColumn &c) {
+    float tot = 0.f;
+#pragma unroll
+    for (int s_ = 0; s_ < 16; ++s_) tot += c.v[s_];
+    return (half_t)tot;
+}
 // four consecutive columns (col % 4 == 0)
 __device__ __forceinline__ h4 qkv_value4(const AttnParams &p, int b, int col) {
     const int cols = (p.H + 2 * p.Hkv) * ATT_D;
@@ -468,24 +483,29 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
     RowRegs q_first;
     int pos = 0;
     if (FUSED) {
-        if (p.suffix_format == SMH_KV_Q40 && gg < len) load_q40_batch(gg, kb0, vb0, ksc0, vsc0);
-        // Everything that does not depend on another load is requested first: the position, the slabs of the new
-        // token's k and v (lane owns the pair (lane, lane + 64)) and of the first query.  k is rotated, both rows
-        // are appended to the branch's suffix cache as Q4_0 and left in LDS as exact fp16 for the pass below.
-        // The query is read like k: lane owns the rotation pair (lane, lane + 64), 2 x ksplit loads of 4 bytes, and
-        // changes to the row layout through LDS.  (Read in the row layout - 8 dims a lane, 16-byte loads - its slabs
-        // alone take 128 registers, and the loads of q, k and v then go out one after the other, each a round trip.)
+        // Two round trips to memory, not more: first everything that depends on no other load - the suffix length
+        // (requested above), the position, the suffix index and the slabs of q, k and v (lane owns the rotation pair
+        // (lane, lane + 64) of each: 2 x ksplit loads of 4 bytes; read in the row layout, 8 dims a lane, q's slabs
+        // alone take 128 registers and the requests leave one after the other) - then what depends on the length
+        // (the first batch of rows) and on the position (the rotation factors).  q changes to the row layout
+        // through LDS; k is rotated, k and v are appended to the branch's suffix cache as Q4_0 and left in LDS as
+        // exact fp16 for the pass below.
         pos = *p.pos_dev;
-        half_t q1 = qkv_value(p, b, h * ATT_D + lane), q2 = qkv_value(p, b, h * ATT_D + lane + 64);
-        half_t k1 = q1, k2 = q1, v1 = q1, v2 = q1;
         int t = -1;
+        SlabColumn cq1, cq2, ck1, ck2, cv1, cv2;
+        qkv_request(p, b, h * ATT_D + lane, cq1);
+        qkv_request(p, b, h * ATT_D + lane + 64, cq2);
         if (sub == 0) {                                            // the wave that owns the new token
             t = p.app_k != nullptr ? *p.app_t : -1;
             const int kcol = (p.H + hk) * ATT_D, vcol = (p.H + p.Hkv + hk) * ATT_D;
-            k1 = qkv_value(p, b, kcol + lane); k2 = qkv_value(p, b, kcol + lane + 64);
-            v1 = qkv_value(p, b, vcol + lane); v2 = qkv_value(p, b, vcol + lane + 64);
+            qkv_request(p, b, kcol + lane, ck1); qkv_request(p, b, kcol + lane + 64, ck2);
+            qkv_request(p, b, vcol + lane, cv1); qkv_request(p, b, vcol + lane + 64, cv2);
         }
+        if (p.suffix_format == SMH_KV_Q40 && gg < len) load_q40_batch(gg, kb0, vb0, ksc0, vsc0);
         const half_t cos_l = p.cos_tab[(long)pos * 64 + lane], sin_l = p.sin_tab[(long)pos * 64 + lane];
+        half_t q1 = qkv_sum(cq1), q2 = qkv_sum(cq2);
+        half_t k1 = q1, k2 = q1, v1 = q1, v2 = q1;
+        if (sub == 0) { k1 = qkv_sum(ck1); k2 = qkv_sum(ck2); v1 = qkv_sum(cv1); v2 = qkv_sum(cv2); }
         rope_pair2(q1, q2, cos_l, sin_l);
         s_kv[wave][2][lane] = q1; s_kv[wave][2][lane + 64] = q2;
         asm volatile("" ::: "memory");                              // the reads below are of another type: keep them behind the writes
