@@ -43,7 +43,7 @@ struct AttnParams {
     float *part_ml;          // [splits][Hkv][Bq][2]
     long suffix_batch_stride_rows;   // rows (tokens) between consecutive branches of the suffix
     int B, H, Hkv, n_rep, Bq;        // Bq = B * n_rep queries per kv head
-    int suffix_waves;                // one-launch kernel: waves that share one query's suffix rows (1, 2 or 4)
+    int suffix_waves;                // waves that share one query's suffix rows (1, 2 or 4)
     int P, tw, splits;
     int suffix_format, lens_stride;
     int causal;                      // prefill mode: branch b attends to suffix rows 0..b
@@ -452,7 +452,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillParams p) {
 // waves (the rows come from the cache after the first), so a wave's chain of memory round trips does not grow with
 // the number of query heads per kv head.  PARTIAL: the pass over the suffix and the new token leaves an un-normalised
 // partial (split index p.splits) for the workgroup that merges, instead of folding in the prefix partials itself.
-// sub, nsub (PARTIAL only): nsub consecutive waves of the workgroup share the query; wave `sub` of them walks every
+// sub, nsub: nsub consecutive waves of the workgroup share the query; wave `sub` of them walks every
 // nsub-th group of four rows, so that a long suffix is a single batch of loads per wave instead of a chain of
 // batches; the waves' results are folded through LDS (every wave of the workgroup must then make this call; a wave
 // without a query of its own passes a valid (b, h) and live = false, and writes nothing).
@@ -460,7 +460,7 @@ template <bool FUSED, bool PARTIAL>
 __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int h, int sub = 0, int nsub = 1, bool live = true) {
     const int hk = h / p.n_rep;
     __shared__ __attribute__((aligned(16))) half_t s_kv[FUSED ? 4 : 1][3][ATT_D];     // FUSED: this wave's new k and v rows, its query
-    __shared__ float s_fold[PARTIAL ? 4 : 1][16][10];                                   // PARTIAL: the waves' states (m, l, o[8])
+    __shared__ float s_fold[4][16][10];                                                 // nsub > 1: the waves' states (m, l, o[8])
     const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
     const int wave = threadIdx.x >> 6;
     int len = 0;
@@ -555,7 +555,7 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
         float pre_m[PRE], pre_l[PRE];
 #pragma unroll
         for (int i = 0; i < PRE; ++i) {
-            const int sp = g + 4 * i;
+            const int sp = gg + gstride * i;
             if (!PARTIAL && sp < p.splits) {
                 const long base = ((long)sp * p.Hkv + hk) * p.Bq + qrow;
                 pre_lo[i] = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 4 * c);
@@ -597,15 +597,15 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
         }
         // ---- the new token's exact K/V (group 0 only) ----
         if (has_cur) soft_add_row(st, row_dot(cur_kr, qr) * p.scale_log2, cur_vr);
-        // ---- prefix partials: group g folds in splits g, g+4, ... ----
+        // ---- prefix partials: the group folds in splits gg, gg + gstride, ... ----
 #pragma unroll
         for (int i = 0; i < PRE; ++i) {
-            if (!PARTIAL && g + 4 * i < p.splits) {
+            if (!PARTIAL && gg + gstride * i < p.splits) {
                 const float o2[8] = {pre_lo[i][0], pre_lo[i][2], pre_lo[i][1], pre_lo[i][3], pre_hi[i][0], pre_hi[i][2], pre_hi[i][1], pre_hi[i][3]};
                 soft_merge(st, pre_m[i], pre_l[i], o2);
             }
         }
-        for (int sp = g + 4 * PRE; !PARTIAL && sp < p.splits; sp += 4) {
+        for (int sp = gg + gstride * PRE; !PARTIAL && sp < p.splits; sp += gstride) {
             const long base = ((long)sp * p.Hkv + hk) * p.Bq + qrow;
             const f4 lo = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 4 * c);
             const f4 hi = *reinterpret_cast<const f4 *>(p.part_o + base * ATT_D + 64 + 4 * c);
@@ -622,7 +622,7 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
             for (int j = 0; j < 8; ++j) o2[j] = __shfl_xor(st.o[j], sh, 64);
             soft_merge(st, m2, l2, o2);
         }
-        if (PARTIAL && nsub > 1) {                     // (uniform over the workgroup)
+        if (nsub > 1) {                                // (uniform over the workgroup)
             if (g == 0) {
                 float *mine = s_fold[wave][c];
                 mine[0] = st.m; mine[1] = st.l;
@@ -639,7 +639,7 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
             st_f4(p.part_o + base * ATT_D + 4 * c, f4{st.o[0], st.o[2], st.o[1], st.o[3]});
             st_f4(p.part_o + base * ATT_D + 64 + 4 * c, f4{st.o[4], st.o[6], st.o[5], st.o[7]});
             if (c == 0) { st_f32(p.part_ml + base * 2, st.m); st_f32(p.part_ml + base * 2 + 1, st.l); }
-        } else if (g == 0) {
+        } else if (g == 0 && sub == 0 && live) {
             const float inv = st.l > 0.f ? 1.0f / st.l : 0.f;
             half_t *op = p.out + ((long)b * p.H + h) * ATT_D;
             h4 lo = {(half_t)(st.o[0] * inv), (half_t)(st.o[2] * inv), (half_t)(st.o[1] * inv), (half_t)(st.o[3] * inv)};
@@ -652,9 +652,13 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
 
 template <bool FUSED>
 __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
-    const long item = (long)blockIdx.x * 4 + (threadIdx.x >> 6);
-    if (item >= (long)p.B * p.H) return;
-    attn_suffix_body<FUSED, false>(p, (int)(item / p.H), (int)(item % p.H));
+    // suffix_waves (1, 2 or 4) waves per (branch, query head): more than one while branches x heads leave CUs idle
+    const int wave = threadIdx.x >> 6, nsub = p.suffix_waves;
+    const long items = (long)p.B * p.H;
+    const long item = ((long)blockIdx.x * 4 + wave) / nsub;
+    if (nsub == 1 && item >= items) return;
+    const long ic = min(item, items - 1);          // with shared queries every wave reaches the fold's barrier
+    attn_suffix_body<FUSED, false>(p, (int)(ic / p.H), (int)(ic % p.H), wave % nsub, nsub, item < items);
 }
 
 // ---- the whole decode attention in ONE launch -----------------------------------------------------------------
@@ -812,6 +816,15 @@ static void attn_plan(int P, int Hkv, int Bq, int *tw_out, int *qgroups_out) {
     *qgroups_out = qg;
 }
 
+// Suffix launch of the two-launch form: waves per (branch, query head) - more than one while the launch still fits
+// the GPU in one round (4 waves of this kernel per SIMD, 1024 SIMDs).
+static int attn_plan_suffix_waves_two(long queries) {
+    static const int most = env_int("SMH_ATTN_SUFFIX_WAVES", 4);
+    int nsub = most >= 4 ? 4 : (most >= 2 ? 2 : 1);
+    while (nsub > 1 && queries * nsub > 4096) nsub >>= 1;
+    return nsub;
+}
+
 // One-launch kernel: waves that share a query's suffix rows - as many as keep the launch within one round of
 // workgroups (two fit a compute unit).
 static int attn_plan_suffix_waves(int splits, int Bq, int Hkv) {
@@ -887,7 +900,8 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
     p.part_ml = p.part_o + n_part * ATT_D;
     if (p.splits > 0)
         hipLaunchKernelGGL(attn_prefix_kernel<false>, dim3(p.splits, Hkv, qgroups), dim3(256), 0, (hipStream_t)stream, p);
-    long items = (long)B * H;
+    p.suffix_waves = attn_plan_suffix_waves_two((long)B * H);
+    long items = (long)B * H * p.suffix_waves;
     hipLaunchKernelGGL(attn_suffix_kernel<false>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
 }
@@ -974,7 +988,8 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
     p.part_ml = p.part_o + n_part * ATT_D;
     if (p.splits > 0)
         hipLaunchKernelGGL(attn_prefix_kernel<true>, dim3(p.splits, Hkv, qgroups), dim3(256), 0, (hipStream_t)stream, p);
-    long items = (long)B * H;
+    p.suffix_waves = attn_plan_suffix_waves_two((long)B * H);
+    long items = (long)B * H * p.suffix_waves;
     hipLaunchKernelGGL(attn_suffix_kernel<true>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
 }
