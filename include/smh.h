@@ -170,6 +170,12 @@ int smh_argmax(const void *logits, int rows, int vocab, long ld, int64_t *out, s
  * numbers take the place of torch.multinomial's generator.  1 <= top_k <= 1024, temperature > 0. */
 int smh_sample_topk(const void *logits, int rows, int vocab, long ld, float temperature, int top_k,
                     const float *uniform, int64_t *out, smh_stream_t stream);
+/* smh_detect_terminal: detectTerminal (mcts.py:14-28) for `rows` branches in place: state[b] counts the tokens of
+ * terminal_seq (int64 [seq_len], "[/PYTHON]" in the reference, mcts.py:12) produced in a row, any other token sends it
+ * back to 0; end[b] = 1 when the sequence is complete or token[b] == eos (2 in the reference), and the state of an ended
+ * branch is 0.  token int64 [rows], state int32 [rows] (read and written), end uint8 [rows]. */
+int smh_detect_terminal(const int64_t *token, int32_t *state, uint8_t *end, const int64_t *terminal_seq, int seq_len,
+                        int64_t eos, int rows, smh_stream_t stream);
 int smh_rope_append_kv(void *q, void *k, const void *v, int B, int H, int Hkv, int D,
                        const void *cos_tab, const void *sin_tab, const int32_t *pos_dev,
                        void *cache_k, void *cache_ks, void *cache_v, void *cache_vs,

@@ -28,6 +28,10 @@ live in tests/test_oracle_*.py):
   topk_probs / sample_topk       candidate values against torch.topk, probabilities against F.softmax of those values,
                                  k = 1 is the argmax, k = vocab with a huge temperature is uniform; the draw against a
                                  brute-force scan in float64 and, over many uniform numbers, its frequencies against p.
+  detect_terminal                a scalar walk over token streams written as plain if / else (tests), known answers:
+                                 the sequence fed in order ends at its last token, end-of-sequence ends at once, a
+                                 wrong token resets, a repeated first token does NOT restart the match (the reference's
+                                 behaviour), every (state, token-class) pair enumerated.
 No function here is "parity unpinned".
 """
 from __future__ import annotations
@@ -186,6 +190,16 @@ def sample_topk(logits: torch.Tensor, temperature: float, top_k: int, u: torch.T
     hit = cdf > target
     j = torch.where(hit.any(-1), hit.float().argmax(-1), torch.full((p.shape[0],), p.shape[1] - 1))
     return order.gather(1, j.unsqueeze(1))[:, 0]
+
+
+def detect_terminal(token: torch.Tensor, state: torch.Tensor, terminal_seq: torch.Tensor, eos: int = 2):
+    """detectTerminal (mcts.py:14-28): mask = terminal_seq[state] == token; state = (state + mask) * mask;
+    end = state == len(terminal_seq) or token == eos; an ended branch restarts at state 0.
+    token int64 [B], state int32 [B] -> (end bool [B], state int32 [B])."""
+    mask = (terminal_seq.gather(0, state.to(torch.int64)) == token).to(torch.int32)
+    state = (state + mask) * mask
+    end = (state == terminal_seq.numel()) | (token == eos)
+    return end, (~end).to(torch.int32) * state
 
 
 def silu_mul(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:

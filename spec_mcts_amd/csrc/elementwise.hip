@@ -383,6 +383,39 @@ extern "C" int smh_sample_topk(const void *logits, int rows, int vocab, long ld,
     return launch_status();
 }
 
+namespace smh {
+
+// detectTerminal of the tree sampler (mcts.py:14-28), one thread per branch: the state counts how many tokens of the
+// terminal sequence the branch has produced in a row; a token that does not continue it sends the state back to 0
+// (also when it equals the sequence's first token, as in the reference); the branch ends when the sequence is
+// complete or the token is the end-of-sequence id, and an ended branch restarts at state 0.
+__global__ __launch_bounds__(256) void detect_terminal_kernel(const int64_t *__restrict__ token, int32_t *__restrict__ state,
+                                                             uint8_t *__restrict__ end, const int64_t *__restrict__ seq, int seq_len,
+                                                             int64_t eos, int rows) {
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i >= rows) return;
+    const int64_t tok = token[i];
+    const int32_t st = state[i];
+    const int32_t match = (st >= 0 && st < seq_len && seq[st] == tok) ? 1 : 0;
+    int32_t nxt = (st + match) * match;
+    const bool done = nxt == seq_len || tok == eos;
+    end[i] = done ? 1 : 0;
+    state[i] = done ? 0 : nxt;
+}
+
+}  // namespace smh
+
+extern "C" int smh_detect_terminal(const int64_t *token, int32_t *state, uint8_t *end, const int64_t *terminal_seq, int seq_len,
+                                   int64_t eos, int rows, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(rows >= 0 && seq_len >= 1, "smh_detect_terminal: rows=%d seq_len=%d", rows, seq_len);
+    if (rows == 0) return 0;
+    SMH_REQUIRE(token && state && end && terminal_seq, "smh_detect_terminal: null pointer");
+    hipLaunchKernelGGL(detect_terminal_kernel, dim3((rows + 255) / 256), dim3(256), 0, (hipStream_t)stream, token, state, end,
+                       terminal_seq, seq_len, eos, rows);
+    return launch_status();
+}
+
 extern "C" int smh_argmax(const void *logits, int rows, int vocab, long ld, int64_t *out, smh_stream_t stream) {
     using namespace smh;
     SMH_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "smh_argmax: rows=%d vocab=%d ld=%ld", rows, vocab, ld);

@@ -425,6 +425,21 @@ def sample_topk(logits: torch.Tensor, temperature: float, top_k: int, uniform: O
     return out
 
 
+def detect_terminal(token: torch.Tensor, state: torch.Tensor, terminal_seq: torch.Tensor, eos: int = 2):
+    """detectTerminal of the reference's tree sampler (mcts.py:14-28) on the device in one launch.
+    token int64 [B], state int32 [B], terminal_seq int64 [L] -> (end bool [B], state int32 [B]); `state` is not modified."""
+    lib = _lib.load()
+    _need_gpu(token, state, terminal_seq)
+    assert token.dtype == torch.int64 and token.dim() == 1 and token.is_contiguous()
+    assert state.shape == token.shape and state.dtype == torch.int32
+    assert terminal_seq.dtype == torch.int64 and terminal_seq.dim() == 1 and terminal_seq.is_contiguous() and terminal_seq.numel() >= 1
+    new_state = state.clone()
+    end = torch.empty(token.shape, dtype=torch.uint8, device=token.device)
+    check(lib.smh_detect_terminal(token.data_ptr(), new_state.data_ptr(), end.data_ptr(), terminal_seq.data_ptr(),
+                                  terminal_seq.numel(), int(eos), token.numel(), _stream()), "smh_detect_terminal")
+    return end.view(torch.bool), new_state
+
+
 def rope(q: torch.Tensor, k: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor, pos0: int) -> None:
     """In-place rotate-half RoPE of q [S,H,128] and k [S,Hkv,128]; token s is at position pos0+s."""
     lib = _lib.load()

@@ -153,3 +153,31 @@ def test_sample_topk_ties_take_the_lowest_indices_and_frequencies_follow_p():
     for j in range(8):
         freq = float((draws == idx[0, j]).float().mean()); pj = float(p[0, j])
         assert abs(freq - pj) < 4 * (pj * (1 - pj) / n) ** 0.5 + 1e-3
+
+
+def test_detect_terminal_matches_the_oracle():
+    """smh_detect_terminal against the oracle's detectTerminal on token streams with the terminal sequence, near
+    matches and end-of-sequence tokens spliced in, 300 branches, 80 steps, state carried on the device: bit-exact"""
+    from spec_mcts_amd import kernels as K
+    seq = torch.tensor([29961, 29914, 20055, 4690, 1164, 29962], dtype=torch.int64)
+    g = torch.Generator().manual_seed(91)
+    B, T = 300, 80
+    toks = torch.randint(0, 50, (B, T), generator=g)
+    toks = torch.where(toks < 18, seq[toks % 6], toks + 100)          # a third of the tokens come from the sequence
+    toks[toks == 131] = 2                                              # some end-of-sequence tokens
+    for b in range(0, B, 3):
+        at = int(torch.randint(0, T - 6, (1,), generator=g))
+        toks[b, at:at + 6] = seq
+    st_o = torch.zeros(B, dtype=torch.int32)
+    st_d = st_o.cuda()
+    seq_d, toks_d = seq.cuda(), toks.cuda()
+    ends = 0
+    for i in range(T):
+        e_o, st_o = O.detect_terminal(toks[:, i].contiguous(), st_o, seq)
+        e_d, st_d = K.detect_terminal(toks_d[:, i].contiguous(), st_d, seq_d)
+        assert torch.equal(e_d.cpu(), e_o) and torch.equal(st_d.cpu(), st_o), f"step {i}"
+        ends += int(e_o.sum())
+    assert ends >= B // 3
+    # no branches: nothing to do
+    e, s_ = K.detect_terminal(toks_d[:0, 0].contiguous(), st_d[:0], seq_d)
+    assert e.numel() == 0 and s_.numel() == 0

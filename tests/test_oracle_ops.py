@@ -249,3 +249,66 @@ def test_sampler_candidates_and_draw():
     for j in range(5):
         freq = float((draws == idx[0, j]).float().mean())
         assert abs(freq - float(p[0, j])) < 4 * (float(p[0, j]) * (1 - float(p[0, j])) / n) ** 0.5 + 1e-3
+
+
+TERMINAL = [29961, 29914, 20055, 4690, 1164, 29962]          # "[/PYTHON]" as the reference tokenises it (mcts.py:12)
+
+
+def scalar_terminal_walk(tokens, seq, eos=2):
+    """a branch's token stream, one token at a time, as plain control flow: returns (ended flags, states)"""
+    ended, states, st = [], [], 0
+    for tok in tokens:
+        if tok == seq[st]:
+            st += 1
+        else:
+            st = 0
+        done = st == len(seq) or tok == eos
+        if done:
+            st = 0
+        ended.append(done)
+        states.append(st)
+    return ended, states
+
+
+def test_terminal_state_machine_known_answers_and_scalar_walk():
+    seq = torch.tensor(TERMINAL, dtype=torch.int64)
+
+    def run(tokens):
+        st = torch.zeros(1, dtype=torch.int32)
+        ended, states = [], []
+        for tok in tokens:
+            e, st = O.detect_terminal(torch.tensor([tok], dtype=torch.int64), st, seq)
+            ended.append(bool(e[0]))
+            states.append(int(st[0]))
+        return ended, states
+
+    # the sequence in order ends at its last token and the state restarts
+    assert run(TERMINAL) == ([False] * 5 + [True], [1, 2, 3, 4, 5, 0])
+    # end-of-sequence ends at once, from any state
+    assert run([7, 2]) == ([False, True], [0, 0])
+    assert run(TERMINAL[:3] + [2]) == ([False, False, False, True], [1, 2, 3, 0])
+    # a wrong token resets; a repeated first token does not restart the match (the reference's transition)
+    assert run(TERMINAL[:2] + [5] + TERMINAL) == ([False] * 8 + [True], [1, 2, 0, 1, 2, 3, 4, 5, 0])
+    assert run([TERMINAL[0], TERMINAL[0], TERMINAL[1]])[1] == [1, 0, 0]
+    # every (state, token class) pair: the expected token, another token of the sequence, a foreign token, eos
+    for st0 in range(6):
+        for tok in TERMINAL + [11, 2]:
+            e, st = O.detect_terminal(torch.tensor([tok], dtype=torch.int64), torch.tensor([st0], dtype=torch.int32), seq)
+            nxt = st0 + 1 if tok == TERMINAL[st0] else 0
+            done = nxt == 6 or tok == 2
+            assert (bool(e[0]), int(st[0])) == (done, 0 if done else nxt)
+    # random streams with the sequence spliced in, batched, against the scalar walk
+    g = torch.Generator().manual_seed(77)
+    streams = []
+    for b in range(16):
+        toks = torch.randint(0, 40, (60,), generator=g).tolist()
+        toks = [TERMINAL[t % 6] if t < 12 else t for t in toks]          # many near-matches
+        at = int(torch.randint(0, 50, (1,), generator=g))
+        toks[at:at + 6] = TERMINAL
+        streams.append(toks[:60])
+    st = torch.zeros(16, dtype=torch.int32)
+    want = [scalar_terminal_walk(s_, TERMINAL) for s_ in streams]
+    for i in range(60):
+        e, st = O.detect_terminal(torch.tensor([s_[i] for s_ in streams], dtype=torch.int64), st, seq)
+        assert e.tolist() == [w[0][i] for w in want]
+        assert st.tolist() == [w[1][i] for w in want]
