@@ -220,6 +220,7 @@ def main():
     ap.add_argument("--persistent", action="store_true", help="batches up to 4 through the persistent step kernel (comparison runs)")
     ap.add_argument("--finish-in-matmul", action="store_true", help="operators after a linear finished inside the matmul launch (comparison runs)")
     ap.add_argument("--no-norm-in-matmul", action="store_true", help="RMSNorm as its own launch at every batch size (comparison runs)")
+    ap.add_argument("--norm-in-rows", type=int, default=-1, help="RMSNorm inside the matmul up to this many rows (comparison runs; default: the model's)")
     ap.add_argument("--batches", default="", help="comma-separated subset of 1,10,100 to run (a partial run is not a valid result)")
     ap.add_argument("--no-roofline", action="store_true", help="skip the matmul roofline legs (profiling runs)")
     ap.add_argument("--roofline-only", type=int, default=0, metavar="M",
@@ -252,6 +253,8 @@ def main():
         model.finish_in_matmul = True
     if a.no_norm_in_matmul:
         model.norm_in_matmul = False
+    if a.norm_in_rows >= 0:
+        model.norm_in_max_rows = a.norm_in_rows
     prompt = torch.randint(0, 32016, (1, prompt_len), generator=torch.Generator().manual_seed(3)).cuda()
 
     if a.roofline_only:

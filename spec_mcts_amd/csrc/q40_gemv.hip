@@ -333,6 +333,9 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
     // weight stages right behind them, so that both are in flight together.
     half_t *xs = reinterpret_cast<half_t *>(lds + WAVES * RING);
     const int slice_k0 = step0 * 32, slice_rows = (step1 - step0) * 32;
+    // a row of xs is 16 bytes longer than its data: the 16 lanes that read one k-octet of 16 different rows would
+    // otherwise hit the same LDS banks whenever the slice is a multiple of 128 bytes long
+    const int xs_pitch = slice_rows + 8;
     if constexpr (SILU_IN) {
         constexpr int MAXQ = SMH_SILU_IN_MAX_M * SMH_SILU_IN_MAX_K / 4 / THREADS;     // quads of columns per thread
         f4 ga[MAXQ], ua[MAXQ];
@@ -366,7 +369,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
                     const half_t sl = (half_t)(gf / (1.0f + expf(-gf)));
                     o[j] = sl * (half_t)ua[i][j];
                 }
-                *reinterpret_cast<h4 *>(xs + (long)(idx / quads) * slice_rows + 4 * (idx % quads)) = o;
+                *reinterpret_cast<h4 *>(xs + (long)(idx / quads) * xs_pitch + 4 * (idx % quads)) = o;
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // xs is complete; the DMA ring stays in flight
@@ -375,7 +378,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         // weights and, in the first threads, of a row's sums of squares go out first, the weight stages right
         // behind them
         constexpr int MAXO = (SMH_NORM_IN_MAX_XS_BYTES / 16 + THREADS - 1) / THREADS;     // k-octets per thread
-        float *s_r = reinterpret_cast<float *>(xs + (long)p.M * slice_rows);           // r[m], behind xs
+        float *s_r = reinterpret_cast<float *>(xs + (long)p.M * xs_pitch);           // r[m], behind xs
         h8 hv[MAXO], wv[MAXO];
         const int octs = slice_rows / 8, total = p.M * octs;
 #pragma unroll
@@ -418,7 +421,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
                     const half_t nv = scale_to_half(hv[i][j], r);
                     o[j] = nv * wv[i][j];
                 }
-                *reinterpret_cast<h8 *>(xs + (long)(idx / octs) * slice_rows + 8 * (idx % octs)) = o;
+                *reinterpret_cast<h8 *>(xs + (long)(idx / octs) * xs_pitch + 8 * (idx % octs)) = o;
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // xs is complete; the DMA ring stays in flight
@@ -427,7 +430,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         for (int i = 0; i < RING_STAGES; ++i)
             if (i < n_steps) issue(ring + i * STAGE, first + i * WAVES);
     }
-    const half_t *xlane = xs + (long)min(c, p.M - 1) * slice_rows + 8 * g;     // X_IN_LDS: this lane's row of xs, its k-octet
+    const half_t *xlane = xs + (long)min(c, p.M - 1) * xs_pitch + 8 * g;     // X_IN_LDS: this lane's row of xs, its k-octet
     // the one step that may lack rows is the last step of K, hence the last one of its wave; it is
     // peeled off so that the loop has a single decoder in it
     const int n_full = first < full_steps ? min(n_steps, (full_steps - first + WAVES - 1) / WAVES) : 0;
@@ -556,7 +559,7 @@ void gemv_fill_plan(MatmulParams &p) {
 }
 
 bool gemv_norm_in_fits(const MatmulParams &p) {
-    return p.M <= SMH_GEMV_MAX_M && (size_t)p.M * p.steps_per_slice * 32 * sizeof(half_t) <= SMH_NORM_IN_MAX_XS_BYTES;
+    return p.M <= SMH_GEMV_MAX_M && (size_t)p.M * (p.steps_per_slice * 32 + 8) * sizeof(half_t) <= SMH_NORM_IN_MAX_XS_BYTES;
 }
 
 int gemv_launch(const MatmulParams &p, hipStream_t stream) {
@@ -565,7 +568,7 @@ int gemv_launch(const MatmulParams &p, hipStream_t stream) {
     size_t lds = (size_t)waves * RING_BYTES;                       // rings, reused for the [waves][M][256] sums
     const size_t red = (size_t)waves * p.M * GEMV_COLS * sizeof(float);
     if (p.tiled && (p.gu_partial != nullptr || p.norm_w != nullptr))   // rings without activation tiles, xs (and r[]) behind them
-        lds = (size_t)waves * RING_BYTES_NO_X + (size_t)p.M * p.steps_per_slice * 32 * sizeof(half_t) + SMH_GEMV_MAX_M * sizeof(float);
+        lds = (size_t)waves * RING_BYTES_NO_X + (size_t)p.M * (p.steps_per_slice * 32 + 8) * sizeof(half_t) + SMH_GEMV_MAX_M * sizeof(float);
     if (red > lds) lds = red;
     if (p.tiled) {
         if (p.fin.mode != 0 || waves != 4) {
