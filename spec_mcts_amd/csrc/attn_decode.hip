@@ -467,8 +467,10 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
     if (p.suffix_format != SMH_KV_NONE) len = p.causal ? b + 1 : p.lens[(long)b * p.lens_stride];
     const int gg = g + 4 * sub, gstride = 4 * nsub;      // this group's first row and the distance to its next one
     const long row0 = (long)b * p.suffix_batch_stride_rows;     // first suffix row of this branch
-    // one batch of Q4_0 suffix rows: group g takes rows t0, t0 + 4, ... (rows past the end repeat the last one)
-    constexpr int UQ = 8;
+    // one batch of Q4_0 suffix rows: group g takes rows t0, t0 + 4, ... (rows past the end repeat the last one).
+    // Four rows a group per batch: eight measured 1-1.5 % slower per decode step at 1, 10 and 100 branches (more
+    // registers, and a short suffix pays for rows it does not have), two 1.5 % slower (more round trips).
+    constexpr int UQ = 4;
     auto load_q40_batch = [&](int t0, uint32_t (&kb)[UQ], uint32_t (&vb)[UQ], uint32_t (&ksc)[UQ], uint32_t (&vsc)[UQ]) {
 #pragma unroll
         for (int u = 0; u < UQ; ++u) {
