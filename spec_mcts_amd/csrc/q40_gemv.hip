@@ -384,11 +384,15 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         float *s_r = reinterpret_cast<float *>(xs + (long)p.M * xs_pitch);           // r[m], behind xs
         h8 hv[MAXO], wv[MAXO];
         const int octs = slice_rows / 8, total = p.M * octs;
+        // item idx = (row idx / octs, octet idx % octs); idx < 1760 and octs <= 1760, so the quotient from a float
+        // reciprocal is exact (an integer division costs ~25 instructions per item here)
+        const float inv_octs = 1.0f / (float)max(octs, 1);
+        auto row_of = [&](int idx) { return (int)(((float)idx + 0.5f) * inv_octs); };
 #pragma unroll
         for (int i = 0; i < MAXO; ++i) {
             const int idx = tid + i * THREADS;
             if (idx < total) {
-                const int m = idx / octs, k = slice_k0 + 8 * (idx % octs);
+                const int m = row_of(idx), k = slice_k0 + 8 * (idx - m * octs);
                 if (k < p.K) {
                     hv[i] = *reinterpret_cast<const h8 *>(p.a + (long)m * p.lda + k);
                     wv[i] = *reinterpret_cast<const h8 *>(p.norm_w + k);
@@ -417,14 +421,15 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         for (int i = 0; i < MAXO; ++i) {
             const int idx = tid + i * THREADS;
             if (idx < total) {
-                const float r = s_r[idx / octs];
+                const int m = row_of(idx);
+                const float r = s_r[m];
                 h8 o;
 #pragma unroll
                 for (int j = 0; j < 8; ++j) {                  // the roundings of partial_rmsnorm_kernel
                     const half_t nv = scale_to_half(hv[i][j], r);
                     o[j] = nv * wv[i][j];
                 }
-                *reinterpret_cast<h8 *>(xs + (long)(idx / octs) * xs_pitch + 8 * (idx % octs)) = o;
+                *reinterpret_cast<h8 *>(xs + (long)m * xs_pitch + 8 * (idx - m * octs)) = o;
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // xs is complete; the DMA ring stays in flight
