@@ -655,12 +655,13 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
 template <bool FUSED>
 __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
     // suffix_waves (1, 2 or 4) waves per (branch, query head): more than one while branches x heads leave CUs idle
+    // grid (groups of four waves of a branch, branches): no division to find the branch
     const int wave = threadIdx.x >> 6, nsub = p.suffix_waves;
-    const long items = (long)p.B * p.H;
-    const long item = ((long)blockIdx.x * 4 + wave) / nsub;
-    if (nsub == 1 && item >= items) return;
-    const long ic = min(item, items - 1);          // with shared queries every wave reaches the fold's barrier
-    attn_suffix_body<FUSED, false>(p, (int)(ic / p.H), (int)(ic % p.H), wave % nsub, nsub, item < items);
+    const int hq = blockIdx.x * 4 + wave;
+    const int h = nsub == 4 ? hq >> 2 : (nsub == 2 ? hq >> 1 : hq);
+    if (nsub == 1 && h >= p.H) return;
+    // with shared queries every wave reaches the fold's barrier: one past the last head repeats it and writes nothing
+    attn_suffix_body<FUSED, false>(p, blockIdx.y, min(h, p.H - 1), hq & (nsub - 1), nsub, h < p.H);
 }
 
 // ---- the whole decode attention in ONE launch -----------------------------------------------------------------
@@ -854,7 +855,7 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
                               void *workspace, size_t workspace_bytes, smh_stream_t stream) {
     using namespace smh;
     SMH_REQUIRE(D == ATT_D, "%s: head dim %d (only 128)", who, D);
-    SMH_REQUIRE(B >= 0 && H > 0 && Hkv > 0 && H % Hkv == 0 && P >= 0, "%s: B=%d H=%d Hkv=%d P=%d", who, B, H, Hkv, P);
+    SMH_REQUIRE(B >= 0 && B <= 65535 && H > 0 && Hkv > 0 && H % Hkv == 0 && P >= 0, "%s: B=%d (at most 65535) H=%d Hkv=%d P=%d", who, B, H, Hkv, P);
     SMH_REQUIRE(suffix_format == SMH_KV_NONE || suffix_format == SMH_KV_FP16 || suffix_format == SMH_KV_Q40,
                 "%s: suffix_format=%d", who, suffix_format);
     if (B == 0) return 0;
@@ -903,8 +904,7 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
     if (p.splits > 0)
         hipLaunchKernelGGL(attn_prefix_kernel<false>, dim3(p.splits, Hkv, qgroups), dim3(256), 0, (hipStream_t)stream, p);
     p.suffix_waves = attn_plan_suffix_waves_two((long)B * H);
-    long items = (long)B * H * p.suffix_waves;
-    hipLaunchKernelGGL(attn_suffix_kernel<false>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL(attn_suffix_kernel<false>, dim3((unsigned)((H * p.suffix_waves + 3) / 4), (unsigned)B), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
 }
 
@@ -991,8 +991,7 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
     if (p.splits > 0)
         hipLaunchKernelGGL(attn_prefix_kernel<true>, dim3(p.splits, Hkv, qgroups), dim3(256), 0, (hipStream_t)stream, p);
     p.suffix_waves = attn_plan_suffix_waves_two((long)B * H);
-    long items = (long)B * H * p.suffix_waves;
-    hipLaunchKernelGGL(attn_suffix_kernel<true>, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL(attn_suffix_kernel<true>, dim3((unsigned)((H * p.suffix_waves + 3) / 4), (unsigned)B), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
 }
 

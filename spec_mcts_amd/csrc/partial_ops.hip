@@ -143,9 +143,9 @@ __global__ __launch_bounds__(64) void partial_residual_sumsq_kernel(const void *
 // slabs hold [gate | up] (2 * n_half columns)
 __global__ __launch_bounds__(256) void partial_silu_mul_kernel(const void *__restrict__ partial, int ksplit, int M, int n_half,
                                                                half_t *__restrict__ out) {
-    const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
-    if (i >= (long)M * n_half) return;
-    const int m = (int)(i / n_half), n = (int)(i % n_half);
+    // grid (quads of a row, rows): no division to find the row (a 64-bit one costs more than the rest of the arithmetic)
+    const int m = blockIdx.y, n = (blockIdx.x * 256 + threadIdx.x) * 4;
+    if (n >= n_half) return;
     const long slab = (long)M * 2 * n_half;
     const f4 ga = slab_sum4(partial, (long)m * 2 * n_half + n, slab, ksplit, slab_is_half(M));
     const f4 ua = slab_sum4(partial, (long)m * 2 * n_half + n_half + n, slab, ksplit, slab_is_half(M));
@@ -171,11 +171,12 @@ __global__ __launch_bounds__(256) void partial_rope_append_kernel(const void *__
     __shared__ float s_row[4][128];
     const int lane = threadIdx.x & 63;
     const int wave = threadIdx.x >> 6;
-    const long item = (long)blockIdx.x * 4 + wave;
+    // grid (groups of four heads, branches)
     const int heads = H + 2 * Hkv;
-    const bool live = item < (long)B * heads;
-    const int b = live ? (int)(item / heads) : 0;
-    const int h = live ? (int)(item % heads) : 0;
+    const int hh = blockIdx.x * 4 + wave;
+    const bool live = hh < heads;
+    const int b = blockIdx.y;
+    const int h = live ? hh : 0;
     const int n_total = heads * 128;
     // the slabs are read two adjacent columns per lane; the rotation pairs column i with i + 64, so the sums
     // change lanes through LDS
@@ -519,8 +520,8 @@ extern "C" int smh_partial_silu_mul(const void *partial, int ksplit, int M, int 
     SMH_REQUIRE(M >= 0 && n_half > 0 && n_half % 4 == 0, "smh_partial_silu_mul: M=%d n_half=%d", M, n_half);
     if (M == 0) return 0;
     SMH_REQUIRE(partial && out, "smh_partial_silu_mul: null pointer");
-    long quads = (long)M * n_half / 4;
-    hipLaunchKernelGGL(partial_silu_mul_kernel, dim3((unsigned)((quads + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+    SMH_REQUIRE(M <= 65535, "smh_partial_silu_mul: M=%d (at most 65535 rows per launch)", M);
+    hipLaunchKernelGGL(partial_silu_mul_kernel, dim3((unsigned)((n_half / 4 + 255) / 256), (unsigned)M), dim3(256), 0, (hipStream_t)stream,
                        partial, ksplit, M, n_half, (half_t *)out);
     return launch_status();
 }
@@ -535,8 +536,8 @@ extern "C" int smh_partial_rope_append_kv(const void *partial, int ksplit, int B
     if (B == 0) return 0;
     SMH_REQUIRE(partial && q && k && v && cos_tab && sin_tab && pos_dev, "smh_partial_rope_append_kv: null pointer");
     SMH_REQUIRE(!cache_k || (cache_ks && cache_v && cache_vs && t_dev && Smax > 0), "smh_partial_rope_append_kv: cache arguments incomplete");
-    long items = (long)B * (H + 2 * Hkv);
-    hipLaunchKernelGGL(partial_rope_append_kernel, dim3((unsigned)((items + 3) / 4)), dim3(256), 0, (hipStream_t)stream,
+    SMH_REQUIRE(B <= 65535, "smh_partial_rope_append_kv: B=%d (at most 65535 branches per launch)", B);
+    hipLaunchKernelGGL(partial_rope_append_kernel, dim3((unsigned)((H + 2 * Hkv + 3) / 4), (unsigned)B), dim3(256), 0, (hipStream_t)stream,
                        partial, ksplit, B, H, Hkv, (half_t *)q, (half_t *)k, (half_t *)v,
                        (const half_t *)cos_tab, (const half_t *)sin_tab, pos_dev, (uint8_t *)cache_k, (half_t *)cache_ks,
                        (uint8_t *)cache_v, (half_t *)cache_vs, Smax, t_dev);

@@ -344,11 +344,14 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         f4 ga[MAXQ], ua[MAXQ];
         const int quads = slice_rows / 4, total = p.M * quads;
         const long gu_slab = (long)p.M * 2 * p.K;
+        // item idx = (row idx / quads, quad idx % quads); idx < 1024, so the quotient from a float reciprocal is exact
+        const float inv_quads = 1.0f / (float)max(quads, 1);
+        auto row_of = [&](int idx) { return (int)(((float)idx + 0.5f) * inv_quads); };
 #pragma unroll
         for (int i = 0; i < MAXQ; ++i) {
             const int idx = tid + i * THREADS;
             if (idx < total) {
-                const int m = idx / quads, k = slice_k0 + 4 * (idx % quads);
+                const int m = row_of(idx), k = slice_k0 + 4 * (idx - m * quads);
                 if (k < p.K) {
                     ga[i] = slab_sum4(p.gu_partial, (long)m * 2 * p.K + k, gu_slab, p.gu_ksplit, false);
                     ua[i] = slab_sum4(p.gu_partial, (long)m * 2 * p.K + p.K + k, gu_slab, p.gu_ksplit, false);
@@ -372,7 +375,8 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
                     const half_t sl = (half_t)(gf / (1.0f + expf(-gf)));
                     o[j] = sl * (half_t)ua[i][j];
                 }
-                *reinterpret_cast<h4 *>(xs + (long)(idx / quads) * xs_pitch + 4 * (idx % quads)) = o;
+                const int m = row_of(idx);
+                *reinterpret_cast<h4 *>(xs + (long)m * xs_pitch + 4 * (idx - m * quads)) = o;
             }
         }
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");      // xs is complete; the DMA ring stays in flight
