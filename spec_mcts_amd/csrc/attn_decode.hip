@@ -62,6 +62,10 @@ struct AttnParams {
     uint32_t *counters;              // one-launch variant: arrivals per kv head (zero between launches)
 };
 
+// x / n_rep and x % n_rep for the query heads per kv head; 1 (multi-head attention) needs no division
+__device__ __forceinline__ int div_rep(const AttnParams &p, int x) { return p.n_rep == 1 ? x : x / p.n_rep; }
+__device__ __forceinline__ int mod_rep(const AttnParams &p, int x) { return p.n_rep == 1 ? 0 : x % p.n_rep; }
+
 // column `col` of branch b in the fused q|k|v product: the slabs added in slice order, rounded once to fp16
 __device__ __forceinline__ half_t qkv_value(const AttnParams &p, int b, int col) {
     const int cols = (p.H + 2 * p.Hkv) * ATT_D;
@@ -148,7 +152,7 @@ __device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split,
     auto load_q = [&](int qt, h8 (&qb)[4]) {
         const int qr = min(qt * 16 + c, p.Bq - 1);
         if (!FUSED) {
-            const int b = qr / p.n_rep, r_ = qr % p.n_rep;
+            const int b = div_rep(p, qr), r_ = mod_rep(p, qr);
             const half_t *qp = p.q + ((long)b * p.H + hk * p.n_rep + r_) * ATT_D + 8 * g;
 #pragma unroll
             for (int k4 = 0; k4 < 4; ++k4) qb[k4] = *reinterpret_cast<const h8 *>(qp + 32 * k4);
@@ -192,7 +196,7 @@ __device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split,
         const int pos = *p.pos_dev;
         for (int qr = tid >> 4; qr < p.Bq; qr += 16) {
             h4 lo, hi;
-            qkv_query(p, qr / p.n_rep, hk * p.n_rep + qr % p.n_rep, pos, cc, lo, hi);
+            qkv_query(p, div_rep(p, qr), hk * p.n_rep + mod_rep(p, qr), pos, cc, lo, hi);
             *reinterpret_cast<h4 *>(&qs[qr][4 * cc]) = lo;
             *reinterpret_cast<h4 *>(&qs[qr][64 + 4 * cc]) = hi;
         }
@@ -458,7 +462,7 @@ __global__ __launch_bounds__(256) void attn_prefill_kernel(PrefillParams p) {
 // without a query of its own passes a valid (b, h) and live = false, and writes nothing).
 template <bool FUSED, bool PARTIAL>
 __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int h, int sub = 0, int nsub = 1, bool live = true) {
-    const int hk = h / p.n_rep;
+    const int hk = div_rep(p, h);
     __shared__ __attribute__((aligned(16))) half_t s_kv[FUSED ? 4 : 1][3][ATT_D];     // FUSED: this wave's new k and v rows, its query
     __shared__ float s_fold[4][16][10];                                                 // nsub > 1: the waves' states (m, l, o[8])
     const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
@@ -680,15 +684,16 @@ __global__ __launch_bounds__(256, 2) void attn_one_kernel(AttnParams p) {
     const int hk = blockIdx.y;
     const int tid = threadIdx.x;
     const int q_tiles = (p.Bq + 15) / 16;
-    const int per_wg = 4 / p.suffix_waves;     // queries of one suffix workgroup (suffix_waves = 1, 2 or 4 waves each)
+    const int sw_shift = p.suffix_waves == 4 ? 2 : (p.suffix_waves == 2 ? 1 : 0);
+    const int per_wg = 4 >> sw_shift;          // queries of one suffix workgroup (suffix_waves = 1, 2 or 4 waves each)
     int tile_lo = 0, tile_hi = q_tiles - 1;    // query tiles this workgroup contributed to
     if ((int)blockIdx.x < p.splits) {
         attn_prefix_body<FUSED, true, ATT_ONE_TW>(p, blockIdx.x, hk);
     } else {
         const int j = (int)blockIdx.x - p.splits, wave_ = tid >> 6;
-        const int qrow = per_wg * j + wave_ / p.suffix_waves;     // query of this kv head: branch qrow / n_rep, its query head qrow % n_rep
+        const int qrow = per_wg * j + (wave_ >> sw_shift);        // query of this kv head: branch qrow / n_rep, its query head qrow % n_rep
         const int qc = min(qrow, p.Bq - 1);
-        attn_suffix_body<FUSED, true>(p, qc / p.n_rep, hk * p.n_rep + qc % p.n_rep, wave_ % p.suffix_waves, p.suffix_waves, qrow < p.Bq);
+        attn_suffix_body<FUSED, true>(p, div_rep(p, qc), hk * p.n_rep + mod_rep(p, qc), wave_ & (p.suffix_waves - 1), p.suffix_waves, qrow < p.Bq);
         tile_lo = tile_hi = (per_wg * j) / 16;  // a workgroup's 1, 2 or 4 consecutive queries never straddle a tile of 16
     }
     wait_vmem();                               // this wave's partials have reached memory ...
@@ -697,7 +702,8 @@ __global__ __launch_bounds__(256, 2) void attn_one_kernel(AttnParams p) {
         uint32_t last = 0u;
         if (tid >= tile_lo && tid <= tile_hi) {
             // arrivals a tile waits for: every prefix slice + the suffix workgroups whose queries fall into it
-            const int j_lo = (16 * tid) / per_wg, j_hi = (min(p.Bq, 16 * tid + 16) - 1) / per_wg;
+            const int pw_shift = 2 - sw_shift;       // per_wg = 1 << pw_shift
+            const int j_lo = (16 * tid) >> pw_shift, j_hi = (min(p.Bq, 16 * tid + 16) - 1) >> pw_shift;
             const uint32_t expected = (uint32_t)(p.splits + j_hi - j_lo + 1);
             uint32_t *cnt = p.counters + hk * q_tiles + tid;
             const uint32_t prev = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -789,7 +795,7 @@ __global__ __launch_bounds__(256, 2) void attn_one_kernel(AttnParams p) {
         }
         if (si != 0 || !live) continue;
         const float inv = l > 0.f ? 1.0f / l : 0.f;
-        const int b = qrow / p.n_rep, h = hk * p.n_rep + qrow % p.n_rep;
+        const int b = div_rep(p, qrow), h = hk * p.n_rep + mod_rep(p, qrow);
         half_t *op = p.out + ((long)b * p.H + h) * ATT_D;
         *reinterpret_cast<h4 *>(op + 4 * cc) = h4{(half_t)(o[0] * inv), (half_t)(o[1] * inv), (half_t)(o[2] * inv), (half_t)(o[3] * inv)};
         *reinterpret_cast<h4 *>(op + 64 + 4 * cc) = h4{(half_t)(o[4] * inv), (half_t)(o[5] * inv), (half_t)(o[6] * inv), (half_t)(o[7] * inv)};
