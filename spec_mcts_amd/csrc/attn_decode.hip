@@ -830,7 +830,8 @@ static void attn_plan(int P, int Hkv, int Bq, int *tw_out, int *qgroups_out) {
 static int attn_plan_suffix_waves_two(long queries) {
     static const int most = env_int("SMH_ATTN_SUFFIX_WAVES", 4);
     int nsub = most >= 4 ? 4 : (most >= 2 ? 2 : 1);
-    while (nsub > 1 && queries * nsub > 4096) nsub >>= 1;
+    static const int cap = env_int("SMH_ATTN_SUFFIX_CAP", 4096);
+    while (nsub > 1 && queries * nsub > cap) nsub >>= 1;
     return nsub;
 }
 
