@@ -39,9 +39,9 @@ ARCHS = {
 }
 # HBM bytes per q40_gemv_kernel launch at M=1: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by a 1 GiB copy
 # (profiles/q40_gemv_m1_hbm_traffic.md has the commands and the factors: 2.0 for reads, 1.0 for writes)
-GEMV_TRAFFIC_BYTES_PER_LAUNCH = 27472929
+GEMV_TRAFFIC_BYTES_PER_LAUNCH = 27473888
 # the same for q40_gemm_kernel at M=100 (profiles/q40_gemm_m100_hbm_traffic.md): 37.25 MB read + 15.13 MB written
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 52400748
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 52400769
 
 
 def q40_bytes(M, N, K):
