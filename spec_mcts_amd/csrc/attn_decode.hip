@@ -815,8 +815,9 @@ static int attn_plan_tw(int P, int Hkv) {
 // slice from the cache but write nothing extra, and only then by narrower slices.
 static void attn_plan(int P, int Hkv, int Bq, int *tw_out, int *qgroups_out) {
     const int rounds = ((Bq + 15) / 16 + 3) / 4;
-    int tw = ATT_TW_MAX, qg = 1;
-    while ((long)((P + tw - 1) / tw) * Hkv * qg < 256) {
+    static const int tw_most = env_int("SMH_ATTN_TW", ATT_TW_MAX), wgs_least = env_int("SMH_ATTN_WGS", 256);
+    int tw = tw_most >= 128 ? 128 : (tw_most >= 64 ? 64 : 32), qg = 1;
+    while ((long)((P + tw - 1) / tw) * Hkv * qg < wgs_least) {
         if (qg < rounds) qg = min(rounds, 2 * qg);
         else if (tw > 32) tw >>= 1;
         else break;
