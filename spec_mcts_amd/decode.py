@@ -36,8 +36,7 @@ class GraphDecoder:
 
     def _step(self):
         logits = self.model._forward_impl(self.tokens, 1, (self.state[0:1], self.state[1:2]))
-        nxt = K.argmax(logits.view(self.B, -1))
-        self.tokens.copy_(nxt.view(self.B, 1))
+        K.argmax(logits.view(self.B, -1), out=self.tokens)      # the next step's input, written in place
         self.state.add_(self.one)
 
     @torch.inference_mode()

@@ -397,13 +397,16 @@ def silu_mul(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def argmax(logits: torch.Tensor) -> torch.Tensor:
-    """Greedy pick over the last dim of fp16 logits [rows, vocab]; lowest index on ties."""
+def argmax(logits: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """Greedy pick over the last dim of fp16 logits [rows, vocab]; lowest index on ties.  `out`: int64, `rows`
+    contiguous elements to write into (a decode loop's token buffer) instead of a fresh tensor."""
     lib = _lib.load()
     _need_gpu(logits)
     assert logits.dim() == 2 and logits.dtype == torch.float16 and logits.stride(1) == 1
     rows, vocab = logits.shape
-    out = torch.empty(rows, device=logits.device, dtype=torch.int64)
+    if out is None:
+        out = torch.empty(rows, device=logits.device, dtype=torch.int64)
+    assert out.dtype == torch.int64 and out.numel() == rows and out.is_contiguous() and out.device == logits.device
     check(lib.smh_argmax(logits.data_ptr(), rows, vocab, logits.stride(0), out.data_ptr(), _stream()), "smh_argmax")
     return out
 
