@@ -235,7 +235,9 @@ int smh_shared_prefix_attn_one(const void *q, void *out, int B, int H, int Hkv, 
  *                       order as the three-launch sequence: results are bit-identical to it;
  *                       workspace as for smh_shared_prefix_attn.
  *   single_launch != 0: ONE launch: prefix slices and the branches' suffixes run side by side, the workgroup
- *                       that completes the count of a tile of 16 queries merges its partials in a fixed order.
+ *                       that completes the count of a tile of 16 queries merges its partials in a fixed order
+ *                       (the faster form up to about 16 queries per kv head, B * H / Hkv; above, the one workgroup
+ *                       that merges a kv head's tiles takes longer than a second launch).
  *                       workspace: smh_attn_qkv_workspace_bytes(B, H, P) bytes whose first 4096 bytes (the
  *                       counters) are zero before the first call; the calls leave them zero.  Calls that
  *                       overlap in time need separate workspaces. */

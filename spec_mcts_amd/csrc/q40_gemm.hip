@@ -3,7 +3,7 @@
 // A workgroup of 4 waves owns 128 rows of A, two adjacent 128-column blocks of the weight (one full
 // 128-byte line of packed nibbles per k) and a slice of K; two workgroups share a compute unit.
 // Everything a 32-row step needs - 4 KB of nibbles, 256 B of scales, the 128 x 32 tile of A - goes
-// global -> LDS by DMA (global_load_lds) into a 6-stage ring shared by the workgroup; one bare
+// global -> LDS by DMA (global_load_lds) into a 4-stage ring shared by the workgroup; one bare
 // s_barrier per step both publishes a stage and frees the oldest one.  (__syncthreads() would wait
 // for every outstanding DMA first, because they write LDS, and so empty the ring at every step.)
 //   * wave w decodes TWO byte positions of ONE block (block w/2, bytes 2(w%2) and 2(w%2)+1 of every
