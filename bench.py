@@ -266,6 +266,15 @@ def main():
         print(json.dumps(matmul_roofline(torch, model, a.roofline_only, 3)))
         return
     batches = tuple(int(x) for x in a.batches.split(",")) if a.batches else BATCHES
+    # the prefill of the shared prompt (once per tree, outside the timed decode steps): reported next to them
+    dec = GraphDecoder(model, 1, use_graph=False)
+    dec.prefill(prompt)
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.prefill(prompt)
+    torch.cuda.synchronize()
+    prefill_ms = (time.perf_counter() - t0) * 1e3
+    del dec
     by_batch = {}
     for B in batches:
         dec = GraphDecoder(model, B, use_graph=not a.no_graph)
@@ -304,6 +313,7 @@ def main():
         "config": {"workload": "codellama%s_arch_q40_decode_prompt%d_shared_prefix" % (a.arch, prompt_len), "branches": head_b,
                    "layers": a.layers, "graph": not a.no_graph},
         "by_batch": {str(B): {k: (round(v, 4) if isinstance(v, float) else v) for k, v in d.items()} for B, d in by_batch.items()},
+        "prefill": {"prompt_tokens": prompt_len, "ms": round(prefill_ms, 3), "tok_s": round(prompt_len / (prefill_ms * 1e-3), 1)},
     }
     if not a.no_roofline:
         rf1 = matmul_roofline(torch, model, 1, 5)
