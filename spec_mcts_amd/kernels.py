@@ -681,6 +681,32 @@ def page_flash_attn(p: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.
                               n_kv_heads=H)
 
 
+def chunk_attn(p: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, P: int, B: int, L: int, H: int,
+               D: int, offset: int) -> torch.Tensor:
+    """The intended result of triton_kernels.chunk_attn (triton_kernels.py:1150-1231): the first `offset` pages of
+    the pools k/v [H,P,D] are one chunk that every branch attends to (no paging: pool rows 0..offset-1 in order),
+    followed by the branch's own pages p[b, offset:L].  p [B,L] integer page ids, q [B,H,D] -> [B,H,D] fp16; equal
+    to page_flash_attn whenever p[b, :offset] == arange(offset).  The reference's two kernels do not combine
+    their softmax states correctly (base-2 against natural maxima, the first kernel's output not reloaded), so
+    this follows the docstring of the reference function, not its output.  The shared chunk is the prefix of the
+    decode attention kernel (read once for all branches), the own pages are gathered into its suffix layout."""
+    _need_gpu(p, q, k, v)
+    assert p.shape == (B, L) and q.shape == (B, H, D) and k.shape == (H, P, D) and v.shape == (H, P, D)
+    assert 0 <= offset <= L and offset <= P
+    pk = k[:, :offset].transpose(0, 1).contiguous() if offset else None     # [offset, H, D]
+    pv = v[:, :offset].transpose(0, 1).contiguous() if offset else None
+    S = L - offset
+    if S:
+        idx = p[:, offset:].to(torch.int64)
+        kt = k.transpose(0, 1)[idx].contiguous()          # [B, S, H, D]
+        vt = v.transpose(0, 1)[idx].contiguous()
+        lens = torch.full((B,), S, dtype=torch.int32, device=q.device)
+    else:
+        kt = vt = lens = None
+    return shared_prefix_attn(q.contiguous(), pk, pv, offset, suffix_k=kt, suffix_v=vt, Smax=S, lens=lens,
+                              lens_stride=1, n_kv_heads=H)
+
+
 class DecodeStepKernel:
     """One decode step (embedding + every layer) of up to 16 branches as a single persistent kernel.
 

@@ -149,7 +149,7 @@ def test_prefill_causal_special_cases():
     assert torch.allclose(out[70:], v[70:71].float().expand(S - 70, H, 128), atol=2e-3, rtol=1e-2)
 
 
-def test_flash_attn_and_page_flash_attn_drop_ins():
+def test_flash_attn_page_flash_attn_and_chunk_attn_drop_ins():
     """the reference's operator names (triton_kernels.py:621, :764) on top of the decode attention kernel, with
     the shapes of its own checks (triton_kernels_bench.py:294-330: B=100, L=512, H=32, D=128, atol 1e-2)"""
     from spec_mcts_amd import kernels as K
@@ -173,6 +173,19 @@ def test_flash_attn_and_page_flash_attn_drop_ins():
     vv = vp.float()[:, idx].permute(1, 0, 2, 3)
     want2 = torch.nn.functional.scaled_dot_product_attention(q2.float()[:, :, None], kk, vv)[:, :, 0]
     assert torch.allclose(got2.float(), want2, rtol=1e-2, atol=2e-3)
+    # chunked: pool rows 0..offset-1 shared by every branch, then the branch's own pages; the shapes of the
+    # reference's tree-attention check (triton_kernels_bench.py:479-493: 27 branches, 512 rows, 256 shared)
+    for offset, L3 in ((256, 512), (0, 40), (40, 40)):
+        pager3 = torch.randint(0, P, (B2, L3), generator=g).to(torch.int16)
+        pager3[:, :offset] = torch.arange(offset, dtype=torch.int16)
+        got3 = K.chunk_attn(pager3.cuda(), q2.cuda(), kp.cuda(), vp.cuda(), P, B2, L3, H, D, offset).cpu()
+        idx3 = pager3.long()
+        want3 = torch.nn.functional.scaled_dot_product_attention(
+            q2.float()[:, :, None], kp.float()[:, idx3].permute(1, 0, 2, 3), vp.float()[:, idx3].permute(1, 0, 2, 3))[:, :, 0]
+        assert got3.dtype == torch.float16 and torch.allclose(got3.float(), want3, rtol=1e-2, atol=2e-3)
+        if offset:
+            same = K.page_flash_attn(pager3.cuda(), q2.cuda(), kp.cuda(), vp.cuda(), P, B2, L3, H, D).cpu()
+            assert torch.allclose(got3.float(), same.float(), rtol=1e-2, atol=2e-3)
 
 
 @pytest.mark.parametrize("B,H,Hkv,P,t", [(1, 4, 4, 40, 0), (3, 4, 4, 40, 5), (16, 8, 2, 100, 9), (5, 8, 8, 0, 3)])
