@@ -42,6 +42,8 @@ ARCHS = {
 GEMV_TRAFFIC_BYTES_PER_LAUNCH = 27473888
 # the same for q40_gemm_kernel at M=100 (profiles/q40_gemm_m100_hbm_traffic.md): 37.25 MB read + 15.13 MB written
 GEMM_TRAFFIC_BYTES_PER_LAUNCH = 52400769
+# the same for one call of the decode attention leg (profiles/attn_decode_hbm_traffic.md): 78.7 MB read + 9.0 MB written
+ATTN_TRAFFIC_BYTES_PER_CALL = 87773495
 
 
 def q40_bytes(M, N, K):
@@ -226,6 +228,9 @@ def main():
     ap.add_argument("--roofline-only", type=int, default=0, metavar="M",
                     help="profiling aid: run only the matmul roofline leg at batch M (eager launches, one pass) after a 1 GiB "
                          "device copy that calibrates the profiler's byte counters, and print that leg's numbers")
+    ap.add_argument("--attention-only", action="store_true",
+                    help="profiling aid: run only the decode attention leg (64 branches, 1024-token shared prefix, ragged Q4_0 suffixes) "
+                         "after the same 1 GiB calibration copy, and print that leg's numbers")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers for a quick functional run (INVALID as a result)")
     ap.add_argument("--arch", choices=sorted(ARCHS), default="7b",
                     help="7b is the headline workload; 70b is the 80-layer GQA architecture with a 2048-token prompt (about 38 GB of Q4_0 "
@@ -257,13 +262,13 @@ def main():
         model.norm_in_max_rows = a.norm_in_rows
     prompt = torch.randint(0, 32016, (1, prompt_len), generator=torch.Generator().manual_seed(3)).cuda()
 
-    if a.roofline_only:
+    if a.roofline_only or a.attention_only:
         src = torch.empty(1 << 29, dtype=torch.float16, device="cuda:0").normal_()
         dst = torch.empty_like(src)
         dst.copy_(src)                                     # 1 GiB read + 1 GiB written by one elementwise kernel
         torch.cuda.synchronize()
         del src, dst
-        print(json.dumps(matmul_roofline(torch, model, a.roofline_only, 3)))
+        print(json.dumps(attention_roofline(torch) if a.attention_only else matmul_roofline(torch, model, a.roofline_only, 3)))
         return
     batches = tuple(int(x) for x in a.batches.split(",")) if a.batches else BATCHES
     # the prefill of the shared prompt (once per tree, outside the timed decode steps): reported next to them
@@ -337,7 +342,7 @@ def main():
             {"kernel": "attn_prefix_kernel + attn_suffix_kernel: 64 branches x 32 heads, shared 1024-token fp16 prefix, ragged Q4_0 "
                        "suffixes of 0..256 rows (the two launches of one call)",
              "bound": "hbm", "achieved": round(att["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-             "frac": round(att["gbs"] / HBM_PEAK_GBS, 4), "avg_call_us": round(att["us"], 2), "bytes_per_call": att["bytes"]})
+             "frac": round(att["gbs"] / HBM_PEAK_GBS, 4), "avg_call_us": round(att["us"], 2), "bytes_per_call": att["bytes"], "traffic": ATTN_TRAFFIC_BYTES_PER_CALL})
         if 1 in by_batch and by_batch[1]["path"].startswith("persistent"):
             # the whole step is one launch: every weight, the prefix KV and the suffix KV once
             b1 = lin_bytes + prefix_bytes + t_mid * suffix_row_bytes
