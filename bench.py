@@ -219,8 +219,6 @@ def main():
     ap.add_argument("--warmup", type=int, default=10)
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--no-graph", action="store_true")
-    ap.add_argument("--persistent", action="store_true", help="batches up to 4 through the persistent step kernel (comparison runs)")
-    ap.add_argument("--finish-in-matmul", action="store_true", help="operators after a linear finished inside the matmul launch (comparison runs)")
     ap.add_argument("--no-norm-in-matmul", action="store_true", help="RMSNorm as its own launch at every batch size (comparison runs)")
     ap.add_argument("--norm-in-rows", type=int, default=-1, help="RMSNorm inside the matmul up to this many rows (comparison runs; default: the model's)")
     ap.add_argument("--batches", default="", help="comma-separated subset of 1,10,100 to run (a partial run is not a valid result)")
@@ -252,10 +250,6 @@ def main():
                    max_prompt_seq_len=prompt_len)
     torch.manual_seed(3)
     model = build_model(torch, args_kw, seed=3)
-    if a.persistent:
-        model.persistent = True
-    if a.finish_in_matmul:
-        model.finish_in_matmul = True
     if a.no_norm_in_matmul:
         model.norm_in_matmul = False
     if a.norm_in_rows >= 0:
@@ -291,9 +285,7 @@ def main():
         dec.decode(steps)
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
-        model.check_step_kernels()
-        by_batch[B] = {"tok_s": B * steps / dt, "ms_per_step": dt / steps * 1e3,
-                       "path": "persistent step kernel" if (model.persistent and B <= model.persistent_max_branches) else "operator kernels"}
+        by_batch[B] = {"tok_s": B * steps / dt, "ms_per_step": dt / steps * 1e3}
         del dec
 
     # per-step algorithmic HBM bytes: Q4 linears + fp16 lm_head + shared prefix KV (once) + suffix KV (Q4 rows)
@@ -343,13 +335,6 @@ def main():
                        "suffixes of 0..256 rows (the two launches of one call)",
              "bound": "hbm", "achieved": round(att["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
              "frac": round(att["gbs"] / HBM_PEAK_GBS, 4), "avg_call_us": round(att["us"], 2), "bytes_per_call": att["bytes"], "traffic": ATTN_TRAFFIC_BYTES_PER_CALL})
-        if 1 in by_batch and by_batch[1]["path"].startswith("persistent"):
-            # the whole step is one launch: every weight, the prefix KV and the suffix KV once
-            b1 = lin_bytes + prefix_bytes + t_mid * suffix_row_bytes
-            result["rooflines_other"].append(
-                {"kernel": "decode_mega_kernel at M=1 (one launch per step; bound from the step time less lm_head/argmax is not separated)",
-                 "bound": "hbm", "achieved": round(b1 / (by_batch[1]["ms_per_step"] * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBS,
-                 "unit": "GB/s", "frac": round(b1 / (by_batch[1]["ms_per_step"] * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
     if not a.no_cpu_baseline:
         cpu, cores, raw = cpu_baseline(torch, args_kw)
         result["cpu_baseline"] = {"value": round(cpu.get(head_b, cpu.get(max(cpu), 0.0)), 4), "unit": "tok/s", "cores": cores, "kind": "port",

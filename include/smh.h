@@ -249,89 +249,6 @@ int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, void *out, i
                                const int32_t *t_dev, int single_launch, void *workspace, size_t workspace_bytes,
                                smh_stream_t stream);
 
-/* ---- matmul with the following operator finished inside the same launch ---------------------------
- * smh_q40_matmul_fused: the product of smh_q40_matmul_partial (same a / segments / partial buffer)
- * followed, in the same launch for M <= 16 and as one more launch above, by the operator that
- * consumes the linear in TransformerBlock.forward (hf_model_q40_kv_shared.py:456-467):
- *   SMH_FIN_STORE            out[M, ldo] = fp16(sum) (+ residual)                       (LinearQ4_0, :228-236)
- *   SMH_FIN_RESIDUAL_RMSNORM h_out = residual + fp16(sum); xn_out = RMSNorm(h_out) * norm_weight
- *                            (the "h + wo(..)" / "h + w2(..)" of :463-466 and the norm of the next
- *                            sub-block, :123-134).  One weight; h_out may be residual (in place).
- *   SMH_FIN_SILU_MUL         out[M, ldo] = fp16(silu(fp16(sum_w1))) * fp16(sum_w3)      (:434)
- *                            two weights of equal width: w1 (gate), w3 (up)
- *   SMH_FIN_ROPE_APPEND      q, k, v = fp16(sum); apply_rotary_emb(q, k) (:173-203); Q4_0 append of k, v
- *                            to row *t_dev of each branch's suffix cache (:365-371).  Three weights wq, wk,
- *                            wv; arguments as smh_rope_append_kv.
- * counters: 32 KiB of device memory zeroed once by the caller and owned by these calls afterwards
- * (arrival counters that reset themselves + per-unit sums of squares).  Calls that share it must not
- * overlap in time.  Same arithmetic and rounding points as smh_q40_matmul_partial + smh_partial_*.
- */
-#define SMH_FIN_STORE 1
-#define SMH_FIN_RESIDUAL_RMSNORM 2
-#define SMH_FIN_SILU_MUL 3
-#define SMH_FIN_ROPE_APPEND 4
-#define SMH_FIN_COUNTER_BYTES 32768
-typedef struct smh_finish {
-    int mode;
-    void *counters;
-    void *out;
-    long ldo;
-    const void *residual;
-    long ldr;
-    void *h_out;
-    const void *norm_weight;
-    float eps;
-    void *xn_out;
-    int H, Hkv, Smax;
-    void *q, *k, *v;
-    const void *cos_tab, *sin_tab;
-    const int32_t *pos_dev, *t_dev;
-    void *cache_k, *cache_ks, *cache_v, *cache_vs;
-} smh_finish;
-int smh_q40_matmul_fused(const void *a, int M, int K, long lda, int nseg, const void *const *w,
-                         const void *const *s, const int *n, void *partial, size_t partial_bytes,
-                         const smh_finish *fin, smh_stream_t stream);
-
-/* ---- whole decode step ------------------------------------------------------------------------
- * smh_decode_step: one decode step (start_pos != 0) of Transformer.forward
- * (hf_model_q40_kv_shared.py:481-512) up to, not including, the final norm and lm_head, for
- * 1..16 branches, as ONE persistent kernel: embedding, then per layer RMSNorm -> wq|wk|wv -> RoPE
- * + Q4_0 KV append -> shared-prefix attention -> wo (+residual) -> RMSNorm -> w1|w3 -> SiLU*up ->
- * w2 (+residual), i.e. TransformerBlock.forward (:456-467) with Attention.forward (:313-405) and
- * FeedForward.forward (:431-436).  Same arithmetic and rounding points as the operator entry
- * points above.  Multi-head attention only (H == Hkv); dim, ffn multiples of 256.
- *   layers_dev  DEVICE array of n_layers descriptors; matrices in the order wq wk wv wo w1 w3 w2
- *               (packed bytes w[i], fp16 scales s[i], checkpoint layout), norm weights fp16 [dim],
- *               prefix_k/v fp16 [P, Hkv, 128], suffix cache as in smh_rope_append_kv
- *   tokens      int64 [M] on the device;  emb fp16 [vocab, dim]
- *   pos_dev, t_dev  int32 on the device: RoPE position and suffix row of this step
- *   h_out       fp16 [M, dim]: hidden state after the last layer (input of the final norm)
- *   workspace   smh_decode_step_workspace_bytes(...) bytes, 256-byte aligned, owned by the step
- *               kernel from smh_decode_prepare on.
- * smh_decode_prepare validates the configuration, clears the workspace and uploads the parameter
- * block into it (synchronous; once per configuration, e.g. after each prefill).  smh_decode_step
- * launches one step on `stream` (asynchronous, capturable in a graph); tokens, pos_dev, t_dev and
- * the caches are read at execution time.  smh_decode_status copies three status words to the
- * host (synchronous): [2] is nonzero if a bounded wait inside a step ran out - the workgroups of
- * a launch must all be resident at once - and the results are then invalid.
- * Steps that share a workspace must not overlap in time.
- */
-typedef struct smh_decode_layer {
-    const void *w[7];
-    const void *s[7];
-    const void *attn_norm, *ffn_norm;
-    const void *prefix_k, *prefix_v;
-    void *cache_k, *cache_v;
-    void *cache_ks, *cache_vs;
-} smh_decode_layer;
-size_t smh_decode_step_workspace_bytes(int n_layers, int M, int dim, int H, int Hkv, int ffn, int P, int Smax);
-int smh_decode_prepare(const smh_decode_layer *layers_dev, int n_layers, int M, int dim, int H, int Hkv,
-                       int ffn, int P, int Smax, float eps, const int64_t *tokens, const void *emb,
-                       const void *cos_tab, const void *sin_tab, const int32_t *pos_dev,
-                       const int32_t *t_dev, void *h_out, void *workspace, size_t workspace_bytes);
-int smh_decode_step(void *workspace, smh_stream_t stream);
-int smh_decode_status(const void *workspace, uint32_t *status3);
-
 #ifdef __cplusplus
 }
 #endif

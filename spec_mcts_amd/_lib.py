@@ -18,18 +18,6 @@ SMH_GEMV_MAX_M = 16
 
 _P = c_void_p
 # name -> (restype, argtypes); must list every symbol of include/smh.h
-class Finish(ctypes.Structure):
-    """struct smh_finish of include/smh.h"""
-    _fields_ = [("mode", c_int), ("counters", c_void_p), ("out", c_void_p), ("ldo", c_long), ("residual", c_void_p),
-                ("ldr", c_long), ("h_out", c_void_p), ("norm_weight", c_void_p), ("eps", c_float), ("xn_out", c_void_p),
-                ("H", c_int), ("Hkv", c_int), ("Smax", c_int), ("q", c_void_p), ("k", c_void_p), ("v", c_void_p),
-                ("cos_tab", c_void_p), ("sin_tab", c_void_p), ("pos_dev", c_void_p), ("t_dev", c_void_p),
-                ("cache_k", c_void_p), ("cache_ks", c_void_p), ("cache_v", c_void_p), ("cache_vs", c_void_p)]
-
-
-SMH_FIN_STORE, SMH_FIN_RESIDUAL_RMSNORM, SMH_FIN_SILU_MUL, SMH_FIN_ROPE_APPEND = 1, 2, 3, 4
-SMH_FIN_COUNTER_BYTES = 32768
-
 SIGNATURES = {
     "smh_version": (c_int, []),
     "smh_last_error_string": (c_char_p, []),
@@ -70,12 +58,6 @@ SIGNATURES = {
     "smh_attn_qkv_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "smh_shared_prefix_attn_qkv": (c_int, [_P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_int,
                                            _P, _P, _P, _P, c_int, _P, c_int, _P, c_size_t, _P]),
-    "smh_decode_step_workspace_bytes": (c_size_t, [c_int] * 8),
-    "smh_q40_matmul_fused": (c_int, [_P, c_int, c_int, c_long, c_int, _P, _P, _P, _P, c_size_t, _P, _P]),
-    "smh_decode_prepare": (c_int, [_P, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, _P, _P, _P, _P, _P, _P, _P, _P,
-                                   c_size_t]),
-    "smh_decode_step": (c_int, [_P, _P]),
-    "smh_decode_status": (c_int, [_P, _P]),
 }
 
 _lib = None

@@ -22,8 +22,6 @@
 
 namespace smh {
 
-int env_int(const char *name, int dflt);      // q40_gemv.hip
-
 constexpr int ATT_D = 128;
 constexpr int ATT_TW_MAX = 128;            // prefix rows per workgroup
 constexpr int ATT_KPITCH = 136;            // halves per LDS row of K (272 B: 16 rows hit distinct banks)
@@ -815,8 +813,8 @@ static int attn_plan_tw(int P, int Hkv) {
 // slice from the cache but write nothing extra, and only then by narrower slices.
 static void attn_plan(int P, int Hkv, int Bq, int *tw_out, int *qgroups_out) {
     const int rounds = ((Bq + 15) / 16 + 3) / 4;
-    static const int tw_most = env_int("SMH_ATTN_TW", ATT_TW_MAX), wgs_least = env_int("SMH_ATTN_WGS", 256);
-    int tw = tw_most >= 128 ? 128 : (tw_most >= 64 ? 64 : 32), qg = 1;
+    constexpr int wgs_least = 256;
+    int tw = ATT_TW_MAX, qg = 1;
     while ((long)((P + tw - 1) / tw) * Hkv * qg < wgs_least) {
         if (qg < rounds) qg = min(rounds, 2 * qg);
         else if (tw > 32) tw >>= 1;
@@ -829,9 +827,8 @@ static void attn_plan(int P, int Hkv, int Bq, int *tw_out, int *qgroups_out) {
 // Suffix launch of the two-launch form: waves per (branch, query head) - more than one while the launch still fits
 // the GPU in one round (4 waves of this kernel per SIMD, 1024 SIMDs).
 static int attn_plan_suffix_waves_two(long queries) {
-    static const int most = env_int("SMH_ATTN_SUFFIX_WAVES", 4);
-    int nsub = most >= 4 ? 4 : (most >= 2 ? 2 : 1);
-    static const int cap = env_int("SMH_ATTN_SUFFIX_CAP", 4096);
+    int nsub = 4;
+    constexpr int cap = 4096;
     while (nsub > 1 && queries * nsub > cap) nsub >>= 1;
     return nsub;
 }
@@ -839,8 +836,7 @@ static int attn_plan_suffix_waves_two(long queries) {
 // One-launch kernel: waves that share a query's suffix rows - as many as keep the launch within one round of
 // workgroups (two fit a compute unit).
 static int attn_plan_suffix_waves(int splits, int Bq, int Hkv) {
-    static const int most = env_int("SMH_ATTN_SUFFIX_WAVES", 4);
-    int nsub = most >= 4 ? 4 : (most >= 2 ? 2 : 1);
+    int nsub = 4;
     while (nsub > 1 && (long)(splits + (Bq + 4 / nsub - 1) / (4 / nsub)) * Hkv > 512) nsub >>= 1;
     return nsub;
 }

@@ -353,80 +353,6 @@ extern "C" int smh_q40_matmul_partial_tiled_norm(const void *h, long ldh, const 
     return gemv_launch(p, (hipStream_t)stream);
 }
 
-extern "C" int smh_q40_matmul_fused(const void *a, int M, int K, long lda, int nseg, const void *const *w,
-                                    const void *const *s, const int *n, void *partial, size_t partial_bytes,
-                                    const smh_finish *fin, smh_stream_t stream) {
-    const char *who = "smh_q40_matmul_fused";
-    MatmulParams p;
-    int st = fill_params(p, a, M, K, lda, nseg, w, s, n, who);
-    if (st) return st;
-    if (M == 0) return 0;
-    SMH_REQUIRE(a && w && s && partial && fin, "%s: null pointer", who);
-    for (int i = 0; i < nseg; ++i) SMH_REQUIRE(w[i] && s[i], "%s: null weight %d", who, i);
-    size_t need = (size_t)p.ksplit * M * p.n_total * sizeof(float);
-    SMH_REQUIRE(partial_bytes >= need, "%s: partial buffer %zu < %zu bytes", who, partial_bytes, need);
-    SMH_REQUIRE(fin->mode >= SMH_FIN_STORE && fin->mode <= SMH_FIN_ROPE_APPEND, "%s: mode %d", who, fin->mode);
-    SMH_REQUIRE(fin->counters != nullptr && p.units <= 1024, "%s: counters missing or too many column units (%d)", who, p.units);
-    const int N = p.n_total;
-    switch (fin->mode) {
-        case SMH_FIN_STORE:
-            SMH_REQUIRE(fin->out && fin->ldo >= N && fin->ldo % 4 == 0 && (!fin->residual || fin->ldr >= N), "%s: STORE arguments", who);
-            break;
-        case SMH_FIN_RESIDUAL_RMSNORM:
-            SMH_REQUIRE(nseg == 1 && fin->residual && fin->ldr >= N && fin->h_out && fin->norm_weight && fin->xn_out && N % 256 == 0,
-                        "%s: RESIDUAL_RMSNORM takes one weight with N %% 256 == 0, residual, h_out, norm_weight, xn_out", who);
-            SMH_REQUIRE((size_t)p.units * M * 4 + 8192 <= SMH_FIN_COUNTER_BYTES || M > SMH_GEMV_MAX_M, "%s: too many units x rows", who);
-            break;
-        case SMH_FIN_SILU_MUL:
-            SMH_REQUIRE(nseg == 2 && n[0] == n[1] && n[0] % 256 == 0 && fin->out && fin->ldo >= n[0], "%s: SILU_MUL takes w1, w3 of equal width (multiple of 256) and out", who);
-            break;
-        default:
-            SMH_REQUIRE(nseg == 3 && fin->H > 0 && fin->Hkv > 0 && n[0] == fin->H * 128 && n[1] == fin->Hkv * 128 && n[2] == n[1] &&
-                        n[0] % 256 == 0 && n[1] % 256 == 0, "%s: ROPE_APPEND takes wq, wk, wv with 128-wide heads in pairs", who);
-            SMH_REQUIRE(fin->q && fin->k && fin->v && fin->cos_tab && fin->sin_tab && fin->pos_dev, "%s: ROPE_APPEND null pointer", who);
-            SMH_REQUIRE(!fin->cache_k || (fin->cache_ks && fin->cache_v && fin->cache_vs && fin->t_dev && fin->Smax > 0), "%s: cache arguments incomplete", who);
-            break;
-    }
-    p.partial = (float *)partial;
-    p.direct = 0;
-    hipStream_t hs = (hipStream_t)stream;
-    if (M <= SMH_GEMV_MAX_M) {
-        MatmulFinish &f = p.fin;
-        uint32_t *cnt = (uint32_t *)fin->counters;
-        f.mode = fin->mode;
-        f.row_cnt = cnt;
-        f.unit_cnt = cnt + 16;
-        f.ssq = (float *)(cnt + 2048);
-        f.out = (half_t *)fin->out; f.ldo = fin->ldo;
-        f.resid = (const half_t *)fin->residual; f.ldr = fin->ldr;
-        f.h_out = (half_t *)fin->h_out; f.norm_w = (const half_t *)fin->norm_weight; f.xn_out = (half_t *)fin->xn_out; f.eps = fin->eps;
-        f.H = fin->H; f.Hkv = fin->Hkv; f.Smax = fin->Smax;
-        f.q = (half_t *)fin->q; f.k = (half_t *)fin->k; f.v = (half_t *)fin->v;
-        f.cos_tab = (const half_t *)fin->cos_tab; f.sin_tab = (const half_t *)fin->sin_tab;
-        f.pos_dev = fin->pos_dev; f.t_dev = fin->t_dev;
-        f.cache_k = (uint8_t *)fin->cache_k; f.cache_v = (uint8_t *)fin->cache_v;
-        f.cache_ks = (half_t *)fin->cache_ks; f.cache_vs = (half_t *)fin->cache_vs;
-        return gemv_launch(p, hs);
-    }
-    // larger M: the slabs of the GEMM are finished by one more launch
-    st = gemm_launch(p, hs);
-    if (st) return st;
-    switch (fin->mode) {
-        case SMH_FIN_STORE:
-            return smh_partial_reduce(partial, p.ksplit, M, N, 0, N, fin->out, fin->ldo, fin->residual ? SMH_EPI_RESIDUAL : SMH_EPI_NONE,
-                                      fin->residual, fin->ldr, stream);
-        case SMH_FIN_RESIDUAL_RMSNORM:
-            SMH_REQUIRE(fin->ldr == N, "%s: residual must be dense for M > %d", who, SMH_GEMV_MAX_M);
-            return smh_partial_rmsnorm(partial, p.ksplit, M, N, fin->residual, fin->norm_weight, fin->eps, fin->h_out, fin->xn_out, stream);
-        case SMH_FIN_SILU_MUL:
-            SMH_REQUIRE(fin->ldo == n[0], "%s: out must be dense for M > %d", who, SMH_GEMV_MAX_M);
-            return smh_partial_silu_mul(partial, p.ksplit, M, n[0], fin->out, stream);
-        default:
-            return smh_partial_rope_append_kv(partial, p.ksplit, M, fin->H, fin->Hkv, 128, fin->q, fin->k, fin->v, fin->cos_tab, fin->sin_tab,
-                                              fin->pos_dev, fin->cache_k, fin->cache_ks, fin->cache_v, fin->cache_vs, fin->Smax, fin->t_dev, stream);
-    }
-}
-
 static int reduce_launch(const void *partial, int ksplit, int M, int n_total, int col0, int N, void *c, long ldc,
                          int epilogue, const void *residual, long ldr, hipStream_t stream) {
     long quads = ((long)M * N + 3) / 4;

@@ -376,11 +376,10 @@ void gemm_fill_plan(MatmulParams &p) {
     // (at least 200 of the 256 units busy): a second co-resident workgroup buys little there and doubles the
     // slabs the next kernel has to read.  Otherwise two per compute unit.  (At M = 100 matrices with few column
     // units still take up to 16 slices: idle compute units cost more than the slab traffic.)
-    static const int capacity = env_int("SMH_GEMM_WGS", 512);
+    constexpr int capacity = 512;
     int ks = (int)(capacity / 2 / tiles);
     if (ks < 1 || tiles * ks < 200) ks = (int)(capacity / tiles);
-    static const int cap_num = env_int("SMH_GEMM_KSCAP", 1600);
-    int cap = cap_num / (p.M > 0 ? p.M : 1);
+    int cap = 1600 / (p.M > 0 ? p.M : 1);
     if (cap > SMH_MAX_KSPLIT) cap = SMH_MAX_KSPLIT;
     if (ks > cap) ks = cap;
     if (ks > steps / GEMM_STAGES) ks = steps / GEMM_STAGES;

@@ -25,14 +25,13 @@
 // blockIdx.x = slice * units_pad + slot with units_pad a multiple of 8: workgroups are dealt round-robin
 // to the 8 XCDs, so all K-slices of a column unit run behind the same L2, and slot -> unit gives every
 // XCD a contiguous run of units (they share the cache lines of the scales).
-#include <stdlib.h>
-
 #include "q40_matmul.hpp"
 #include "slab_sum.hpp"
 
 namespace smh {
 
 constexpr int GEMV_COLS = 256;             // columns per workgroup
+constexpr int GEMV_WAVES = 4;              // waves per workgroup, each with its own ring
 
 // ---- per-wave ring of 32-row steps in LDS ----------------------------------------------------------
 // The loads of a step go straight from global memory to LDS (global_load_lds, no VGPRs held while
@@ -241,14 +240,13 @@ __device__ __forceinline__ void gemv_consume_tiled(const uint8_t *stage, int k0,
         }
 }
 
-// FINISH: the workgroup that completes a column unit also applies the operator that follows the linear
-// (matmul_finish.hpp); a separate instantiation, so that the plain kernel keeps its register budget
 // LAYOUT 0: checkpoint layout; 1: tiled weights (smh_q40_tile); 2: tiled weights and activations made from the
 // gate|up slabs by the workgroup itself (p.gu_partial): SiLU(gate) * up needs no launch of its own; 3: tiled weights
 // and activations made from the residual stream by the workgroup itself (p.norm_w, p.norm_ss): RMSNorm needs only
 // the small launch that adds the slabs and leaves the sums of squares
-template <int WAVES, bool FINISH, int LAYOUT>
-__global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
+template <int LAYOUT>
+__global__ __launch_bounds__(GEMV_WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
+    constexpr int WAVES = GEMV_WAVES;
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];   // WAVES rings, then reused as red[WAVES][M][256]
     constexpr int THREADS = WAVES * 64;
     constexpr bool TILED = LAYOUT != 0;
@@ -493,7 +491,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
 
     const int outputs = p.M * GEMV_COLS;
     float *slab = p.partial + (long)slice * p.M * p.n_total;
-    if (!FINISH && !p.direct) {
+    if (!p.direct) {
         // slabs: four consecutive columns per thread (segment widths are multiples of 128, so a quad is inside or outside)
         for (int q = tid; q < outputs / 4; q += THREADS) {
             f4 sum = {0.f, 0.f, 0.f, 0.f};
@@ -512,15 +510,7 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
         const int m = idx >> 8, n_seg = col0 + (idx & 255);
         if (n_seg >= seg.N) continue;
         const int n = seg.col0 + n_seg;
-        if (p.direct) p.c[(long)m * p.ldc + n] = matmul_epilogue(p, sum, m, n);
-        else if (FINISH) st_f32(slab + (long)m * p.n_total + n, sum);              // another workgroup of this launch reads it
-        else slab[(long)m * p.n_total + n] = sum;
-    }
-    if constexpr (FINISH) {
-        uint32_t *s_flag = reinterpret_cast<uint32_t *>(lds);      // the sums in LDS have been consumed ...
-        __syncthreads();                                           // ... by every thread
-        matmul_finish<THREADS>(p.fin, p.partial, p.ksplit, p.M, p.n_total, unit, p.units, seg.col0 + col0,
-                               min(GEMV_COLS, seg.N - col0), sg, col0, s_flag);
+        p.c[(long)m * p.ldc + n] = matmul_epilogue(p, sum, m, n);
     }
 }
 
@@ -528,17 +518,12 @@ __global__ __launch_bounds__(WAVES * 64) void q40_gemv_kernel(MatmulParams p) {
 
 namespace smh {
 
-int env_int(const char *name, int dflt) {
-    const char *v = getenv(name);
-    return v ? atoi(v) : dflt;
-}
-
 // K is cut into slices so that the launch fills the GPU in ONE round of workgroups: two
 // workgroups (two sets of LDS rings) fit a CU, 256 CUs, so at most 512 workgroups; a launch of a
 // few more than that would run a second, nearly empty round and take twice as long.
 void gemv_plan(int n_total_units, int K, int waves, int *ksplit, int *steps_per_slice) {
     const int steps = (K + 31) / 32;
-    static const int capacity = env_int("SMH_GEMV_WGS", 512);
+    constexpr int capacity = 512;
     int ks = capacity / n_total_units;              // floor: never exceed one round
     if (ks < 1) ks = 1;
     if (ks > SMH_MAX_KSPLIT) ks = SMH_MAX_KSPLIT;
@@ -547,13 +532,6 @@ void gemv_plan(int n_total_units, int K, int waves, int *ksplit, int *steps_per_
     const int sps = (steps + ks - 1) / ks;
     *ksplit = (steps + sps - 1) / sps;
     *steps_per_slice = sps;
-}
-
-int gemv_waves(int M) {
-    static const int waves_pref = env_int("SMH_GEMV_WAVES", 4);
-    int waves = waves_pref;
-    (void)M;
-    return waves;
 }
 
 void gemv_fill_plan(MatmulParams &p) {
@@ -567,7 +545,7 @@ void gemv_fill_plan(MatmulParams &p) {
     p.units = unit0;
     p.units_pad = (unit0 + 7) / 8 * 8;
     p.n_total = col0;
-    gemv_plan(p.units, p.K, gemv_waves(p.M), &p.ksplit, &p.steps_per_slice);
+    gemv_plan(p.units, p.K, GEMV_WAVES, &p.ksplit, &p.steps_per_slice);
 }
 
 bool gemv_norm_in_fits(const MatmulParams &p) {
@@ -575,7 +553,7 @@ bool gemv_norm_in_fits(const MatmulParams &p) {
 }
 
 int gemv_launch(const MatmulParams &p, hipStream_t stream) {
-    const int waves = gemv_waves(p.M);
+    constexpr int waves = GEMV_WAVES;
     dim3 grid((unsigned)(p.units_pad * p.ksplit));
     size_t lds = (size_t)waves * RING_BYTES;                       // rings, reused for the [waves][M][256] sums
     const size_t red = (size_t)waves * p.M * GEMV_COLS * sizeof(float);
@@ -583,10 +561,6 @@ int gemv_launch(const MatmulParams &p, hipStream_t stream) {
         lds = (size_t)waves * RING_BYTES_NO_X + (size_t)p.M * (p.steps_per_slice * 32 + 8) * sizeof(half_t) + SMH_GEMV_MAX_M * sizeof(float);
     if (red > lds) lds = red;
     if (p.tiled) {
-        if (p.fin.mode != 0 || waves != 4) {
-            set_error("q40 gemv: tiled weights run with 4 waves and without a finishing operator");
-            return -1;
-        }
         if (p.gu_partial != nullptr) {
             if (p.M > SMH_SILU_IN_MAX_M || p.steps_per_slice * 32 > SMH_SILU_IN_MAX_K) {
                 set_error("q40 gemv: activations from the gate|up slabs need M <= %d and K-slices of at most %d rows", SMH_SILU_IN_MAX_M,
@@ -594,27 +568,26 @@ int gemv_launch(const MatmulParams &p, hipStream_t stream) {
                 return -1;
             }
             // more than 64 KB of dynamic LDS has to be allowed once (not stream work: fine under graph capture)
-            static const hipError_t lds_ok = hipFuncSetAttribute((const void *)q40_gemv_kernel<4, false, 2>, hipFuncAttributeMaxDynamicSharedMemorySize,
+            static const hipError_t lds_ok = hipFuncSetAttribute((const void *)q40_gemv_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                                                  80 * 1024);
             if (lds_ok != hipSuccess) return (int)lds_ok;
-            hipLaunchKernelGGL((q40_gemv_kernel<4, false, 2>), grid, dim3(256), lds, stream, p);
+            hipLaunchKernelGGL((q40_gemv_kernel<2>), grid, dim3(256), lds, stream, p);
         } else if (p.norm_w != nullptr) {
             if (!gemv_norm_in_fits(p)) {
                 set_error("q40 gemv: %d rows x K-slices of %d rows do not fit next to the weight rings (RMSNorm inside the matmul)", p.M,
                           p.steps_per_slice * 32);
                 return -1;
             }
-            static const hipError_t lds_ok = hipFuncSetAttribute((const void *)q40_gemv_kernel<4, false, 3>, hipFuncAttributeMaxDynamicSharedMemorySize,
+            static const hipError_t lds_ok = hipFuncSetAttribute((const void *)q40_gemv_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                                                  80 * 1024);
             if (lds_ok != hipSuccess) return (int)lds_ok;
-            hipLaunchKernelGGL((q40_gemv_kernel<4, false, 3>), grid, dim3(256), lds, stream, p);
+            hipLaunchKernelGGL((q40_gemv_kernel<3>), grid, dim3(256), lds, stream, p);
         } else {
-            hipLaunchKernelGGL((q40_gemv_kernel<4, false, 1>), grid, dim3(256), lds, stream, p);
+            hipLaunchKernelGGL((q40_gemv_kernel<1>), grid, dim3(256), lds, stream, p);
         }
-    } else if (p.fin.mode != 0) hipLaunchKernelGGL((q40_gemv_kernel<4, true, 0>), grid, dim3(256), lds, stream, p);
-    else if (waves == 2) hipLaunchKernelGGL((q40_gemv_kernel<2, false, 0>), grid, dim3(128), lds, stream, p);
-    else if (waves == 8) hipLaunchKernelGGL((q40_gemv_kernel<8, false, 0>), grid, dim3(512), lds, stream, p);
-    else hipLaunchKernelGGL((q40_gemv_kernel<4, false, 0>), grid, dim3(256), lds, stream, p);
+    } else {
+        hipLaunchKernelGGL((q40_gemv_kernel<0>), grid, dim3(256), lds, stream, p);
+    }
     return launch_status();
 }
 

@@ -17,8 +17,6 @@
 #define SMH_NORM_SUMS 16            /* partial sums of squares per row that smh_partial_residual_sumsq leaves */
 #define SMH_NORM_IN_MAX_XS_BYTES 28160   /* M x K-slice fp16 activations next to the weight rings, two workgroups per CU */
 
-#include "matmul_finish.hpp"
-
 namespace smh {
 
 // ---- tiled weight layout ---------------------------------------------------------------------------
@@ -76,7 +74,6 @@ struct MatmulParams {
     const half_t *norm_w;
     const float *norm_ss;
     float norm_eps;
-    MatmulFinish fin;        // fin.mode == 0: leave the slabs to another launch
 };
 
 __device__ __forceinline__ half_t matmul_epilogue(const MatmulParams &p, float acc, int m, int n) {
@@ -88,7 +85,6 @@ __device__ __forceinline__ half_t matmul_epilogue(const MatmulParams &p, float a
 // The dtype of the slabs follows from the row count alone, so producer and consumer agree without a flag.
 __host__ __device__ inline bool slab_is_half(int M) { return M > SMH_GEMV_MAX_M; }
 
-int env_int(const char *name, int dflt);
 void gemv_fill_plan(MatmulParams &p);
 int gemv_launch(const MatmulParams &p, hipStream_t stream);
 bool gemv_norm_in_fits(const MatmulParams &p);     // after gemv_fill_plan: can RMSNorm be made inside the launch

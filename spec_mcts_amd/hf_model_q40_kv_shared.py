@@ -276,10 +276,7 @@ class Transformer(nn.Module):
         self._step_state = None       # int32 [2] on the device: (position, suffix index t)
         self._step_host = None
         self.fused = True             # fused decode-layer launches; False runs module by module
-        self.finish_in_matmul = False # decode: finish the operator after each linear inside the matmul launch (6 launches per
-                                      # layer instead of 10; measured slower at B=10: the finisher's round trips are serial)
         self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
-        self.persistent = False       # True: decode steps of few branches as one persistent kernel (needs fused); the operator kernels are faster
         self.fused_sampler = True          # generate(): temperature / top-k / draw as one kernel instead of five torch ops
         self.silu_in_matmul = True         # up to 2 rows: w2's launch makes its own SiLU(gate)*up activations
         self.tiled_weights = True          # the fused path streams tiled copies of the weights (LinearQ4_0.operand)
@@ -289,8 +286,6 @@ class Transformer(nn.Module):
         self.norm_in_max_rows = 2          # ... up to this many rows: at 10 rows the matmul's longer prologue costs more than it saves
         self._norm_in_ok = {}
         self.attn_from_qkv = True          # up to 16 branches the attention takes the wq|wk|wv product itself, in one launch
-        self.persistent_max_branches = 4   # with persistent = True: largest batch that uses the kernel (it takes up to 16)
-        self._step_kernels = {}       # branches -> K.DecodeStepKernel
 
     # -- helpers -------------------------------------------------------------------------------
     def _tables(self, device):
@@ -335,17 +330,8 @@ class Transformer(nn.Module):
         bsz, seqlen = tokens.shape
         M = bsz * seqlen
         p = self.params
-        if start_pos != 0 and seqlen == 1 and self.persistent and bsz <= self.persistent_max_branches:
-            sk = self._step_kernel(bsz, tokens.device)
-            if sk is not None:
-                pos_dev, t_dev = step_state
-                sk.prepare(self.layers[0].attention.cache_prompt_len, pos_dev, t_dev)
-                hn = K.rmsnorm(sk.launch(tokens), self.norm.weight, self.norm.eps)
-                return self.output(hn.view(bsz, 1, p.dim)).to(DTYPE)
         h = self.tok_embeddings(tokens).to(DTYPE).reshape(M, p.dim)
         cos, sin = self._tables(h.device)
-        if start_pos != 0 and seqlen == 1 and self.finish_in_matmul and self._finish_shapes_ok():
-            return self._forward_decode_finished(h, cos, sin, step_state, bsz)
         pending = None                      # product of the previous layer's w2, not yet added to h
         for layer in self.layers:
             att, ff = layer.attention, layer.feed_forward
@@ -423,65 +409,6 @@ class Transformer(nn.Module):
         if ok is None:
             ok = self._norm_in_ok[key] = K.norm_in_fits(M, Kd, list(key[2]))
         return ok
-
-    def _finish_shapes_ok(self) -> bool:
-        """the in-launch finishers work on 256-column units: every linear's width must be a multiple of 256"""
-        att, ff = self.layers[0].attention, self.layers[0].feed_forward
-        widths = (self.params.dim, ff.w1.shape[0], att.n_local_heads * att.head_dim, att.n_local_kv_heads * att.head_dim)
-        return all(w % 256 == 0 for w in widths)
-
-    def _forward_decode_finished(self, h, cos, sin, step_state, bsz):
-        """One decode step with six launches per layer: wq|wk|wv (+RoPE, KV append), the two attention kernels,
-        wo (+residual, RMSNorm), w1|w3 (+SiLU*up), w2 (+residual, RMSNorm of the next sub-block); for more
-        than 16 rows each matmul is followed by its small finishing launch instead."""
-        p = self.params
-        pos_dev, t_dev = step_state
-        seg = lambda lin: (lin.w, lin.s, lin.shape[0])
-        xn = K.rmsnorm(h, self.layers[0].attention_norm.weight, self.layers[0].attention_norm.eps)
-        n_layers = len(self.layers)
-        for i, layer in enumerate(self.layers):
-            att, ff = layer.attention, layer.feed_forward
-            H, Hkv = att.n_local_heads, att.n_local_kv_heads
-            q, k, v = K.matmul_q40_rope_append_kv(xn, seg(att.wq), seg(att.wk), seg(att.wv), H, Hkv, cos, sin, pos_dev,
-                                                  att.cache_k, att.cache_k_s, att.cache_v, att.cache_v_s, p.max_seq_len, t_dev)
-            o = K.shared_prefix_attn(q, att.cache_prompt_k[0], att.cache_prompt_v[0], att.cache_prompt_len,
-                                     suffix_k=att.cache_k, suffix_v=att.cache_v, suffix_ks=att.cache_k_s,
-                                     suffix_vs=att.cache_v_s, Smax=p.max_seq_len, lens=t_dev, lens_stride=0,
-                                     cur_k=k, cur_v=v).view(bsz, H * att.head_dim)
-            h, xn = K.matmul_q40_residual_rmsnorm(o, seg(att.wo), h, layer.ffn_norm.weight, layer.ffn_norm.eps)
-            act = K.matmul_q40_silu_mul(xn, seg(ff.w1), seg(ff.w3))
-            nxt = self.layers[i + 1].attention_norm if i + 1 < n_layers else self.norm
-            h, xn = K.matmul_q40_residual_rmsnorm(act, seg(ff.w2), h, nxt.weight, nxt.eps)
-        return self.output(xn.view(bsz, 1, p.dim)).to(DTYPE)
-
-    def _step_kernel(self, bsz: int, device):
-        """The persistent decode kernel for `bsz` branches, or None when the model shape is outside it."""
-        if bsz in self._step_kernels:
-            return self._step_kernels[bsz]
-        p = self.params
-        att0, ff0 = self.layers[0].attention, self.layers[0].feed_forward
-        H, Hkv, ffn = att0.n_local_heads, att0.n_local_kv_heads, ff0.w1.shape[0]
-        sk = None
-        if K.DecodeStepKernel.supports(bsz, p.dim, H, Hkv, ffn):
-            rows = []
-            for layer in self.layers:
-                a, f = layer.attention, layer.feed_forward
-                lins = [a.wq, a.wk, a.wv, a.wo, f.w1, f.w3, f.w2]
-                rows.append([l.w.data_ptr() for l in lins] + [l.s.data_ptr() for l in lins] +
-                            [layer.attention_norm.weight.data_ptr(), layer.ffn_norm.weight.data_ptr(),
-                             a.cache_prompt_k.data_ptr(), a.cache_prompt_v.data_ptr(),
-                             a.cache_k.data_ptr(), a.cache_v.data_ptr(), a.cache_k_s.data_ptr(), a.cache_v_s.data_ptr()])
-            cos, sin = self._tables(device)
-            sk = K.DecodeStepKernel(rows, bsz, p.dim, H, Hkv, ffn, p.max_seq_len, p.max_prompt_seq_len, self.norm.eps,
-                                    self.tok_embeddings.weight, cos, sin)
-        self._step_kernels[bsz] = sk
-        return sk
-
-    def check_step_kernels(self):
-        """Raises if a persistent decode step reported a time-out (call after synchronising)."""
-        for sk in self._step_kernels.values():
-            if sk is not None and sk.bound is not None:
-                sk.check_status()
 
     @torch.inference_mode()
     def forward(self, tokens: torch.Tensor, start_pos: int):

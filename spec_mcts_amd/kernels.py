@@ -574,83 +574,6 @@ def prefill_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Ten
 
 
 
-_fin_counters: Dict[str, torch.Tensor] = {}
-
-
-def _finish_counters(device: torch.device) -> torch.Tensor:
-    key = str(device)
-    t = _fin_counters.get(key)
-    if t is None:
-        t = _fin_counters[key] = torch.zeros(_lib.SMH_FIN_COUNTER_BYTES, dtype=torch.uint8, device=device)
-    return t
-
-
-def _fused(a: torch.Tensor, linears, fin: "_lib.Finish") -> None:
-    import ctypes
-    lib = _lib.load()
-    _need_gpu(a)
-    assert a.dtype == torch.float16 and a.dim() == 2 and a.stride(1) == 1
-    M, Kd = a.shape
-    ns = [int(n) for _, _, n in linears]
-    ks = matmul_plan(M, Kd, ns)
-    ws = matmul_workspace(a.device, max(M, 16), sum(ns))
-    need = ks * M * sum(ns) * 4
-    assert ws.numel() >= need, "matmul workspace too small"
-    nseg = len(linears)
-    wp = (ctypes.c_void_p * nseg)(*[w.data_ptr() for w, _, _ in linears])
-    sp = (ctypes.c_void_p * nseg)(*[s_.data_ptr() for _, s_, _ in linears])
-    np_ = (ctypes.c_int * nseg)(*ns)
-    fin.counters = _finish_counters(a.device).data_ptr()
-    check(lib.smh_q40_matmul_fused(a.data_ptr(), M, Kd, a.stride(0), nseg, wp, sp, np_, ws.data_ptr(), ws.numel(),
-                                   ctypes.byref(fin), _stream()), "smh_q40_matmul_fused")
-
-
-def matmul_q40_store(a: torch.Tensor, linears, residual: Optional[torch.Tensor] = None) -> torch.Tensor:
-    """fp16 product of `a` with the concatenated Q4_0 weights (+ residual), finished inside the matmul launch."""
-    N = sum(int(n) for _, _, n in linears)
-    out = torch.empty((a.shape[0], N), dtype=torch.float16, device=a.device)
-    fin = _lib.Finish(mode=_lib.SMH_FIN_STORE, out=out.data_ptr(), ldo=N, residual=_ptr(residual),
-                      ldr=residual.stride(0) if residual is not None else 0)
-    _fused(a, linears, fin)
-    return out
-
-
-def matmul_q40_residual_rmsnorm(a: torch.Tensor, linear, h_in: torch.Tensor, weight: torch.Tensor, eps: float):
-    """h = h_in + a . W (fp16, rounded as the reference rounds), xn = RMSNorm(h) * weight; one launch for M <= 16."""
-    N = int(linear[2])
-    assert h_in.is_contiguous() and h_in.shape == (a.shape[0], N) and weight.numel() == N
-    h = torch.empty_like(h_in)
-    xn = torch.empty_like(h_in)
-    fin = _lib.Finish(mode=_lib.SMH_FIN_RESIDUAL_RMSNORM, residual=h_in.data_ptr(), ldr=N, h_out=h.data_ptr(),
-                      norm_weight=weight.data_ptr(), eps=float(eps), xn_out=xn.data_ptr())
-    _fused(a, [linear], fin)
-    return h, xn
-
-
-def matmul_q40_silu_mul(a: torch.Tensor, w1, w3) -> torch.Tensor:
-    """fp16(silu(a . W1)) * (a . W3); one launch for M <= 16."""
-    n_half = int(w1[2])
-    out = torch.empty((a.shape[0], n_half), dtype=torch.float16, device=a.device)
-    fin = _lib.Finish(mode=_lib.SMH_FIN_SILU_MUL, out=out.data_ptr(), ldo=n_half)
-    _fused(a, [w1, w3], fin)
-    return out
-
-
-def matmul_q40_rope_append_kv(a: torch.Tensor, wq, wk, wv, H: int, Hkv: int, cos: torch.Tensor, sin: torch.Tensor,
-                              pos_dev: torch.Tensor, cache_k, cache_ks, cache_v, cache_vs, Smax: int, t_dev):
-    """q, k, v = a . [Wq|Wk|Wv]; RoPE(q, k) at *pos_dev; Q4_0 append of k, v at suffix row *t_dev; one launch for
-    M <= 16.  Returns q [M,H,128], k, v [M,Hkv,128] (the exact fp16 rows of the new token)."""
-    M = a.shape[0]
-    q = torch.empty((M, H, 128), dtype=torch.float16, device=a.device)
-    k = torch.empty((M, Hkv, 128), dtype=torch.float16, device=a.device)
-    v = torch.empty((M, Hkv, 128), dtype=torch.float16, device=a.device)
-    fin = _lib.Finish(mode=_lib.SMH_FIN_ROPE_APPEND, H=H, Hkv=Hkv, Smax=int(Smax), q=q.data_ptr(), k=k.data_ptr(), v=v.data_ptr(),
-                      cos_tab=cos.data_ptr(), sin_tab=sin.data_ptr(), pos_dev=pos_dev.data_ptr(), t_dev=_ptr(t_dev),
-                      cache_k=_ptr(cache_k), cache_ks=_ptr(cache_ks), cache_v=_ptr(cache_v), cache_vs=_ptr(cache_vs))
-    _fused(a, [wq, wk, wv], fin)
-    return q, k, v
-
-
 def flash_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, B: int, L: int, H: int, D: int) -> torch.Tensor:
     """Drop-in for triton_kernels.flash_attn (triton_kernels.py:621-647): one query per (branch, head) against
     that branch's own L keys.  q [B,H,D], k/v [B,H,L,D] fp16 -> [B,H,D] fp16.  The keys are brought into the
@@ -705,68 +628,3 @@ def chunk_attn(p: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
         kt = vt = lens = None
     return shared_prefix_attn(q.contiguous(), pk, pv, offset, suffix_k=kt, suffix_v=vt, Smax=S, lens=lens,
                               lens_stride=1, n_kv_heads=H)
-
-
-class DecodeStepKernel:
-    """One decode step (embedding + every layer) of up to 16 branches as a single persistent kernel.
-
-    Owns the layer descriptor table, the workspace and the output buffer; `prepare` binds a prompt
-    length and the device-side step state, `launch` runs one step on the current stream and returns
-    the hidden state that enters the final norm.  The caller checks `status()` after synchronising.
-    """
-
-    MAX_BRANCHES = 16
-
-    @staticmethod
-    def supports(M: int, dim: int, H: int, Hkv: int, ffn: int) -> bool:
-        return 1 <= M <= DecodeStepKernel.MAX_BRANCHES and H == Hkv and dim % 256 == 0 and ffn % 256 == 0 and (H * 128) % 256 == 0
-
-    def __init__(self, layer_rows: Sequence[Sequence[int]], M: int, dim: int, H: int, Hkv: int, ffn: int, Smax: int,
-                 P_max: int, eps: float, emb: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor):
-        lib = _lib.load()
-        _need_gpu(emb, cos, sin)
-        self.dev = emb.device
-        self.M, self.dim, self.H, self.Hkv, self.ffn, self.Smax, self.eps = M, dim, H, Hkv, ffn, Smax, float(eps)
-        self.n_layers = len(layer_rows)
-        assert all(len(r) == 22 for r in layer_rows), "a layer descriptor is 22 pointers"
-        self.table = torch.tensor(layer_rows, dtype=torch.int64).to(self.dev)
-        need = lib.smh_decode_step_workspace_bytes(self.n_layers, M, dim, H, Hkv, ffn, P_max, Smax)
-        if need == 0:
-            raise _lib.SmhError("smh_decode_step_workspace_bytes: " + lib.smh_last_error_string().decode())
-        self.workspace = torch.zeros(need + 256, dtype=torch.uint8, device=self.dev)
-        off = (-self.workspace.data_ptr()) % 256
-        self.ws_ptr = self.workspace.data_ptr() + off
-        self.ws_bytes = need
-        self.tokens = torch.zeros(M, dtype=torch.int64, device=self.dev)
-        self.h = torch.empty((M, dim), dtype=torch.float16, device=self.dev)
-        self.emb, self.cos, self.sin = emb, cos, sin
-        self.bound = None
-
-    def prepare(self, P: int, pos_dev: torch.Tensor, t_dev: torch.Tensor) -> None:
-        key = (P, pos_dev.data_ptr(), t_dev.data_ptr())
-        if self.bound == key:
-            return
-        lib = _lib.load()
-        check(lib.smh_decode_prepare(self.table.data_ptr(), self.n_layers, self.M, self.dim, self.H, self.Hkv, self.ffn, P,
-                                     self.Smax, self.eps, self.tokens.data_ptr(), self.emb.data_ptr(), self.cos.data_ptr(),
-                                     self.sin.data_ptr(), pos_dev.data_ptr(), t_dev.data_ptr(), self.h.data_ptr(),
-                                     self.ws_ptr, self.ws_bytes), "smh_decode_prepare")
-        self.bound = key
-
-    def launch(self, tokens: torch.Tensor) -> torch.Tensor:
-        assert self.bound is not None, "prepare() first"
-        self.tokens.copy_(tokens.reshape(-1))
-        check(_lib.load().smh_decode_step(self.ws_ptr, _stream()), "smh_decode_step")
-        return self.h
-
-    def status(self) -> Tuple[int, int, int]:
-        import ctypes
-        out = (ctypes.c_uint32 * 3)()
-        check(_lib.load().smh_decode_status(self.ws_ptr, out), "smh_decode_status")
-        return int(out[0]), int(out[1]), int(out[2])
-
-    def check_status(self) -> None:
-        st = self.status()
-        if st[2] != 0:
-            raise _lib.SmhError("the persistent decode kernel timed out waiting for its own workgroups "
-                                "(they must all be resident at once); results are invalid")

@@ -193,55 +193,3 @@ def test_fused_rope_append_consumer_bit_exact():
     assert torch.equal(cv.cpu().view(B, Smax, Hkv, 64)[:, t], wv.view(B, Hkv, 64))
     assert torch.equal(cks.cpu().view(B, Smax, Hkv, 2)[:, t].view(torch.int16), sk.view(B, Hkv, 2).view(torch.int16))
     assert torch.equal(cvs.cpu().view(B, Smax, Hkv, 2)[:, t].view(torch.int16), sv.view(B, Hkv, 2).view(torch.int16))
-
-
-@pytest.mark.parametrize("M", [1, 3, 10, 16, 40])
-def test_operator_finished_inside_the_matmul_launch(M):
-    """smh_q40_matmul_fused against smh_q40_matmul_partial + the partial_* kernels: same slabs, same slice
-    order, same roundings -> identical results (the RMSNorm's sum of squares is added in another order: the
-    normalised output may differ in the last bit of a few elements).  M = 40 takes the two-launch route."""
-    from spec_mcts_amd import kernels as K
-    Kd = 1024
-    dev = "cuda:0"
-    # STORE with residual, one weight
-    w, s = _weights(768, Kd, 90)
-    lin = (w.to(dev), s.to(dev), 768)
-    a = _acts(M, Kd, 91).to(dev)
-    r = _acts(M, 768, 92).to(dev)
-    pp = K.matmul_q40_partial(a, [lin])
-    assert torch.equal(K.matmul_q40_store(a, [lin], residual=r), K.partial_reduce(pp, residual=r))
-    assert torch.equal(K.matmul_q40_store(a, [lin]), K.partial_reduce(pp))
-    # RESIDUAL + RMSNorm (N = 1024: four units, second-level counter), called twice: the counters reset themselves
-    w2, s2 = _weights(1024, Kd, 93)
-    lin2 = (w2.to(dev), s2.to(dev), 1024)
-    wt = (1 + 0.1 * torch.randn(1024, generator=torch.Generator().manual_seed(94))).to(torch.float16).to(dev)
-    hin = _acts(M, 1024, 95).to(dev)
-    h_want, xn_want = K.partial_rmsnorm(K.matmul_q40_partial(a, [lin2]), hin, wt, 1e-5)
-    for _ in range(2):
-        h, xn = K.matmul_q40_residual_rmsnorm(a, lin2, hin, wt, 1e-5)
-        assert torch.equal(h, h_want)
-        assert torch.allclose(xn.float(), xn_want.float(), rtol=2e-3, atol=1e-4) and (xn != xn_want).float().mean() < 0.01
-    # SiLU(gate) * up
-    wg, sg = _weights(512, Kd, 96)
-    wu, su = _weights(512, Kd, 97)
-    l1, l3 = (wg.to(dev), sg.to(dev), 512), (wu.to(dev), su.to(dev), 512)
-    assert torch.equal(K.matmul_q40_silu_mul(a, l1, l3), K.partial_silu_mul(K.matmul_q40_partial(a, [l1, l3])))
-    # RoPE + KV append
-    H, Hkv, D, Smax = 4, 2, 128, 4
-    ws = [_weights(n, Kd, 100 + i, std=0.05) for i, n in enumerate((H * D, Hkv * D, Hkv * D))]
-    lins = [(x.to(dev), y.to(dev), n) for (x, y), n in zip(ws, (H * D, Hkv * D, Hkv * D))]
-    fc = O.precompute_freqs_cis(D, 32, 1e6)
-    cos, sin = fc.real.to(torch.float16).contiguous().to(dev), fc.imag.to(torch.float16).contiguous().to(dev)
-    rows = M * Smax * Hkv
-    st = torch.tensor([9, 2], dtype=torch.int32).to(dev)
-
-    def caches():
-        return [torch.zeros((rows, 64), dtype=torch.int8, device=dev), torch.zeros((rows * 2, 1), dtype=torch.float16, device=dev),
-                torch.zeros((rows, 64), dtype=torch.int8, device=dev), torch.zeros((rows * 2, 1), dtype=torch.float16, device=dev)]
-    c1, c2 = caches(), caches()
-    want = K.partial_rope_append_kv(K.matmul_q40_partial(a, lins), H, Hkv, D, cos, sin, st[0:1], c1[0], c1[1], c1[2], c1[3], Smax, st[1:2])
-    got = K.matmul_q40_rope_append_kv(a, lins[0], lins[1], lins[2], H, Hkv, cos, sin, st[0:1], c2[0], c2[1], c2[2], c2[3], Smax, st[1:2])
-    for x, y in zip(got, want):
-        assert torch.equal(x, y)
-    for x, y in zip(c1, c2):
-        assert torch.equal(x, y)
