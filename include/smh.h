@@ -211,6 +211,21 @@ int smh_shared_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int 
 int smh_prefill_attn(const void *q, const void *k, const void *v, void *out, int S, int H, int Hkv,
                      int D, smh_stream_t stream);
 
+/* smh_shared_prefix_attn_static: smh_shared_prefix_attn (same arguments without the workspace, same kernels, bit-identical
+ * results) for callers that cannot allocate device memory or pass a workspace: code under HIP graph capture, tight
+ * serving loops, harnesses that forbid hipMalloc.  It has no counterpart in the reference.  The prefix partials live in
+ * a static device array of smh_attn_static_scratch_bytes() = 16 MiB that every GPU the library runs on holds until the
+ * process ends; shapes that need more (prefix slices x B x H x 520 bytes) are rejected with an error.  The call allocates
+ * and frees nothing; the first call on a device looks the array's address up (make that call outside a graph capture).
+ * All calls on one GPU share the array: calls that overlap in time on one GPU race - keep them on one stream. */
+size_t smh_attn_static_scratch_bytes(void);
+int smh_shared_prefix_attn_static(const void *q, void *out, int B, int H, int Hkv, int D,
+                                  const void *prefix_k, const void *prefix_v, int P,
+                                  int suffix_format, const void *suffix_k, const void *suffix_v,
+                                  const void *suffix_ks, const void *suffix_vs, int Smax,
+                                  const int32_t *lens, int lens_stride, const void *cur_k, const void *cur_v,
+                                  smh_stream_t stream);
+
 /* smh_shared_prefix_attn_one: smh_shared_prefix_attn (same arguments, same attention) in ONE launch instead of
  * two: prefix slices and the branches' suffix passes run side by side and the workgroup that completes a
  * tile of 16 queries merges its partials in a fixed order (deterministic; equal to the two-launch result up

@@ -54,6 +54,9 @@ SIGNATURES = {
                                        _P, c_int, _P, _P, _P, c_size_t, _P]),
     "smh_shared_prefix_attn_one": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, c_int, _P, _P, _P, _P, c_int,
                                        _P, c_int, _P, _P, _P, c_size_t, _P]),
+    "smh_attn_static_scratch_bytes": (c_size_t, []),
+    "smh_shared_prefix_attn_static": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, c_int, _P, _P, _P, _P, c_int,
+                                              _P, c_int, _P, _P, _P]),
     "smh_prefill_attn": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     "smh_attn_qkv_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "smh_shared_prefix_attn_qkv": (c_int, [_P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_int,

@@ -17,6 +17,8 @@
 //
 // Algorithmic HBM traffic: prefix 2*P*Hkv*D*2 B once + per branch its suffix rows
 // (512 B fp16 or 136 B Q4_0 per row and kv head) + q/out.
+#include <mutex>
+
 #include "attn_rows.hpp"
 #include "rope_kv.hpp"
 
@@ -920,6 +922,61 @@ extern "C" int smh_shared_prefix_attn(const void *q, void *out, int B, int H, in
                                       void *workspace, size_t workspace_bytes, smh_stream_t stream) {
     return shared_prefix_attn("smh_shared_prefix_attn", false, q, out, B, H, Hkv, D, prefix_k, prefix_v, P, suffix_format, suffix_k,
                               suffix_v, suffix_ks, suffix_vs, Smax, lens, lens_stride, cur_k, cur_v, workspace, workspace_bytes, stream);
+}
+
+// ---- the same attention for callers that cannot allocate ---------------------------------------------------------
+// The prefix partials of smh_shared_prefix_attn_static live in this array instead of a caller's workspace.  Every GPU
+// the library runs on holds its own copy at its own address for the life of the process; host code never uses the
+// array's name as an address, only what hipGetSymbolAddress returned for the current device.
+constexpr size_t ATT_STATIC_SCRATCH_BYTES = (size_t)16 << 20;
+static __device__ __align__(256) unsigned char scratch[ATT_STATIC_SCRATCH_BYTES];
+constexpr int ATT_STATIC_MAX_DEVICES = 64;
+static std::mutex g_scratch_mutex;
+static void *g_scratch_ptr[ATT_STATIC_MAX_DEVICES] = {};
+
+// Device address of `scratch` on the current device, looked up once per device.
+static int static_scratch(void **ptr_out) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) { smh::set_error("smh_shared_prefix_attn_static: hipGetDevice: %s", hipGetErrorString(e)); return (int)e; }
+    if (dev < 0 || dev >= ATT_STATIC_MAX_DEVICES) { smh::set_error("smh_shared_prefix_attn_static: device %d outside [0,%d)", dev, ATT_STATIC_MAX_DEVICES); return -1; }
+    std::lock_guard<std::mutex> lock(g_scratch_mutex);
+    if (g_scratch_ptr[dev] == nullptr) {
+        void *ptr = nullptr;
+        e = hipGetSymbolAddress((void **)&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || ptr == nullptr) {
+            smh::set_error("smh_shared_prefix_attn_static: hipGetSymbolAddress: %s", hipGetErrorString(e));
+            return e != hipSuccess ? (int)e : -1;
+        }
+        g_scratch_ptr[dev] = ptr;
+    }
+    *ptr_out = g_scratch_ptr[dev];
+    return 0;
+}
+
+extern "C" size_t smh_attn_static_scratch_bytes(void) { return ATT_STATIC_SCRATCH_BYTES; }
+
+extern "C" int smh_shared_prefix_attn_static(const void *q, void *out, int B, int H, int Hkv, int D,
+                                             const void *prefix_k, const void *prefix_v, int P,
+                                             int suffix_format, const void *suffix_k, const void *suffix_v,
+                                             const void *suffix_ks, const void *suffix_vs, int Smax,
+                                             const int32_t *lens, int lens_stride, const void *cur_k, const void *cur_v,
+                                             smh_stream_t stream) {
+    using namespace smh;
+    const char *who = "smh_shared_prefix_attn_static";
+    SMH_REQUIRE(B >= 0 && B <= 65535 && H > 0 && Hkv > 0 && H % Hkv == 0 && P >= 0, "%s: B=%d (at most 65535) H=%d Hkv=%d P=%d", who, B, H, Hkv, P);
+    // the partials the two launches exchange: one (max, sum, o[128]) per prefix slice and query, as smh_shared_prefix_attn plans them
+    int tw = ATT_TW_MAX, qgroups = 1;
+    attn_plan(P, Hkv, B * (H / Hkv), &tw, &qgroups);
+    const size_t splits = P > 0 ? (size_t)(P + tw - 1) / tw : 0;
+    const size_t need = splits * (size_t)B * H * (ATT_D + 2) * sizeof(float);
+    SMH_REQUIRE(need <= ATT_STATIC_SCRATCH_BYTES, "%s: B=%d H=%d P=%d needs %zu bytes of scratch, the static array holds %zu (use smh_shared_prefix_attn with a workspace)",
+                who, B, H, P, need, ATT_STATIC_SCRATCH_BYTES);
+    void *ws = nullptr;
+    const int st = static_scratch(&ws);
+    if (st) return st;
+    return shared_prefix_attn(who, false, q, out, B, H, Hkv, D, prefix_k, prefix_v, P, suffix_format, suffix_k, suffix_v, suffix_ks, suffix_vs,
+                              Smax, lens, lens_stride, cur_k, cur_v, ws, ATT_STATIC_SCRATCH_BYTES, stream);
 }
 
 extern "C" int smh_shared_prefix_attn_one(const void *q, void *out, int B, int H, int Hkv, int D,

@@ -492,12 +492,14 @@ def shared_prefix_attn(q: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix
                        suffix_ks: Optional[torch.Tensor] = None, suffix_vs: Optional[torch.Tensor] = None,
                        Smax: int = 0, lens: Optional[torch.Tensor] = None, lens_stride: int = 1,
                        cur_k: Optional[torch.Tensor] = None, cur_v: Optional[torch.Tensor] = None,
-                       n_kv_heads: Optional[int] = None, single_launch: bool = False) -> torch.Tensor:
+                       n_kv_heads: Optional[int] = None, single_launch: bool = False, out: Optional[torch.Tensor] = None,
+                       static_scratch: bool = False) -> torch.Tensor:
     """out[b,h] = softmax(q[b,h] . K_b^T / sqrt(D)) . V_b with K_b = prefix[:P] (shared) ||
     suffix[b, :lens[b]] || cur_k[b].  The suffix is fp16 [B,Smax,Hkv,D] or Q4_0 (int8 rows +
     fp16 scales, the model's cache layout); `lens` is int32 on the device.
     single_launch: one launch instead of two (at most 128 queries per kv head; same result up to fp32
-    summation order)."""
+    summation order).  static_scratch: the two-launch form on the library's own static scratch array: with `out`
+    given the call allocates nothing (smh_shared_prefix_attn_static)."""
     lib = _lib.load()
     _need_gpu(q)
     assert q.is_contiguous() and q.dtype == torch.float16 and q.dim() == 3
@@ -521,7 +523,15 @@ def shared_prefix_attn(q: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix
             fmt = SMH_KV_Q40
     if cur_k is not None:
         assert cur_k.is_contiguous() and cur_v.is_contiguous() and cur_k.dtype == torch.float16
-    out = torch.empty_like(q)
+    if out is None:
+        out = torch.empty_like(q)
+    assert out.shape == q.shape and out.dtype == torch.float16 and out.is_contiguous() and out.device == q.device
+    if static_scratch:
+        check(lib.smh_shared_prefix_attn_static(q.data_ptr(), out.data_ptr(), B, H, Hkv, D, _ptr(prefix_k), _ptr(prefix_v), int(P),
+                                                fmt, _ptr(suffix_k), _ptr(suffix_v), _ptr(suffix_ks), _ptr(suffix_vs), int(Smax),
+                                                _ptr(lens), int(lens_stride), _ptr(cur_k), _ptr(cur_v), _stream()),
+              "smh_shared_prefix_attn_static")
+        return out
     one = bool(single_launch) and B * (H // Hkv) <= 128
     ws = attn_qkv_workspace(q.device, B, H, P) if one else attn_workspace(q.device, B, H, P)
     fn = lib.smh_shared_prefix_attn_one if one else lib.smh_shared_prefix_attn

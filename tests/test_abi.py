@@ -43,6 +43,11 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert 1 <= ks <= 16
     assert lib.smh_q40_matmul_plan(1, 4096, 1, (ctypes.c_int * 1)(100)) < 0      # N not a multiple of 128
     assert lib.smh_attn_workspace_bytes(64, 32, 1024) >= 32 * 64 * 32 * 130 * 4
+    # the entry point without a workspace refuses shapes beyond its static array before anything touches the device
+    assert lib.smh_attn_static_scratch_bytes() == 16 << 20
+    st = lib.smh_shared_prefix_attn_static(None, None, 4096, 64, 64, 128, None, None, 4096, 0, None, None, None, None, 0, None, 0,
+                                           None, None, None)
+    assert st < 0 and b"static array holds" in lib.smh_last_error_string()
 
 
 def test_host_quantiser_matches_oracle():
