@@ -32,7 +32,10 @@ class GraphDecoder:
         self.state = torch.zeros(2, dtype=torch.int32, device=self.device)     # (position, suffix index)
         self.one = torch.ones(2, dtype=torch.int32, device=self.device)
         self.graph: Optional[torch.cuda.CUDAGraph] = None
+        self._graph_key = None        # what the captured launches were planned for: (prompt length, model switches)
+        self._pinned = []             # workspaces whose addresses are inside the graph: kept alive as long as it is
         self.prompt_len = 0
+        self.t = 0                    # suffix rows written so far (host mirror of state[1])
 
     def _step(self):
         logits = self.model._forward_impl(self.tokens, 1, (self.state[0:1], self.state[1:2]))
@@ -45,14 +48,24 @@ class GraphDecoder:
         m = self.model
         m.resetSeq()
         logits = m(prompt[:1].to(self.device), 0)[:, -1]
-        self.prompt_len = prompt.shape[1]
+        self.prompt_len = m.layers[0].attention.cache_prompt_len      # (a prompt longer than the cache was cropped by the model)
         first = K.argmax(logits.contiguous())
         self.tokens.copy_(first.view(1, 1).expand(self.B, 1))
         self._reset_state()
+        if self.graph is not None and self._graph_key != self._key():
+            # the prompt length decides the attention's slices, grid and workspace layout, all constants of the
+            # recorded launches: a graph captured for another prompt length is dropped and captured again
+            self.graph = None
         return first
+
+    def _key(self):
+        m = self.model
+        return (self.prompt_len, self.B, m.fused, m.tiled_weights, m.silu_in_matmul, m.norm_in_matmul, m.norm_in_max_rows,
+                m.attn_from_qkv, m.attn_single_launch, m.per_branch_kv, m._forked)
 
     def _reset_state(self):
         self.state.copy_(torch.tensor([self.prompt_len, 0], dtype=torch.int32))
+        self.t = 0
 
     @torch.inference_mode()
     def capture(self):
@@ -69,9 +82,13 @@ class GraphDecoder:
         self._reset_state()
         self.tokens.copy_(saved)
         if self.use_graph:
+            # the warm-up grew the shared workspaces to what this step needs; the graph records their addresses, so
+            # they must outlive it even if a later, larger call replaces them in the operators' table
+            self._pinned = list(K._workspaces.values())
             self.graph = torch.cuda.CUDAGraph()
             with torch.cuda.graph(self.graph):
                 self._step()
+            self._graph_key = self._key()
             # the capture pass itself does not execute; state and tokens are untouched
         torch.cuda.synchronize()
 
@@ -80,6 +97,13 @@ class GraphDecoder:
         """Run `steps` decode steps; returns the tokens produced, int64 [B, steps]."""
         if out is None:
             out = torch.empty((self.B, steps), dtype=torch.int64, device=self.device)
+        p = self.model.params
+        # the kernels take position and suffix row from device counters and do not know the caches' ends
+        assert self.t + steps <= p.max_seq_len, f"suffix cache exhausted: {self.t} + {steps} rows of {p.max_seq_len}"
+        assert self.prompt_len + self.t + steps <= self.model.freqs_cis.shape[0], "position beyond the rotation table"
+        assert self.graph is None or self._graph_key == self._key(), "the graph was captured for another prompt length or configuration"
+        self.t += steps
+        self.model._rows_written = self.t
         for i in range(steps):
             if self.graph is not None:
                 self.graph.replay()

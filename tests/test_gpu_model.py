@@ -155,3 +155,35 @@ def test_hf_model_q40_flavour_matches_oracle():
     # greedy generation API of this flavour
     res, lens = model.generate(prompt[:1].cuda(), 2, 5, temperature=0.0)
     assert res.shape[0] == 2 and torch.equal(res[0], res[1])
+
+
+def test_graph_decoder_serves_prompts_of_different_length():
+    """One GraphDecoder, two prompts of different length: the graph captured for the first prompt is not replayed
+    for the second (the prompt length is a constant of the recorded attention launches); tokens equal the eager loop."""
+    from spec_mcts_amd.decode import GraphDecoder
+    oargs, sd, model = _build(SMALL, 40)
+    dec = GraphDecoder(model, 3)
+    for P, seed in ((11, 140), (29, 141), (11, 142)):
+        prompt = torch.randint(0, SMALL["vocab_size"], (1, P), generator=torch.Generator().manual_seed(seed))
+        got = dec.generate(prompt, 7).cpu()
+        want = _greedy_gpu(model, prompt, 3, 7)
+        assert torch.equal(got, want), f"prompt of {P} tokens"
+        assert dec.graph is not None and dec._graph_key[0] == P
+
+
+def test_graph_decoder_refuses_to_run_past_the_caches():
+    """Position and suffix row live in device counters the kernels trust: the host refuses steps that would run past
+    the suffix cache or the rotation table before anything is launched."""
+    from spec_mcts_amd.decode import GraphDecoder
+    oargs, sd, model = _build(SMALL, 41)
+    dec = GraphDecoder(model, 2)
+    prompt = torch.randint(0, SMALL["vocab_size"], (1, 9), generator=torch.Generator().manual_seed(143))
+    dec.generate(prompt, 5)                                  # 4 decode steps: suffix rows 0..3
+    assert dec.t == 4
+    with pytest.raises(AssertionError, match="suffix cache exhausted"):
+        dec.decode(SMALL["max_seq_len"] - 3)                 # 4 + 21 > 24 rows
+    dec.decode(SMALL["max_seq_len"] - 4)                     # exactly to the end of the cache is fine
+    with pytest.raises(AssertionError, match="suffix cache exhausted"):
+        dec.decode(1)
+    with pytest.raises(AssertionError, match="suffix cache exhausted"):
+        model(torch.zeros((2, 1), dtype=torch.int64, device="cuda:0"), 9 + SMALL["max_seq_len"])
