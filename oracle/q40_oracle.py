@@ -213,16 +213,21 @@ def silu_mul(g: torch.Tensor, u: torch.Tensor) -> torch.Tensor:
 # --------------------------------------------------------------------------------------------
 def shared_prefix_attention(q: torch.Tensor, prefix_k: torch.Tensor, prefix_v: torch.Tensor,
                             suffix_k: Optional[torch.Tensor], suffix_v: Optional[torch.Tensor],
-                            lens: Optional[List[int]]) -> torch.Tensor:
+                            lens: Optional[List[int]], acc_dtype=torch.float32, p_half_prefix: bool = False) -> torch.Tensor:
     """One query per branch over [shared prefix || that branch's own suffix].
 
     q [B,H,D]; prefix_k/v [P,Hkv,D]; suffix_k/v [B,S,Hkv,D] with lens[b] valid rows.
     softmax(q.K^T/sqrt(D)).V with fp32 scores/softmax/accumulation, fp16 result: what
     F.scaled_dot_product_attention computes at hf_model_q40_kv_shared.py:375-405 (there the prefix
-    is expanded per branch and all lens are equal)."""
+    is expanded per branch and all lens are equal).
+    The two keyword arguments are instruments for noise studies, not part of the reference's arithmetic: `acc_dtype`
+    float64 evaluates the same formula in double precision; `p_half_prefix` rounds the un-normalised probabilities of the
+    PREFIX keys to fp16 before they multiply V (what a matrix-core P.V product with fp16 operands does), the
+    denominator keeping the unrounded values."""
     B, H, D = q.shape
     Hkv = prefix_k.shape[1]
     n_rep = H // Hkv
+    P = prefix_k.shape[0]
     out = torch.empty((B, H, D), dtype=q.dtype)
     for b in range(B):
         k = prefix_k
@@ -230,24 +235,35 @@ def shared_prefix_attention(q: torch.Tensor, prefix_k: torch.Tensor, prefix_v: t
         if suffix_k is not None and lens is not None and lens[b] > 0:
             k = torch.cat((k, suffix_k[b, : lens[b]]), dim=0)
             v = torch.cat((v, suffix_v[b, : lens[b]]), dim=0)
-        kf = k.float().repeat_interleave(n_rep, dim=1)       # [L, H, D]
-        vf = v.float().repeat_interleave(n_rep, dim=1)
-        scores = torch.einsum("hd,lhd->hl", q[b].float(), kf) / math.sqrt(D)
-        p = torch.softmax(scores, dim=-1)
+        kf = k.to(acc_dtype).repeat_interleave(n_rep, dim=1)       # [L, H, D]
+        vf = v.to(acc_dtype).repeat_interleave(n_rep, dim=1)
+        scores = torch.einsum("hd,lhd->hl", q[b].to(acc_dtype), kf) / math.sqrt(D)
+        if not p_half_prefix:
+            p = torch.softmax(scores, dim=-1)
+        else:
+            e = torch.exp(scores - scores.max(dim=-1, keepdim=True).values)
+            den = e.sum(dim=-1, keepdim=True)
+            e = torch.cat((e[:, :P].to(DTYPE).to(acc_dtype), e[:, P:]), dim=1)
+            p = e / den
         out[b] = torch.einsum("hl,lhd->hd", p, vf).to(q.dtype)
     return out
 
 
-def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor) -> torch.Tensor:
+def causal_attention(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, acc_dtype=torch.float32, p_half: bool = False) -> torch.Tensor:
     """Prefill attention: q,k,v [S,H(kv),D]; additive -inf above the diagonal
-    (hf_model_q40_kv_shared.py:499-504, 405)."""
+    (hf_model_q40_kv_shared.py:499-504, 405).  acc_dtype / p_half: as in shared_prefix_attention (noise studies)."""
     S, H, D = q.shape
     n_rep = H // k.shape[1]
-    kf = k.float().repeat_interleave(n_rep, dim=1)
-    vf = v.float().repeat_interleave(n_rep, dim=1)
-    scores = torch.einsum("shd,lhd->hsl", q.float(), kf) / math.sqrt(D)
-    mask = torch.full((S, S), float("-inf")).triu(diagonal=1)
-    p = torch.softmax(scores + mask, dim=-1)
+    kf = k.to(acc_dtype).repeat_interleave(n_rep, dim=1)
+    vf = v.to(acc_dtype).repeat_interleave(n_rep, dim=1)
+    scores = torch.einsum("shd,lhd->hsl", q.to(acc_dtype), kf) / math.sqrt(D)
+    mask = torch.full((S, S), float("-inf"), dtype=acc_dtype).triu(diagonal=1)
+    scores = scores + mask
+    if not p_half:
+        p = torch.softmax(scores, dim=-1)
+    else:
+        e = torch.exp(scores - scores.max(dim=-1, keepdim=True).values)
+        p = e.to(DTYPE).to(acc_dtype) / e.sum(dim=-1, keepdim=True)
     return torch.einsum("hsl,lhd->shd", p, vf).to(q.dtype)
 
 
@@ -292,7 +308,20 @@ class OracleTransformer:
                "feed_forward.w1", "feed_forward.w2", "feed_forward.w3")
 
     def __init__(self, args: OracleArgs, sd: Dict[str, torch.Tensor], dense: bool = True,
-                 quantize_kv: bool = True, per_branch_kv: bool = False):
+                 quantize_kv: bool = True, per_branch_kv: bool = False, acc_dtype=torch.float32,
+                 scale_on_x_max_rows: int = 0, p_half_prefix: bool = False, slab_half_ksplit=None, share_dense=None):
+        # The last five arguments are instruments for noise studies (how far may two faithful implementations of the
+        # same cast points drift apart on a deep random model), not the reference's arithmetic; the defaults are the oracle.
+        #   acc_dtype float64        every matrix product and the attention accumulate in double precision
+        #   scale_on_x_max_rows = R  linears of at most R rows round fp16(x * scale) and multiply by the integer code,
+        #                            instead of x by fp16(code * scale): same values before rounding, the rounding on the other operand
+        #   p_half_prefix            see shared_prefix_attention (prefill: all keys)
+        #   slab_half_ksplit(key, K, N) -> number of K-slices whose partial sums are rounded to fp16 before they are added
+        #   share_dense              another oracle whose dequantised matrices are reused (same weights, no second copy)
+        self.acc_dtype = acc_dtype
+        self.scale_on_x_max_rows = scale_on_x_max_rows
+        self.p_half_prefix = p_half_prefix
+        self.slab_half_ksplit = slab_half_ksplit
         # per_branch_kv=True restates hf_model_q40.Transformer instead (hf_model_q40.py:236-372): no shared
         # prompt cache, EVERY position of every batch row lives in that row's Q4_0 cache, the rows of the
         # tokens being processed are used exact (:313-314) and stored quantised (:322-343); a prefill takes
@@ -307,18 +336,31 @@ class OracleTransformer:
         self.freqs_cis = precompute_freqs_cis(self.head_dim, args.max_seq_len + args.max_prompt_seq_len,
                                               args.rope_theta)
         self._dense: Dict[str, torch.Tensor] = {}
-        if dense:
+        self._codes: Dict[str, Tuple[torch.Tensor, torch.Tensor]] = {}
+        if share_dense is not None and share_dense.acc_dtype == acc_dtype:
+            self._dense = share_dense._dense
+        elif dense:
             for i in range(args.n_layers):
                 for name in self.LINEARS:
                     key = f"layers.{i}.{name}"
                     N, K = tuple(sd[key + ".shape"])
                     self._dense[key] = dequantize_q40(sd[key + ".w"], sd[key + ".s"], GROUP_SIZE,
-                                                      (K, N), DTYPE).float()
-        self._out_w = sd["output.weight"].float()
+                                                      (K, N), DTYPE).to(acc_dtype)
+        if scale_on_x_max_rows > 0:
+            assert dense, "the scale-on-x variant keeps the dense matrices for calls with more rows"
+            for i in range(args.n_layers):
+                for name in self.LINEARS:
+                    key = f"layers.{i}.{name}"
+                    N, K = tuple(sd[key + ".shape"])
+                    # codes [N/64, K, 64] (group-major, ready for a batched product), scales fp16 [K, N/64]
+                    codes = unpack_codes(sd[key + ".w"]).view(K, N // GROUP_SIZE, GROUP_SIZE).permute(1, 0, 2).to(acc_dtype).contiguous()
+                    self._codes[key] = (codes, sd[key + ".s"].view(K, N // GROUP_SIZE))
+        self._out_w = sd["output.weight"].to(acc_dtype)
         self.reset()
 
     def reset(self):
         a = self.args
+        self.kv_codes = {}
         self.prompt_len = 0
         self.prompt_k = [None] * a.n_layers      # fp16 [P, Hkv, D]
         self.prompt_v = [None] * a.n_layers
@@ -336,19 +378,36 @@ class OracleTransformer:
     def _linear(self, key: str, x: torch.Tensor) -> torch.Tensor:
         shp = x.shape
         x2 = x.reshape(-1, shp[-1])
-        if self.dense:
-            y = (x2.float() @ self._dense[key]).to(DTYPE)
+        if self.dense and x2.shape[0] <= self.scale_on_x_max_rows:
+            codes, scales = self._codes[key]
+            a = (x2[:, :, None] * scales[None]).to(self.acc_dtype)            # fp16 product, rounded to fp16: [M, K, G]
+            y = torch.bmm(a.permute(2, 0, 1), codes).permute(1, 0, 2).reshape(x2.shape[0], -1).to(DTYPE)
+        elif self.dense and self.slab_half_ksplit is not None:
+            W = self._dense[key]
+            K, N = W.shape
+            ks = int(self.slab_half_ksplit(key, K, N))
+            steps = (K + 31) // 32
+            per = (steps + ks - 1) // ks * 32                             # rows of a slice: whole 32-row steps
+            y = torch.zeros((x2.shape[0], N), dtype=self.acc_dtype)
+            for k0 in range(0, K, per):
+                y += (x2[:, k0:k0 + per].to(self.acc_dtype) @ W[k0:k0 + per]).to(DTYPE).to(self.acc_dtype)
+            y = y.to(DTYPE)
+        elif self.dense:
+            y = (x2.to(self.acc_dtype) @ self._dense[key]).to(DTYPE)
         else:
             N, K = tuple(self.sd[key + ".shape"])
             y = matmul_q40(x2, self.sd[key + ".w"], self.sd[key + ".s"], (K, N))
         return y.reshape(*shp[:-1], -1)
 
-    def _kv_roundtrip(self, x: torch.Tensor) -> torch.Tensor:
+    def _kv_roundtrip(self, x: torch.Tensor, tag=None) -> torch.Tensor:
         """What later steps see of a stored K/V vector: quantise + dequantise
-        (hf_model_q40_kv_shared.py:365-366 then :352-353 on the next step)."""
+        (hf_model_q40_kv_shared.py:365-366 then :352-353 on the next step).  `tag`: the packed rows and scales of this call
+        are kept in self.kv_codes[tag] (what the reference writes into cache_k / cache_k_s), for tests that copy them."""
         if not self.quantize_kv:
             return x
         w, s = quantize_q40(x, GROUP_SIZE)
+        if tag is not None:
+            self.kv_codes[tag] = (w, s)
         return dequantize_q40(w, s, GROUP_SIZE, x.shape, DTYPE)
 
     def forward(self, tokens: torch.Tensor, start_pos: int) -> torch.Tensor:
@@ -377,12 +436,12 @@ class OracleTransformer:
                     attn = shared_prefix_attention(xq[:, 0], none, none, sk, sv, [start_pos + 1] * B)[:, None]
                 else:
                     assert start_pos == 0, "multi-token calls are prefills"
-                    attn = torch.stack([causal_attention(xq[b], xk[b], xv[b]) for b in range(B)])
+                    attn = torch.stack([causal_attention(xq[b], xk[b], xv[b], self.acc_dtype, self.p_half_prefix) for b in range(B)])
             elif start_pos == 0:
                 # prefill: prompt KV taken from row 0 only, kept in fp16 (:324-329)
                 self.prompt_k[i] = xk[0].clone()
                 self.prompt_v[i] = xv[0].clone()
-                attn = torch.stack([causal_attention(xq[b], xk[b], xv[b]) for b in range(B)])
+                attn = torch.stack([causal_attention(xq[b], xk[b], xv[b], self.acc_dtype, self.p_half_prefix) for b in range(B)])
             else:
                 assert S == 1
                 t = start_pos - self.prompt_len
@@ -391,10 +450,10 @@ class OracleTransformer:
                 sk = torch.cat((ck[:B, :t], xk), dim=1)
                 sv = torch.cat((cv[:B, :t], xv), dim=1)
                 # ... and later steps see its Q4 round trip (:365-371)
-                ck[:B, t] = self._kv_roundtrip(xk[:, 0])
-                cv[:B, t] = self._kv_roundtrip(xv[:, 0])
+                ck[:B, t] = self._kv_roundtrip(xk[:, 0], (i, "k"))
+                cv[:B, t] = self._kv_roundtrip(xv[:, 0], (i, "v"))
                 attn = shared_prefix_attention(xq[:, 0], self.prompt_k[i], self.prompt_v[i],
-                                               sk, sv, [t + 1] * B)[:, None]
+                                               sk, sv, [t + 1] * B, self.acc_dtype, self.p_half_prefix)[:, None]
             attn = attn.reshape(B, S, H * D)
             h = h + self._linear(p + "attention.wo", attn)
             xn = rmsnorm(h, sd[p + "ffn_norm.weight"], a.norm_eps)
@@ -404,7 +463,17 @@ class OracleTransformer:
         if start_pos == 0 and not self.per_branch_kv:
             self.prompt_len = S
         h = rmsnorm(h, sd["norm.weight"], a.norm_eps)
-        return (h.float() @ self._out_w.t()).to(DTYPE)
+        return (h.to(self.acc_dtype) @ self._out_w.t()).to(DTYPE)
+
+    def forced(self, prompt: torch.Tensor, tokens: torch.Tensor) -> torch.Tensor:
+        """Teacher-forced run of one branch: prefill, then step s is fed tokens[s-1] whatever this model would have
+        picked.  Returns the fp32 view of the fp16 logits of every step, [len(tokens), vocab]; row 0 is the prefill's."""
+        self.reset()
+        P = prompt.shape[1]
+        rows = [self.forward(prompt[:1], 0)[0, -1].float()]
+        for sidx in range(1, tokens.numel()):
+            rows.append(self.forward(tokens[sidx - 1].view(1, 1), P + sidx - 1)[0, -1].float())
+        return torch.stack(rows)
 
     def greedy(self, prompt: torch.Tensor, batch_size: int, steps: int):
         """Prefill once at B=1, fork to `batch_size` branches, greedy decode `steps` tokens

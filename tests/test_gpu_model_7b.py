@@ -1,16 +1,18 @@
-"""Greedy decoding of the 7B-architecture random-init Q4_0 model (BASELINE configs[3]) against the oracle's
-tokens held in tests/golden/greedy_7b.json (made by tests/golden/make_7b_greedy.py: dense fp32 CPU
-restatement of the model on the same generated weights).
+"""Greedy decoding of the 7B-architecture random-init Q4_0 model (BASELINE configs[3]) against the oracle's tokens held
+in tests/golden/greedy_7b.json (made by tests/golden/make_7b_greedy.py: dense fp32 CPU restatement of the model on the
+same generated weights, plus a noise study).
 
-The GPU model is fed the ORACLE's previous token at every step (teacher forcing), so each of the 64 steps
-is checked on its own: a step counts when the oracle's top-1/top-2 logit margin is above NEAR_TIE; below
-it the argmax is decided by rounding noise and the step is only reported.
-
-How large that noise is was measured, not guessed: this random-init model is chaotic (32 layers of random
-weights and Q4_0-quantised KV rows), and the two GPU paths of this package - the persistent step kernel and
-the operator kernels, which round at the same points and differ ONLY in the order of fp32 partial sums -
-disagree by 0.03 to 0.09 in the largest logit difference of a step (logits are fp16 numbers up to 6.5, one
-ulp is 0.004 to 0.008).  NEAR_TIE is set to the top of that band."""
+Every path the benchmark times is held against the fixture: one branch (tiled GEMV with the RMSNorm and SiLU made inside
+the matmul launches, the one-launch attention), ten branches (GEMV, separate small kernels) and a hundred (the MFMA
+GEMM, the two-launch attention).  Two runs per path:
+  teacher-forced  the GPU model is fed the ORACLE's previous token, so each of the 64 steps is checked on its own.  A step
+                  counts when the oracle's top-1/top-2 logit margin is at least the fixture's `near_tie`; below it the
+                  argmax is only reported.  near_tie comes from the oracle alone: twice the largest change of that margin
+                  between the fp32 oracle and the same oracle accumulating in double precision (two faithful evaluations
+                  of the reference's cast points drift that far apart on this chaotic 32-layer random model).
+  free-running    the GPU model is fed its own tokens, as the benchmark runs it; the length of the common prefix with the
+                  oracle's tokens is printed (after the first near-tie that falls the other way the sequences are unrelated)
+                  and must reach the first step whose margin is below near_tie."""
 import json
 import os
 
@@ -19,7 +21,6 @@ import torch
 
 pytestmark = pytest.mark.gpu
 
-NEAR_TIE = 0.09
 FIXTURE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "greedy_7b.json")
 
 
@@ -28,31 +29,46 @@ def test_7b_greedy_tokens_match_oracle():
     from spec_mcts_amd import kernels as K
     fx = json.load(open(FIXTURE))
     seed, P, steps = fx["seed"], fx["prompt_len"], fx["steps"]
+    near_tie = fx["near_tie"]
+    assert near_tie == pytest.approx(2.0 * max(fx["noise"]["acc64"]["gap_shift"]), abs=1e-4)
     want = torch.tensor(fx["tokens"], dtype=torch.int64)
     margins = fx["margins"]
     torch.manual_seed(seed)
-    model = bench.build_model(torch, fx["args"], seed=seed)
+    model = bench.build_model(torch, dict(fx["args"], max_batch_size=100), seed=seed)
     prompt = torch.randint(0, fx["args"]["vocab_size"], (1, P), generator=torch.Generator().manual_seed(seed)).cuda()
-    decidable = [i for i, m in enumerate(margins) if m >= NEAR_TIE]
+    decidable = [i for i, m in enumerate(margins) if m >= near_tie]
+    first_near_tie = next(i for i, m in enumerate(margins) if m < near_tie)
     assert len(decidable) >= steps * 2 // 3, "fixture has too many near-ties to be a test"
-    for B in (1, 3, 10):
-        print(f"B={B}", flush=True)
+    print(f"near_tie {near_tie}: {len(decidable)} of {steps} steps decidable, first near-tie at step {first_near_tie}", flush=True)
+    for B in (1, 10, 100):
+        # ---- teacher-forced ----
         model.resetSeq()
         logits = model(prompt, 0)[:, -1]
         got = torch.zeros((B, steps), dtype=torch.int64)
         got[:, 0] = int(K.argmax(logits.contiguous())[0])
-        gaps = []
         for s in range(1, steps):
             tok = want[s - 1].expand(B, 1).contiguous().cuda()            # the oracle's token, not the model's own
             lg = model(tok, P + s - 1)[:, -1]
             got[:, s] = K.argmax(lg.contiguous()).cpu()
-            top2 = lg[0].float().topk(2).values
-            gaps.append(float(top2[0] - top2[1]))
         torch.cuda.synchronize()
         for b in range(1, B):
             assert torch.equal(got[b], got[0]), "identical branches must produce identical tokens"
-        wrong = [i for i in decidable if int(got[0, i]) != int(want[i])]
-        free_run = next((i for i in range(steps) if int(got[0, i]) != int(want[i])), steps)
-        print(f"  matches {int((got[0] == want).sum())}/{steps}; decidable {len(decidable)}; first difference at step {free_run}; "
-              f"oracle margins at differing steps {[margins[i] for i in range(steps) if int(got[0, i]) != int(want[i])]}", flush=True)
-        assert not wrong, f"tokens differ at steps {wrong} where the oracle's margin is {[margins[i] for i in wrong]}"
+        differing = [i for i in range(steps) if int(got[0, i]) != int(want[i])]
+        print(f"B={B} teacher-forced: {steps - len(differing)}/{steps} tokens equal the oracle's; differing steps and their oracle margins "
+              f"{[(i, margins[i]) for i in differing]}", flush=True)
+        wrong = [i for i in differing if margins[i] >= near_tie]
+        assert not wrong, f"B={B}: tokens differ at steps {wrong} where the oracle's margin is {[margins[i] for i in wrong]} >= {near_tie}"
+        # ---- free-running ----
+        model.resetSeq()
+        logits = model(prompt, 0)[:, -1]
+        free = torch.zeros((B, steps), dtype=torch.int64, device="cuda:0")
+        free[:, 0] = K.argmax(logits.contiguous())[0]
+        for s in range(1, steps):
+            lg = model(free[:, s - 1:s].contiguous(), P + s - 1)[:, -1]
+            free[:, s] = K.argmax(lg.contiguous())
+        free = free.cpu()
+        for b in range(1, B):
+            assert torch.equal(free[b], free[0])
+        run = next((i for i in range(steps) if int(free[0, i]) != int(want[i])), steps)
+        print(f"B={B} free-running: first {run} tokens equal the oracle's" + (f" (oracle margin at step {run}: {margins[run]})" if run < steps else ""), flush=True)
+        assert run >= first_near_tie, f"B={B}: free-running tokens leave the oracle's at step {run}, before the first near-tie (step {first_near_tie})"

@@ -312,3 +312,51 @@ def test_terminal_state_machine_known_answers_and_scalar_walk():
         e, st = O.detect_terminal(torch.tensor([s_[i] for s_ in streams], dtype=torch.int64), st, seq)
         assert e.tolist() == [w[0][i] for w in want]
         assert st.tolist() == [w[1][i] for w in want]
+
+
+def test_noise_study_instruments_reduce_to_the_oracle_where_they_must():
+    """The oracle's noise-study switches (double-precision accumulation, scale on the activation side, fp16 prefix
+    probabilities, fp16 K-slice partial sums) change WHERE a rounding happens, never the value before rounding: each
+    must reproduce the plain oracle on inputs where that rounding is exact, and stay within fp16 noise otherwise."""
+    cfg = dict(dim=256, n_layers=2, n_heads=2, vocab_size=320, multiple_of=128, max_batch_size=2, max_seq_len=8, max_prompt_seq_len=16)
+    args = O.OracleArgs(**cfg)
+    sd = O.random_q40_state_dict(args, seed=70, std=0.05)
+    g = torch.Generator().manual_seed(71)
+    prompt = torch.randint(0, 320, (1, 12), generator=g)
+    base = O.OracleTransformer(args, sd, dense=True)
+    toks, _ = base.greedy(prompt, 1, 6)
+    want = base.forced(prompt, toks[0])
+    assert want.shape == (6, 320)
+    assert torch.equal(want.argmax(-1), toks[0])                      # forced on its own tokens = its greedy run
+    # one K-slice: the fp16 rounding of the only partial sum is the result's own rounding
+    one = O.OracleTransformer(args, sd, dense=True, slab_half_ksplit=lambda key, K, N: 1, share_dense=base)
+    assert torch.equal(one.forced(prompt, toks[0]), want)
+    # several slices, double precision: close, not necessarily equal
+    for kw in (dict(slab_half_ksplit=lambda key, K, N: 4, share_dense=base), dict(acc_dtype=torch.float64), dict(p_half_prefix=True, share_dense=base),
+               dict(scale_on_x_max_rows=16, share_dense=base)):
+        got = O.OracleTransformer(args, sd, dense=True, **kw).forced(prompt, toks[0])
+        assert torch.allclose(got, want, rtol=0, atol=0.05) and float((got - want).abs().max()) > 0.0, kw
+    # power-of-two scales: x * scale and code * scale are both exact in fp16, so moving the rounding changes nothing
+    # (double-precision accumulation on both sides, so that the summation order does not matter either)
+    sd2 = dict(sd)
+    for k in list(sd2):
+        if k.endswith(".s"):
+            s = sd2[k].float()
+            sd2[k] = torch.where(s > 0, torch.exp2(torch.round(torch.log2(s.clamp_min(1e-8)))), s).to(torch.float16)
+    a64 = O.OracleTransformer(args, sd2, dense=True, acc_dtype=torch.float64)
+    b64 = O.OracleTransformer(args, sd2, dense=True, acc_dtype=torch.float64, scale_on_x_max_rows=16)
+    x = ((torch.rand((3, 256), generator=g) * 1.9 + 0.1) * torch.where(torch.rand((3, 256), generator=g) < 0.5, -1.0, 1.0)).half()    # no product underflows
+    for key in ("layers.0.attention.wq", "layers.1.feed_forward.w1"):
+        assert torch.equal(a64._linear(key, x), b64._linear(key, x))
+    x20 = torch.cat([x] * 7)[:20]                                     # 20 rows: above the limit, the dense path in both
+    assert torch.equal(a64._linear("layers.0.attention.wo", x20), b64._linear("layers.0.attention.wo", x20))
+    # uniform scores: every prefix probability is exp(0) = 1, exact in fp16
+    q = torch.zeros((2, 2, 128), dtype=torch.float16)
+    pk, pv = torch.randn((9, 2, 128), generator=g).half(), torch.randn((9, 2, 128), generator=g).half()
+    sk, sv = torch.randn((2, 3, 2, 128), generator=g).half(), torch.randn((2, 3, 2, 128), generator=g).half()
+    assert torch.equal(O.shared_prefix_attention(q, pk, pv, sk, sv, [3, 1], p_half_prefix=True), O.shared_prefix_attention(q, pk, pv, sk, sv, [3, 1]))
+    qq = torch.randn((2, 2, 128), generator=g).half()
+    d = (O.shared_prefix_attention(qq, pk, pv, sk, sv, [3, 1], p_half_prefix=True).float() - O.shared_prefix_attention(qq, pk, pv, sk, sv, [3, 1]).float()).abs().max()
+    assert float(d) <= 2e-3
+    d = (O.shared_prefix_attention(qq, pk, pv, sk, sv, [3, 1], acc_dtype=torch.float64).float() - O.shared_prefix_attention(qq, pk, pv, sk, sv, [3, 1]).float()).abs().max()
+    assert float(d) <= 2e-3
