@@ -124,24 +124,32 @@ __device__ __forceinline__ void gemv_issue_tiled(const GemvLane &L, uint8_t *sta
     }
 }
 
-// The two masks and the two fp16 magic numbers of the decoder, held in registers the compiler cannot
-// see through: (bits & mask) | magic then becomes ONE v_and_or_b32 (that instruction takes no
-// literal operands, so with visible constants the compiler emits an AND and an OR).
+// The two masks, the two fp16 magic numbers and the two offsets of the decoder, held in registers the compiler cannot
+// see through: (bits & mask) | magic then becomes ONE v_and_or_b32 (that instruction takes no literal operands, so
+// with visible constants the compiler emits an AND and an OR).
 struct GemvConsts {
     uint32_t mask_hi, mask_lo, magic_hi, magic_lo;
+    h2 off_hi, off_lo;
 };
 
-// Decoding without a per-weight multiply or subtract.  With u = nibble ^ 8 = code + 8:
-//   high nibble: (bits & 0x00F0) | 0x5400 is the fp16 number 64 + u,   code = (64 + u) - 72
-//   low  nibble: (bits & 0x000F) | 0x6400 is the fp16 number 1024 + u, code = (1024 + u) - 1032
-// These offset codes go into the matrix core as they are.  The scales move to the other operand,
-// A[m][k] = fp16(x[m][k] * s[k]) for the (block, nibble half) the 16 columns of an MFMA share, and the
-// offsets are taken out at the end:  sum_k A (v - off) = sum_k A v - off * sum_k A,  where sum_k A
-// comes from one more MFMA per (block, half) against a B operand of ones.
-// acc[blk][h][b]: column 128*blk + 64*h + 4c + b;  corr[blk*2 + h] = sum_k A.
+// Decoding.  With u = nibble ^ 8 = code + 8:
+//   high nibble: (bits & 0x00F0) | 0x5400 is the fp16 number 64 + u,   code = (64 + u) - 72     (exact)
+//   low  nibble: (bits & 0x000F) | 0x6400 is the fp16 number 1024 + u, code = (1024 + u) - 1032 (exact)
+// and ONE fp16 multiply by the group's scale gives the weight exactly as the reference's dequantiser rounds it,
+// fp16(code * scale) (fp16_to_int4.py:90-96) - three packed instructions per two weights - which enters the matrix core as
+// the B operand (lane = column, 8 consecutive k per lane) against the unscaled activations: the products the reference's
+// kernel forms (triton_kernels.py:444-449), accumulated in fp32.
+__device__ __forceinline__ uint32_t gemv_weights_high(uint32_t pr, h2 scale, const GemvConsts &C) {
+    return as_u32((as_h2((pr & C.mask_hi) | C.magic_hi) + C.off_hi) * scale);
+}
+__device__ __forceinline__ uint32_t gemv_weights_low(uint32_t pr, h2 scale, const GemvConsts &C) {
+    return as_u32((as_h2((pr & C.mask_lo) | C.magic_lo) + C.off_lo) * scale);
+}
+
+// acc[blk][h][b]: column 128*blk + 64*h + 4c + b.
 template <bool RAGGED>
 __device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K, int c, int g, const GemvConsts &C,
-                                             f4 (&acc)[2][2][4], f4 (&corr)[4]) {
+                                             f4 (&acc)[2][2][4]) {
     uint32_t u0[8], u1[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) {
@@ -155,36 +163,29 @@ __device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K
             for (int i = 0; i < 8; ++i) xv[i] = (half_t)0.f;
         }
     }
-    // scales of this lane's 8 rows: sv[i] = ((hi, lo) of block 0, (hi, lo) of block 1); regroup them per
-    // (block, half) into the k-pair order of xv and scale the activations
+    // scales of this lane's 8 rows: sv[i] = ((hi, lo) of block 0, (hi, lo) of block 1), regrouped per (block, half)
+    // into the row pairs (2j, 2j+1) of the B operands
     u32x2 sv[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) sv[i] = *reinterpret_cast<const u32x2 *>(stage + STAGE_W_BYTES + (8 * g + i) * 8);
-    h8 a[4];
+    h2 sc[2][2][4];
 #pragma unroll
-    for (int blk = 0; blk < 2; ++blk) {
-        u32x4 s_hi, s_lo;
+    for (int blk = 0; blk < 2; ++blk)
 #pragma unroll
         for (int j = 0; j < 4; ++j) {
-            s_hi[j] = pack_lo16(sv[2 * j][blk], sv[2 * j + 1][blk]);
-            s_lo[j] = pack_hi16(sv[2 * j][blk], sv[2 * j + 1][blk]);
+            sc[blk][0][j] = as_h2(pack_lo16(sv[2 * j][blk], sv[2 * j + 1][blk]));
+            sc[blk][1][j] = as_h2(pack_hi16(sv[2 * j][blk], sv[2 * j + 1][blk]));
         }
-        a[2 * blk] = xv * __builtin_bit_cast(h8, s_hi);
-        a[2 * blk + 1] = xv * __builtin_bit_cast(h8, s_lo);
-    }
-    const h8 ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
-#pragma unroll
-    for (int bh = 0; bh < 4; ++bh) corr[bh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[bh], ones, corr[bh], 0, 0, 0);
 #define SMH_GEMV_BYTE(U, BLK, B)                                                                 \
     {                                                                                            \
         u32x4 vh, vl;                                                                            \
         _Pragma("unroll") for (int j = 0; j < 4; ++j) {                                          \
             const uint32_t pr = pair_bytes<B>(U[2 * j], U[2 * j + 1]);                           \
-            vh[j] = (pr & C.mask_hi) | C.magic_hi;                                               \
-            vl[j] = (pr & C.mask_lo) | C.magic_lo;                                               \
+            vh[j] = gemv_weights_high(pr, sc[BLK][0][j], C);                                     \
+            vl[j] = gemv_weights_low(pr, sc[BLK][1][j], C);                                      \
         }                                                                                        \
-        acc[BLK][0][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * BLK], __builtin_bit_cast(h8, vh), acc[BLK][0][B], 0, 0, 0);     \
-        acc[BLK][1][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * BLK + 1], __builtin_bit_cast(h8, vl), acc[BLK][1][B], 0, 0, 0); \
+        acc[BLK][0][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv, __builtin_bit_cast(h8, vh), acc[BLK][0][B], 0, 0, 0);     \
+        acc[BLK][1][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv, __builtin_bit_cast(h8, vl), acc[BLK][1][B], 0, 0, 0);     \
     }
     SMH_GEMV_BYTE(u0, 0, 0)
     SMH_GEMV_BYTE(u0, 0, 1)
@@ -198,12 +199,12 @@ __device__ __forceinline__ void gemv_consume(const uint8_t *stage, int k0, int K
 }
 
 // The same products from a tile (q40_matmul.hpp): the lane's 64 bytes are four linear 16-byte reads, the row
-// pairs come out of (x, x2, x >> 8, x2 >> 8) and the scales arrive in the register order of the A operands.
+// pairs come out of (x, x2, x >> 8, x2 >> 8) and the scales arrive in the order of the row pairs.
 // Same operands into the same MFMAs in the same order as gemv_consume: the results are bit-identical.
 // `xrow`: the 8 activations k0 + 8g .. of this lane's batch row when they do not come from the stage (nullptr otherwise)
 template <bool RAGGED, bool XROW = false>
 __device__ __forceinline__ void gemv_consume_tiled(const uint8_t *stage, int k0, int K, int lane, const GemvConsts &C,
-                                                   f4 (&acc)[2][2][4], f4 (&corr)[4], const half_t *xrow = nullptr) {
+                                                   f4 (&acc)[2][2][4], const half_t *xrow = nullptr) {
     const int c = lane & 15, g = lane >> 4;
     u32x4 wq[4];
 #pragma unroll
@@ -217,12 +218,10 @@ __device__ __forceinline__ void gemv_consume_tiled(const uint8_t *stage, int k0,
             for (int i = 0; i < 8; ++i) xv[i] = (half_t)0.f;
         }
     }
-    h8 a[4];
+    // sc[grp][j]: scales of rows (2j, 2j+1) of this lane's k-octet for the unit's 64-column group grp = 2 blk + half
+    u32x4 sc[4];
 #pragma unroll
-    for (int grp = 0; grp < 4; ++grp) a[grp] = xv * *reinterpret_cast<const h8 *>(stage + STAGE_W_BYTES + g * 64 + grp * 16);
-    const h8 ones = {(half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f, (half_t)1.f};
-#pragma unroll
-    for (int bh = 0; bh < 4; ++bh) corr[bh] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[bh], ones, corr[bh], 0, 0, 0);
+    for (int grp = 0; grp < 4; ++grp) sc[grp] = *reinterpret_cast<const u32x4 *>(stage + STAGE_W_BYTES + g * 64 + grp * 16);
 #pragma unroll
     for (int q = 0; q < 4; ++q)
 #pragma unroll
@@ -232,11 +231,11 @@ __device__ __forceinline__ void gemv_consume_tiled(const uint8_t *stage, int k0,
             u32x4 vh, vl;
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
-                vh[j] = (pr[j] & C.mask_hi) | C.magic_hi;
-                vl[j] = (pr[j] & C.mask_lo) | C.magic_lo;
+                vh[j] = gemv_weights_high(pr[j], as_h2(sc[2 * blk][j]), C);
+                vl[j] = gemv_weights_low(pr[j], as_h2(sc[2 * blk + 1][j]), C);
             }
-            acc[blk][0][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * blk], __builtin_bit_cast(h8, vh), acc[blk][0][B], 0, 0, 0);
-            acc[blk][1][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a[2 * blk + 1], __builtin_bit_cast(h8, vl), acc[blk][1][B], 0, 0, 0);
+            acc[blk][0][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv, __builtin_bit_cast(h8, vh), acc[blk][0][B], 0, 0, 0);
+            acc[blk][1][B] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xv, __builtin_bit_cast(h8, vl), acc[blk][1][B], 0, 0, 0);
         }
 }
 
@@ -301,19 +300,17 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void q40_gemv_kernel(MatmulParams 
     }
     uint8_t *ring = lds + wave * RING;
 
-    GemvConsts C{0x00F000F0u, 0x000F000Fu, 0x54005400u, 0x64006400u};
+    GemvConsts C{0x00F000F0u, 0x000F000Fu, 0x54005400u, 0x64006400u, h2{(half_t)-72.f, (half_t)-72.f}, h2{(half_t)-1032.f, (half_t)-1032.f}};
     asm volatile("" : "+s"(C.mask_hi), "+s"(C.mask_lo));
     asm volatile("" : "+v"(C.magic_hi), "+v"(C.magic_lo));
 
-    f4 acc[2][2][4], corr[4];
+    f4 acc[2][2][4];
 #pragma unroll
     for (int d = 0; d < 2; ++d)
 #pragma unroll
         for (int h = 0; h < 2; ++h)
 #pragma unroll
             for (int b = 0; b < 4; ++b) acc[d][h][b] = f4{0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-    for (int bh = 0; bh < 4; ++bh) corr[bh] = f4{0.f, 0.f, 0.f, 0.f};
 
     // this wave's steps: first, first + WAVES, ...
     const int step0 = slice * p.steps_per_slice;
@@ -450,9 +447,9 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void q40_gemv_kernel(MatmulParams 
         if (later >= 2) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(2 * PER_STAGE) : "memory");
         else if (later == 1) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(PER_STAGE) : "memory");
         else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if constexpr (X_IN_LDS) gemv_consume_tiled<false, true>(ring + stage * STAGE, 0, p.K, lane, C, acc, corr, xlane + (first + i * WAVES - step0) * 32);
-        else if constexpr (TILED) gemv_consume_tiled<false>(ring + stage * STAGE, 0, p.K, lane, C, acc, corr);
-        else gemv_consume<false>(ring + stage * STAGE, 0, p.K, c, g, C, acc, corr);
+        if constexpr (X_IN_LDS) gemv_consume_tiled<false, true>(ring + stage * STAGE, 0, p.K, lane, C, acc, xlane + (first + i * WAVES - step0) * 32);
+        else if constexpr (TILED) gemv_consume_tiled<false>(ring + stage * STAGE, 0, p.K, lane, C, acc);
+        else gemv_consume<false>(ring + stage * STAGE, 0, p.K, c, g, C, acc);
         if (i + RING_STAGES < n_steps) {
             asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");        // this stage's LDS reads are done
             issue(ring + stage * STAGE, first + (i + RING_STAGES) * WAVES);
@@ -461,15 +458,15 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void q40_gemv_kernel(MatmulParams 
     }
     if (n_full < n_steps) {
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if constexpr (X_IN_LDS) gemv_consume_tiled<true, true>(ring + stage * STAGE, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr, xlane + (first + n_full * WAVES - step0) * 32);
-        else if constexpr (TILED) gemv_consume_tiled<true>(ring + stage * STAGE, (first + n_full * WAVES) * 32, p.K, lane, C, acc, corr);
-        else gemv_consume<true>(ring + stage * STAGE, (first + n_full * WAVES) * 32, p.K, c, g, C, acc, corr);
+        if constexpr (X_IN_LDS) gemv_consume_tiled<true, true>(ring + stage * STAGE, (first + n_full * WAVES) * 32, p.K, lane, C, acc, xlane + (first + n_full * WAVES - step0) * 32);
+        else if constexpr (TILED) gemv_consume_tiled<true>(ring + stage * STAGE, (first + n_full * WAVES) * 32, p.K, lane, C, acc);
+        else gemv_consume<true>(ring + stage * STAGE, (first + n_full * WAVES) * 32, p.K, c, g, C, acc);
     }
     __syncthreads();                        // every wave is done with its ring: reuse LDS for the sums
 
     // ---- add the waves' partial sums through LDS ----
     // accumulator element r of acc[blk][h][b] in lane (g, c) is row m = 4g + r,
-    // column 128*blk + 64h + 4c + b of the workgroup's 256; the nibble offsets (72 / 1032) leave here
+    // column 128*blk + 64h + 4c + b of the workgroup's 256
     float *red = reinterpret_cast<float *>(lds);
 #pragma unroll
     for (int d = 0; d < 2; ++d)
@@ -478,12 +475,10 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void q40_gemv_kernel(MatmulParams 
 #pragma unroll
             for (int r = 0; r < 4; ++r) {
                 const int m = 4 * g + r;
-                const float off = h ? 1032.f : 72.f;
                 if (r < p.M) {                      // uniform: with fewer than 4 rows whole store instructions drop out
                     if (m < p.M) {                  // the four columns 4c .. 4c+3 of (block d, half h) as one 16-byte store
-                        const float cr = off * corr[2 * d + h][r];
                         *reinterpret_cast<f4 *>(&red[(wave * p.M + m) * GEMV_COLS + 128 * d + 64 * h + 4 * c]) =
-                            f4{acc[d][h][0][r] - cr, acc[d][h][1][r] - cr, acc[d][h][2][r] - cr, acc[d][h][3][r] - cr};
+                            f4{acc[d][h][0][r], acc[d][h][1][r], acc[d][h][2][r], acc[d][h][3][r]};
                     }
                 }
             }
