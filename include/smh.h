@@ -185,6 +185,16 @@ int smh_rope(void *q, void *k, int S, int H, int Hkv, int D, const void *cos_tab
 int smh_kv_fork(void *cache, void *cache_s, int Bmax, long row_bytes, long row_scales,
                 int origin, int curr, int forks, smh_stream_t stream);
 
+/* ---- fp16 vocabulary projection and embedding -------------------------------------------------------
+ * smh_f16_linear: out[M, N] = x[M, K] . w[N, K]^T, fp16 operands, fp32 accumulation, one rounding to fp16: the
+ *   `self.output(h)` of Transformer.forward (hf_model_q40_kv_shared.py:509; nn.Linear without bias, weight [vocab, dim]
+ *   as the checkpoint holds it, :484).  x rows ldx apart, out rows ldo apart; K % 64 == 0, ldx % 8 == 0, x and w 16-byte
+ *   aligned.  N need not be a multiple of anything (vocab 32016).
+ * smh_embedding: out[m, :] = table[tokens[m], :], the `self.tok_embeddings(tokens)` of Transformer.forward (:495; table
+ *   [vocab, dim] fp16, :477).  tokens int64 [M] on the device; dim % 8 == 0. */
+int smh_f16_linear(const void *x, int M, int K, long ldx, const void *w, int N, void *out, long ldo, smh_stream_t stream);
+int smh_embedding(const int64_t *tokens, int M, const void *table, int vocab, int dim, void *out, smh_stream_t stream);
+
 /* ---- attention -----------------------------------------------------------------------------
  * smh_shared_prefix_attn: the decode attention of Attention.forward
  * (hf_model_q40_kv_shared.py:375-405) without materialising or copying the prefix per branch:
@@ -210,6 +220,31 @@ int smh_shared_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int 
                            void *workspace, size_t workspace_bytes, smh_stream_t stream);
 int smh_prefill_attn(const void *q, const void *k, const void *v, void *out, int S, int H, int Hkv,
                      int D, smh_stream_t stream);
+
+/* ---- paged / tree attention --------------------------------------------------------------------------------------
+ * smh_paged_prefix_attn: smh_shared_prefix_attn whose per-branch rows are looked up in a page table inside the
+ * kernel, one token per page: the reference's tree attention page_flash_attn (triton_kernels.py:649-789, pager[B, L] ->
+ * page pool) and the intent of chunk_attn (:1150-1231: a shared first chunk, then the branch's own pages).  Branches
+ * forked from a common ancestor share the ancestor's pages, so Attention.fork (hf_model_q40_kv_shared.py:282-297)
+ * becomes a copy of page ids (smh_page_fork) instead of a copy of K/V rows.
+ *   out[b,h,:] = softmax(q[b,h,:] . K_b^T / sqrt(D)) . V_b,  K_b = [prefix rows 0..P-1 (shared) || pool rows
+ *                pages[b, 0 .. lens[b]-1] || cur_k[b] (optional)]
+ *   prefix_k/v   fp16, element strides prefix_row_stride between rows and prefix_head_stride between kv heads
+ *                (0, 0 = token-major [P, Hkv, D]; a head-major pool [Hkv, rows, D] is (D, rows * D))
+ *   pool         SMH_KV_FP16: pool_k/v fp16 with pool_row_stride / pool_head_stride as above;
+ *                SMH_KV_Q40: the model's cache rows, bytes [rows, Hkv, 64] + scales fp16 [rows, Hkv, 2] (strides 0)
+ *   pages        page ids [B, pages_stride] of page_bytes = 2, 4 or 8 bytes each (int16 as in the reference, int32, int64)
+ *   lens         int32 [B] (lens_stride 1) or one shared int32 (lens_stride 0): pages of the branch that are valid
+ *   single_launch, workspace: as smh_shared_prefix_attn_one (counters zeroed once) when != 0, else as smh_shared_prefix_attn
+ * smh_page_fork: table[curr + i, 0..n-1] = table[origin, 0..n-1] for i < forks; table int32 [rows, stride]. */
+int smh_paged_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int D,
+                          const void *prefix_k, const void *prefix_v, int P, long prefix_row_stride, long prefix_head_stride,
+                          int pool_format, const void *pool_k, const void *pool_v, const void *pool_ks, const void *pool_vs,
+                          long pool_row_stride, long pool_head_stride,
+                          const void *pages, int page_bytes, long pages_stride, const int32_t *lens, int lens_stride,
+                          const void *cur_k, const void *cur_v, int single_launch,
+                          void *workspace, size_t workspace_bytes, smh_stream_t stream);
+int smh_page_fork(int32_t *table, int rows, long stride, int origin, int curr, int forks, int n, smh_stream_t stream);
 
 /* smh_shared_prefix_attn_static: smh_shared_prefix_attn (same arguments without the workspace, same kernels, bit-identical
  * results) for callers that cannot allocate device memory or pass a workspace: code under HIP graph capture, tight
@@ -255,14 +290,18 @@ int smh_shared_prefix_attn_one(const void *q, void *out, int B, int H, int Hkv, 
  *                       that merges a kv head's tiles takes longer than a second launch).
  *                       workspace: smh_attn_qkv_workspace_bytes(B, H, P) bytes whose first 4096 bytes (the
  *                       counters) are zero before the first call; the calls leave them zero.  Calls that
- *                       overlap in time need separate workspaces. */
+ *                       overlap in time need separate workspaces.
+ *   pages               NULL, or a page table int32 [B, pages_stride] (pages_stride >= Smax): suffix row j of branch b is
+ *                       read from cache row pages[b * pages_stride + j] (rows counted over all branches, i.e. branch b's own
+ *                       row j is b * Smax + j) - branches forked from a common ancestor share its rows instead of holding
+ *                       copies (see smh_paged_prefix_attn).  The new token's row is still appended at b * Smax + *t_dev. */
 size_t smh_attn_qkv_workspace_bytes(int B, int H, int P);
 int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, void *out, int B, int H, int Hkv, int D,
                                const void *cos_tab, const void *sin_tab, const int32_t *pos_dev,
                                const void *prefix_k, const void *prefix_v, int P,
                                void *cache_k, void *cache_ks, void *cache_v, void *cache_vs, int Smax,
-                               const int32_t *t_dev, int single_launch, void *workspace, size_t workspace_bytes,
-                               smh_stream_t stream);
+                               const int32_t *t_dev, const int32_t *pages, int pages_stride, int single_launch,
+                               void *workspace, size_t workspace_bytes, smh_stream_t stream);
 
 #ifdef __cplusplus
 }

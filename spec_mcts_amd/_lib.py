@@ -49,6 +49,8 @@ SIGNATURES = {
     "smh_rope_append_kv": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, c_int, _P, _P]),
     "smh_rope": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, _P]),
     "smh_kv_fork": (c_int, [_P, _P, c_int, c_long, c_long, c_int, c_int, c_int, _P]),
+    "smh_f16_linear": (c_int, [_P, c_int, c_int, c_long, _P, c_int, _P, c_long, _P]),
+    "smh_embedding": (c_int, [_P, c_int, _P, c_int, c_int, _P, _P]),
     "smh_attn_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "smh_shared_prefix_attn": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, c_int, _P, _P, _P, _P, c_int,
                                        _P, c_int, _P, _P, _P, c_size_t, _P]),
@@ -60,7 +62,11 @@ SIGNATURES = {
     "smh_prefill_attn": (c_int, [_P, _P, _P, _P, c_int, c_int, c_int, c_int, _P]),
     "smh_attn_qkv_workspace_bytes": (c_size_t, [c_int, c_int, c_int]),
     "smh_shared_prefix_attn_qkv": (c_int, [_P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_int,
-                                           _P, _P, _P, _P, c_int, _P, c_int, _P, c_size_t, _P]),
+                                           _P, _P, _P, _P, c_int, _P, _P, c_int, c_int, _P, c_size_t, _P]),
+    "smh_paged_prefix_attn": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, c_long, c_long,
+                                      c_int, _P, _P, _P, _P, c_long, c_long, _P, c_int, c_long, _P, c_int, _P, _P, c_int,
+                                      _P, c_size_t, _P]),
+    "smh_page_fork": (c_int, [_P, c_int, c_long, c_int, c_int, c_int, c_int, _P]),
 }
 
 _lib = None

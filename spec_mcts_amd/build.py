@@ -13,7 +13,7 @@ import sys
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libsmh.so")
-SOURCES = ["smh_api.hip", "q40_codec.hip", "q40_gemv.hip", "q40_gemm.hip", "partial_ops.hip", "elementwise.hip", "attn_decode.hip"]
+SOURCES = ["smh_api.hip", "q40_codec.hip", "q40_gemv.hip", "q40_gemm.hip", "partial_ops.hip", "elementwise.hip", "attn_decode.hip", "f16_head.hip"]
 # packed fp32 VALU ops are disabled on purpose (device code only; the host pass ignores the feature)
 FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-Wall", "-Wno-unused-function",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops"]

@@ -42,6 +42,15 @@ struct AttnParams {
     float *part_o;           // [splits][Hkv][Bq][128]
     float *part_ml;          // [splits][Hkv][Bq][2]
     long suffix_batch_stride_rows;   // rows (tokens) between consecutive branches of the suffix
+    // paged suffix: row j of branch b is pool row pages[b * pages_stride + j] instead of b * suffix_batch_stride_rows + j
+    // (page ids of page_bytes = 2, 4 or 8 bytes each); pages == nullptr: contiguous rows per branch
+    const void *pages;
+    long pages_stride;
+    int page_bytes;
+    // element strides of the fp16 K/V tensors: between consecutive rows (tokens) and between kv heads.  Token-major
+    // [rows, Hkv, 128] is (Hkv * 128, 128); a head-major pool [Hkv, rows, 128] is (128, rows * 128).  Q4_0 rows are token-major.
+    long pfx_row_stride, pfx_head_stride;
+    long sfx_row_stride, sfx_head_stride;
     int B, H, Hkv, n_rep, Bq;        // Bq = B * n_rep queries per kv head
     int suffix_waves;                // waves that share one query's suffix rows (1, 2 or 4)
     int P, tw, splits;
@@ -176,7 +185,7 @@ __device__ __forceinline__ void attn_prefix_body(const AttnParams &p, int split,
             const int t = 4 * kg + e;
             kv[e] = u32x4{0, 0, 0, 0}; vv[e] = u32x4{0, 0, 0, 0};
             if (t < cnt) {
-                const long off = ((long)(t0 + t) * p.Hkv + hk) * ATT_D + ch * 8;
+                const long off = (long)(t0 + t) * p.pfx_row_stride + (long)hk * p.pfx_head_stride + ch * 8;
                 kv[e] = *reinterpret_cast<const u32x4 *>(p.prefix_k + off);
                 vv[e] = *reinterpret_cast<const u32x4 *>(p.prefix_v + off);
             }
@@ -468,9 +477,18 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
     const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
     const int wave = threadIdx.x >> 6;
     int len = 0;
-    if (p.suffix_format != SMH_KV_NONE) len = p.causal ? b + 1 : p.lens[(long)b * p.lens_stride];
+    // a length beyond the branch's rows (a device counter that ran past the cache) is cut at the cache's end
+    if (p.suffix_format != SMH_KV_NONE) len = p.causal ? b + 1 : min(p.lens[(long)b * p.lens_stride], (int)p.suffix_batch_stride_rows);
     const int gg = g + 4 * sub, gstride = 4 * nsub;      // this group's first row and the distance to its next one
     const long row0 = (long)b * p.suffix_batch_stride_rows;     // first suffix row of this branch
+    // pool row that holds suffix position t of this branch
+    auto row_of = [&](int t) -> long {
+        if (p.pages == nullptr) return row0 + t;
+        const long i = (long)b * p.pages_stride + t;
+        if (p.page_bytes == 4) return reinterpret_cast<const int32_t *>(p.pages)[i];
+        if (p.page_bytes == 2) return reinterpret_cast<const int16_t *>(p.pages)[i];
+        return reinterpret_cast<const int64_t *>(p.pages)[i];
+    };
     // one batch of Q4_0 suffix rows: group g takes rows t0, t0 + 4, ... (rows past the end repeat the last one).
     // Four rows a group per batch: eight measured 1-1.5 % slower per decode step at 1, 10 and 100 branches (more
     // registers, and a short suffix pays for rows it does not have), two 1.5 % slower (more round trips).
@@ -478,7 +496,7 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
     auto load_q40_batch = [&](int t0, uint32_t (&kb)[UQ], uint32_t (&vb)[UQ], uint32_t (&ksc)[UQ], uint32_t (&vsc)[UQ]) {
 #pragma unroll
         for (int u = 0; u < UQ; ++u) {
-            const long row = (row0 + min(t0 + gstride * u, len - 1)) * p.Hkv + hk;
+            const long row = row_of(min(t0 + gstride * u, len - 1)) * p.Hkv + hk;
             kb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_k + row * 64 + 4 * c);
             vb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_v + row * 64 + 4 * c);
             ksc[u] = *reinterpret_cast<const uint32_t *>(p.suffix_ks + row * 2);
@@ -577,9 +595,9 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
                 RowRegs kr[U], vr[U];
 #pragma unroll
                 for (int u = 0; u < U; ++u) {
-                    const long row = (row0 + min(t0 + gstride * u, len - 1)) * p.Hkv + hk;
-                    kr[u] = row_from_fp16((const half_t *)p.suffix_k + row * ATT_D, c);
-                    vr[u] = row_from_fp16((const half_t *)p.suffix_v + row * ATT_D, c);
+                    const long off = row_of(min(t0 + gstride * u, len - 1)) * p.sfx_row_stride + (long)hk * p.sfx_head_stride;
+                    kr[u] = row_from_fp16((const half_t *)p.suffix_k + off, c);
+                    vr[u] = row_from_fp16((const half_t *)p.suffix_v + off, c);
                 }
 #pragma unroll
                 for (int u = 0; u < U; ++u)
@@ -853,12 +871,20 @@ extern "C" size_t smh_attn_workspace_bytes(int B, int H, int P) {
 
 constexpr size_t ATT_COUNTER_BYTES = 4096;     // one-launch variants: arrival counters at the start of the workspace
 
+// what the paged entry point adds to the arguments of smh_shared_prefix_attn (zero strides: token-major tensors)
+struct AttnExtras {
+    const void *pages = nullptr;
+    long pages_stride = 0;
+    int page_bytes = 4;
+    long pfx_row = 0, pfx_head = 0, sfx_row = 0, sfx_head = 0;
+};
+
 static int shared_prefix_attn(const char *who, bool one, const void *q, void *out, int B, int H, int Hkv, int D,
                               const void *prefix_k, const void *prefix_v, int P,
                               int suffix_format, const void *suffix_k, const void *suffix_v,
                               const void *suffix_ks, const void *suffix_vs, int Smax,
                               const int32_t *lens, int lens_stride, const void *cur_k, const void *cur_v,
-                              void *workspace, size_t workspace_bytes, smh_stream_t stream) {
+                              void *workspace, size_t workspace_bytes, smh_stream_t stream, const AttnExtras &ex = AttnExtras()) {
     using namespace smh;
     SMH_REQUIRE(D == ATT_D, "%s: head dim %d (only 128)", who, D);
     SMH_REQUIRE(B >= 0 && B <= 65535 && H > 0 && Hkv > 0 && H % Hkv == 0 && P >= 0, "%s: B=%d (at most 65535) H=%d Hkv=%d P=%d", who, B, H, Hkv, P);
@@ -881,6 +907,9 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
     p.lens = lens; p.lens_stride = lens_stride;
     p.cur_k = (const half_t *)cur_k; p.cur_v = (const half_t *)cur_v;
     p.suffix_batch_stride_rows = Smax;
+    p.pages = ex.pages; p.pages_stride = ex.pages_stride; p.page_bytes = ex.page_bytes;
+    p.pfx_row_stride = ex.pfx_row ? ex.pfx_row : (long)Hkv * ATT_D; p.pfx_head_stride = ex.pfx_head ? ex.pfx_head : ATT_D;
+    p.sfx_row_stride = ex.sfx_row ? ex.sfx_row : (long)Hkv * ATT_D; p.sfx_head_stride = ex.sfx_head ? ex.sfx_head : ATT_D;
     p.B = B; p.H = H; p.Hkv = Hkv; p.n_rep = H / Hkv; p.Bq = B * p.n_rep;
     p.P = P; p.suffix_format = suffix_format; p.causal = 0;
     p.scale_log2 = LOG2E / sqrtf((float)D);
@@ -922,6 +951,48 @@ extern "C" int smh_shared_prefix_attn(const void *q, void *out, int B, int H, in
                                       void *workspace, size_t workspace_bytes, smh_stream_t stream) {
     return shared_prefix_attn("smh_shared_prefix_attn", false, q, out, B, H, Hkv, D, prefix_k, prefix_v, P, suffix_format, suffix_k,
                               suffix_v, suffix_ks, suffix_vs, Smax, lens, lens_stride, cur_k, cur_v, workspace, workspace_bytes, stream);
+}
+
+extern "C" int smh_paged_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int D,
+                                     const void *prefix_k, const void *prefix_v, int P, long prefix_row_stride, long prefix_head_stride,
+                                     int pool_format, const void *pool_k, const void *pool_v, const void *pool_ks, const void *pool_vs,
+                                     long pool_row_stride, long pool_head_stride,
+                                     const void *pages, int page_bytes, long pages_stride, const int32_t *lens, int lens_stride,
+                                     const void *cur_k, const void *cur_v, int single_launch,
+                                     void *workspace, size_t workspace_bytes, smh_stream_t stream) {
+    using namespace smh;
+    const char *who = "smh_paged_prefix_attn";
+    SMH_REQUIRE(pool_format == SMH_KV_FP16 || pool_format == SMH_KV_Q40, "%s: pool_format=%d", who, pool_format);
+    SMH_REQUIRE(pages != nullptr && (page_bytes == 2 || page_bytes == 4 || page_bytes == 8) && pages_stride >= 1,
+                "%s: pages=%p page_bytes=%d (2, 4 or 8) pages_stride=%ld", who, pages, page_bytes, pages_stride);
+    SMH_REQUIRE(pages_stride <= 0x7fffffffL, "%s: pages_stride=%ld", who, pages_stride);
+    SMH_REQUIRE(prefix_row_stride >= 0 && prefix_head_stride >= 0 && pool_row_stride >= 0 && pool_head_stride >= 0 &&
+                prefix_row_stride % 8 == 0 && prefix_head_stride % 8 == 0 && pool_row_stride % 4 == 0 && pool_head_stride % 4 == 0,
+                "%s: strides must be non-negative (0 = token-major), prefix strides multiples of 8 and pool strides multiples of 4 elements", who);
+    SMH_REQUIRE(pool_format != SMH_KV_Q40 || (pool_row_stride == 0 && pool_head_stride == 0), "%s: Q4_0 pools are token-major (strides 0)", who);
+    AttnExtras ex;
+    ex.pages = pages; ex.page_bytes = page_bytes; ex.pages_stride = pages_stride;
+    ex.pfx_row = prefix_row_stride; ex.pfx_head = prefix_head_stride; ex.sfx_row = pool_row_stride; ex.sfx_head = pool_head_stride;
+    return shared_prefix_attn(who, single_launch != 0, q, out, B, H, Hkv, D, prefix_k, prefix_v, P, pool_format, pool_k, pool_v, pool_ks, pool_vs,
+                              (int)pages_stride, lens, lens_stride, cur_k, cur_v, workspace, workspace_bytes, stream, ex);
+}
+
+// copies entries 0 .. n - 1 of row `origin` of a page table [rows, stride] to rows curr .. curr + forks - 1
+__global__ __launch_bounds__(256) void page_fork_kernel(int32_t *table, long stride, int origin, int curr, int n) {
+    const int32_t *src = table + (long)origin * stride;
+    int32_t *dst = table + (long)(curr + blockIdx.y) * stride;
+    const int i = blockIdx.x * 256 + threadIdx.x;
+    if (i < n) dst[i] = src[i];
+}
+
+extern "C" int smh_page_fork(int32_t *table, int rows, long stride, int origin, int curr, int forks, int n, smh_stream_t stream) {
+    SMH_REQUIRE(table && rows > 0 && stride > 0 && n >= 0 && n <= stride, "smh_page_fork: table=%p rows=%d stride=%ld n=%d", (void *)table, rows, stride, n);
+    SMH_REQUIRE(origin >= 0 && origin < rows && forks >= 0 && curr >= 0 && curr + forks <= rows && forks <= 65535,
+                "smh_page_fork: origin=%d curr=%d forks=%d outside the table's %d rows", origin, curr, forks, rows);
+    SMH_REQUIRE(origin < curr || origin >= curr + forks, "smh_page_fork: the origin row lies inside the rows it is copied to");
+    if (forks == 0 || n == 0) return 0;
+    hipLaunchKernelGGL(page_fork_kernel, dim3((unsigned)((n + 255) / 256), (unsigned)forks), dim3(256), 0, (hipStream_t)stream, table, stride, origin, curr, n);
+    return smh::launch_status();
 }
 
 // ---- the same attention for callers that cannot allocate ---------------------------------------------------------
@@ -1000,10 +1071,11 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
                                           const void *cos_tab, const void *sin_tab, const int32_t *pos_dev,
                                           const void *prefix_k, const void *prefix_v, int P,
                                           void *cache_k, void *cache_ks, void *cache_v, void *cache_vs, int Smax,
-                                          const int32_t *t_dev, int single_launch, void *workspace, size_t workspace_bytes,
-                                          smh_stream_t stream) {
+                                          const int32_t *t_dev, const int32_t *pages, int pages_stride, int single_launch,
+                                          void *workspace, size_t workspace_bytes, smh_stream_t stream) {
     using namespace smh;
     const char *who = "smh_shared_prefix_attn_qkv";
+    SMH_REQUIRE(pages == nullptr || pages_stride >= Smax, "%s: pages_stride=%d must cover the %d rows of a branch", who, pages_stride, Smax);
     SMH_REQUIRE(D == ATT_D, "%s: head dim %d (only 128)", who, D);
     SMH_REQUIRE(B >= 0 && B <= 16 && H > 0 && Hkv > 0 && H % Hkv == 0 && P >= 0, "%s: B=%d (at most 16) H=%d Hkv=%d P=%d", who, B, H, Hkv, P);
     SMH_REQUIRE(ksplit >= 1 && ksplit <= 16, "%s: ksplit=%d", who, ksplit);
@@ -1019,6 +1091,9 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
     p.suffix_ks = (const half_t *)cache_ks; p.suffix_vs = (const half_t *)cache_vs;
     p.lens = t_dev; p.lens_stride = 0;
     p.suffix_batch_stride_rows = Smax;
+    p.pages = pages; p.pages_stride = pages_stride; p.page_bytes = 4;
+    p.pfx_row_stride = (long)Hkv * ATT_D; p.pfx_head_stride = ATT_D;
+    p.sfx_row_stride = (long)Hkv * ATT_D; p.sfx_head_stride = ATT_D;
     p.B = B; p.H = H; p.Hkv = Hkv; p.n_rep = H / Hkv; p.Bq = B * p.n_rep;
     p.P = P; p.suffix_format = SMH_KV_Q40; p.causal = 0;
     p.scale_log2 = LOG2E / sqrtf((float)D);

@@ -171,7 +171,21 @@ class Attention(nn.Module):
         """Sets sequence length = 0"""
         self.cache_prompt_len = 0
 
-    def forward(self, x: torch.Tensor, start_pos: int, freqs_cis, mask, residual=None, step_state=None):
+    def decode_attention(self, q, k, v, t_dev, pages, single_launch):
+        """One query per branch over the shared prompt rows, the branch's suffix rows 0 .. *t_dev - 1 (its own, or those its
+        page-table row names) and the new token's exact k, v."""
+        P = self.cache_prompt_len
+        if pages is None:
+            return K.shared_prefix_attn(q, self.cache_prompt_k[0], self.cache_prompt_v[0], P, suffix_k=self.cache_k, suffix_v=self.cache_v,
+                                        suffix_ks=self.cache_k_s, suffix_vs=self.cache_v_s, Smax=self.args.max_seq_len, lens=t_dev,
+                                        lens_stride=0, cur_k=k, cur_v=v, single_launch=single_launch)
+        Hkv = self.n_local_kv_heads
+        return K.paged_prefix_attn(q, pages, t_dev, self.cache_k.view(-1, Hkv, 64), self.cache_v.view(-1, Hkv, 64),
+                                   self.cache_k_s.view(-1, Hkv, 2), self.cache_v_s.view(-1, Hkv, 2),
+                                   prefix_k=self.cache_prompt_k[0], prefix_v=self.cache_prompt_v[0], P=P, cur_k=k, cur_v=v,
+                                   lens_stride=0, single_launch=single_launch)
+
+    def forward(self, x: torch.Tensor, start_pos: int, freqs_cis, mask, residual=None, step_state=None, pages=None):
         """x [B,S,dim] (already normalised); returns residual + wo(attention) when `residual` is given."""
         bsz, seqlen, _ = x.shape
         global QKVO_TIME, ATTN_TIME
@@ -203,11 +217,7 @@ class Attention(nn.Module):
             K.rope_append_kv(q_b, k_b, v_b, cos, sin, pos_dev, self.cache_k, self.cache_k_s,
                              self.cache_v, self.cache_v_s, self.args.max_seq_len, t_dev)
             t1 = _tick()
-            output = K.shared_prefix_attn(
-                q_b, self.cache_prompt_k[0], self.cache_prompt_v[0], self.cache_prompt_len,
-                suffix_k=self.cache_k, suffix_v=self.cache_v, suffix_ks=self.cache_k_s, suffix_vs=self.cache_v_s,
-                Smax=self.args.max_seq_len, lens=t_dev, lens_stride=0, cur_k=k_b, cur_v=v_b)
-            output = output.view(bsz, 1, H * D)
+            output = self.decode_attention(q_b, k_b, v_b, t_dev, pages, False).view(bsz, 1, H * D)
         if PROFILE:
             t2 = _tick()
             QKVO_TIME += t1 - t0
@@ -249,9 +259,9 @@ class TransformerBlock(nn.Module):
         self.attention_norm = RMSNorm(args.dim, eps=args.norm_eps)
         self.ffn_norm = RMSNorm(args.dim, eps=args.norm_eps)
 
-    def forward(self, x, start_pos, freqs_cis, mask, step_state=None):
+    def forward(self, x, start_pos, freqs_cis, mask, step_state=None, pages=None):
         # the residual adds are fused into the epilogues of wo and w2
-        h = self.attention.forward(self.attention_norm(x), start_pos, freqs_cis, mask, residual=x, step_state=step_state)
+        h = self.attention.forward(self.attention_norm(x), start_pos, freqs_cis, mask, residual=x, step_state=step_state, pages=pages)
         return self.feed_forward.forward(self.ffn_norm(h), residual=h)
 
 
@@ -286,6 +296,10 @@ class Transformer(nn.Module):
         self.norm_in_max_rows = 2          # ... up to this many rows: at 10 rows the matmul's longer prologue costs more than it saves
         self._norm_in_ok = {}
         self.attn_from_qkv = True          # up to 16 branches the attention takes the wq|wk|wv product itself, in one launch
+        self.paged_kv = True               # fork = a copy of page ids: forked branches share their ancestor's suffix rows
+        self._page_table = None            # int32 [max_batch_size, max_seq_len]: cache row that holds position j of branch b
+        self._forked = False               # a fork happened since the last resetSeq (until then every branch reads its own rows)
+        self._rows_written = 0             # suffix rows every live branch has after the last decode step
 
     # -- helpers -------------------------------------------------------------------------------
     def _tables(self, device):
@@ -314,12 +328,13 @@ class Transformer(nn.Module):
         function issues no host-to-device traffic and can be captured in a HIP graph."""
         if self.fused:
             return self._forward_fused(tokens, start_pos, step_state)
-        h = self.tok_embeddings(tokens).to(DTYPE)
+        h = K.embedding(tokens, self.tok_embeddings.weight)
         freqs = self._tables(h.device)
+        pages = self._pages(h.device) if start_pos != 0 else None
         for layer in self.layers:
-            h = layer(h, start_pos, freqs, None, step_state=step_state)
+            h = layer(h, start_pos, freqs, None, step_state=step_state, pages=pages)
         h = self.norm(h)
-        return self.output(h).to(DTYPE)
+        return K.f16_linear(h, self.output.weight)
 
     def _forward_fused(self, tokens: torch.Tensor, start_pos: int, step_state):
         """Same arithmetic as the module-by-module path, with the launches of a layer fused:
@@ -330,9 +345,10 @@ class Transformer(nn.Module):
         bsz, seqlen = tokens.shape
         M = bsz * seqlen
         p = self.params
-        h = self.tok_embeddings(tokens).to(DTYPE).reshape(M, p.dim)
+        h = K.embedding(tokens, self.tok_embeddings.weight).view(M, p.dim)
         cos, sin = self._tables(h.device)
         pending = None                      # product of the previous layer's w2, not yet added to h
+        pages = self._pages(h.device) if start_pos != 0 else None
         for layer in self.layers:
             att, ff = layer.attention, layer.feed_forward
             H, Hkv, D = att.n_local_heads, att.n_local_kv_heads, att.head_dim
@@ -373,15 +389,12 @@ class Transformer(nn.Module):
                     o = K.shared_prefix_attn_qkv(qkv, H, Hkv, D, cos, sin, pos_dev, att.cache_prompt_k[0], att.cache_prompt_v[0],
                                                  att.cache_prompt_len, att.cache_k, att.cache_k_s, att.cache_v, att.cache_v_s,
                                                  p.max_seq_len, t_dev,
-                                                 single_launch=self.attn_single_launch and M * (H // Hkv) <= 16).view(M, H * D)
+                                                 single_launch=self.attn_single_launch and M * (H // Hkv) <= 16,
+                                                 pages=pages).view(M, H * D)
                 else:
                     q, k, v = K.partial_rope_append_kv(qkv, H, Hkv, D, cos, sin, pos_dev, att.cache_k, att.cache_k_s,
                                                        att.cache_v, att.cache_v_s, p.max_seq_len, t_dev)
-                    o = K.shared_prefix_attn(q, att.cache_prompt_k[0], att.cache_prompt_v[0], att.cache_prompt_len,
-                                             suffix_k=att.cache_k, suffix_v=att.cache_v, suffix_ks=att.cache_k_s,
-                                             suffix_vs=att.cache_v_s, Smax=p.max_seq_len, lens=t_dev, lens_stride=0,
-                                             cur_k=k, cur_v=v,
-                                             single_launch=self.attn_single_launch and M * (H // Hkv) <= 16).view(M, H * D)
+                    o = att.decode_attention(q, k, v, t_dev, pages, self.attn_single_launch and M * (H // Hkv) <= 16).view(M, H * D)
             po = K.matmul_q40_partial(o, [att.wo.operand(tiled)])
             gu_ops = [ff.w1.operand(tiled), ff.w3.operand(tiled)]
             if self._norm_in(M, p.dim, gu_ops):
@@ -396,7 +409,19 @@ class Transformer(nn.Module):
                 act = K.partial_silu_mul(gu)
                 pending = K.matmul_q40_partial(act, [ff.w2.operand(tiled)])
         _, hn = K.partial_rmsnorm(pending, h, self.norm.weight, self.norm.eps, want_h=False)
-        return self.output(hn.view(bsz, seqlen, p.dim)).to(DTYPE)
+        return K.f16_linear(hn.view(bsz, seqlen, p.dim), self.output.weight)
+
+    def _pages(self, device):
+        """The page table the attention kernels read suffix rows through, or None while no branch shares rows."""
+        if not (self.paged_kv and self._forked) or self.per_branch_kv:
+            return None
+        return self._table(device)
+
+    def _table(self, device):
+        p = self.params
+        if self._page_table is None or self._page_table.device != device:
+            self._page_table = torch.arange(p.max_batch_size * p.max_seq_len, dtype=torch.int32, device=device).view(p.max_batch_size, p.max_seq_len)
+        return self._page_table
 
     def _norm_in(self, M: int, Kd: int, ops) -> bool:
         """RMSNorm inside the matmul that follows it: tiled weights, few rows, and rows x K-slice small enough for the
@@ -418,14 +443,25 @@ class Transformer(nn.Module):
         if start_pos != 0:
             t = start_pos - self.layers[0].attention.cache_prompt_len
             assert 0 <= t < self.params.max_seq_len, "suffix cache exhausted"
+            assert start_pos < self.freqs_cis.shape[0], "position beyond the rotation table"
             assert _bsz <= self.params.max_batch_size
             step_state = self._set_step(tokens.device, start_pos)
+            self._rows_written = t + 1
         else:
             assert seqlen <= self.params.max_prompt_seq_len
+            self._rows_written = 0
         return self._forward_impl(tokens, start_pos, step_state)
 
     def fork(self, origin: int, curr_batch: int, forks: int):
-        """Forks the process, such that kv-cache is copied from origin batch number to all the list of new batches"""
+        """Forks the process, such that kv-cache is copied from origin batch number to all the list of new batches.
+        With paged_kv (the default) nothing of the cache moves: the new branches' page-table rows take the ids of the
+        origin's rows written so far, one small launch for the whole model; later rows go to each branch's own slots."""
+        assert 0 <= origin < self.params.max_batch_size and forks >= 0 and 0 <= curr_batch and curr_batch + forks <= self.params.max_batch_size
+        if self.paged_kv and not self.per_branch_kv:
+            if forks > 0 and self._rows_written > 0:
+                K.page_fork(self._table(self.layers[0].attention.cache_k.device), origin, curr_batch, forks, self._rows_written)
+                self._forked = True
+            return
         for layer in self.layers:
             layer.attention.fork(origin, curr_batch, forks)
 
@@ -433,6 +469,10 @@ class Transformer(nn.Module):
         """Sets all sequence length = 0"""
         for layer in self.layers:
             layer.attention.resetSeq()
+        if self._forked:
+            self._page_table = None          # back to every branch reading its own rows
+            self._forked = False
+        self._rows_written = 0
 
     def resetTimers(self):
         global COMP_TIME, DEQ_TIME, QKVO_TIME, ATTN_TIME, MLP_TIME, Q_TIME, DQ_TIME

@@ -485,6 +485,37 @@ def kv_fork(cache: torch.Tensor, cache_s: torch.Tensor, Bmax: int, origin: int, 
 
 
 # ---------------------------------------------------------------------------------------------
+# fp16 vocabulary projection, embedding
+# ---------------------------------------------------------------------------------------------
+def f16_linear(x: torch.Tensor, weight: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """x [..., K] . weight [N, K]^T -> [..., N] fp16 (fp32 accumulation, one rounding): nn.Linear without bias, as the
+    reference's lm_head (hf_model_q40_kv_shared.py:484,509)."""
+    lib = _lib.load()
+    _need_gpu(x, weight)
+    assert x.dtype == torch.float16 and weight.dtype == torch.float16 and weight.dim() == 2 and weight.is_contiguous()
+    N, Kd = weight.shape
+    assert x.shape[-1] == Kd and x.is_contiguous()
+    M = x.numel() // Kd
+    if out is None:
+        out = torch.empty(x.shape[:-1] + (N,), dtype=torch.float16, device=x.device)
+    assert out.dtype == torch.float16 and out.is_contiguous() and out.numel() == M * N
+    check(lib.smh_f16_linear(x.data_ptr(), M, Kd, Kd, weight.data_ptr(), N, out.data_ptr(), N, _stream()), "smh_f16_linear")
+    return out
+
+
+def embedding(tokens: torch.Tensor, table: torch.Tensor) -> torch.Tensor:
+    """table[tokens]: int64 tokens [...] -> fp16 [..., dim] (nn.Embedding of the reference, hf_model_q40_kv_shared.py:477,495)."""
+    lib = _lib.load()
+    _need_gpu(tokens, table)
+    assert tokens.dtype == torch.int64 and table.dtype == torch.float16 and table.dim() == 2 and table.is_contiguous()
+    tokens = tokens.contiguous()
+    vocab, dim = table.shape
+    out = torch.empty(tokens.shape + (dim,), dtype=torch.float16, device=table.device)
+    check(lib.smh_embedding(tokens.data_ptr(), tokens.numel(), table.data_ptr(), vocab, dim, out.data_ptr(), _stream()), "smh_embedding")
+    return out
+
+
+# ---------------------------------------------------------------------------------------------
 # attention
 # ---------------------------------------------------------------------------------------------
 def shared_prefix_attn(q: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix_v: Optional[torch.Tensor], P: int,
@@ -545,13 +576,18 @@ def shared_prefix_attn(q: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix
 def shared_prefix_attn_qkv(p: PartialProduct, H: int, Hkv: int, D: int, cos: torch.Tensor, sin: torch.Tensor,
                            pos_dev: torch.Tensor, prefix_k: Optional[torch.Tensor], prefix_v: Optional[torch.Tensor], P: int,
                            cache_k: torch.Tensor, cache_ks: torch.Tensor, cache_v: torch.Tensor, cache_vs: torch.Tensor,
-                           Smax: int, t_dev: torch.Tensor, single_launch: bool = True) -> torch.Tensor:
+                           Smax: int, t_dev: torch.Tensor, single_launch: bool = True,
+                           pages: Optional[torch.Tensor] = None) -> torch.Tensor:
     """partial_rope_append_kv + shared_prefix_attn without the RoPE launch and without q/k/v tensors, for up to
     16 branches: the q|k|v product `p` goes straight into the attention kernels.  Returns out [B,H,D].
     single_launch: everything in one launch (the workgroup that finishes last merges); otherwise two launches
-    whose result is bit-identical to the separate operators."""
+    whose result is bit-identical to the separate operators.  pages: int32 [>= B, >= Smax] page table (suffix row j of
+    branch b is cache row pages[b, j]); None = every branch reads its own rows."""
     lib = _lib.load()
     B = p.M
+    if pages is not None:
+        assert pages.is_cuda and pages.dtype == torch.int32 and pages.dim() == 2 and pages.stride(1) == 1
+        assert pages.shape[0] >= B and pages.shape[1] >= Smax
     assert B <= SMH_GEMV_MAX_M and p.n_total == (H + 2 * Hkv) * D and p.buf.dtype == torch.float32
     _need_gpu(p.buf, cache_k, cache_v, cache_ks, cache_vs, t_dev, pos_dev)
     if prefix_k is not None:
@@ -564,7 +600,8 @@ def shared_prefix_attn_qkv(p: PartialProduct, H: int, Hkv: int, D: int, cos: tor
     check(lib.smh_shared_prefix_attn_qkv(p.buf.data_ptr(), p.ksplit, out.data_ptr(), B, H, Hkv, D, cos.data_ptr(), sin.data_ptr(),
                                          pos_dev.data_ptr(), _ptr(prefix_k), _ptr(prefix_v), int(P),
                                          cache_k.data_ptr(), cache_ks.data_ptr(), cache_v.data_ptr(), cache_vs.data_ptr(), int(Smax),
-                                         t_dev.data_ptr(), int(bool(single_launch)), ws.data_ptr(), ws.numel(), _stream()),
+                                         t_dev.data_ptr(), _ptr(pages), pages.stride(0) if pages is not None else 0,
+                                         int(bool(single_launch)), ws.data_ptr(), ws.numel(), _stream()),
           "smh_shared_prefix_attn_qkv")
     return out
 
@@ -598,20 +635,80 @@ def flash_attn(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, B: int, L: int
                               n_kv_heads=H)
 
 
+def paged_prefix_attn(q: torch.Tensor, pages: torch.Tensor, lens: torch.Tensor, pool_k: torch.Tensor, pool_v: torch.Tensor,
+                      pool_ks: Optional[torch.Tensor] = None, pool_vs: Optional[torch.Tensor] = None, head_major: bool = False,
+                      prefix_k: Optional[torch.Tensor] = None, prefix_v: Optional[torch.Tensor] = None, P: int = 0,
+                      prefix_head_major: bool = False, cur_k: Optional[torch.Tensor] = None, cur_v: Optional[torch.Tensor] = None,
+                      lens_stride: int = 1, single_launch: bool = False) -> torch.Tensor:
+    """Tree attention: out[b,h] = softmax(q[b,h] . K_b^T / sqrt(D)) . V_b with K_b = prefix[:P] (shared) || the pool rows
+    pages[b, :lens[b]] || cur_k[b].  The rows are looked up inside the kernel (nothing is gathered or copied).
+    pool: fp16 [rows, Hkv, D] (or [Hkv, rows, D] with head_major) or Q4_0 rows int8 [rows, Hkv, 64] + scales fp16
+    [rows, Hkv, 2]; pages: int16 / int32 / int64 [B, L]; lens int32 on the device."""
+    lib = _lib.load()
+    _need_gpu(q, pages, lens, pool_k, pool_v)
+    assert q.is_contiguous() and q.dtype == torch.float16 and q.dim() == 3
+    B, H, D = q.shape
+    assert pages.dim() == 2 and pages.shape[0] >= B and pages.stride(1) == 1 and pages.dtype in (torch.int16, torch.int32, torch.int64)
+    assert lens.dtype == torch.int32
+    assert pool_k.is_contiguous() and pool_v.is_contiguous() and pool_k.shape == pool_v.shape
+    if pool_k.dtype == torch.float16:
+        fmt = SMH_KV_FP16
+        assert pool_k.dim() == 3 and pool_k.shape[2] == D
+        Hkv = pool_k.shape[0] if head_major else pool_k.shape[1]
+        rows = pool_k.shape[1] if head_major else pool_k.shape[0]
+        row_stride, head_stride = (D, rows * D) if head_major else (0, 0)
+    else:
+        fmt = SMH_KV_Q40
+        assert pool_k.dtype == torch.int8 and pool_ks is not None and pool_vs is not None and not head_major
+        assert pool_ks.dtype == torch.float16 and pool_vs.dtype == torch.float16 and pool_ks.is_contiguous() and pool_vs.is_contiguous()
+        assert pool_k.dim() == 3 and pool_k.shape[2] == 64
+        Hkv = pool_k.shape[1]
+        row_stride = head_stride = 0
+    assert H % Hkv == 0
+    p_row = p_head = 0
+    if prefix_k is not None and P > 0:
+        assert prefix_k.is_contiguous() and prefix_v.is_contiguous() and prefix_k.dtype == torch.float16 and prefix_k.dim() == 3
+        if prefix_head_major:
+            assert prefix_k.shape[0] == Hkv and P <= prefix_k.shape[1]
+            p_row, p_head = D, prefix_k.shape[1] * D
+        else:
+            assert prefix_k.shape[1] == Hkv and P <= prefix_k.shape[0]
+    else:
+        P = 0
+    if cur_k is not None:
+        assert cur_k.is_contiguous() and cur_v.is_contiguous() and cur_k.dtype == torch.float16 and cur_k.shape == (B, Hkv, D)
+    out = torch.empty_like(q)
+    one = bool(single_launch) and B * (H // Hkv) <= 128
+    ws = attn_qkv_workspace(q.device, B, H, P) if one else attn_workspace(q.device, B, H, P)
+    check(lib.smh_paged_prefix_attn(q.data_ptr(), out.data_ptr(), B, H, Hkv, D, _ptr(prefix_k) if P else None, _ptr(prefix_v) if P else None,
+                                    int(P), p_row, p_head, fmt, pool_k.data_ptr(), pool_v.data_ptr(), _ptr(pool_ks), _ptr(pool_vs),
+                                    row_stride, head_stride, pages.data_ptr(), pages.element_size(), pages.stride(0),
+                                    lens.data_ptr(), int(lens_stride), _ptr(cur_k), _ptr(cur_v), int(one), ws.data_ptr(), ws.numel(), _stream()),
+          "smh_paged_prefix_attn")
+    return out
+
+
+def page_fork(table: torch.Tensor, origin: int, curr: int, forks: int, n: int) -> None:
+    """table[curr : curr + forks, :n] = table[origin, :n] for an int32 page table [rows, stride]: the fork of a branch
+    when its rows are shared through the table instead of copied."""
+    lib = _lib.load()
+    _need_gpu(table)
+    assert table.dtype == torch.int32 and table.dim() == 2 and table.is_contiguous()
+    check(lib.smh_page_fork(table.data_ptr(), table.shape[0], table.shape[1], int(origin), int(curr), int(forks), int(n), _stream()),
+          "smh_page_fork")
+
+
 def page_flash_attn(p: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, P: int, B: int, L: int, H: int,
                     D: int) -> torch.Tensor:
     """Drop-in for triton_kernels.page_flash_attn (triton_kernels.py:764-789): branch b attends to the L pages
-    p[b, :] of the page pools k/v [H,P,D].  p [B,L] integer page ids, q [B,H,D] -> [B,H,D] fp16.  The pages of
-    each branch are gathered (one indexed copy) into the token-major suffix layout and attended to by the
-    decode attention kernel."""
+    p[b, :] of the page pools k/v [H,P,D].  p [B,L] integer page ids, q [B,H,D] -> [B,H,D] fp16.  The pools are read
+    where they lie, through the page table (no gather, no layout copy); scores and the softmax state are fp32 (the
+    reference keeps them in fp16)."""
     _need_gpu(p, q, k, v)
     assert p.shape == (B, L) and q.shape == (B, H, D) and k.shape == (H, P, D) and v.shape == (H, P, D)
-    idx = p.to(torch.int64)
-    kt = k.transpose(0, 1)[idx].contiguous()              # [B, L, H, D]
-    vt = v.transpose(0, 1)[idx].contiguous()
-    lens = torch.full((B,), L, dtype=torch.int32, device=q.device)
-    return shared_prefix_attn(q.contiguous(), None, None, 0, suffix_k=kt, suffix_v=vt, Smax=L, lens=lens, lens_stride=1,
-                              n_kv_heads=H)
+    lens = torch.full((1,), L, dtype=torch.int32, device=q.device)
+    return paged_prefix_attn(q.contiguous(), p if p.stride(1) == 1 else p.contiguous(), lens, k.contiguous(), v.contiguous(),
+                             head_major=True, lens_stride=0)
 
 
 def chunk_attn(p: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, P: int, B: int, L: int, H: int,
@@ -622,19 +719,14 @@ def chunk_attn(p: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tenso
     to page_flash_attn whenever p[b, :offset] == arange(offset).  The reference's two kernels do not combine
     their softmax states correctly (base-2 against natural maxima, the first kernel's output not reloaded), so
     this follows the docstring of the reference function, not its output.  The shared chunk is the prefix of the
-    decode attention kernel (read once for all branches), the own pages are gathered into its suffix layout."""
+    decode attention kernel (staged once in LDS for all branches, read from the pool in place), the own pages are looked
+    up through the page table inside the kernel."""
     _need_gpu(p, q, k, v)
     assert p.shape == (B, L) and q.shape == (B, H, D) and k.shape == (H, P, D) and v.shape == (H, P, D)
     assert 0 <= offset <= L and offset <= P
-    pk = k[:, :offset].transpose(0, 1).contiguous() if offset else None     # [offset, H, D]
-    pv = v[:, :offset].transpose(0, 1).contiguous() if offset else None
-    S = L - offset
-    if S:
-        idx = p[:, offset:].to(torch.int64)
-        kt = k.transpose(0, 1)[idx].contiguous()          # [B, S, H, D]
-        vt = v.transpose(0, 1)[idx].contiguous()
-        lens = torch.full((B,), S, dtype=torch.int32, device=q.device)
-    else:
-        kt = vt = lens = None
-    return shared_prefix_attn(q.contiguous(), pk, pv, offset, suffix_k=kt, suffix_v=vt, Smax=S, lens=lens,
-                              lens_stride=1, n_kv_heads=H)
+    k, v = k.contiguous(), v.contiguous()
+    p = p if p.stride(1) == 1 else p.contiguous()
+    lens = torch.full((1,), L - offset, dtype=torch.int32, device=q.device)
+    own = p[:, offset:] if offset < L else p[:, :1]                    # a view: same table, first own page
+    return paged_prefix_attn(q.contiguous(), own, lens, k, v, head_major=True, prefix_k=k, prefix_v=v, P=offset,
+                             prefix_head_major=True, lens_stride=0)
