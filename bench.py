@@ -135,6 +135,53 @@ def matmul_roofline(torch, model, M, iters):
             "tflops": flops / (ms * 1e-3) / 1e12}
 
 
+SWEEP_SHAPES = ((4096, 4096), (11008, 4096), (4096, 11008), (32128, 4096))     # (N, K); 32128 = vocab 32016 padded to 251 x 128 columns
+
+
+def matmul_sweep(torch, iters=3):
+    """BASELINE configs[1]: the Q4_0 matmul kernel alone at M = 1, 10, 100 on every CodeLlama-7B shape (the vocabulary
+    projection zero-padded from 32016 to 32128 columns, the next multiple of 128 - the reference's format cannot hold 32016).
+    Each point cycles through distinct weight copies that together exceed the 256 MB Infinity Cache, launched back to back
+    in one HIP graph and timed with HIP events on its stream; weights in the tiled streaming layout, as the model holds
+    them.  Bytes per launch: packed nibbles + scales + activations + fp16 outputs."""
+    from spec_mcts_amd import kernels as K
+    dev = torch.device("cuda:0")
+    out = []
+    for N, Kd in SWEEP_SHAPES:
+        wbytes = N * Kd // 2 + N * Kd // 32
+        copies = max(2, -(-300_000_000 // wbytes))
+        tiled = []
+        for _ in range(copies):
+            w = torch.randint(-128, 128, (Kd * N // 128, 64), device=dev, dtype=torch.int16).to(torch.int8)
+            s = (torch.rand((Kd * N // 64,), device=dev) * 0.01).half()
+            tiled.append(K.tile_q40(w, s, Kd, N))
+            del w, s
+        for M in (1, 10, 100):
+            x = torch.randn((M, Kd), device=dev).half()
+
+            def run():
+                for t in tiled:
+                    K.matmul_q40_partial(x, [t])
+
+            run()
+            torch.cuda.synchronize()
+            graph = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(graph):
+                run()
+            for _ in range(3):
+                graph.replay()
+            us = time_region(torch, graph.replay, iters) * 1e3 / copies
+            nbytes = q40_bytes(M, N, Kd)
+            flops = 2.0 * M * N * Kd
+            out.append({"M": M, "N": N, "K": Kd, "us": round(us, 2), "bytes": nbytes, "gbs": round(nbytes / us / 1e3, 1),
+                        "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "tflops": round(flops / us / 1e6, 1),
+                        "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "weight_copies": copies})
+            del graph
+        del tiled
+        torch.cuda.empty_cache()
+    return out
+
+
 def attention_roofline(torch, iters=5, copies=3):
     """The shared-prefix decode attention alone on the reference's tree-attention shape: 64 branches, 32 heads,
     head_dim 128, one 1024-token fp16 prefix shared by all branches, ragged suffixes of 0..256 rows per branch held
@@ -223,6 +270,7 @@ def main():
     ap.add_argument("--norm-in-rows", type=int, default=-1, help="RMSNorm inside the matmul up to this many rows (comparison runs; default: the model's)")
     ap.add_argument("--batches", default="", help="comma-separated subset of 1,10,100 to run (a partial run is not a valid result)")
     ap.add_argument("--no-roofline", action="store_true", help="skip the matmul roofline legs (profiling runs)")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the per-shape matmul sweep and the eager-loop timing")
     ap.add_argument("--roofline-only", type=int, default=0, metavar="M",
                     help="profiling aid: run only the matmul roofline leg at batch M (eager launches, one pass) after a 1 GiB "
                          "device copy that calibrates the profiler's byte counters, and print that leg's numbers")
@@ -287,6 +335,18 @@ def main():
         dt = time.perf_counter() - t0
         by_batch[B] = {"tok_s": B * steps / dt, "ms_per_step": dt / steps * 1e3}
         del dec
+        if not a.no_sweep:
+            # the same steps issued launch by launch from Python, as mcts.search's model(tokens, pos) calls would issue them
+            dec = GraphDecoder(model, B, use_graph=False)
+            dec.prefill(prompt)
+            dec.decode(3)
+            torch.cuda.synchronize()
+            n_eager = min(20, max_seq - 5)
+            t0 = time.perf_counter()
+            dec.decode(n_eager)
+            torch.cuda.synchronize()
+            by_batch[B]["eager_ms_per_step"] = (time.perf_counter() - t0) / n_eager * 1e3
+            del dec
 
     # per-step algorithmic HBM bytes: Q4 linears + fp16 lm_head + shared prefix KV (once) + suffix KV (Q4 rows)
     lin_bytes = sum(q40_bytes(0, n, k_in) for k_in, segs in step_matmuls(model) for _, n in segs)
@@ -335,6 +395,8 @@ def main():
                        "suffixes of 0..256 rows (the two launches of one call)",
              "bound": "hbm", "achieved": round(att["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
              "frac": round(att["gbs"] / HBM_PEAK_GBS, 4), "avg_call_us": round(att["us"], 2), "bytes_per_call": att["bytes"], "traffic": ATTN_TRAFFIC_BYTES_PER_CALL})
+    if not a.no_sweep and a.arch == "7b":
+        result["matmul_sweep"] = matmul_sweep(torch)
     if not a.no_cpu_baseline:
         cpu, cores, raw = cpu_baseline(torch, args_kw)
         result["cpu_baseline"] = {"value": round(cpu.get(head_b, cpu.get(max(cpu), 0.0)), 4), "unit": "tok/s", "cores": cores, "kind": "port",

@@ -184,6 +184,10 @@ int smh_rope(void *q, void *k, int S, int H, int Hkv, int D, const void *cos_tab
              const void *sin_tab, int pos0, smh_stream_t stream);
 int smh_kv_fork(void *cache, void *cache_s, int Bmax, long row_bytes, long row_scales,
                 int origin, int curr, int forks, smh_stream_t stream);
+/* smh_set_step: state[0] = pos, state[1] = t (int32 on the device), the `start_pos` of Transformer.forward
+ * (hf_model_q40_kv_shared.py:492) and the suffix row start_pos - prompt length (:333-336) that the decode kernels read
+ * through pos_dev / t_dev.  The values travel as kernel arguments: no host buffer, no copy, nothing the host waits for. */
+int smh_set_step(int32_t *state, int pos, int t, smh_stream_t stream);
 
 /* ---- fp16 vocabulary projection and embedding -------------------------------------------------------
  * smh_f16_linear: out[M, N] = x[M, K] . w[N, K]^T, fp16 operands, fp32 accumulation, one rounding to fp16: the

@@ -48,6 +48,7 @@ SIGNATURES = {
     "smh_sample_topk": (c_int, [_P, c_int, c_int, c_long, c_float, c_int, _P, _P, _P]),
     "smh_rope_append_kv": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, c_int, _P, _P]),
     "smh_rope": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, _P]),
+    "smh_set_step": (c_int, [_P, c_int, c_int, _P]),
     "smh_kv_fork": (c_int, [_P, _P, c_int, c_long, c_long, c_int, c_int, c_int, _P]),
     "smh_f16_linear": (c_int, [_P, c_int, c_int, c_long, _P, c_int, _P, c_long, _P]),
     "smh_embedding": (c_int, [_P, c_int, _P, c_int, c_int, _P, _P]),

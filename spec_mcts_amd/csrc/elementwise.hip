@@ -455,6 +455,19 @@ extern "C" int smh_rope(void *q, void *k, int S, int H, int Hkv, int D, const vo
     return launch_status();
 }
 
+namespace smh {
+__global__ void set_step_kernel(int32_t *state, int pos, int t) {
+    state[0] = pos;
+    state[1] = t;
+}
+}  // namespace smh
+
+extern "C" int smh_set_step(int32_t *state, int pos, int t, smh_stream_t stream) {
+    SMH_REQUIRE(state != nullptr && pos >= 0 && t >= 0, "smh_set_step: state=%p pos=%d t=%d", (void *)state, pos, t);
+    hipLaunchKernelGGL(smh::set_step_kernel, dim3(1), dim3(1), 0, (hipStream_t)stream, state, pos, t);
+    return smh::launch_status();
+}
+
 extern "C" int smh_kv_fork(void *cache, void *cache_s, int Bmax, long row_bytes, long row_scales,
                            int origin, int curr, int forks, smh_stream_t stream) {
     using namespace smh;

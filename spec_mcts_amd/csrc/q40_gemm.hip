@@ -29,6 +29,10 @@
 
 namespace smh {
 
+// most K-slices of a launch = SMH_GEMM_KSCAP / rows (every slice leaves an fp32 slab of rows x columns)
+#ifndef SMH_GEMM_KSCAP
+#define SMH_GEMM_KSCAP 1600
+#endif
 constexpr int GEMM_BM = 128;
 constexpr int GEMM_WAVES = 4;
 constexpr int GEMM_THREADS = GEMM_WAVES * 64;
@@ -379,7 +383,7 @@ void gemm_fill_plan(MatmulParams &p) {
     constexpr int capacity = 512;
     int ks = (int)(capacity / 2 / tiles);
     if (ks < 1 || tiles * ks < 200) ks = (int)(capacity / tiles);
-    int cap = 1600 / (p.M > 0 ? p.M : 1);
+    int cap = SMH_GEMM_KSCAP / (p.M > 0 ? p.M : 1);
     if (cap > SMH_MAX_KSPLIT) cap = SMH_MAX_KSPLIT;
     if (ks > cap) ks = cap;
     if (ks > steps / GEMM_STAGES) ks = steps / GEMM_STAGES;

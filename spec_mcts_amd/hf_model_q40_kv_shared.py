@@ -284,7 +284,6 @@ class Transformer(nn.Module):
                                               params.rope_theta)
         self._rope_tables = None      # (cos, sin) fp16 [T, 64] on the device
         self._step_state = None       # int32 [2] on the device: (position, suffix index t)
-        self._step_host = None
         self.fused = True             # fused decode-layer launches; False runs module by module
         self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
         self.fused_sampler = True          # generate(): temperature / top-k / draw as one kernel instead of five torch ops
@@ -314,11 +313,8 @@ class Transformer(nn.Module):
         """Publish (position, suffix index) to the device for the decode kernels."""
         if self._step_state is None or self._step_state.device != device:
             self._step_state = torch.zeros(2, dtype=torch.int32, device=device)
-            self._step_host = torch.zeros(2, dtype=torch.int32).pin_memory() if device.type == "cuda" else torch.zeros(2, dtype=torch.int32)
         prompt_len = self.layers[0].attention.cache_prompt_len
-        self._step_host[0] = start_pos
-        self._step_host[1] = start_pos - prompt_len
-        self._step_state.copy_(self._step_host, non_blocking=False)
+        K.set_step(self._step_state, start_pos, start_pos - prompt_len)      # a one-thread launch: nothing the host waits for
         return self._step_state[0:1], self._step_state[1:2]
 
     # -- the hot path ----------------------------------------------------------------------------

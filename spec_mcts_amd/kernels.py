@@ -473,6 +473,13 @@ def rope_append_kv(q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cos: torch
                                  _stream()), "smh_rope_append_kv")
 
 
+def set_step(state: torch.Tensor, pos: int, t: int) -> None:
+    """state[0] = pos, state[1] = t on the device, asynchronously (the values are kernel arguments)."""
+    _need_gpu(state)
+    assert state.dtype == torch.int32 and state.numel() >= 2 and state.is_contiguous()
+    check(_lib.load().smh_set_step(state.data_ptr(), int(pos), int(t), _stream()), "smh_set_step")
+
+
 def kv_fork(cache: torch.Tensor, cache_s: torch.Tensor, Bmax: int, origin: int, curr: int, forks: int) -> None:
     """Copy branch `origin`'s Q4_0 cache rows to branches curr..curr+forks-1."""
     lib = _lib.load()
