@@ -51,6 +51,11 @@ const char *smh_last_error_string(void);
  * rounding: scale = fp16(absmax/7), code = rint(fp16(x/scale)), 0/0 -> 0. groups must be even. */
 int smh_q40_dequant(const void *w, const void *s, void *out, long rows, smh_stream_t stream);
 int smh_q40_quantize(const void *in, void *w, void *s, long groups, smh_stream_t stream);
+/* smh_q40_quantize_f32: the same quantiser for checkpoint weights held in fp32 or bfloat16 (fp16_to_int4.py:169-184 runs
+ * quantize_q40 on the checkpoint's own dtype; HF CodeLlama shards are bfloat16).  `in` holds the values widened to fp32;
+ * src_bf16 != 0 says they were bfloat16.  torch's roundings for those types: scale = fp16(T(absmax / 7)) with T the source
+ * type, code = rint(x / scale) with the quotient in fp32. */
+int smh_q40_quantize_f32(const void *in, int src_bf16, void *w, void *s, long groups, smh_stream_t stream);
 
 /* ---- Q4_0 matmul ---------------------------------------------------------------------------
  * c[M,N] = a[M,K] . deq(b_w, b_s)[K,N], fp16 operands, fp32 accumulation, one fp16 rounding;

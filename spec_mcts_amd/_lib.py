@@ -23,6 +23,7 @@ SIGNATURES = {
     "smh_last_error_string": (c_char_p, []),
     "smh_q40_dequant": (c_int, [_P, _P, _P, c_long, _P]),
     "smh_q40_quantize": (c_int, [_P, _P, _P, c_long, _P]),
+    "smh_q40_quantize_f32": (c_int, [_P, c_int, _P, _P, c_long, _P]),
     "smh_q40_matmul_workspace_bytes": (c_size_t, [c_int, c_int]),
     "smh_q40_gemv": (c_int, [_P, c_int, c_int, c_long, _P, _P, c_int, _P, c_long, c_int, _P, c_long, _P, c_size_t, _P]),
     "smh_q40_gemm": (c_int, [_P, c_int, c_int, c_long, _P, _P, c_int, _P, c_long, c_int, _P, c_long, _P, c_size_t, _P]),

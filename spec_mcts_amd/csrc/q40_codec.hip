@@ -100,6 +100,56 @@ __global__ __launch_bounds__(256) void q40_quantize_kernel(const u32x4 *__restri
     }
 }
 
+// The same quantiser for checkpoint weights held in fp32 or bfloat16 (passed widened to fp32, which is exact).  torch's
+// arithmetic for those types (fp16_to_int4.py:60-70 run on such a tensor): wmax / 7.0 is rounded to the tensor's own
+// type (fp32, or bfloat16) and then to fp16; w / scale promotes to fp32, so the quotient is NOT rounded to fp16 before
+// round-half-even; 0 / 0 -> NaN -> code 0.  SRC_BF16 selects the intermediate bfloat16 rounding of the scale.
+__device__ __forceinline__ float round_to_bf16(float x) {
+    uint32_t u = __builtin_bit_cast(uint32_t, x);
+    if ((u & 0x7F800000u) == 0x7F800000u) return x;                  // inf / nan stay
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return __builtin_bit_cast(float, u & 0xFFFF0000u);
+}
+template <bool SRC_BF16>
+__global__ __launch_bounds__(256) void q40_quantize_f32_kernel(const f4 *__restrict__ in, uint8_t *__restrict__ w,
+                                                               half_t *__restrict__ s, long groups) {
+    long t = (long)blockIdx.x * blockDim.x + threadIdx.x;
+    long g = t >> 3;
+    int c = (int)(t & 7);
+    bool live = g < groups;
+    f4 a = live ? in[2 * t] : f4{0.f, 0.f, 0.f, 0.f}, b = live ? in[2 * t + 1] : f4{0.f, 0.f, 0.f, 0.f};
+    const float x[8] = {a[0], a[1], a[2], a[3], b[0], b[1], b[2], b[3]};
+    float amax = 0.f;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) amax = fmaxf(amax, fabsf(x[j]));
+#pragma unroll
+    for (int o = 4; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+    float q7 = amax / 7.0f;
+    if (SRC_BF16) q7 = round_to_bf16(q7);
+    const half_t scale_h = (half_t)q7;
+    const float scale = (float)scale_h;
+    uint32_t nib = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const float qf = x[j] / scale;
+        const int code = (qf == qf) ? (int)__builtin_rintf(qf) : 0;
+        nib |= (uint32_t)(code & 15) << (4 * j);
+    }
+    uint32_t other = (uint32_t)__shfl_xor((int)nib, 8, 64);
+    if (!live) return;
+    if (c == 0) s[g] = scale_h;
+    if ((g & 1) == 0) {
+        uint32_t hi = nib, lo = other;
+        uint32_t b0 = 0, b1 = 0;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            b0 |= ((((hi >> (4 * j)) & 15) << 4) | ((lo >> (4 * j)) & 15)) << (8 * j);
+            b1 |= ((((hi >> (4 * j + 16)) & 15) << 4) | ((lo >> (4 * j + 16)) & 15)) << (8 * j);
+        }
+        *reinterpret_cast<u32x2 *>(w + (g >> 1) * 64 + c * 8) = u32x2{b0, b1};
+    }
+}
+
 // One thread per output dword of the tiled layout (q40_matmul.hpp): 1024 nibble dwords + 64 scale dwords per tile.
 __global__ __launch_bounds__(256) void q40_tile_kernel(const uint8_t *__restrict__ w, const half_t *__restrict__ s,
                                                        int K, int N, uint32_t *__restrict__ tiled, long tiles) {
@@ -180,5 +230,17 @@ extern "C" int smh_q40_quantize(const void *in, void *w, void *s, long groups, s
     dim3 grid((unsigned)((threads + 255) / 256));
     hipLaunchKernelGGL(q40_quantize_kernel, grid, dim3(256), 0, (hipStream_t)stream,
                        (const u32x4 *)in, (uint8_t *)w, (half_t *)s, groups);
+    return launch_status();
+}
+
+extern "C" int smh_q40_quantize_f32(const void *in, int src_bf16, void *w, void *s, long groups, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(groups >= 0 && (groups & 1) == 0, "smh_q40_quantize_f32: groups=%ld must be even", groups);
+    if (groups == 0) return 0;
+    SMH_REQUIRE(in && w && s && ((uintptr_t)in & 15) == 0, "smh_q40_quantize_f32: null or misaligned pointer");
+    long threads = groups * 8;
+    dim3 grid((unsigned)((threads + 255) / 256));
+    if (src_bf16) hipLaunchKernelGGL(q40_quantize_f32_kernel<true>, grid, dim3(256), 0, (hipStream_t)stream, (const f4 *)in, (uint8_t *)w, (half_t *)s, groups);
+    else hipLaunchKernelGGL(q40_quantize_f32_kernel<false>, grid, dim3(256), 0, (hipStream_t)stream, (const f4 *)in, (uint8_t *)w, (half_t *)s, groups);
     return launch_status();
 }

@@ -295,6 +295,7 @@ class Transformer(nn.Module):
         self.norm_in_max_rows = 2          # ... up to this many rows: at 10 rows the matmul's longer prologue costs more than it saves
         self._norm_in_ok = {}
         self.attn_from_qkv = True          # up to 16 branches the attention takes the wq|wk|wv product itself, in one launch
+        self._q40_output = None            # quantize_lm_head(): (w, s, padded vocab) of a Q4_0 vocabulary projection
         self.paged_kv = True               # fork = a copy of page ids: forked branches share their ancestor's suffix rows
         self._page_table = None            # int32 [max_batch_size, max_seq_len]: cache row that holds position j of branch b
         self._forked = False               # a fork happened since the last resetSeq (until then every branch reads its own rows)
@@ -330,7 +331,7 @@ class Transformer(nn.Module):
         for layer in self.layers:
             h = layer(h, start_pos, freqs, None, step_state=step_state, pages=pages)
         h = self.norm(h)
-        return K.f16_linear(h, self.output.weight)
+        return self._lm_head(h)
 
     def _forward_fused(self, tokens: torch.Tensor, start_pos: int, step_state):
         """Same arithmetic as the module-by-module path, with the launches of a layer fused:
@@ -405,7 +406,34 @@ class Transformer(nn.Module):
                 act = K.partial_silu_mul(gu)
                 pending = K.matmul_q40_partial(act, [ff.w2.operand(tiled)])
         _, hn = K.partial_rmsnorm(pending, h, self.norm.weight, self.norm.eps, want_h=False)
-        return K.f16_linear(hn.view(bsz, seqlen, p.dim), self.output.weight)
+        return self._lm_head(hn.view(bsz, seqlen, p.dim))
+
+    def quantize_lm_head(self, enable: bool = True):
+        """Optional: run the vocabulary projection as a Q4_0 matmul.  The reference keeps `output` in fp16 because its format
+        needs out_features % 128 == 0 and the vocabulary has 32016 entries (hf_model_q40_kv_shared.py:484); here the weight is
+        zero-padded to the next multiple of 128 rows (32128), quantised like every other linear (the transpose, groups of 64
+        along the outputs) and the padded logits are cut off.  69.7 MB instead of 262 MB per step; logits differ from the
+        fp16 projection by the quantisation error of the weight, so this is off unless asked for."""
+        if not enable:
+            self._q40_output = None
+            return
+        W = self.output.weight
+        K._need_gpu(W)
+        vocab, dim = W.shape
+        padded = (vocab + 127) // 128 * 128
+        Wp = torch.zeros((padded, dim), dtype=DTYPE, device=W.device)
+        Wp[:vocab] = W.detach().to(DTYPE)
+        w, s = K.quantize_q40(Wp.t().contiguous(), GROUP_SIZE)
+        self._q40_output = (w, s, padded)
+
+    def _lm_head(self, hn: torch.Tensor) -> torch.Tensor:
+        """hn [..., dim] -> logits fp16 [..., vocab]"""
+        if self._q40_output is None:
+            return K.f16_linear(hn, self.output.weight)
+        w, s, padded = self._q40_output
+        dim = hn.shape[-1]
+        logits = K.matmul_q40(hn.reshape(-1, dim), w, s, (dim, padded))
+        return logits.view(hn.shape[:-1] + (padded,))[..., : self.vocab_size]
 
     def _pages(self, device):
         """The page table the attention kernels read suffix rows through, or None while no branch shares rows."""

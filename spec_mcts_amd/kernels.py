@@ -359,11 +359,30 @@ def q_int40(w: torch.Tensor, group_size: int = GROUP_SIZE) -> Tuple[torch.Tensor
     return q, s
 
 
+def q_int40_wide(w: torch.Tensor, group_size: int = GROUP_SIZE) -> Tuple[torch.Tensor, torch.Tensor]:
+    """bfloat16 or fp32 -> Q4_0 on the GPU with the roundings torch's CPU quantiser has for those types (scale through
+    the tensor's own type, quotient in fp32): what converting a bfloat16 HF checkpoint on the host produces."""
+    lib = _lib.load()
+    assert group_size == GROUP_SIZE
+    _need_gpu(w)
+    assert w.dtype in (torch.bfloat16, torch.float32)
+    wide = w.contiguous().float()
+    n = wide.numel()
+    assert n % 128 == 0
+    q = torch.empty((n // 128, 64), device=w.device, dtype=torch.int8)
+    s = torch.empty((n // 64, 1), device=w.device, dtype=torch.float16)
+    check(lib.smh_q40_quantize_f32(wide.data_ptr(), int(w.dtype == torch.bfloat16), q.data_ptr(), s.data_ptr(), n // 64, _stream()),
+          "smh_q40_quantize_f32")
+    return q, s
+
+
 def quantize_q40(w: torch.Tensor, group_size: int = GROUP_SIZE) -> Tuple[torch.Tensor, torch.Tensor]:
-    """reference: triton_kernels.py:12-41.  fp16 GPU tensors use the HIP kernel; anything else
-    (checkpoint conversion of bf16/fp32 weights on the host) uses the torch formulation."""
+    """reference: triton_kernels.py:12-41.  GPU tensors use the HIP kernels (fp16, or bfloat16 / fp32 with torch's
+    roundings for those types); host tensors use the torch formulation."""
     if w.is_cuda and w.dtype == torch.float16:
         return q_int40(w, group_size)
+    if w.is_cuda and w.dtype in (torch.bfloat16, torch.float32):
+        return q_int40_wide(w, group_size)
     return quantize_q40_torch(w, group_size)
 
 

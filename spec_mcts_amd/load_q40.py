@@ -10,7 +10,7 @@ from typing import Dict, Optional, Union
 
 import torch
 
-from .fp16_to_int4 import remap_state_dict
+from .fp16_to_int4 import _is_quantised_key, iter_checkpoint_tensors, quantize_linear_weight_gpu, remap_state_dict
 from .hf_model_q40_kv_shared import ModelArgs, Transformer
 
 DTYPE = torch.float16
@@ -49,6 +49,33 @@ def load_q40(model_file: Union[str, Dict[str, torch.Tensor]], params: Optional[M
     plain = {k: v for k, v in model_dict.items() if k.split(".")[-1] not in ("w", "s", "shape")}
     model.load_state_dict(plain, strict=False, assign=True)
     assign_q40(model, model_dict, device)
+    model.to(device=device, dtype=DTYPE)
+    model.eval()
+    return model
+
+
+def load_hf_q40(model_dir: str, params: Optional[ModelArgs] = None, device: str = "cuda:0", model_cls=None) -> Transformer:
+    """Build the Q4_0 model straight from an unconverted HF checkpoint directory (fp16 / bf16 shards): every linear is
+    sent to the GPU, quantised there and assigned, one tensor at a time, so the 16-bit weights are never held as a whole
+    on the host or on the device (a 70B-class checkpoint is ~140 GB in bf16, ~36 GB as Q4_0).  Equivalent to
+    fp16_to_int4.convert_checkpoint followed by load_q40."""
+    if model_cls is None:
+        model_cls = Transformer
+    model = model_cls(params if params is not None else ModelArgs())
+    plain: Dict[str, torch.Tensor] = {}
+    seen = set()
+    for name, v in iter_checkpoint_tensors(model_dir):
+        if _is_quantised_key(name):
+            _, i, block, lname, _ = name.split(".")
+            lin = getattr(getattr(model.layers[int(i)], block), lname)
+            lin.w, lin.s, lin.shape = quantize_linear_weight_gpu(v, device)
+            seen.add((int(i), block, lname))
+        else:
+            plain[name] = v.to(device=device, dtype=DTYPE) if v.is_floating_point() else v
+    missing = [(i, b, n) for i in range(len(model.layers)) for b, n in LINEARS if (i, b, n) not in seen]
+    if missing:
+        raise ValueError(f"checkpoint lacks {len(missing)} linear weights, first: layers.{missing[0][0]}.{missing[0][1]}.{missing[0][2]}")
+    model.load_state_dict(plain, strict=False, assign=True)
     model.to(device=device, dtype=DTYPE)
     model.eval()
     return model
