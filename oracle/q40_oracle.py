@@ -28,6 +28,9 @@ live in tests/test_oracle_*.py):
   topk_probs / sample_topk       candidate values against torch.topk, probabilities against F.softmax of those values,
                                  k = 1 is the argmax, k = vocab with a huge temperature is uniform; the draw against a
                                  brute-force scan in float64 and, over many uniform numbers, its frequencies against p.
+  sample_topk_counts / tree_fork the draws against sample_topk row by row; the bookkeeping against hand-computed known answers
+                                 (every row of a small tree written out), conservation of the multiplicities while rows are
+                                 left, truncation when they run out, dead branches untouched, histories of forked rows.
   detect_terminal                a scalar walk over token streams written as plain if / else (tests), known answers:
                                  the sequence fed in order ends at its last token, end-of-sequence ends at once, a
                                  wrong token resets, a repeated first token does NOT restart the match (the reference's
@@ -190,6 +193,56 @@ def sample_topk(logits: torch.Tensor, temperature: float, top_k: int, u: torch.T
     hit = cdf > target
     j = torch.where(hit.any(-1), hit.float().argmax(-1), torch.full((p.shape[0],), p.shape[1] - 1))
     return order.gather(1, j.unsqueeze(1))[:, 0]
+
+
+def sample_topk_counts(logits: torch.Tensor, temperature: float, top_k: int, counts, u: torch.Tensor) -> torch.Tensor:
+    """counts[r] draws per row (mcts.py:128: torch.multinomial(probs[r], num_samples=output_counts[1, r], replacement=True)
+    followed by the gather of :129), each an inverse-CDF draw as in sample_topk; row r uses u[sum(counts[:r]) ...]."""
+    out = []
+    off = 0
+    for r in range(logits.shape[0]):
+        n = int(counts[r])
+        if n:
+            out.append(sample_topk(logits[r:r + 1].expand(n, -1), temperature, top_k, u[off:off + n]))
+        off += n
+    return torch.cat(out) if out else torch.zeros(0, dtype=torch.int64)
+
+
+def tree_fork(draws: torch.Tensor, output_counts: torch.Tensor, alive: torch.Tensor, curr_batch: int, batch_size: int,
+              results: torch.Tensor, t: int, pages: Optional[torch.Tensor] = None, n_rows: int = 0):
+    """The per-branch loop of the tree sampler's expansion step (mcts.py:127-152) and the masking of :160, on host tensors,
+    in place.  draws: the tokens the live branches sampled, branch after branch (output_counts[1, i] each).  Returns
+    (new curr_batch, origin list: the branch each row was forked from in this call, else -1)."""
+    origin = [-1] * batch_size
+    off = 0
+    segs = []
+    for i in range(curr_batch):
+        n = int(output_counts[1, i])
+        segs.append(draws[off:off + n])
+        off += n
+    for i in range(curr_batch):
+        next_token = segs[i]
+        if next_token.numel() == 0:
+            continue
+        unique_idx, counts = torch.unique(next_token, return_counts=True, dim=0)      # ascending (:131)
+        if alive[i]:                                                                 # :135-138
+            output_counts[0, i] = unique_idx[0]
+            output_counts[1, i] = counts[0]
+            results[i, t] = unique_idx[0]
+        forks = min(len(counts) - 1, batch_size - curr_batch)                        # :141-142
+        if forks > 0 and curr_batch < batch_size and alive[i]:                       # :143
+            for j in range(forks):                                                   # model.fork(i, curr_batch, forks) + :146-150
+                r = curr_batch + j
+                origin[r] = i
+                if pages is not None:
+                    pages[r, :n_rows] = pages[i, :n_rows]
+                results[r] = results[i]
+                output_counts[0, r] = unique_idx[1 + j]
+                output_counts[1, r] = counts[1 + j]
+                results[r, t] = unique_idx[1 + j]
+            curr_batch += forks
+    results[:, t] *= alive.to(results.dtype)                                         # :160
+    return curr_batch, origin
 
 
 def detect_terminal(token: torch.Tensor, state: torch.Tensor, terminal_seq: torch.Tensor, eos: int = 2):

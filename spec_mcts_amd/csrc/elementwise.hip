@@ -264,8 +264,11 @@ __device__ __forceinline__ void sample_pick_bin(int *bins, int want, int *out_bi
     __syncthreads();
 }
 
+// counts == nullptr: one draw per row, uniform[row] -> out[row].  Otherwise row r makes counts[r] draws with replacement from
+// its candidates, with the uniform numbers (and into the slots of out) that start at counts[0] + ... + counts[r-1].
 __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restrict__ logits, int vocab, long ld, float temperature,
-                                                           int top_k, const float *__restrict__ uniform, int64_t *__restrict__ out) {
+                                                           int top_k, const float *__restrict__ uniform, int64_t *__restrict__ out,
+                                                           const int32_t *__restrict__ counts) {
     __shared__ int bins[256];
     __shared__ int s_bin, s_above, s_count;
     __shared__ int scan[1024];
@@ -360,11 +363,105 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
         cdf[tid] += v;
         __syncthreads();
     }
-    const float target = uniform[blockIdx.x] * cdf[k - 1];
+    long first = blockIdx.x;
+    int draws = 1;
+    if (counts != nullptr) {
+        first = 0;
+        for (int r = 0; r < (int)blockIdx.x; ++r) first += counts[r];
+        draws = counts[blockIdx.x];
+    }
     if (tid < k) {
         const float before = tid == 0 ? 0.f : cdf[tid - 1];
-        // first candidate whose cumulative probability exceeds the target (the last one if rounding leaves none)
-        if ((before <= target && target < cdf[tid]) || (tid == k - 1 && target >= cdf[tid])) out[blockIdx.x] = o_idx[tid];
+        for (int j = 0; j < draws; ++j) {
+            const float target = uniform[first + j] * cdf[k - 1];
+            // first candidate whose cumulative probability exceeds the target (the last one if rounding leaves none)
+            if ((before <= target && target < cdf[tid]) || (tid == k - 1 && target >= cdf[tid])) out[first + j] = o_idx[tid];
+        }
+    }
+}
+
+// The bookkeeping of one step of the tree sampler (mcts.py:127-152) for all branches in one launch, one workgroup.
+//   draws   the tokens every live branch drew this step (sample_topk_kernel with counts): branch i owns cnt[i] of them,
+//           in branch order
+//   per branch i < *curr_b, in order: its distinct tokens in ascending order with their multiplicities (torch.unique,
+//           :131); if the branch is alive the smallest stays on row i with its multiplicity (:135-138) and each further
+//           distinct token opens a new row while rows are left (:141-150): the new row takes the origin's token
+//           history, the token, its multiplicity, and - instead of a copy of K/V rows - the origin's page ids of the
+//           suffix rows written so far.  Dead branches change nothing.  Then the step's column of every dead row is
+//           zeroed (:160).
+//   tok / cnt = output_counts[0] / [1] of the reference; origin[r] = the branch row r was forked from in this step, else -1.
+constexpr int TREE_MAX_BATCH = 1024;
+__global__ __launch_bounds__(256) void tree_fork_kernel(const int64_t *__restrict__ draws, int32_t *__restrict__ tok, int32_t *__restrict__ cnt,
+                                                        const uint8_t *__restrict__ alive, int32_t *__restrict__ curr_b, int batch_size,
+                                                        int64_t *__restrict__ results, long ld, int t,
+                                                        int32_t *__restrict__ pages, long pages_stride, int n_rows,
+                                                        int32_t *__restrict__ origin) {
+    __shared__ int64_t u_tok[TREE_MAX_BATCH];      // the draws, then per branch its distinct tokens (at the segment's start)
+    __shared__ int u_cnt[TREE_MAX_BATCH];
+    __shared__ int seg_off[TREE_MAX_BATCH + 1];    // first draw of branch i
+    __shared__ int seg_uniq[TREE_MAX_BATCH];       // distinct tokens of branch i
+    __shared__ int s_new;                          // branches after the step
+    const int tid = threadIdx.x;
+    const int c0 = *curr_b;
+    if (tid == 0) {
+        int off = 0;
+        for (int i = 0; i < c0; ++i) { seg_off[i] = off; off += cnt[i]; }
+        seg_off[c0] = off;
+    }
+    __syncthreads();
+    const int total = min(seg_off[c0], TREE_MAX_BATCH);
+    for (int i = tid; i < total; i += 256) u_tok[i] = draws[i];
+    for (int r = tid; r < batch_size; r += 256) origin[r] = -1;
+    __syncthreads();
+    // one thread per branch: insertion sort of its draws, then run-length encoding in place
+    for (int i = tid; i < c0; i += 256) {
+        const int lo = seg_off[i], hi = min(seg_off[i + 1], TREE_MAX_BATCH);
+        for (int a = lo + 1; a < hi; ++a) {
+            const int64_t v = u_tok[a];
+            int b = a - 1;
+            while (b >= lo && u_tok[b] > v) { u_tok[b + 1] = u_tok[b]; --b; }
+            u_tok[b + 1] = v;
+        }
+        int n = 0;
+        for (int a = lo; a < hi; ++a) {
+            if (n > 0 && u_tok[lo + n - 1] == u_tok[a]) { ++u_cnt[lo + n - 1]; }
+            else { u_tok[lo + n] = u_tok[a]; u_cnt[lo + n] = 1; ++n; }
+        }
+        seg_uniq[i] = n;
+    }
+    __syncthreads();
+    // rows are handed out in branch order (what is left depends on every earlier branch): one thread walks the branches
+    if (tid == 0) {
+        int cur = c0;
+        for (int i = 0; i < c0; ++i) {
+            if (!alive[i] || seg_uniq[i] == 0) continue;
+            const int lo = seg_off[i];
+            tok[i] = (int32_t)u_tok[lo];
+            cnt[i] = u_cnt[lo];
+            const int forks = min(seg_uniq[i] - 1, batch_size - cur);
+            for (int j = 0; j < forks; ++j) {
+                origin[cur + j] = i;
+                tok[cur + j] = (int32_t)u_tok[lo + 1 + j];
+                cnt[cur + j] = u_cnt[lo + 1 + j];
+            }
+            cur += max(forks, 0);
+        }
+        s_new = cur;
+        *curr_b = cur;
+    }
+    __syncthreads();
+    const int c1 = s_new;
+    // token histories and page ids of the new rows, then this step's column
+    for (int r = c0; r < c1; ++r) {
+        const int o = origin[r];
+        for (long j = tid; j < ld; j += 256) results[(long)r * ld + j] = results[(long)o * ld + j];
+        if (pages != nullptr)
+            for (int j = tid; j < n_rows; j += 256) pages[(long)r * pages_stride + j] = pages[(long)o * pages_stride + j];
+    }
+    __syncthreads();
+    for (int r = tid; r < batch_size; r += 256) {
+        if (!alive[r]) results[(long)r * ld + t] = 0;
+        else if (r < c1 && (r >= c0 || seg_uniq[r] > 0)) results[(long)r * ld + t] = tok[r];
     }
 }
 
@@ -379,7 +476,33 @@ extern "C" int smh_sample_topk(const void *logits, int rows, int vocab, long ld,
     if (rows == 0) return 0;
     SMH_REQUIRE(logits && uniform && out, "smh_sample_topk: null pointer");
     hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, temperature,
-                       top_k, uniform, out);
+                       top_k, uniform, out, (const int32_t *)nullptr);
+    return launch_status();
+}
+
+extern "C" int smh_sample_topk_counts(const void *logits, int rows, int vocab, long ld, float temperature, int top_k,
+                                      const float *uniform, const int32_t *counts, int64_t *out, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(rows >= 0 && rows <= TREE_MAX_BATCH && vocab > 0 && ld >= vocab, "smh_sample_topk_counts: rows=%d (at most %d) vocab=%d ld=%ld", rows, TREE_MAX_BATCH, vocab, ld);
+    SMH_REQUIRE(top_k >= 1 && top_k <= SAMPLE_MAX_K, "smh_sample_topk_counts: top_k=%d outside [1,%d]", top_k, SAMPLE_MAX_K);
+    SMH_REQUIRE(temperature > 0.f, "smh_sample_topk_counts: temperature=%g must be positive", (double)temperature);
+    if (rows == 0) return 0;
+    SMH_REQUIRE(logits && uniform && counts && out, "smh_sample_topk_counts: null pointer");
+    hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, temperature,
+                       top_k, uniform, out, counts);
+    return launch_status();
+}
+
+extern "C" int smh_tree_fork(const int64_t *draws, int32_t *tok, int32_t *cnt, const uint8_t *alive, int32_t *curr_b, int batch_size,
+                             int64_t *results, long ld, int t, int32_t *pages, long pages_stride, int n_rows, int32_t *origin,
+                             smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(batch_size >= 1 && batch_size <= TREE_MAX_BATCH, "smh_tree_fork: batch_size=%d outside [1,%d]", batch_size, TREE_MAX_BATCH);
+    SMH_REQUIRE(draws && tok && cnt && alive && curr_b && results && origin, "smh_tree_fork: null pointer");
+    SMH_REQUIRE(ld >= 1 && t >= 0 && t < ld, "smh_tree_fork: column %d outside the %ld of a row", t, ld);
+    SMH_REQUIRE(pages == nullptr || (pages_stride >= n_rows && n_rows >= 0), "smh_tree_fork: n_rows=%d pages_stride=%ld", n_rows, pages_stride);
+    hipLaunchKernelGGL(tree_fork_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, draws, tok, cnt, alive, curr_b, batch_size, results, ld, t,
+                       pages, pages_stride, n_rows, origin);
     return launch_status();
 }
 

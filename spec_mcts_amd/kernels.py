@@ -447,6 +447,48 @@ def sample_topk(logits: torch.Tensor, temperature: float, top_k: int, uniform: O
     return out
 
 
+def sample_topk_counts(logits: torch.Tensor, temperature: float, top_k: int, counts: torch.Tensor, uniform: torch.Tensor,
+                       out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """sample_topk with counts[r] draws for row r (torch.multinomial(probs[r], num_samples=counts[r], replacement=True) of
+    the tree sampler, mcts.py:128): int64 [uniform.numel()] with row r's tokens at counts[:r].sum() onwards.  counts int32
+    [rows] and uniform fp32 [>= counts.sum()] on the device."""
+    lib = _lib.load()
+    _need_gpu(logits, counts, uniform)
+    assert logits.dim() == 2 and logits.dtype == torch.float16 and logits.stride(1) == 1
+    rows, vocab = logits.shape
+    assert counts.dtype == torch.int32 and counts.is_contiguous() and counts.numel() >= rows
+    assert uniform.dtype == torch.float32 and uniform.is_contiguous()
+    if out is None:
+        out = torch.zeros(uniform.numel(), device=logits.device, dtype=torch.int64)
+    assert out.dtype == torch.int64 and out.is_contiguous() and out.numel() >= uniform.numel()
+    check(lib.smh_sample_topk_counts(logits.data_ptr(), rows, vocab, logits.stride(0), float(temperature), int(min(top_k, vocab)),
+                                     uniform.data_ptr(), counts.data_ptr(), out.data_ptr(), _stream()), "smh_sample_topk_counts")
+    return out
+
+
+def tree_fork(draws: torch.Tensor, output_counts: torch.Tensor, alive: torch.Tensor, curr_b: torch.Tensor, results: torch.Tensor, t: int,
+              pages: Optional[torch.Tensor] = None, n_rows: int = 0, origin: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One expansion step of the tree sampler's bookkeeping (mcts.py:127-152) on the device, in place: output_counts int32
+    [2, batch] (tokens, multiplicities), alive bool/uint8 [batch], curr_b int32 [1], results int64 [batch, steps], pages int32
+    [batch, stride] or None.  Returns origin int32 [batch] (-1, or the branch a row was forked from in this call)."""
+    lib = _lib.load()
+    _need_gpu(draws, output_counts, alive, curr_b, results)
+    batch = results.shape[0]
+    assert output_counts.dtype == torch.int32 and output_counts.shape == (2, batch) and output_counts.is_contiguous()
+    assert draws.dtype == torch.int64 and draws.is_contiguous()
+    assert alive.numel() == batch and alive.is_contiguous() and alive.element_size() == 1
+    assert curr_b.dtype == torch.int32 and curr_b.numel() == 1
+    assert results.dtype == torch.int64 and results.dim() == 2 and results.is_contiguous()
+    if pages is not None:
+        assert pages.is_cuda and pages.dtype == torch.int32 and pages.dim() == 2 and pages.is_contiguous() and pages.shape[0] >= batch
+    if origin is None:
+        origin = torch.empty(batch, dtype=torch.int32, device=results.device)
+    check(lib.smh_tree_fork(draws.data_ptr(), output_counts[0].data_ptr(), output_counts[1].data_ptr(), alive.data_ptr(), curr_b.data_ptr(),
+                            batch, results.data_ptr(), results.shape[1], int(t), _ptr(pages), pages.shape[1] if pages is not None else 0,
+                            int(n_rows), origin.data_ptr(), _stream()), "smh_tree_fork")
+    return origin
+
+
 def detect_terminal(token: torch.Tensor, state: torch.Tensor, terminal_seq: torch.Tensor, eos: int = 2):
     """detectTerminal of the reference's tree sampler (mcts.py:14-28) on the device in one launch.
     token int64 [B], state int32 [B], terminal_seq int64 [L] -> (end bool [B], state int32 [B]); `state` is not modified."""

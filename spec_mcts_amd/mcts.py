@@ -1,0 +1,90 @@
+"""Tree sampler of the reference (mcts.py: class mcts, search) on the device operators of this package.
+
+Same constructor and call: mcts(model, depth, nodes, top_k, temp).search(prompt, batch_size) returns
+(results[:curr_batch], results_len, batch_stats) as mcts.py:67-182 does.  What differs is where the work runs: the
+expansion step - counts[i] draws per branch, torch.unique, one new row per further distinct token, Transformer.fork per
+branch in a Python loop with a host round trip per tensor element (mcts.py:127-152) - is two launches
+(kernels.sample_topk_counts, kernels.tree_fork), a fork is a copy of page ids inside the second of them, and the host
+reads back one integer per step (the number of live branches, which sizes the next forward).
+
+Randomness: the draws are inverse-CDF draws over uniform numbers from torch.rand (the generator may be passed in) in place
+of torch.multinomial's stream, so token sequences differ from the reference's for the same seed while the distribution
+of every draw is the same.  Only a positive temperature is supported (the reference's temp <= 0 mode divides the logits by
+a per-branch ramp of the multiplicities).
+"""
+from __future__ import annotations
+
+from typing import Optional
+
+import torch
+
+from . import kernels as K
+
+TERMINAL_SEQ = (29961, 29914, 20055, 4690, 1164, 29962)       # "[/PYTHON]" (mcts.py:12)
+EOS = 2
+
+
+class mcts:
+    def __init__(self, model, depth, nodes: int = 1024 ** 2, top_k: int = 32, temp: float = 0.3):
+        self.max_nodes = nodes
+        self.top_k = top_k
+        self.max_depth = depth
+        self.max_batch = model.params.max_batch_size
+        self.model = model
+        self.temp = temp
+        self.generator: Optional[torch.Generator] = None
+        self.verbose = False
+
+    @torch.inference_mode()
+    def search(self, prompt: torch.Tensor, batch_size: int):
+        """Grow up to batch_size branches from one prompt until every live branch has ended or max_depth tokens exist."""
+        m = self.model
+        assert self.temp > 0.0, "only the fixed-temperature mode is provided"
+        assert m.paged_kv, "the device-side fork copies page ids: paged_kv must be on"
+        m.resetTimers()
+        m.resetSeq()
+        assert m.params.max_batch_size >= batch_size
+        dev = m.norm.weight.device
+        idx = prompt[:1].to(dev)
+        assert m.params.max_prompt_seq_len >= idx.shape[1]
+        steps = min(self.max_depth, m.params.max_seq_len)
+        results = torch.zeros((batch_size, steps), dtype=torch.int64, device=dev)
+        results_len = torch.zeros(batch_size, dtype=torch.int32, device=dev)
+        alive = torch.ones(batch_size, dtype=torch.bool, device=dev)                 # results_mask
+        output_counts = torch.zeros((2, batch_size), dtype=torch.int32, device=dev)
+        output_counts[1, 0] = batch_size
+        curr_b = torch.ones(1, dtype=torch.int32, device=dev)
+        curr = 1
+        batch_stats = torch.zeros(steps, dtype=torch.uint8, device=dev)
+        state = torch.zeros(batch_size, dtype=torch.int32, device=dev)               # end_stateMachine
+        terminal = torch.tensor(TERMINAL_SEQ, dtype=torch.int64, device=dev)
+        draws = torch.zeros(batch_size, dtype=torch.int64, device=dev)
+        origin = torch.empty(batch_size, dtype=torch.int32, device=dev)
+        pos = 0
+        for t in range(steps):
+            if pos == 0:
+                logits = m(idx, 0)
+                pos = idx.shape[1]
+            else:
+                logits = m(results[:curr, t - 1:t], pos)
+                pos += 1
+            logits = logits[:, -1, :]
+            u = torch.rand(batch_size, device=dev, dtype=torch.float32, generator=self.generator)
+            K.sample_topk_counts(logits, self.temp, self.top_k, output_counts[1], u, out=draws)
+            # the new rows read their ancestors' suffix rows through the model's page table: rows 0 .. t-1 exist so far
+            K.tree_fork(draws, output_counts, alive, curr_b, results, t, pages=m._table(dev), n_rows=m._rows_written, origin=origin)
+            new_curr = int(curr_b.item())                                            # the step's one host read
+            if new_curr > curr and m._rows_written > 0:
+                m._forked = True
+            curr = new_curr
+            ends, state = K.detect_terminal(results[:, t].contiguous(), state, terminal, EOS)
+            results_len += alive.int()
+            alive = ~(ends | ~alive)
+            batch_stats[t] = curr
+            if self.verbose:
+                print(f"step {t}: {curr} branches, {int(alive[:curr].sum())} alive")
+            if int((~alive).sum()) == curr:                                          # mcts.py:174 (counts ended rows over the whole batch)
+                m.printTimers()
+                return results[:curr, :t + 1], results_len, batch_stats[:t + 1]
+        m.printTimers()
+        return results[:curr, :], results_len, batch_stats

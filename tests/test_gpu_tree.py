@@ -1,0 +1,131 @@
+"""The expansion step of the tree sampler on the device (multi-draw top-k sampler, unique / fork bookkeeping) against the
+oracle's restatement of mcts.py:115-152, and the whole search loop against a host loop that does the same bookkeeping
+with the oracle and forks by copying K/V rows."""
+import pytest
+import torch
+
+from oracle import q40_oracle as O
+
+pytestmark = pytest.mark.gpu
+
+
+def test_multi_draw_sampler_matches_oracle_and_single_draws():
+    from spec_mcts_amd import kernels as K
+    g = torch.Generator().manual_seed(80)
+    logits = (torch.randn((5, 32016), generator=g) * 2).half()
+    counts = torch.tensor([3, 0, 40, 1, 6], dtype=torch.int32)
+    u = torch.rand(50, generator=g)
+    got = K.sample_topk_counts(logits.cuda(), 0.3, 32, counts.cuda(), u.cuda()).cpu()
+    want = O.sample_topk_counts(logits, 0.3, 32, counts.tolist(), u)
+    assert torch.equal(got, want)
+    # the same draws one row at a time through the single-draw kernel
+    rows = torch.repeat_interleave(torch.arange(5), counts.long())
+    single = K.sample_topk(logits[rows].cuda(), 0.3, 32, uniform=u.cuda()).cpu()
+    assert torch.equal(got, single)
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_tree_fork_kernel_matches_oracle(seed):
+    """random trees: random multiplicities that sum to the batch size, a few dead branches, few distinct tokens (many
+    duplicates) or many (rows run out), with and without a page table"""
+    from spec_mcts_amd import kernels as K
+    g = torch.Generator().manual_seed(900 + seed)
+    B = int(torch.randint(1, 120, (1,), generator=g))
+    steps, t = 7, int(torch.randint(0, 7, (1,), generator=g))
+    cur = int(torch.randint(1, B + 1, (1,), generator=g))
+    # multiplicities: cur positive integers that sum to B
+    cuts = torch.sort(torch.randperm(B - 1, generator=g)[: cur - 1] + 1).values.tolist() if B > 1 else []
+    cnt = [b - a for a, b in zip([0] + cuts, cuts + [B])]
+    oc = torch.zeros((2, B), dtype=torch.int32)
+    oc[1, :cur] = torch.tensor(cnt, dtype=torch.int32)
+    oc[0, :cur] = torch.randint(0, 1000, (cur,), generator=g, dtype=torch.int32)
+    vocab = 3 if seed % 2 == 0 else 32016
+    draws = torch.randint(0, vocab, (B,), generator=g)
+    alive = torch.rand(B, generator=g) > 0.2
+    results = torch.zeros((B, steps), dtype=torch.int64)
+    results[:cur, :t] = torch.randint(1, 32016, (cur, t), generator=g)
+    use_pages = seed % 3 != 0
+    Smax = 9
+    pages = (torch.arange(B * Smax, dtype=torch.int32).view(B, Smax) * 7 % 1000) if use_pages else None
+    n_rows = min(t, Smax)
+    want_oc, want_res, want_pages = oc.clone(), results.clone(), pages.clone() if use_pages else None
+    want_cur, want_origin = O.tree_fork(draws, want_oc, alive, cur, B, want_res, t, want_pages, n_rows)
+    d_oc, d_res, d_cur = oc.cuda(), results.cuda(), torch.tensor([cur], dtype=torch.int32).cuda()
+    d_pages = pages.cuda() if use_pages else None
+    origin = K.tree_fork(draws.cuda(), d_oc, alive.cuda(), d_cur, d_res, t, pages=d_pages, n_rows=n_rows)
+    assert int(d_cur) == want_cur
+    assert origin.cpu().tolist() == want_origin
+    assert torch.equal(d_oc.cpu(), want_oc)
+    assert torch.equal(d_res.cpu(), want_res)
+    if use_pages:
+        assert torch.equal(d_pages.cpu(), want_pages)
+
+
+CFG = dict(dim=256, n_layers=2, n_heads=2, vocab_size=320, multiple_of=128, max_batch_size=12, max_seq_len=10, max_prompt_seq_len=16)
+
+
+def _host_search(model, prompt, batch_size, depth, top_k, temp, uniforms):
+    """The reference's search loop (mcts.py:67-182) with the oracle's bookkeeping on the host and row-copy forks."""
+    from spec_mcts_amd import kernels as K
+    model.resetSeq()
+    steps = min(depth, model.params.max_seq_len)
+    results = torch.zeros((batch_size, steps), dtype=torch.int64)
+    alive = torch.ones(batch_size, dtype=torch.bool)
+    oc = torch.zeros((2, batch_size), dtype=torch.int32)
+    oc[1, 0] = batch_size
+    state = torch.zeros(batch_size, dtype=torch.int32)
+    results_len = torch.zeros(batch_size, dtype=torch.int32)
+    terminal = torch.tensor((29961, 29914, 20055, 4690, 1164, 29962))
+    cur, pos, stats = 1, 0, []
+    for t in range(steps):
+        if pos == 0:
+            logits = model(prompt.cuda(), 0)
+            pos = prompt.shape[1]
+        else:
+            logits = model(results[:cur, t - 1:t].cuda(), pos)
+            pos += 1
+        # (the draws come from the device sampler, held against the oracle's in the test above: a probability on a rounding
+        # boundary must not decide whether the two LOOPS agree)
+        draws = K.sample_topk_counts(logits[:, -1].contiguous(), temp, top_k, oc[1].cuda(), uniforms[t].cuda()).cpu()
+        new_cur, origin = O.tree_fork(draws, oc, alive, cur, batch_size, results, t)
+        r = cur
+        while r < new_cur:                                   # consecutive new rows of one origin = one model.fork call
+            n = 1
+            while r + n < new_cur and origin[r + n] == origin[r]:
+                n += 1
+            model.fork(origin[r], r, n)
+            r += n
+        cur = new_cur
+        ends, state = O.detect_terminal(results[:, t], state, terminal, 2)
+        results_len += alive.int()
+        alive = ~(ends | ~alive)
+        stats.append(cur)
+        if int((~alive).sum()) == cur:
+            return results[:cur, :t + 1], results_len, stats
+    return results[:cur], results_len, stats
+
+
+@pytest.mark.parametrize("seed,temp", [(0, 0.8), (1, 1.5), (2, 3.0)])
+def test_device_search_equals_host_search(seed, temp):
+    from spec_mcts_amd import ModelArgs
+    from spec_mcts_amd.load_q40 import load_q40
+    from spec_mcts_amd.mcts import mcts
+    sd = O.random_q40_state_dict(O.OracleArgs(**CFG), seed=60 + seed, std=0.05)
+    dev_model = load_q40(dict(sd), ModelArgs(**CFG))
+    host_model = load_q40(dict(sd), ModelArgs(**CFG))
+    host_model.paged_kv = False                                # forks copy K/V rows, as the reference's do
+    prompt = torch.randint(0, CFG["vocab_size"], (1, 9), generator=torch.Generator().manual_seed(seed))
+    B, depth = 12, 8
+    tree = mcts(dev_model, depth, top_k=8, temp=temp)
+    tree.generator = torch.Generator(device="cuda:0").manual_seed(1234 + seed)
+    res, res_len, stats = tree.search(prompt, B)
+    # the same uniform numbers, step by step, for the host loop
+    gen = torch.Generator(device="cuda:0").manual_seed(1234 + seed)
+    uniforms = [torch.rand(B, device="cuda:0", dtype=torch.float32, generator=gen).cpu() for _ in range(depth)]
+    want, want_len, want_stats = _host_search(host_model, prompt, B, depth, 8, temp, uniforms)
+    assert stats.cpu().tolist() == want_stats
+    assert torch.equal(res.cpu(), want)
+    assert torch.equal(res_len.cpu(), want_len)
+    assert want_stats[-1] > 1, "the tree did not branch: the test would not exercise the fork"
+    # every row's history up to its fork point is its ancestor's: rows share first tokens
+    assert int((res[:, 0] == res[0, 0]).sum()) >= 1

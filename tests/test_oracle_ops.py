@@ -360,3 +360,50 @@ def test_noise_study_instruments_reduce_to_the_oracle_where_they_must():
     assert float(d) <= 2e-3
     d = (O.shared_prefix_attention(qq, pk, pv, sk, sv, [3, 1], acc_dtype=torch.float64).float() - O.shared_prefix_attention(qq, pk, pv, sk, sv, [3, 1]).float()).abs().max()
     assert float(d) <= 2e-3
+
+
+def test_tree_fork_known_answers():
+    """The expansion bookkeeping of the tree sampler (mcts.py:127-152) on a tree small enough to write every row out by hand."""
+    B, steps = 6, 4
+    results = torch.zeros((B, steps), dtype=torch.int64)
+    results[0, 0], results[1, 0] = 11, 12
+    oc = torch.zeros((2, B), dtype=torch.int32)
+    oc[0, 0], oc[1, 0], oc[0, 1], oc[1, 1] = 11, 4, 12, 2
+    alive = torch.tensor([True, True, True, True, True, True])
+    pages = torch.arange(B * 5, dtype=torch.int32).view(B, 5)
+    # branch 0 drew 7, 5, 7, 9 -> distinct 5 (x1), 7 (x2), 9 (x1); branch 1 drew 3, 3 -> distinct 3 (x2)
+    draws = torch.tensor([7, 5, 7, 9, 3, 3])
+    cur, origin = O.tree_fork(draws, oc, alive, 2, B, results, 1, pages, n_rows=2)
+    assert cur == 4 and origin == [-1, -1, 0, 0, -1, -1]
+    assert results[:, :2].tolist() == [[11, 5], [12, 3], [11, 7], [11, 9], [0, 0], [0, 0]]
+    assert oc.tolist() == [[5, 3, 7, 9, 0, 0], [1, 2, 2, 1, 0, 0]] and int(oc[1].sum()) == 6       # multiplicities conserved
+    assert pages[2, :2].tolist() == pages[0, :2].tolist() == [0, 1] and pages[2, 2:].tolist() == [12, 13, 14]
+    assert pages[3, :2].tolist() == [0, 1]
+    # next step: branch 1 is dead (its draws change nothing, its column is zeroed), branch 2 forks once more
+    alive = torch.tensor([True, False, True, True, True, True])
+    draws = torch.tensor([8,   4, 4,   6, 2,   1])       # branch 0: 8 | branch 1: 4 4 | branch 2: 6 2 | branch 3: 1
+    oc2 = oc.clone()
+    cur, origin = O.tree_fork(draws, oc2, alive, 4, B, results, 2, pages, n_rows=3)
+    assert cur == 5 and origin == [-1, -1, -1, -1, 2, -1]
+    assert results[:, :3].tolist() == [[11, 5, 8], [12, 3, 0], [11, 7, 2], [11, 9, 1], [11, 7, 6], [0, 0, 0]]
+    assert oc2[0].tolist() == [8, 3, 2, 1, 6, 0] and oc2[1].tolist() == [1, 2, 1, 1, 1, 0]
+    assert pages[4, :3].tolist() == pages[2, :3].tolist() == [0, 1, 12] and pages[4, 3:].tolist() == [23, 24]
+    # rows run out: branch 0 draws three distinct tokens with one row left; the last distinct token and its multiplicity
+    # are dropped, as in the reference (forks = min(len(counts) - 1, batch_size - curr_batch_size), mcts.py:141-142)
+    r4 = torch.zeros((3, 2), dtype=torch.int64)
+    oc4 = torch.tensor([[0, 0, 0], [3, 1, 0]], dtype=torch.int32)
+    cur, origin = O.tree_fork(torch.tensor([7, 5, 6, 9]), oc4, torch.ones(3, dtype=torch.bool), 2, 3, r4, 0)
+    assert cur == 3 and origin == [-1, -1, 0] and r4[:, 0].tolist() == [5, 9, 6] and oc4.tolist() == [[5, 9, 6], [1, 1, 1]]
+    # a full tree: nothing forks any more
+    alive6 = torch.ones(6, dtype=torch.bool)
+    oc3 = torch.tensor([[0] * 6, [1, 1, 1, 1, 1, 1]], dtype=torch.int32)
+    r3 = torch.zeros((6, 2), dtype=torch.int64)
+    cur, origin = O.tree_fork(torch.arange(6) + 20, oc3, alive6, 6, 6, r3, 0)
+    assert cur == 6 and origin == [-1] * 6 and r3[:, 0].tolist() == [20, 21, 22, 23, 24, 25]
+    # draws per row against the single-draw sampler
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn((3, 50), generator=g).half()
+    u = torch.rand(7, generator=g)
+    got = O.sample_topk_counts(logits, 0.7, 8, [2, 0, 5], u)
+    want = torch.cat([O.sample_topk(logits[0:1].expand(2, -1), 0.7, 8, u[:2]), O.sample_topk(logits[2:3].expand(5, -1), 0.7, 8, u[2:])])
+    assert torch.equal(got, want)
