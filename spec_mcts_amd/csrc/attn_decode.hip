@@ -676,14 +676,21 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
 
 template <bool FUSED>
 __global__ __launch_bounds__(256) void attn_suffix_kernel(AttnParams p) {
-    // suffix_waves (1, 2 or 4) waves per (branch, query head): more than one while branches x heads leave CUs idle
-    // grid (groups of four waves of a branch, branches): no division to find the branch
+    // suffix_waves (1, 2 or 4) waves per (branch, query head): more than one while branches x heads leave CUs idle.
+    // Workgroups are dealt round-robin to the 8 XCDs (8 L2s); the heads of one branch share the 128-byte lines of that
+    // branch's scales (2 fp16 per head and position), so ALL workgroups of a branch go to one XCD: workgroup L of the 1-D
+    // grid sits on XCD L % 8 and takes branch 8 (L / 8 / per_branch) + L % 8, head group (L / 8) % per_branch.
     const int wave = threadIdx.x >> 6, nsub = p.suffix_waves;
-    const int hq = blockIdx.x * 4 + wave;
+    const int per_branch = (p.H * nsub + 3) >> 2;              // workgroups (four waves) per branch
+    const int L = blockIdx.x, j = L >> 3;
+    const int grp = j / per_branch;
+    const int b = 8 * grp + (L & 7);
+    if (b >= p.B) return;
+    const int hq = (j - grp * per_branch) * 4 + wave;
     const int h = nsub == 4 ? hq >> 2 : (nsub == 2 ? hq >> 1 : hq);
     if (nsub == 1 && h >= p.H) return;
     // with shared queries every wave reaches the fold's barrier: one past the last head repeats it and writes nothing
-    attn_suffix_body<FUSED, false>(p, blockIdx.y, min(h, p.H - 1), hq & (nsub - 1), nsub, h < p.H);
+    attn_suffix_body<FUSED, false>(p, b, min(h, p.H - 1), hq & (nsub - 1), nsub, h < p.H);
 }
 
 // ---- the whole decode attention in ONE launch -----------------------------------------------------------------
@@ -939,7 +946,7 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
     if (p.splits > 0)
         hipLaunchKernelGGL(attn_prefix_kernel<false>, dim3(p.splits, Hkv, qgroups), dim3(256), 0, (hipStream_t)stream, p);
     p.suffix_waves = attn_plan_suffix_waves_two((long)B * H);
-    hipLaunchKernelGGL(attn_suffix_kernel<false>, dim3((unsigned)((H * p.suffix_waves + 3) / 4), (unsigned)B), dim3(256), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL(attn_suffix_kernel<false>, dim3((unsigned)(((H * p.suffix_waves + 3) / 4) * ((B + 7) / 8 * 8))), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
 }
 
@@ -1127,7 +1134,7 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
     if (p.splits > 0)
         hipLaunchKernelGGL(attn_prefix_kernel<true>, dim3(p.splits, Hkv, qgroups), dim3(256), 0, (hipStream_t)stream, p);
     p.suffix_waves = attn_plan_suffix_waves_two((long)B * H);
-    hipLaunchKernelGGL(attn_suffix_kernel<true>, dim3((unsigned)((H * p.suffix_waves + 3) / 4), (unsigned)B), dim3(256), 0, (hipStream_t)stream, p);
+    hipLaunchKernelGGL(attn_suffix_kernel<true>, dim3((unsigned)(((H * p.suffix_waves + 3) / 4) * ((B + 7) / 8 * 8))), dim3(256), 0, (hipStream_t)stream, p);
     return launch_status();
 }
 
