@@ -340,13 +340,12 @@ def main():
             # the same steps issued launch by launch from Python, as mcts.search's model(tokens, pos) calls would issue them
             dec = GraphDecoder(model, B, use_graph=False)
             dec.prefill(prompt)
-            dec.decode(3)
+            dec.decode(warmup)                              # the same suffix positions as the graph's timed steps
             torch.cuda.synchronize()
-            n_eager = min(20, max_seq - 5)
             t0 = time.perf_counter()
-            dec.decode(n_eager)
+            dec.decode(steps)
             torch.cuda.synchronize()
-            by_batch[B]["eager_ms_per_step"] = (time.perf_counter() - t0) / n_eager * 1e3
+            by_batch[B]["eager_ms_per_step"] = (time.perf_counter() - t0) / steps * 1e3
             del dec
 
     # per-step algorithmic HBM bytes: Q4 linears + fp16 lm_head + shared prefix KV (once) + suffix KV (Q4 rows)

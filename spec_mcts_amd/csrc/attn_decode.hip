@@ -474,7 +474,18 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
     const int hk = div_rep(p, h);
     __shared__ __attribute__((aligned(16))) half_t s_kv[FUSED ? 4 : 1][3][ATT_D];     // FUSED: this wave's new k and v rows, its query
     __shared__ float s_fold[4][16][10];                                                 // nsub > 1: the waves' states (m, l, o[8])
-    const int lane = threadIdx.x & 63, c = lane & 15, g = lane >> 4;
+    // Lane = 16 g + Q4_LPR rl + e.  In the Q4_0 walk below a row belongs to the Q4_LPR lanes (g, rl, 0..Q4_LPR-1), lane e
+    // holding bytes (64 / Q4_LPR) e .. of it; everywhere else the 16 lanes of group g share a row in eight-dim pieces, lane
+    // (rl, e) taking piece c = Q4_DW e + rl - a piece whose dims are among those the lane holds in the walk, so that the
+    // walk's result needs no exchange between lanes with different e.
+    // Measured (64 branches x 32 heads, ragged suffixes of 0..256 rows / 100 branches at ~55 rows): 8 lanes a row and 2 passes a
+    // chunk 22.1 / 14.2 us; 4 lanes 23.6 / 16.2 (more registers, 64 lane exchanges at the end); 16 lanes 26.6 / 14.3; 4 passes
+    // a chunk 23.9 / 15.8, 1 pass 23.7 / 13.8.  Before (16 lanes, 4 rows a batch, no request ahead): 28.6 / 14.8 us.
+    constexpr int Q4_LPR = 8;                              // lanes per row (4, 8 or 16)
+    constexpr int Q4_DW = 16 / Q4_LPR;                     // dwords of a row's 64 bytes per lane = row slots per group
+    constexpr int Q4_ROWS = 4 * Q4_DW;                     // rows per pass of the wave
+    constexpr int Q4_CH = 2;                               // passes per chunk
+    const int lane = threadIdx.x & 63, g = lane >> 4, e = lane & (Q4_LPR - 1), rl = (lane & 15) / Q4_LPR, c = Q4_DW * e + rl;
     const int wave = threadIdx.x >> 6;
     int len = 0;
     // a length beyond the branch's rows (a device counter that ran past the cache) is cut at the cache's end
@@ -489,21 +500,41 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
         if (p.page_bytes == 2) return reinterpret_cast<const int16_t *>(p.pages)[i];
         return reinterpret_cast<const int64_t *>(p.pages)[i];
     };
-    // one batch of Q4_0 suffix rows: group g takes rows t0, t0 + 4, ... (rows past the end repeat the last one).
-    // Four rows a group per batch: eight measured 1-1.5 % slower per decode step at 1, 10 and 100 branches (more
-    // registers, and a short suffix pays for rows it does not have), two 1.5 % slower (more round trips).
-    constexpr int UQ = 4;
-    auto load_q40_batch = [&](int t0, uint32_t (&kb)[UQ], uint32_t (&vb)[UQ], uint32_t (&ksc)[UQ], uint32_t (&vsc)[UQ]) {
+    // ---- Q4_0 suffix rows: a wave takes Q4_ROWS rows per pass (row slot Q4_DW g + rl) and Q4_CH passes per chunk; wave
+    // `sub` of the nsub that share a query takes every nsub-th pass.  All loads of a chunk are requested together, and
+    // the next chunk's before this one is used: the time of this walk is its dependent trips to memory (page id -> row)
+    // and its instructions, not its bytes. ----
+    typedef uint32_t q4_dw_t __attribute__((ext_vector_type(Q4_DW > 1 ? Q4_DW : 2)));
+    struct Q4One { uint32_t x; __device__ uint32_t operator[](int) const { return x; } };
+    typedef std::conditional_t<Q4_DW == 1, Q4One, q4_dw_t> q4_reg_t;
+    struct Q4Chunk { q4_reg_t k[Q4_CH], v[Q4_CH]; uint32_t ks[Q4_CH], vs[Q4_CH]; };
+    const int q4_passes = p.suffix_format == SMH_KV_Q40 ? (len + Q4_ROWS - 1) / Q4_ROWS : 0;     // passes over all waves of the query
+    const int q4_mine = q4_passes > sub ? (q4_passes - sub + nsub - 1) / nsub : 0;                // passes of this wave
+    const int q4_chunks = (q4_mine + Q4_CH - 1) / Q4_CH;
+    auto q4_pos = [&](int n, int u) { return Q4_ROWS * (sub + nsub * (Q4_CH * n + u)) + Q4_DW * g + rl; };  // suffix position of this lane's row
+    auto q4_ids = [&](int n, long (&id)[Q4_CH]) {
 #pragma unroll
-        for (int u = 0; u < UQ; ++u) {
-            const long row = row_of(min(t0 + gstride * u, len - 1)) * p.Hkv + hk;
-            kb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_k + row * 64 + 4 * c);
-            vb[u] = *reinterpret_cast<const uint32_t *>((const uint8_t *)p.suffix_v + row * 64 + 4 * c);
-            ksc[u] = *reinterpret_cast<const uint32_t *>(p.suffix_ks + row * 2);
-            vsc[u] = *reinterpret_cast<const uint32_t *>(p.suffix_vs + row * 2);
+        for (int u = 0; u < Q4_CH; ++u) id[u] = row_of(min(q4_pos(n, u), len - 1));               // rows past the end repeat the last one
+    };
+    auto q4_rows = [&](const long (&id)[Q4_CH], Q4Chunk &ck) {
+#pragma unroll
+        for (int u = 0; u < Q4_CH; ++u) {
+            const long row = id[u] * p.Hkv + hk;
+            ck.k[u] = *reinterpret_cast<const q4_reg_t *>((const uint8_t *)p.suffix_k + row * 64 + 4 * Q4_DW * e);
+            ck.v[u] = *reinterpret_cast<const q4_reg_t *>((const uint8_t *)p.suffix_v + row * 64 + 4 * Q4_DW * e);
+            ck.ks[u] = *reinterpret_cast<const uint32_t *>(p.suffix_ks + row * 2);
+            ck.vs[u] = *reinterpret_cast<const uint32_t *>(p.suffix_vs + row * 2);
         }
     };
-    uint32_t kb0[UQ], vb0[UQ], ksc0[UQ], vsc0[UQ];              // FUSED: the first batch, requested up front
+    Q4Chunk q4_first;                                       // chunk 0, requested as early as the length is known
+    long q4_next_id[Q4_CH];                                 // page ids of the chunk after the one in flight
+    auto q4_prime = [&]() {
+        if (q4_chunks > 0) {
+            q4_ids(0, q4_next_id);
+            q4_rows(q4_next_id, q4_first);
+            if (q4_chunks > 1) q4_ids(1, q4_next_id);
+        }
+    };
     RowRegs q_first;
     int pos = 0;
     if (FUSED) {
@@ -525,7 +556,7 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
             qkv_request(p, b, kcol + lane, ck1); qkv_request(p, b, kcol + lane + 64, ck2);
             qkv_request(p, b, vcol + lane, cv1); qkv_request(p, b, vcol + lane + 64, cv2);
         }
-        if (p.suffix_format == SMH_KV_Q40 && gg < len) load_q40_batch(gg, kb0, vb0, ksc0, vsc0);
+        q4_prime();
         const half_t cos_l = p.cos_tab[(long)pos * 64 + lane], sin_l = p.sin_tab[(long)pos * 64 + lane];
         half_t q1 = qkv_sum(cq1), q2 = qkv_sum(cq2);
         half_t k1 = q1, k2 = q1, v1 = q1, v2 = q1;
@@ -603,20 +634,90 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
                 for (int u = 0; u < U; ++u)
                     if (t0 + gstride * u < len) soft_add_row(st, row_dot(kr[u], qr) * p.scale_log2, vr[u]);
             }
-        } else {
-            constexpr int U = UQ;
-            for (int t0 = gg; t0 < len; t0 += gstride * U) {
-                uint32_t kb[U], vb[U], ksc[U], vsc[U];
-                if (FUSED && t0 == gg) {
+        } else if (q4_chunks > 0) {
+            if (!FUSED) q4_prime();
+            RowRegs qj[Q4_DW];                              // the query's dims this lane holds of a row: pieces Q4_DW e + j
 #pragma unroll
-                    for (int u = 0; u < U; ++u) { kb[u] = kb0[u]; vb[u] = vb0[u]; ksc[u] = ksc0[u]; vsc[u] = vsc0[u]; }
-                } else {
-                    load_q40_batch(t0, kb, vb, ksc, vsc);
+            for (int j = 0; j < Q4_DW; ++j)
+                qj[j] = FUSED ? row_from_fp16(&s_kv[wave][2][0], Q4_DW * e + j) : row_from_fp16(p.q + ((long)b * p.H + h) * ATT_D, Q4_DW * e + j);
+            float m = -INFINITY, l = 0.f;                   // m: common to the group; l, o: of this lane's row slot
+            float o[Q4_DW][8];
+#pragma unroll
+            for (int j = 0; j < Q4_DW; ++j)
+#pragma unroll
+                for (int k = 0; k < 8; ++k) o[j][k] = 0.f;
+            Q4Chunk cur = q4_first;
+            for (int n = 0; n < q4_chunks; ++n) {
+                Q4Chunk nxt;
+                if (n + 1 < q4_chunks) {
+                    q4_rows(q4_next_id, nxt);
+                    if (n + 2 < q4_chunks) q4_ids(n + 2, q4_next_id);
                 }
+                float sc[Q4_CH];
 #pragma unroll
-                for (int u = 0; u < U; ++u)
-                    if (t0 + gstride * u < len)
-                        soft_add_row(st, row_dot(row_from_q40(kb[u], ksc[u]), qr) * p.scale_log2, row_from_q40(vb[u], vsc[u]));
+                for (int u = 0; u < Q4_CH; ++u) {
+                    float d = 0.f;
+#pragma unroll
+                    for (int j = 0; j < Q4_DW; ++j) {
+                        const RowRegs kr = row_from_q40(cur.k[u][j], cur.ks[u]);
+                        d = __builtin_amdgcn_fdot2(kr.a02, qj[j].a02, d, false);
+                        d = __builtin_amdgcn_fdot2(kr.a13, qj[j].a13, d, false);
+                        d = __builtin_amdgcn_fdot2(kr.b02, qj[j].b02, d, false);
+                        d = __builtin_amdgcn_fdot2(kr.b13, qj[j].b13, d, false);
+                    }
+                    d += dpp_move<DPP_QUAD_XOR1>(d);        // the lanes that share the row
+                    d += dpp_move<DPP_QUAD_XOR2>(d);
+                    if (Q4_LPR >= 8) d += dpp_move<DPP_ROW_HALF_MIRROR>(d);
+                    if (Q4_LPR == 16) d += dpp_move<DPP_ROW_ROR8>(d);
+                    sc[u] = q4_pos(n, u) < len ? d * p.scale_log2 : -INFINITY;
+                }
+                float mx = sc[0];
+#pragma unroll
+                for (int u = 1; u < Q4_CH; ++u) mx = fmaxf(mx, sc[u]);
+                if (Q4_LPR <= 8) mx = fmaxf(mx, dpp_move<DPP_ROW_ROR8>(mx)); // the row slots of the group
+                if (Q4_LPR == 4) mx = fmaxf(mx, dpp_move<DPP_ROW_ROR4>(mx));
+                const float m_new = fmaxf(m, mx);
+                const float m_ref = m_new == -INFINITY ? 0.f : m_new;    // a group without a row yet: every factor below is exp2(-inf) = 0
+                const float corr = exp2f(m - m_ref);
+                m = m_new;
+                l *= corr;
+#pragma unroll
+                for (int j = 0; j < Q4_DW; ++j)
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) o[j][k] *= corr;
+#pragma unroll
+                for (int u = 0; u < Q4_CH; ++u) {
+                    const float pr = exp2f(sc[u] - m_ref);
+                    l += pr;
+#pragma unroll
+                    for (int j = 0; j < Q4_DW; ++j) {
+                        const RowRegs vr = row_from_q40(cur.v[u][j], cur.vs[u]);
+                        o[j][0] += pr * (float)vr.a02.x; o[j][1] += pr * (float)vr.a02.y;
+                        o[j][2] += pr * (float)vr.a13.x; o[j][3] += pr * (float)vr.a13.y;
+                        o[j][4] += pr * (float)vr.b02.x; o[j][5] += pr * (float)vr.b02.y;
+                        o[j][6] += pr * (float)vr.b13.x; o[j][7] += pr * (float)vr.b13.y;
+                    }
+                }
+                cur = nxt;
+            }
+            // the group's row slots added up, then lane (rl, e) keeps piece Q4_DW e + rl = c
+            if (Q4_LPR <= 8) l += dpp_move<DPP_ROW_ROR8>(l);
+            if (Q4_LPR == 4) l += dpp_move<DPP_ROW_ROR4>(l);
+#pragma unroll
+            for (int j = 0; j < Q4_DW; ++j)
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    if (Q4_LPR <= 8) o[j][k] += dpp_move<DPP_ROW_ROR8>(o[j][k]);
+                    if (Q4_LPR == 4) o[j][k] += dpp_move<DPP_ROW_ROR4>(o[j][k]);
+                }
+            st.m = m;
+            st.l = l;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                float v = o[0][k];
+#pragma unroll
+                for (int j = 1; j < Q4_DW; ++j) v = rl == j ? o[j][k] : v;
+                st.o[k] = v;
             }
         }
         // ---- the new token's exact K/V (group 0 only) ----
@@ -855,7 +956,7 @@ static void attn_plan(int P, int Hkv, int Bq, int *tw_out, int *qgroups_out) {
 // the GPU in one round (4 waves of this kernel per SIMD, 1024 SIMDs).
 static int attn_plan_suffix_waves_two(long queries) {
     int nsub = 4;
-    constexpr int cap = 4096;
+    constexpr int cap = 4096;                  // measured again with the 8-lanes-a-row walk: 2048 and 8192 are both slower
     while (nsub > 1 && queries * nsub > cap) nsub >>= 1;
     return nsub;
 }

@@ -90,11 +90,30 @@ __device__ __forceinline__ float wave_max(float v) {
     for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
     return v;
 }
-// reductions over the 16 lanes that share lane/16 (one DPP row)
+
+// The value another lane holds, through a data-parallel-primitive move (no LDS, folds into the instruction that uses it).
+// Controls: a permutation of each four consecutive lanes, a rotation of each 16 consecutive lanes (lane i reads i - n), or a
+// reversal of each 8 consecutive lanes.
+constexpr int DPP_QUAD_XOR1 = 0xB1, DPP_QUAD_XOR2 = 0x4E, DPP_ROW_ROR4 = 0x124, DPP_ROW_ROR8 = 0x128;
+constexpr int DPP_ROW_HALF_MIRROR = 0x141;      // lane i of each 8 consecutive lanes reads lane 7 - i
+template <int CTRL>
+__device__ __forceinline__ float dpp_move(float v) {
+    return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xf, 0xf, false));
+}
+
+// sum over the 16 lanes that share lane/16 (one DPP row)
 __device__ __forceinline__ float row16_sum(float v) {
+#ifdef SMH_ROW16_DPP
+    v += dpp_move<DPP_ROW_ROR8>(v);
+    v += dpp_move<DPP_ROW_ROR4>(v);
+    v += dpp_move<DPP_QUAD_XOR2>(v);
+    v += dpp_move<DPP_QUAD_XOR1>(v);
+    return v;
+#else
 #pragma unroll
     for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
     return v;
+#endif
 }
 
 // ---- RMSNorm arithmetic shared by every kernel that normalises ---------------------------------------
