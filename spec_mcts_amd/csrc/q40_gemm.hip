@@ -33,6 +33,9 @@ namespace smh {
 #ifndef SMH_GEMM_KSCAP
 #define SMH_GEMM_KSCAP 1600
 #endif
+#ifndef SMH_GEMM_WAVES
+#define SMH_GEMM_WAVES 8
+#endif
 constexpr int GEMM_BM = 128;
 constexpr int GEMM_WAVES = 4;
 constexpr int GEMM_THREADS = GEMM_WAVES * 64;
@@ -54,15 +57,29 @@ typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
 
-// Waits until at most `stages` younger stages (4 DMA instructions each) of this wave are still in flight.
+// Waits until at most `stages` younger stages (PER DMA instructions each: 4 with four waves, 2 with eight) of this wave
+// are still in flight.
+template <int PER>
 __device__ __forceinline__ void gemm_wait_dma(int stages) {
-    switch (stages) {
-        case 5: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
-        case 4: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
-        case 3: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
-        case 2: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
-        case 1: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
-        default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+    static_assert(PER == 4 || PER == 2, "DMA instructions per wave and stage");
+    if (PER == 4) {
+        switch (stages) {
+            case 5: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
+            case 4: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
+            case 3: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
+            case 2: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+            case 1: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+            default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        }
+    } else {
+        switch (stages) {
+            case 5: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
+            case 4: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
+            case 3: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
+            case 2: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
+            case 1: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
+            default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
+        }
     }
 }
 
@@ -73,12 +90,20 @@ __device__ __forceinline__ void gemm_barrier() { asm volatile("s_waitcnt lgkmcnt
 // TILED: the weights are in the tiled layout (q40_matmul.hpp).  Wave w then moves and decodes piece w of a
 // tile (its two byte positions of its block, already paired by rows): one 16-byte LDS read instead of eight
 // dword reads, shifts instead of byte permutes, the scales already in operand order; rows past K hold zeros.
-template <int TILES, bool RAGGED, bool TILED>
-__global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams p) {
+// WAVES = 8 (tiled weights only): waves w and w + 4 share piece w of a tile; wave w multiplies the columns of its HIGH
+// nibbles, wave w + 4 those of the low nibbles (two B operands and half the accumulators each, the same A tiles), so
+// that every SIMD holds two waves of the workgroup and the decode of one runs under the MFMAs of the other.
+template <int TILES, bool RAGGED, bool TILED, int WAVES>
+__global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kernel(MatmulParams p) {
+    static_assert(WAVES == 4 || (WAVES == 8 && TILED && !RAGGED), "eight waves: tiled weights, K a multiple of 32");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    constexpr int NB = WAVES == 8 ? 2 : 4;     // B operands (16 columns each) per wave
+    constexpr int DMA_PER = WAVES == 8 ? 2 : 4;
 
     const int tid = threadIdx.x;
-    const int wave = tid >> 6;
+    const int wave8 = tid >> 6;                // 0 .. WAVES-1
+    const int wave = wave8 & 3;                // piece of the tile / rows of the ring this wave serves
+    const int hh = wave8 >> 2;                 // eight waves: 0 = high nibbles (columns c), 1 = low nibbles (columns c + 64)
     const int lane = tid & 63;
     const int c = lane & 15;
     const int g = lane >> 4;
@@ -113,7 +138,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     const int w_lrow = 8 * wave + (lane >> 3), w_lcol = 16 * (two_blocks ? (lane & 7) : (lane & 3));
     const int s_lrow = 8 * wave + ((lane & 15) >> 1), s_lcol = 4 * (two_blocks ? (lane & 1) : 0);
     const int a_chunk = (lane & 3) ^ ((lane >> 4) & 3);                   // logical 16-byte chunk stored in slot lane&3
-    const long a_r0 = (long)min(m0 + 32 * wave + (lane >> 2), p.M - 1) * p.lda * 2;
+    const long a_r0 = (long)min(m0 + (WAVES == 8 ? 16 * wave8 : 32 * wave) + (lane >> 2), p.M - 1) * p.lda * 2;
     const long a_r1 = (long)min(m0 + 32 * wave + 16 + (lane >> 2), p.M - 1) * p.lda * 2;
     const uint32_t w_voff = (uint32_t)(w_lrow * w_row + w_lcol);
     const uint32_t s_voff = (uint32_t)(s_lrow * s_row + s_lcol);
@@ -122,7 +147,13 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     auto issue = [&](int step, int slot_) {
         uint8_t *st = lds + slot_ * GS_BYTES;
         const long k0 = (long)step * 32;
-        if (TILED) {
+        if (TILED && WAVES == 8) {
+            // two DMA instructions a wave: waves 0-3 their piece of the nibbles, waves 4-7 its scales; every wave 16 rows of A
+            const uint8_t *tile = w_base + (long)step * TILE_BYTES;
+            if (hh == 0) __builtin_amdgcn_global_load_lds((gptr_t)(tile + wave * 1024 + lane * 16), (lptr_t)(st + wave * 1024), 16, 0, 0);
+            else if (lane < 16) __builtin_amdgcn_global_load_lds((gptr_t)(tile + TILE_W_BYTES + (16 * wave + lane) * 4), (lptr_t)(st + GS_W + wave * 64), 4, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(a_base + k0 * 2 + a_voff0), (lptr_t)(st + GS_W + GS_S + wave8 * 1024), 16, 0, 0);
+        } else if (TILED) {
             const uint8_t *tile = w_base + (long)step * TILE_BYTES;
             __builtin_amdgcn_global_load_lds((gptr_t)(tile + wave * 1024 + lane * 16), (lptr_t)(st + wave * 1024), 16, 0, 0);
             if (lane < 16)
@@ -153,9 +184,9 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
         }
     };
 
-    f4 acc[4][TILES];
+    f4 acc[NB][TILES];
 #pragma unroll
-    for (int h = 0; h < 4; ++h)
+    for (int h = 0; h < NB; ++h)
 #pragma unroll
         for (int t = 0; t < TILES; ++t) acc[h][t] = f4{0.f, 0.f, 0.f, 0.f};
 
@@ -180,6 +211,17 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             // wv[0..3] = (x, x2) of byte 2bp, (x, x2) of byte 2bp+1; sv[0..3] / sv[4..7] = the row pairs' scales of the
             // block's first / second 64 columns
             const u32x4 wq = *reinterpret_cast<const u32x4 *>(st + wave * 1024 + lane * 16);
+            if (WAVES == 8) {                  // the scales of this wave's nibble only
+                const u32x4 sc = *reinterpret_cast<const u32x4 *>(st + GS_W + g * 64 + (2 * blk + hh) * 16);
+#pragma unroll
+                for (int r = 0; r < 4; ++r) {
+                    wv[r] = wq[r];
+                    wv[4 + r] = 0;
+                    sv[r] = sc[r];
+                    sv[4 + r] = 0;
+                }
+                return;
+            }
             const u32x4 sh = *reinterpret_cast<const u32x4 *>(st + GS_W + g * 64 + (2 * blk) * 16);
             const u32x4 sl = *reinterpret_cast<const u32x4 *>(st + GS_W + g * 64 + (2 * blk + 1) * 16);
 #pragma unroll
@@ -198,8 +240,25 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
         }
     };
     // exact fp16 code * scale, as the four B operands (byte 2bp high / low, byte 2bp+1 high / low)
-    auto decode = [&](const uint32_t (&wv)[8], const uint32_t (&sv)[8], bool dead, h8 (&b)[4]) {
+    // eight waves: the nibble this wave decodes, as constants of one and-or + one packed fma (code = fp16 bits * mul + off)
+    const uint32_t nib_mask = hh == 0 ? 0x00F000F0u : 0x000F000Fu;
+    const h2 nib_mul = hh == 0 ? h2{(half_t)0.0625f, (half_t)0.0625f} : h2{(half_t)1.0f, (half_t)1.0f};
+    const h2 nib_off = hh == 0 ? h2{(half_t)-72.0f, (half_t)-72.0f} : h2{(half_t)-1032.0f, (half_t)-1032.0f};
+    auto decode = [&](const uint32_t (&wv)[8], const uint32_t (&sv)[8], bool dead, h8 (&b)[NB]) {
         u32x4 v0h, v0l, v1h, v1l;
+        if (TILED && WAVES == 8) {
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const uint32_t pr0 = j < 2 ? wv[j] : wv[j - 2] >> 8;           // rows (2j, 2j+1) of byte 2bp, codes + 8
+                const uint32_t pr1 = j < 2 ? wv[2 + j] : wv[j] >> 8;           // ... of byte 2bp+1
+                const h2 sc = as_h2(sv[j]);
+                v0h[j] = as_u32(__builtin_elementwise_fma(as_h2((pr0 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
+                v1h[j] = as_u32(__builtin_elementwise_fma(as_h2((pr1 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
+            }
+            b[0] = __builtin_bit_cast(h8, v0h);
+            b[1] = __builtin_bit_cast(h8, v1h);
+            return;
+        }
         if (TILED) {
 #pragma unroll
             for (int j = 0; j < 4; ++j) {
@@ -211,10 +270,12 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
                 v1h[j] = as_u32(codes_high(pr1) * s_hi);
                 v1l[j] = as_u32(codes_low(pr1) * s_lo);
             }
-            b[0] = __builtin_bit_cast(h8, v0h);
-            b[1] = __builtin_bit_cast(h8, v0l);
-            b[2] = __builtin_bit_cast(h8, v1h);
-            b[3] = __builtin_bit_cast(h8, v1l);
+            if constexpr (NB == 4) {
+                b[0] = __builtin_bit_cast(h8, v0h);
+                b[1] = __builtin_bit_cast(h8, v0l);
+                b[2] = __builtin_bit_cast(h8, v1h);
+                b[3] = __builtin_bit_cast(h8, v1l);
+            }
             return;
         }
 #pragma unroll
@@ -229,10 +290,12 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             v1l[j] = as_u32(codes_low(pr1) * s_lo);
         }
         if (RAGGED && dead) v0h = v0l = v1h = v1l = u32x4{0u, 0u, 0u, 0u};     // k >= K: no contribution
-        b[0] = __builtin_bit_cast(h8, v0h);
-        b[1] = __builtin_bit_cast(h8, v0l);
-        b[2] = __builtin_bit_cast(h8, v1h);
-        b[3] = __builtin_bit_cast(h8, v1l);
+        if constexpr (NB == 4) {
+            b[0] = __builtin_bit_cast(h8, v0h);
+            b[1] = __builtin_bit_cast(h8, v0l);
+            b[2] = __builtin_bit_cast(h8, v1h);
+            b[3] = __builtin_bit_cast(h8, v1l);
+        }
     };
     auto k_dead = [&](int step) { return step * 32 + 8 * g >= p.K; };      // only in the last step when K % 32 != 0
     // While the matrix pipe multiplies step i (A tile read from stage i, B operands decoded one iteration
@@ -246,19 +309,19 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             av[t] = *reinterpret_cast<const h8 *>(at + r * 64 + ((g ^ ((r >> 2) & 3)) << 4));
         }
     };
-    auto multiply = [&](const h8 (&av)[TILES], const h8 (&b)[4]) {
+    auto multiply = [&](const h8 (&av)[TILES], const h8 (&b)[NB]) {
 #pragma unroll
         for (int t = 0; t < TILES; ++t) {
 #pragma unroll
-            for (int o = 0; o < 4; ++o) acc[o][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], b[o], acc[o][t], 0, 0, 0);
+            for (int o = 0; o < NB; ++o) acc[o][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], b[o], acc[o][t], 0, 0, 0);
         }
     };
     if (n_steps > 0) {
-        h8 bq[4];
+        h8 bq[NB];
         int cur = step0 + rot;                 // step being multiplied
         int slot = 0;                          // its ring slot
         {
-            gemm_wait_dma(min(GEMM_STAGES - 2, n_steps - 1));
+            gemm_wait_dma<DMA_PER>(min(GEMM_STAGES - 2, n_steps - 1));
             gemm_barrier();
             uint32_t wv[8], sv[8];
             load_ws(lds, wv, sv);
@@ -268,8 +331,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
         // compile-time flag so that the body of the main loop is one basic block with its DMA inside
         auto iterate = [&](int i, auto refill) {
             // stage i+1 has landed for this wave (the three younger ones may still be in flight) ...
-            if (refill.value) gemm_wait_dma(GEMM_STAGES - 3);
-            else gemm_wait_dma(min(GEMM_STAGES - 3, max(n_steps - 2 - i, 0)));
+            if (refill.value) gemm_wait_dma<DMA_PER>(GEMM_STAGES - 3);
+            else gemm_wait_dma<DMA_PER>(min(GEMM_STAGES - 3, max(n_steps - 2 - i, 0)));
             gemm_barrier();                    // ... and for everyone; everyone is done with stage i-1
             if (refill.value) fetch_next(slot == 0 ? GEMM_STAGES - 1 : slot - 1);
             const uint8_t *st = lds + slot * GS_BYTES;
@@ -277,13 +340,13 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             cur = cur + 1 == step1 ? step0 : cur + 1;
             // past the last step the next slot holds stale bytes: read, decoded and never used
             uint32_t wv[8], sv[8];
-            h8 av[TILES], bn[4];
+            h8 av[TILES], bn[NB];
             load_a(st, av);
             load_ws(lds + slot * GS_BYTES, wv, sv);
             multiply(av, bq);
             decode(wv, sv, k_dead(cur), bn);
 #pragma unroll
-            for (int o = 0; o < 4; ++o) bq[o] = bn[o];
+            for (int o = 0; o < NB; ++o) bq[o] = bn[o];
             // issue order asked of the scheduler: LDS reads first, then MFMAs with the decode's VALU between them (the matrix
             // pipe works 16 cycles per MFMA and the wave's next instructions issue meanwhile); it follows this in part
             // (the reads move to the front, about a third of the VALU between the MFMAs) and the launch is 3 % shorter
@@ -292,7 +355,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
 #pragma unroll
             for (int t = 0; t < TILES; ++t) {
 #pragma unroll
-                for (int o = 0; o < 4; ++o) {
+                for (int o = 0; o < NB; ++o) {
                     __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
                     __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
                 }
@@ -317,7 +380,8 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     constexpr int OTILE_BYTES = 16 * OP * 4;
     static_assert(2 * OTILE_BYTES <= GEMM_LDS, "two output tiles must fit in the ring");
     float *slab = p.partial + (long)slice * p.M * p.n_total;
-    const int o_row = tid >> 4;                 // 0..15
+    const int o_row = (tid & 255) >> 4;         // 0..15
+    const int o_half = tid >> 8;                // eight waves: the second 256 threads store the second half of the columns
     const int o_lane = tid & 15;                // store q of this lane: columns 64q + 4*o_lane .. (fp16: 128q + 8*o_lane ..),
                                                 // so that one store instruction writes whole contiguous rows
     gemm_barrier();                             // every wave has left the main loop: the ring is free
@@ -325,17 +389,23 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
     for (int t = 0; t < TILES; ++t) {
         float *otile = reinterpret_cast<float *>(lds + (t & 1) * OTILE_BYTES);
         // operands o and o + 2 are neighbouring columns: one 8-byte LDS store for the pair
-#pragma unroll
-        for (int o = 0; o < 2; ++o)
+        if constexpr (WAVES == 8) {
 #pragma unroll
             for (int r = 0; r < 4; ++r)
-                *reinterpret_cast<f2 *>(&otile[(4 * g + r) * OP + 128 * blk + 64 * o + 4 * c + 2 * bp]) = f2{acc[o][t][r], acc[o + 2][t][r]};
+                *reinterpret_cast<f2 *>(&otile[(4 * g + r) * OP + 128 * blk + 64 * hh + 4 * c + 2 * bp]) = f2{acc[0][t][r], acc[1][t][r]};
+        } else {
+#pragma unroll
+            for (int o = 0; o < 2; ++o)
+#pragma unroll
+                for (int r = 0; r < 4; ++r)
+                    *reinterpret_cast<f2 *>(&otile[(4 * g + r) * OP + 128 * blk + 64 * o + 4 * c + 2 * bp]) = f2{acc[o][t][r], acc[o + 2][t][r]};
+        }
         gemm_barrier();
         const int m = m0 + 16 * t + o_row;
         if (m < p.M) {
             if (p.direct) {
 #pragma unroll
-                for (int q = 0; q < 2; ++q) {
+                for (int q = (WAVES == 8 ? o_half : 0); q < (WAVES == 8 ? o_half + 1 : 2); ++q) {
                     const int n_seg = col0 + 128 * q + 8 * o_lane;
                     if (n_seg < seg.N) {
                         const int n = seg.col0 + n_seg;
@@ -353,7 +423,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             } else if (p.slab_half) {
                 half_t *dst = reinterpret_cast<half_t *>(p.partial) + ((long)slice * p.M + m) * p.n_total + seg.col0 + col0;
 #pragma unroll
-                for (int q = 0; q < 2; ++q) {
+                for (int q = (WAVES == 8 ? o_half : 0); q < (WAVES == 8 ? o_half + 1 : 2); ++q) {
                     const int cq = 128 * q + 8 * o_lane;
                     if (col0 + cq < seg.N) {
                         const f4 v0 = *reinterpret_cast<const f4 *>(otile + o_row * OP + cq);
@@ -367,7 +437,7 @@ __global__ __launch_bounds__(GEMM_THREADS, 2) void q40_gemm_kernel(MatmulParams 
             } else {
                 float *dst = slab + (long)m * p.n_total + seg.col0 + col0;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
+                for (int q = (WAVES == 8 ? 2 * o_half : 0); q < (WAVES == 8 ? 2 * o_half + 2 : 4); ++q) {
                     const int cq = 64 * q + 4 * o_lane;
                     if (col0 + cq < seg.N) *reinterpret_cast<f4 *>(dst + cq) = *reinterpret_cast<const f4 *>(otile + o_row * OP + cq);
                 }
@@ -412,11 +482,12 @@ template <bool TILED>
 static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
     // one instantiation per number of 16-row tiles (M <= 128) keeps the step free of branches; K % 32 != 0
     // takes the masked variant with all 8 tiles
-    static const gemm_kernel_t exact[9] = {nullptr, q40_gemm_kernel<2, false, TILED>, q40_gemm_kernel<2, false, TILED>,
-                                           q40_gemm_kernel<3, false, TILED>, q40_gemm_kernel<4, false, TILED>,
-                                           q40_gemm_kernel<5, false, TILED>, q40_gemm_kernel<6, false, TILED>,
-                                           q40_gemm_kernel<7, false, TILED>, q40_gemm_kernel<8, false, TILED>};
-    static const gemm_kernel_t ragged = q40_gemm_kernel<8, true, TILED>;
+    constexpr int W = TILED ? SMH_GEMM_WAVES : 4;
+    static const gemm_kernel_t exact[9] = {nullptr, q40_gemm_kernel<2, false, TILED, W>, q40_gemm_kernel<2, false, TILED, W>,
+                                           q40_gemm_kernel<3, false, TILED, W>, q40_gemm_kernel<4, false, TILED, W>,
+                                           q40_gemm_kernel<5, false, TILED, W>, q40_gemm_kernel<6, false, TILED, W>,
+                                           q40_gemm_kernel<7, false, TILED, W>, q40_gemm_kernel<8, false, TILED, W>};
+    static const gemm_kernel_t ragged = q40_gemm_kernel<8, true, TILED, 4>;
     // more than 64 KB of dynamic LDS has to be allowed once per kernel (the attribute is not stream work,
     // so a launch under graph capture is not affected)
     static const hipError_t lds_ok = [] {
@@ -430,7 +501,7 @@ static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
     const int tiles = p.mblocks > 1 ? 8 : (p.M + 15) / 16;
     const gemm_kernel_t kern = (p.K % 32 != 0) ? ragged : exact[tiles < 2 ? 2 : tiles];
     dim3 grid((unsigned)((long)p.units_pad * p.mblocks * p.ksplit));
-    hipLaunchKernelGGL(kern, grid, dim3(GEMM_THREADS), GEMM_LDS, stream, p);
+    hipLaunchKernelGGL(kern, grid, dim3(kern == ragged ? GEMM_THREADS : 64 * W), GEMM_LDS, stream, p);
     return launch_status();
 }
 
