@@ -191,6 +191,12 @@ int smh_sample_topk(const void *logits, int rows, int vocab, long ld, float temp
  *   batch_size <= 1024. */
 int smh_sample_topk_counts(const void *logits, int rows, int vocab, long ld, float temperature, int top_k,
                            const float *uniform, const int32_t *counts, int64_t *out, smh_stream_t stream);
+/* smh_sample_topk_rowtemp: smh_sample_topk_counts with a temperature per row, row_temps fp32 [rows] on the device, all
+ * positive - the tree sampler's temp <= 0 mode, where the logits of branch i are divided by a ramp of its multiplicity
+ * (mcts.py:110-114).  There the divisor is a float32 TENSOR, which promotes the fp16 logits: quotients, softmax and
+ * probabilities are fp32 here too (no fp16 rounding of x or p); the candidates are the top_k largest logits. */
+int smh_sample_topk_rowtemp(const void *logits, int rows, int vocab, long ld, const float *row_temps, int top_k,
+                            const float *uniform, const int32_t *counts, int64_t *out, smh_stream_t stream);
 int smh_tree_fork(const int64_t *draws, int32_t *tok, int32_t *cnt, const uint8_t *alive, int32_t *curr_b, int batch_size,
                   int64_t *results, long ld, int t, int32_t *pages, long pages_stride, int n_rows, int32_t *origin,
                   smh_stream_t stream);

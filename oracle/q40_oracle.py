@@ -172,10 +172,24 @@ def apply_rotary_emb(q: torch.Tensor, k: torch.Tensor, freqs_cis: torch.Tensor):
     return q_embed, k_embed
 
 
-def topk_probs(logits: torch.Tensor, temperature: float, top_k: int) -> Tuple[torch.Tensor, torch.Tensor]:
+def ramp_temperature(temp: float, batch_size: int, counts: torch.Tensor) -> torch.Tensor:
+    """The per-branch temperature of the tree sampler's temp <= 0 mode (mcts.py:113, the lambda f applied to
+    output_counts[1, :curr]): a line from 0.1 at multiplicity 1 to |temp| at multiplicity batch_size; counts int32 ->
+    float32, as torch promotes int32 * Python float."""
+    return (abs(temp) - 0.1) / (batch_size - 1) * (counts - 1) + 0.1
+
+
+def topk_probs(logits: torch.Tensor, temperature, top_k: int) -> Tuple[torch.Tensor, torch.Tensor]:
     """The candidates of the reference's sampling step (hf_model_q40_kv_shared.py:580-586): `logits / temperature` on
     the fp16 tensor, `torch.topk`, `F.softmax` (fp16 in, fp16 out).  Returns (p [rows, k] fp16, idx [rows, k]) in
-    descending order of value; equal values are ordered by index (torch.topk leaves that order open)."""
+    descending order of value; equal values are ordered by index (torch.topk leaves that order open).
+    temperature may be a float32 tensor [rows] (mcts.py:114, `(logits.t() / f(..)).t()`): torch then promotes the
+    quotient, and with it the softmax, to float32."""
+    if isinstance(temperature, torch.Tensor):
+        x = (logits.t() / temperature).t()                     # fp16 tensor / fp32 tensor: fp32 result
+        k = min(top_k, x.shape[-1])
+        order = torch.argsort(x, dim=-1, descending=True, stable=True)[:, :k]
+        return F.softmax(torch.gather(x, 1, order), dim=-1), order
     x = logits / temperature                                   # fp16 tensor / python float: fp16 result
     k = min(top_k, x.shape[-1])
     order = torch.argsort(x.float(), dim=-1, descending=True, stable=True)[:, :k]
@@ -195,7 +209,7 @@ def sample_topk(logits: torch.Tensor, temperature: float, top_k: int, u: torch.T
     return order.gather(1, j.unsqueeze(1))[:, 0]
 
 
-def sample_topk_counts(logits: torch.Tensor, temperature: float, top_k: int, counts, u: torch.Tensor) -> torch.Tensor:
+def sample_topk_counts(logits: torch.Tensor, temperature, top_k: int, counts, u: torch.Tensor) -> torch.Tensor:
     """counts[r] draws per row (mcts.py:128: torch.multinomial(probs[r], num_samples=output_counts[1, r], replacement=True)
     followed by the gather of :129), each an inverse-CDF draw as in sample_topk; row r uses u[sum(counts[:r]) ...]."""
     out = []
@@ -203,7 +217,8 @@ def sample_topk_counts(logits: torch.Tensor, temperature: float, top_k: int, cou
     for r in range(logits.shape[0]):
         n = int(counts[r])
         if n:
-            out.append(sample_topk(logits[r:r + 1].expand(n, -1), temperature, top_k, u[off:off + n]))
+            tr = temperature[r:r + 1].expand(n) if isinstance(temperature, torch.Tensor) else temperature
+            out.append(sample_topk(logits[r:r + 1].expand(n, -1), tr, top_k, u[off:off + n]))
         off += n
     return torch.cat(out) if out else torch.zeros(0, dtype=torch.int64)
 

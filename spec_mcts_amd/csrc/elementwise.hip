@@ -268,7 +268,12 @@ __device__ __forceinline__ void sample_pick_bin(int *bins, int want, int *out_bi
 // its candidates, with the uniform numbers (and into the slots of out) that start at counts[0] + ... + counts[r-1].
 __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restrict__ logits, int vocab, long ld, float temperature,
                                                            int top_k, const float *__restrict__ uniform, int64_t *__restrict__ out,
-                                                           const int32_t *__restrict__ counts) {
+                                                           const int32_t *__restrict__ counts, const float *__restrict__ row_temps) {
+    // row_temps: a temperature per row, applied in fp32 (a tensor divisor promotes the fp16 logits to fp32 in torch, a
+    // Python scalar does not): candidates by the raw logits (division by a positive number keeps their order, and two
+    // different fp16 values stay different in fp32), softmax and probabilities in fp32
+    const bool wide = row_temps != nullptr;
+    if (wide) temperature = row_temps[blockIdx.x];
     __shared__ int bins[256];
     __shared__ int s_bin, s_above, s_count;
     __shared__ int scan[1024];
@@ -280,7 +285,8 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
     const int tid = threadIdx.x;
     const half_t *row = logits + (long)blockIdx.x * ld;
     const int k = min(top_k, vocab);
-    auto key_at = [&](int i) { return sample_key((half_t)((float)row[i] / temperature)); };
+    auto key_at = [&](int i) { return sample_key(wide ? row[i] : (half_t)((float)row[i] / temperature)); };
+    auto value_of = [&](uint32_t key) { return wide ? (float)sample_unkey(key) / temperature : (float)sample_unkey(key); };
 
     // ---- the k-th largest key: high byte, then low byte ----
     if (tid < 256) bins[tid] = 0;
@@ -342,8 +348,8 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
     __syncthreads();
 
     // ---- p = fp16(softmax), inverse CDF ----
-    const float xmax = (float)sample_unkey(o_key[0]);
-    const float e = tid < k ? expf((float)sample_unkey(o_key[tid]) - xmax) : 0.f;
+    const float xmax = value_of(o_key[0]);
+    const float e = tid < k ? expf(value_of(o_key[tid]) - xmax) : 0.f;
     cdf[tid] = e;
     __syncthreads();
     for (int off = 1; off < 1024; off <<= 1) {
@@ -354,7 +360,7 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
     }
     const float total = cdf[k - 1];
     __syncthreads();
-    const float pr = tid < k ? (float)(half_t)(e / total) : 0.f;
+    const float pr = tid < k ? (wide ? e / total : (float)(half_t)(e / total)) : 0.f;
     cdf[tid] = pr;
     __syncthreads();
     for (int off = 1; off < 1024; off <<= 1) {
@@ -476,7 +482,7 @@ extern "C" int smh_sample_topk(const void *logits, int rows, int vocab, long ld,
     if (rows == 0) return 0;
     SMH_REQUIRE(logits && uniform && out, "smh_sample_topk: null pointer");
     hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, temperature,
-                       top_k, uniform, out, (const int32_t *)nullptr);
+                       top_k, uniform, out, (const int32_t *)nullptr, (const float *)nullptr);
     return launch_status();
 }
 
@@ -489,7 +495,19 @@ extern "C" int smh_sample_topk_counts(const void *logits, int rows, int vocab, l
     if (rows == 0) return 0;
     SMH_REQUIRE(logits && uniform && counts && out, "smh_sample_topk_counts: null pointer");
     hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, temperature,
-                       top_k, uniform, out, counts);
+                       top_k, uniform, out, counts, (const float *)nullptr);
+    return launch_status();
+}
+
+extern "C" int smh_sample_topk_rowtemp(const void *logits, int rows, int vocab, long ld, const float *row_temps, int top_k,
+                                       const float *uniform, const int32_t *counts, int64_t *out, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(rows >= 0 && rows <= TREE_MAX_BATCH && vocab > 0 && ld >= vocab, "smh_sample_topk_rowtemp: rows=%d (at most %d) vocab=%d ld=%ld", rows, TREE_MAX_BATCH, vocab, ld);
+    SMH_REQUIRE(top_k >= 1 && top_k <= SAMPLE_MAX_K, "smh_sample_topk_rowtemp: top_k=%d outside [1,%d]", top_k, SAMPLE_MAX_K);
+    if (rows == 0) return 0;
+    SMH_REQUIRE(logits && row_temps && uniform && counts && out, "smh_sample_topk_rowtemp: null pointer");
+    hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, 1.0f,
+                       top_k, uniform, out, counts, row_temps);
     return launch_status();
 }
 

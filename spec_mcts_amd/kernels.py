@@ -447,11 +447,13 @@ def sample_topk(logits: torch.Tensor, temperature: float, top_k: int, uniform: O
     return out
 
 
-def sample_topk_counts(logits: torch.Tensor, temperature: float, top_k: int, counts: torch.Tensor, uniform: torch.Tensor,
+def sample_topk_counts(logits: torch.Tensor, temperature, top_k: int, counts: torch.Tensor, uniform: torch.Tensor,
                        out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """sample_topk with counts[r] draws for row r (torch.multinomial(probs[r], num_samples=counts[r], replacement=True) of
     the tree sampler, mcts.py:128): int64 [uniform.numel()] with row r's tokens at counts[:r].sum() onwards.  counts int32
-    [rows] and uniform fp32 [>= counts.sum()] on the device."""
+    [rows] and uniform fp32 [>= counts.sum()] on the device.  temperature: a positive number (logits / temperature stays
+    fp16, as in torch) or a float32 tensor [rows] of positive numbers on the device (the sampler's per-branch ramp,
+    mcts.py:110-114: a tensor divisor promotes to fp32, so quotients and probabilities are fp32)."""
     lib = _lib.load()
     _need_gpu(logits, counts, uniform)
     assert logits.dim() == 2 and logits.dtype == torch.float16 and logits.stride(1) == 1
@@ -461,6 +463,12 @@ def sample_topk_counts(logits: torch.Tensor, temperature: float, top_k: int, cou
     if out is None:
         out = torch.zeros(uniform.numel(), device=logits.device, dtype=torch.int64)
     assert out.dtype == torch.int64 and out.is_contiguous() and out.numel() >= uniform.numel()
+    if isinstance(temperature, torch.Tensor):
+        _need_gpu(temperature)
+        assert temperature.dtype == torch.float32 and temperature.is_contiguous() and temperature.numel() >= rows
+        check(lib.smh_sample_topk_rowtemp(logits.data_ptr(), rows, vocab, logits.stride(0), temperature.data_ptr(), int(min(top_k, vocab)),
+                                          uniform.data_ptr(), counts.data_ptr(), out.data_ptr(), _stream()), "smh_sample_topk_rowtemp")
+        return out
     check(lib.smh_sample_topk_counts(logits.data_ptr(), rows, vocab, logits.stride(0), float(temperature), int(min(top_k, vocab)),
                                      uniform.data_ptr(), counts.data_ptr(), out.data_ptr(), _stream()), "smh_sample_topk_counts")
     return out

@@ -5,12 +5,13 @@ Same constructor and call: mcts(model, depth, nodes, top_k, temp).search(prompt,
 expansion step - counts[i] draws per branch, torch.unique, one new row per further distinct token, Transformer.fork per
 branch in a Python loop with a host round trip per tensor element (mcts.py:127-152) - is two launches
 (kernels.sample_topk_counts, kernels.tree_fork), a fork is a copy of page ids inside the second of them, and the host
-reads back one integer per step (the number of live branches, which sizes the next forward).
+reads back two integers per step in one copy (the number of live branches, which sizes the next forward, and the
+number of ended rows, which stops the search).
 
 Randomness: the draws are inverse-CDF draws over uniform numbers from torch.rand (the generator may be passed in) in place
 of torch.multinomial's stream, so token sequences differ from the reference's for the same seed while the distribution
-of every draw is the same.  Only a positive temperature is supported (the reference's temp <= 0 mode divides the logits by
-a per-branch ramp of the multiplicities).
+of every draw is the same.  temp > 0: one temperature for all branches; temp <= 0: the reference's ramp, branch i at
+0.1 + (|temp| - 0.1) (n_i - 1) / (batch_size - 1) for multiplicity n_i (mcts.py:110-114), in float32 as there.
 """
 from __future__ import annotations
 
@@ -39,7 +40,6 @@ class mcts:
     def search(self, prompt: torch.Tensor, batch_size: int):
         """Grow up to batch_size branches from one prompt until every live branch has ended or max_depth tokens exist."""
         m = self.model
-        assert self.temp > 0.0, "only the fixed-temperature mode is provided"
         assert m.paged_kv, "the device-side fork copies page ids: paged_kv must be on"
         m.resetTimers()
         m.resetSeq()
@@ -70,20 +70,24 @@ class mcts:
                 pos += 1
             logits = logits[:, -1, :]
             u = torch.rand(batch_size, device=dev, dtype=torch.float32, generator=self.generator)
-            K.sample_topk_counts(logits, self.temp, self.top_k, output_counts[1], u, out=draws)
+            if self.temp > 0.0:
+                temperature = self.temp
+            else:       # mcts.py:113-114, the expression itself: int32 tensor -> float32 (ZeroDivisionError at batch_size 1, as there)
+                temperature = ((abs(self.temp) - 0.1) / (batch_size - 1) * (output_counts[1] - 1) + 0.1).contiguous()
+            K.sample_topk_counts(logits, temperature, self.top_k, output_counts[1], u, out=draws)
             # the new rows read their ancestors' suffix rows through the model's page table: rows 0 .. t-1 exist so far
             K.tree_fork(draws, output_counts, alive, curr_b, results, t, pages=m._table(dev), n_rows=m._rows_written, origin=origin)
-            new_curr = int(curr_b.item())                                            # the step's one host read
-            if new_curr > curr and m._rows_written > 0:
-                m._forked = True
-            curr = new_curr
             ends, state = K.detect_terminal(results[:, t].contiguous(), state, terminal, EOS)
             results_len += alive.int()
             alive = ~(ends | ~alive)
+            new_curr, ended = torch.stack((curr_b[0], (~alive).sum().int())).tolist()     # the step's one host read
+            if new_curr > curr and m._rows_written > 0:
+                m._forked = True
+            curr = new_curr
             batch_stats[t] = curr
             if self.verbose:
                 print(f"step {t}: {curr} branches, {int(alive[:curr].sum())} alive")
-            if int((~alive).sum()) == curr:                                          # mcts.py:174 (counts ended rows over the whole batch)
+            if ended == curr:                                                        # mcts.py:174 (counts ended rows over the whole batch)
                 m.printTimers()
                 return results[:curr, :t + 1], results_len, batch_stats[:t + 1]
         m.printTimers()

@@ -24,6 +24,26 @@ def test_multi_draw_sampler_matches_oracle_and_single_draws():
     assert torch.equal(got, single)
 
 
+def test_row_temperature_sampler_matches_oracle():
+    """The sampler's temp <= 0 mode: one temperature per branch, quotients and probabilities in float32."""
+    from spec_mcts_amd import kernels as K
+    g = torch.Generator().manual_seed(81)
+    logits = (torch.randn((6, 32016), generator=g) * 2).half()
+    counts = torch.tensor([5, 1, 0, 30, 2, 12], dtype=torch.int32)
+    temps = O.ramp_temperature(-0.9, 50, counts)
+    assert temps.dtype == torch.float32 and float(temps[1]) == pytest.approx(0.1) and float(temps.max()) < 0.9
+    u = torch.rand(50, generator=g)
+    got = K.sample_topk_counts(logits.cuda(), temps.cuda(), 32, counts.cuda(), u.cuda()).cpu()
+    want = O.sample_topk_counts(logits, temps, 32, counts.tolist(), u)
+    assert torch.equal(got, want)
+    # one temperature for all rows, a power of two (the fp16 quotient is exact): the float32 mode draws what the fp16 mode
+    # draws wherever the fp16 rounding of the probabilities does not move a boundary across the uniform number
+    flat = torch.full((6,), 0.5)
+    a = K.sample_topk_counts(logits.cuda(), flat.cuda(), 32, counts.cuda(), u.cuda()).cpu()
+    b = K.sample_topk_counts(logits.cuda(), 0.5, 32, counts.cuda(), u.cuda()).cpu()
+    assert int((a != b).sum()) <= 1
+
+
 @pytest.mark.parametrize("seed", range(8))
 def test_tree_fork_kernel_matches_oracle(seed):
     """random trees: random multiplicities that sum to the batch size, a few dead branches, few distinct tokens (many
@@ -64,6 +84,10 @@ def test_tree_fork_kernel_matches_oracle(seed):
 CFG = dict(dim=256, n_layers=2, n_heads=2, vocab_size=320, multiple_of=128, max_batch_size=12, max_seq_len=10, max_prompt_seq_len=16)
 
 
+def _temperature(temp, batch_size, counts):
+    return temp if temp > 0.0 else O.ramp_temperature(temp, batch_size, counts)
+
+
 def _host_search(model, prompt, batch_size, depth, top_k, temp, uniforms):
     """The reference's search loop (mcts.py:67-182) with the oracle's bookkeeping on the host and row-copy forks."""
     from spec_mcts_amd import kernels as K
@@ -86,7 +110,8 @@ def _host_search(model, prompt, batch_size, depth, top_k, temp, uniforms):
             pos += 1
         # (the draws come from the device sampler, held against the oracle's in the test above: a probability on a rounding
         # boundary must not decide whether the two LOOPS agree)
-        draws = K.sample_topk_counts(logits[:, -1].contiguous(), temp, top_k, oc[1].cuda(), uniforms[t].cuda()).cpu()
+        tt = _temperature(temp, batch_size, oc[1])
+        draws = K.sample_topk_counts(logits[:, -1].contiguous(), tt.cuda() if isinstance(tt, torch.Tensor) else tt, top_k, oc[1].cuda(), uniforms[t].cuda()).cpu()
         new_cur, origin = O.tree_fork(draws, oc, alive, cur, batch_size, results, t)
         r = cur
         while r < new_cur:                                   # consecutive new rows of one origin = one model.fork call
@@ -105,7 +130,7 @@ def _host_search(model, prompt, batch_size, depth, top_k, temp, uniforms):
     return results[:cur], results_len, stats
 
 
-@pytest.mark.parametrize("seed,temp", [(0, 0.8), (1, 1.5), (2, 3.0)])
+@pytest.mark.parametrize("seed,temp", [(0, 0.8), (1, 1.5), (2, 3.0), (3, -2.5)])
 def test_device_search_equals_host_search(seed, temp):
     from spec_mcts_amd import ModelArgs
     from spec_mcts_amd.load_q40 import load_q40

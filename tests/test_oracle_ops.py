@@ -362,6 +362,33 @@ def test_noise_study_instruments_reduce_to_the_oracle_where_they_must():
     assert float(d) <= 2e-3
 
 
+def test_row_temperature_known_answers():
+    """The temp <= 0 mode of the tree sampler (mcts.py:110-114): the ramp's end points, and draws whose probabilities are
+    worked out by hand.  Two candidates with logits (0, T ln 3) at temperature T have probabilities (1/4, 3/4); in
+    descending order the cumulative sums are (3/4, 1): a uniform number below 3/4 picks the larger logit."""
+    counts = torch.tensor([1, 12, 4], dtype=torch.int32)
+    t = O.ramp_temperature(-0.7, 12, counts)
+    assert t.dtype == torch.float32
+    assert float(t[0]) == pytest.approx(0.1, abs=1e-7) and float(t[1]) == pytest.approx(0.7, abs=1e-6)
+    assert float(t[2]) == pytest.approx(0.1 + 0.6 * 3 / 11, abs=1e-6)
+    assert torch.equal(O.ramp_temperature(0.7, 12, counts), t)                 # the sign only selects the mode
+    ln3 = 1.0986328125                                                        # fp16(ln 3)
+    logits = torch.full((2, 8), -30.0, dtype=torch.float16)
+    logits[:, 5] = 0.0
+    logits[0, 2] = 0.5 * ln3                                                  # row 0 at T = 0.5
+    logits[1, 2] = 0.5 * ln3                                                  # row 1 at T = 1: p = (0.634, 0.366)
+    temps = torch.tensor([0.5, 1.0])
+    p, order = O.topk_probs(logits, temps, 2)
+    assert p.dtype == torch.float32 and order.tolist() == [[2, 5], [2, 5]]
+    assert float(p[0, 0]) == pytest.approx(0.75, abs=2e-4) and float(p[1, 0]) == pytest.approx(3 ** 0.5 / (1 + 3 ** 0.5), abs=2e-4)
+    u = torch.tensor([0.70, 0.80, 0.60, 0.70])
+    got = O.sample_topk_counts(logits, temps, 2, [2, 2], u)
+    assert got.tolist() == [2, 5, 2, 5]                                       # row 0: 0.70 < 3/4 <= 0.80; row 1: 0.60 < 0.634 <= 0.70
+    # a scalar temperature keeps the fp16 path: same candidates, probabilities rounded to fp16
+    p16, order16 = O.topk_probs(logits[:1], 0.5, 2)
+    assert p16.dtype == torch.float16 and order16.tolist() == [[2, 5]] and float(p16[0, 0]) == pytest.approx(0.75, abs=1e-3)
+
+
 def test_tree_fork_known_answers():
     """The expansion bookkeeping of the tree sampler (mcts.py:127-152) on a tree small enough to write every row out by hand."""
     B, steps = 6, 4
