@@ -347,20 +347,6 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
             decode(wv, sv, k_dead(cur), bn);
 #pragma unroll
             for (int o = 0; o < NB; ++o) bq[o] = bn[o];
-            // issue order asked of the scheduler: LDS reads first, then MFMAs with the decode's VALU between them (the matrix
-            // pipe works 16 cycles per MFMA and the wave's next instructions issue meanwhile); it follows this in part
-            // (the reads move to the front, about a third of the VALU between the MFMAs) and the launch is 3 % shorter
-            // at 100 rows; one or three VALU per MFMA measured slower than two
-            __builtin_amdgcn_sched_group_barrier(0x100, 3 + (TILES > 1 ? 2 : 1), 0);
-#pragma unroll
-            for (int t = 0; t < TILES; ++t) {
-#pragma unroll
-                for (int o = 0; o < NB; ++o) {
-                    __builtin_amdgcn_sched_group_barrier(0x008, 1, 0);
-                    __builtin_amdgcn_sched_group_barrier(0x002, 2, 0);
-                }
-                if (t + 2 < TILES) __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
-            }
         };
         typedef std::integral_constant<bool, true> yes;
         typedef std::integral_constant<bool, false> no;
