@@ -1,11 +1,11 @@
 // Q4_0 dequant + matmul for large batches (decode at B = 100, prefill): c[M,N] = a[M,K] . deq(W)[K,N].
 //
-// A workgroup of 4 waves owns 128 rows of A, two adjacent 128-column blocks of the weight (one full
-// 128-byte line of packed nibbles per k) and a slice of K; two workgroups share a compute unit.
-// Everything a 32-row step needs - 4 KB of nibbles, 256 B of scales, the 128 x 32 tile of A - goes
-// global -> LDS by DMA (global_load_lds) into a 4-stage ring shared by the workgroup; one bare
-// s_barrier per step both publishes a stage and frees the oldest one.  (__syncthreads() would wait
-// for every outstanding DMA first, because they write LDS, and so empty the ring at every step.)
+// A workgroup of 4 waves (8 on tiled weights, see the kernel) owns 128 rows of A, two adjacent 128-column blocks
+// of the weight (one full 128-byte line of packed nibbles per k) and a slice of K; two workgroups share a
+// compute unit.  Everything a 32-row step needs - 4 KB of nibbles, 256 B of scales, the 128 x 32 tile of A -
+// goes global -> LDS by DMA (global_load_lds) into a 6-slot ring shared by the workgroup; one bare s_barrier
+// per TWO steps both publishes stages and frees the oldest ones.  (__syncthreads() would wait for every
+// outstanding DMA first, because they write LDS, and so empty the ring at every barrier.)
 //   * wave w decodes TWO byte positions of ONE block (block w/2, bytes 2(w%2) and 2(w%2)+1 of every
 //     dword): perm pairs the byte of two consecutive rows, and-or drops the nibbles into fp16
 //     mantissas, one packed op recovers the exact code and one packed multiply applies the scales -
@@ -19,7 +19,7 @@
 //     row tiles and the ragged-K handling are template parameters), and the DMA addresses are a
 //     scalar base per step plus lane offsets that never change, so issuing a stage costs no VALU work;
 //   * the accumulators leave through LDS one row tile at a time, so global stores are 64-byte
-//     contiguous per lane; K-slices are written as slabs (fp16 above 16 rows) and added by the consuming kernel.
+//     contiguous per lane; K-slices are written as fp32 slabs and added by the consuming kernel.
 //
 // At M = 100 the work sits on the ridge of the roofline: 2*M*N*K flops against
 // N*K*0.53125 + 2*M*(K+N) bytes.
@@ -39,9 +39,10 @@ namespace smh {
 constexpr int GEMM_BM = 128;
 constexpr int GEMM_WAVES = 4;
 constexpr int GEMM_THREADS = GEMM_WAVES * 64;
-// stages of the DMA ring: four measured 2 % faster per launch at M=100 than six (five in between)
+// slots of the DMA ring (with a barrier per step, four slots measured 2 % faster per launch at M=100 than six; with a
+// barrier per two steps, six slots are 3 % faster than that)
 #ifndef SMH_GEMM_STAGES
-#define SMH_GEMM_STAGES 4
+#define SMH_GEMM_STAGES 6
 #endif
 constexpr int GEMM_STAGES = SMH_GEMM_STAGES;
 constexpr int GS_WBLOCK = 8 * 128 + 64;        // the 8 rows one wave fetches, padded by 16 banks: the four row groups a
@@ -202,7 +203,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
         fetch = fetch + 1 == step1 ? step0 : fetch + 1;
     };
 #pragma unroll
-    for (int i = 0; i < GEMM_STAGES - 1; ++i)
+    for (int i = 0; i < 4; ++i)
         if (i < n_steps) fetch_next(i);
 
     // the eight dwords of this lane's column bytes and of their scales, for one step
@@ -316,25 +317,24 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
             for (int o = 0; o < NB; ++o) acc[o][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], b[o], acc[o][t], 0, 0, 0);
         }
     };
+    // Steps go in pairs: ONE wait + barrier per two steps.  Six slots; at the barrier before steps i, i+1 the stages of
+    // steps i .. i+2 have landed (the B operands of step i+2 are decoded during step i+1), step i+3 may be in flight, and
+    // the slots of steps i-2, i-1 are refilled with steps i+4, i+5.  A stage has the same two steps of time to land as
+    // with a barrier per step; the waves meet half as often.
     if (n_steps > 0) {
+        static_assert(GEMM_STAGES == 6, "the paired loop counts on six slots");
         h8 bq[NB];
         int cur = step0 + rot;                 // step being multiplied
         int slot = 0;                          // its ring slot
         {
-            gemm_wait_dma<DMA_PER>(min(GEMM_STAGES - 2, n_steps - 1));
+            gemm_wait_dma<DMA_PER>(min(3, n_steps - 1));
             gemm_barrier();
             uint32_t wv[8], sv[8];
             load_ws(lds, wv, sv);
             decode(wv, sv, k_dead(cur), bq);
         }
-        // one iteration: multiply step i with bq while the B operands of step i+1 are decoded; REFILL is a
-        // compile-time flag so that the body of the main loop is one basic block with its DMA inside
-        auto iterate = [&](int i, auto refill) {
-            // stage i+1 has landed for this wave (the three younger ones may still be in flight) ...
-            if (refill.value) gemm_wait_dma<DMA_PER>(GEMM_STAGES - 3);
-            else gemm_wait_dma<DMA_PER>(min(GEMM_STAGES - 3, max(n_steps - 2 - i, 0)));
-            gemm_barrier();                    // ... and for everyone; everyone is done with stage i-1
-            if (refill.value) fetch_next(slot == 0 ? GEMM_STAGES - 1 : slot - 1);
+        // multiply the step in `slot` with bq while the B operands of the next step are decoded
+        auto one_step = [&]() {
             const uint8_t *st = lds + slot * GS_BYTES;
             slot = slot == GEMM_STAGES - 1 ? 0 : slot + 1;
             cur = cur + 1 == step1 ? step0 : cur + 1;
@@ -348,13 +348,26 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
 #pragma unroll
             for (int o = 0; o < NB; ++o) bq[o] = bn[o];
         };
-        typedef std::integral_constant<bool, true> yes;
-        typedef std::integral_constant<bool, false> no;
+        auto back = [&](int k) { return slot >= k ? slot - k : slot + GEMM_STAGES - k; };
         int i = 0;
 #pragma unroll 1
-        for (; i + GEMM_STAGES - 1 < n_steps; ++i) iterate(i, yes{});
+        for (; i + 5 < n_steps; i += 2) {      // both refills exist: the body is one basic block
+            gemm_wait_dma<DMA_PER>(1);
+            gemm_barrier();
+            fetch_next(back(2));
+            fetch_next(back(1));
+            one_step();
+            one_step();
+        }
 #pragma unroll 1
-        for (; i < n_steps; ++i) iterate(i, no{});
+        for (; i < n_steps; i += 2) {
+            gemm_wait_dma<DMA_PER>(i + 3 <= n_steps - 1 ? 1 : 0);
+            gemm_barrier();
+            if (i + 4 < n_steps) fetch_next(back(2));
+            if (i + 5 < n_steps) fetch_next(back(1));
+            one_step();
+            if (i + 1 < n_steps) one_step();
+        }
     }
 
     // ---- results leave one 16-row tile at a time through LDS: [16][256 + 4] floats, two buffers in turn ----
