@@ -83,7 +83,8 @@ def test_one_hot_rows_are_bit_exact(M):
     assert bool((zero == 0).all())
 
 
-@pytest.mark.parametrize("M,N,Kd", [(2, 128, 8), (5, 256, 40), (16, 128, 72), (40, 256, 200), (129, 128, 1000)])
+@pytest.mark.parametrize("M,N,Kd", [(2, 128, 8), (5, 256, 40), (16, 128, 72), (40, 256, 200), (129, 128, 1000),
+                                    (33, 128, 32), (40, 256, 96), (100, 128, 160), (17, 256, 224), (100, 384, 416)])
 def test_ragged_k_and_small_shapes(M, N, Kd):
     """K not a multiple of the 32-row step, single column block, M around the tile sizes"""
     from spec_mcts_amd import kernels as K

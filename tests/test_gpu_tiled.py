@@ -54,7 +54,9 @@ def test_tiles_match_the_layout_definition(K, N):
 
 @pytest.mark.parametrize("M", [1, 3, 10, 16, 17, 100, 130])
 @pytest.mark.parametrize("K,ns", [(64, [128]), (40, [384]), (4096, [4096]), (1000, [256, 128, 128]), (4096, [1024, 256, 256]),
-                                  (11008, [4096]), (4096, [11008, 11008])])
+                                  (11008, [4096]), (4096, [11008, 11008]),
+                                  # 1, 3, 5 and 7 steps of 32 rows: the ends of a loop that takes its steps in pairs
+                                  (32, [128]), (96, [256]), (160, [128]), (224, [384]), (416, [256])])
 def test_tiled_products_equal_checkpoint_layout_products(M, K, ns):
     """same operands into the same MFMAs in the same order: the slabs are bit-identical"""
     from spec_mcts_amd import kernels as Kn
