@@ -178,26 +178,27 @@ int smh_sample_topk(const void *logits, int rows, int vocab, long ld, float temp
 /* The expansion step of the tree sampler (mcts.py:115-152) without its per-branch Python loop and host round trips.
  * smh_sample_topk_counts: smh_sample_topk where row r makes counts[r] draws with replacement (torch.multinomial with
  *   num_samples = output_counts[1, r], :128): the draws of row r use uniform[o .. o + counts[r]) and fill out[o ..) with
- *   o = counts[0] + ... + counts[r-1].  counts int32 [rows] on the device; at most 1024 rows.
+ *   o = counts[0] + ... + counts[r-1].  counts int32 [rows] on the device; at most 1024 rows.  uniform and out hold
+ *   n_draws entries: draws beyond them (counts that add up to more) are not made.
  * smh_tree_fork: the bookkeeping of :127-152 for all *curr_b live branches in one launch: per branch, in order, the
  *   distinct drawn tokens in ascending order with their multiplicities (torch.unique, :131); an alive branch keeps the
  *   smallest on its row and opens one new row per further distinct token while rows are left (:141-150).  A new row
  *   receives the origin's token history (results row), token and multiplicity, and the origin's page ids of the
  *   n_rows suffix rows written so far (what Transformer.fork copies as K/V rows, hf_model_q40_kv_shared.py:282-297;
  *   pages may be NULL).  Then column t of every dead row is zeroed (:160).
- *     draws int64 [sum of cnt over live branches]; tok, cnt int32 [batch_size] = output_counts[0], [1] (:88-89);
+ *     draws int64 [n_draws] (the sum of cnt over the live branches; draws past n_draws are ignored); tok, cnt int32 [batch_size] = output_counts[0], [1] (:88-89);
  *     alive uint8 [batch_size] = results_mask; curr_b int32 on the device, updated; results int64 [batch_size, ld];
  *     pages int32 [batch_size, pages_stride]; origin int32 [batch_size]: the branch a row was forked from in this call, else -1.
  *   batch_size <= 1024. */
 int smh_sample_topk_counts(const void *logits, int rows, int vocab, long ld, float temperature, int top_k,
-                           const float *uniform, const int32_t *counts, int64_t *out, smh_stream_t stream);
+                           const float *uniform, const int32_t *counts, int64_t *out, int n_draws, smh_stream_t stream);
 /* smh_sample_topk_rowtemp: smh_sample_topk_counts with a temperature per row, row_temps fp32 [rows] on the device, all
  * positive - the tree sampler's temp <= 0 mode, where the logits of branch i are divided by a ramp of its multiplicity
  * (mcts.py:110-114).  There the divisor is a float32 TENSOR, which promotes the fp16 logits: quotients, softmax and
  * probabilities are fp32 here too (no fp16 rounding of x or p); the candidates are the top_k largest logits. */
 int smh_sample_topk_rowtemp(const void *logits, int rows, int vocab, long ld, const float *row_temps, int top_k,
-                            const float *uniform, const int32_t *counts, int64_t *out, smh_stream_t stream);
-int smh_tree_fork(const int64_t *draws, int32_t *tok, int32_t *cnt, const uint8_t *alive, int32_t *curr_b, int batch_size,
+                            const float *uniform, const int32_t *counts, int64_t *out, int n_draws, smh_stream_t stream);
+int smh_tree_fork(const int64_t *draws, int n_draws, int32_t *tok, int32_t *cnt, const uint8_t *alive, int32_t *curr_b, int batch_size,
                   int64_t *results, long ld, int t, int32_t *pages, long pages_stride, int n_rows, int32_t *origin,
                   smh_stream_t stream);
 /* smh_detect_terminal: detectTerminal (mcts.py:14-28) for `rows` branches in place: state[b] counts the tokens of

@@ -268,7 +268,7 @@ __device__ __forceinline__ void sample_pick_bin(int *bins, int want, int *out_bi
 // its candidates, with the uniform numbers (and into the slots of out) that start at counts[0] + ... + counts[r-1].
 __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restrict__ logits, int vocab, long ld, float temperature,
                                                            int top_k, const float *__restrict__ uniform, int64_t *__restrict__ out,
-                                                           const int32_t *__restrict__ counts, const float *__restrict__ row_temps) {
+                                                           const int32_t *__restrict__ counts, const float *__restrict__ row_temps, int n_draws) {
     // row_temps: a temperature per row, applied in fp32 (a tensor divisor promotes the fp16 logits to fp32 in torch, a
     // Python scalar does not): candidates by the raw logits (division by a positive number keeps their order, and two
     // different fp16 values stay different in fp32), softmax and probabilities in fp32
@@ -373,8 +373,9 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
     int draws = 1;
     if (counts != nullptr) {
         first = 0;
-        for (int r = 0; r < (int)blockIdx.x; ++r) first += counts[r];
-        draws = counts[blockIdx.x];
+        for (int r = 0; r < (int)blockIdx.x; ++r) first += max(counts[r], 0);
+        draws = max(counts[blockIdx.x], 0);
+        draws = (int)max(min((long)draws, (long)n_draws - first), 0L);       // counts that add up to more than the buffers hold are cut
     }
     if (tid < k) {
         const float before = tid == 0 ? 0.f : cdf[tid - 1];
@@ -397,7 +398,7 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
 //           zeroed (:160).
 //   tok / cnt = output_counts[0] / [1] of the reference; origin[r] = the branch row r was forked from in this step, else -1.
 constexpr int TREE_MAX_BATCH = 1024;
-__global__ __launch_bounds__(256) void tree_fork_kernel(const int64_t *__restrict__ draws, int32_t *__restrict__ tok, int32_t *__restrict__ cnt,
+__global__ __launch_bounds__(256) void tree_fork_kernel(const int64_t *__restrict__ draws, int n_draws, int32_t *__restrict__ tok, int32_t *__restrict__ cnt,
                                                         const uint8_t *__restrict__ alive, int32_t *__restrict__ curr_b, int batch_size,
                                                         int64_t *__restrict__ results, long ld, int t,
                                                         int32_t *__restrict__ pages, long pages_stride, int n_rows,
@@ -408,20 +409,20 @@ __global__ __launch_bounds__(256) void tree_fork_kernel(const int64_t *__restric
     __shared__ int seg_uniq[TREE_MAX_BATCH];       // distinct tokens of branch i
     __shared__ int s_new;                          // branches after the step
     const int tid = threadIdx.x;
-    const int c0 = *curr_b;
+    const int c0 = min(max(*curr_b, 0), batch_size);             // (a counter outside the batch is cut, never followed)
     if (tid == 0) {
         int off = 0;
-        for (int i = 0; i < c0; ++i) { seg_off[i] = off; off += cnt[i]; }
+        for (int i = 0; i < c0; ++i) { seg_off[i] = off; off = min(off + max(cnt[i], 0), TREE_MAX_BATCH); }
         seg_off[c0] = off;
     }
     __syncthreads();
-    const int total = min(seg_off[c0], TREE_MAX_BATCH);
+    const int total = min(seg_off[c0], min(n_draws, TREE_MAX_BATCH));   // draws the buffer does not hold do not exist
     for (int i = tid; i < total; i += 256) u_tok[i] = draws[i];
     for (int r = tid; r < batch_size; r += 256) origin[r] = -1;
     __syncthreads();
     // one thread per branch: insertion sort of its draws, then run-length encoding in place
     for (int i = tid; i < c0; i += 256) {
-        const int lo = seg_off[i], hi = min(seg_off[i + 1], TREE_MAX_BATCH);
+        const int lo = min(seg_off[i], total), hi = min(seg_off[i + 1], total);
         for (int a = lo + 1; a < hi; ++a) {
             const int64_t v = u_tok[a];
             int b = a - 1;
@@ -482,44 +483,44 @@ extern "C" int smh_sample_topk(const void *logits, int rows, int vocab, long ld,
     if (rows == 0) return 0;
     SMH_REQUIRE(logits && uniform && out, "smh_sample_topk: null pointer");
     hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, temperature,
-                       top_k, uniform, out, (const int32_t *)nullptr, (const float *)nullptr);
+                       top_k, uniform, out, (const int32_t *)nullptr, (const float *)nullptr, rows);
     return launch_status();
 }
 
 extern "C" int smh_sample_topk_counts(const void *logits, int rows, int vocab, long ld, float temperature, int top_k,
-                                      const float *uniform, const int32_t *counts, int64_t *out, smh_stream_t stream) {
+                                      const float *uniform, const int32_t *counts, int64_t *out, int n_draws, smh_stream_t stream) {
     using namespace smh;
     SMH_REQUIRE(rows >= 0 && rows <= TREE_MAX_BATCH && vocab > 0 && ld >= vocab, "smh_sample_topk_counts: rows=%d (at most %d) vocab=%d ld=%ld", rows, TREE_MAX_BATCH, vocab, ld);
     SMH_REQUIRE(top_k >= 1 && top_k <= SAMPLE_MAX_K, "smh_sample_topk_counts: top_k=%d outside [1,%d]", top_k, SAMPLE_MAX_K);
     SMH_REQUIRE(temperature > 0.f, "smh_sample_topk_counts: temperature=%g must be positive", (double)temperature);
     if (rows == 0) return 0;
-    SMH_REQUIRE(logits && uniform && counts && out, "smh_sample_topk_counts: null pointer");
+    SMH_REQUIRE(logits && uniform && counts && out && n_draws >= 0, "smh_sample_topk_counts: null pointer or n_draws=%d", n_draws);
     hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, temperature,
-                       top_k, uniform, out, counts, (const float *)nullptr);
+                       top_k, uniform, out, counts, (const float *)nullptr, n_draws);
     return launch_status();
 }
 
 extern "C" int smh_sample_topk_rowtemp(const void *logits, int rows, int vocab, long ld, const float *row_temps, int top_k,
-                                       const float *uniform, const int32_t *counts, int64_t *out, smh_stream_t stream) {
+                                       const float *uniform, const int32_t *counts, int64_t *out, int n_draws, smh_stream_t stream) {
     using namespace smh;
     SMH_REQUIRE(rows >= 0 && rows <= TREE_MAX_BATCH && vocab > 0 && ld >= vocab, "smh_sample_topk_rowtemp: rows=%d (at most %d) vocab=%d ld=%ld", rows, TREE_MAX_BATCH, vocab, ld);
     SMH_REQUIRE(top_k >= 1 && top_k <= SAMPLE_MAX_K, "smh_sample_topk_rowtemp: top_k=%d outside [1,%d]", top_k, SAMPLE_MAX_K);
     if (rows == 0) return 0;
-    SMH_REQUIRE(logits && row_temps && uniform && counts && out, "smh_sample_topk_rowtemp: null pointer");
+    SMH_REQUIRE(logits && row_temps && uniform && counts && out && n_draws >= 0, "smh_sample_topk_rowtemp: null pointer or n_draws=%d", n_draws);
     hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, 1.0f,
-                       top_k, uniform, out, counts, row_temps);
+                       top_k, uniform, out, counts, row_temps, n_draws);
     return launch_status();
 }
 
-extern "C" int smh_tree_fork(const int64_t *draws, int32_t *tok, int32_t *cnt, const uint8_t *alive, int32_t *curr_b, int batch_size,
+extern "C" int smh_tree_fork(const int64_t *draws, int n_draws, int32_t *tok, int32_t *cnt, const uint8_t *alive, int32_t *curr_b, int batch_size,
                              int64_t *results, long ld, int t, int32_t *pages, long pages_stride, int n_rows, int32_t *origin,
                              smh_stream_t stream) {
     using namespace smh;
     SMH_REQUIRE(batch_size >= 1 && batch_size <= TREE_MAX_BATCH, "smh_tree_fork: batch_size=%d outside [1,%d]", batch_size, TREE_MAX_BATCH);
-    SMH_REQUIRE(draws && tok && cnt && alive && curr_b && results && origin, "smh_tree_fork: null pointer");
+    SMH_REQUIRE(draws && n_draws >= 0 && tok && cnt && alive && curr_b && results && origin, "smh_tree_fork: null pointer or n_draws=%d", n_draws);
     SMH_REQUIRE(ld >= 1 && t >= 0 && t < ld, "smh_tree_fork: column %d outside the %ld of a row", t, ld);
     SMH_REQUIRE(pages == nullptr || (pages_stride >= n_rows && n_rows >= 0), "smh_tree_fork: n_rows=%d pages_stride=%ld", n_rows, pages_stride);
-    hipLaunchKernelGGL(tree_fork_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, draws, tok, cnt, alive, curr_b, batch_size, results, ld, t,
+    hipLaunchKernelGGL(tree_fork_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, draws, n_draws, tok, cnt, alive, curr_b, batch_size, results, ld, t,
                        pages, pages_stride, n_rows, origin);
     return launch_status();
 }

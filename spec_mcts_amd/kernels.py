@@ -467,10 +467,10 @@ def sample_topk_counts(logits: torch.Tensor, temperature, top_k: int, counts: to
         _need_gpu(temperature)
         assert temperature.dtype == torch.float32 and temperature.is_contiguous() and temperature.numel() >= rows
         check(lib.smh_sample_topk_rowtemp(logits.data_ptr(), rows, vocab, logits.stride(0), temperature.data_ptr(), int(min(top_k, vocab)),
-                                          uniform.data_ptr(), counts.data_ptr(), out.data_ptr(), _stream()), "smh_sample_topk_rowtemp")
+                                          uniform.data_ptr(), counts.data_ptr(), out.data_ptr(), uniform.numel(), _stream()), "smh_sample_topk_rowtemp")
         return out
     check(lib.smh_sample_topk_counts(logits.data_ptr(), rows, vocab, logits.stride(0), float(temperature), int(min(top_k, vocab)),
-                                     uniform.data_ptr(), counts.data_ptr(), out.data_ptr(), _stream()), "smh_sample_topk_counts")
+                                     uniform.data_ptr(), counts.data_ptr(), out.data_ptr(), uniform.numel(), _stream()), "smh_sample_topk_counts")
     return out
 
 
@@ -491,7 +491,7 @@ def tree_fork(draws: torch.Tensor, output_counts: torch.Tensor, alive: torch.Ten
         assert pages.is_cuda and pages.dtype == torch.int32 and pages.dim() == 2 and pages.is_contiguous() and pages.shape[0] >= batch
     if origin is None:
         origin = torch.empty(batch, dtype=torch.int32, device=results.device)
-    check(lib.smh_tree_fork(draws.data_ptr(), output_counts[0].data_ptr(), output_counts[1].data_ptr(), alive.data_ptr(), curr_b.data_ptr(),
+    check(lib.smh_tree_fork(draws.data_ptr(), draws.numel(), output_counts[0].data_ptr(), output_counts[1].data_ptr(), alive.data_ptr(), curr_b.data_ptr(),
                             batch, results.data_ptr(), results.shape[1], int(t), _ptr(pages), pages.shape[1] if pages is not None else 0,
                             int(n_rows), origin.data_ptr(), _stream()), "smh_tree_fork")
     return origin

@@ -24,6 +24,31 @@ def test_multi_draw_sampler_matches_oracle_and_single_draws():
     assert torch.equal(got, single)
 
 
+def test_counts_beyond_the_buffers_are_cut():
+    """counts that add up to more than uniform / out hold: the draws that fit are made, nothing is written past them;
+    the bookkeeping kernel likewise ignores draws its buffer does not hold and a branch counter outside the batch"""
+    from spec_mcts_amd import kernels as K
+    g = torch.Generator().manual_seed(82)
+    logits = (torch.randn((4, 4096), generator=g) * 2).half()
+    counts = torch.tensor([6, 9, 30, 5], dtype=torch.int32)
+    u = torch.rand(50, generator=g)
+    full = K.sample_topk_counts(logits.cuda(), 0.7, 16, counts.cuda(), u.cuda()).cpu()
+    out = torch.full((40,), -1, dtype=torch.int64, device="cuda:0")
+    K.sample_topk_counts(logits.cuda(), 0.7, 16, counts.cuda(), u[:20].contiguous().cuda(), out=out)
+    assert torch.equal(out[:20].cpu(), full[:20]) and bool((out[20:] == -1).all())
+    # bookkeeping: 4 branches want 50 draws, the buffer holds 8 (6 of branch 0, 2 of branch 1); curr_b says 9 of a batch of 6
+    draws = full[:8].contiguous().cuda()
+    oc = torch.zeros((2, 6), dtype=torch.int32)
+    oc[1, :4] = counts
+    oc_d = oc.cuda()
+    alive = torch.ones(6, dtype=torch.bool, device="cuda:0")
+    curr = torch.tensor([9], dtype=torch.int32, device="cuda:0")
+    results = torch.zeros((6, 4), dtype=torch.int64, device="cuda:0")
+    K.tree_fork(draws, oc_d, alive, curr, results, 0)
+    assert 1 <= int(curr) <= 6
+    assert int(results[0, 0]) == int(full[:6].min())              # branch 0 keeps its smallest distinct draw
+
+
 def test_row_temperature_sampler_matches_oracle():
     """The sampler's temp <= 0 mode: one temperature per branch, quotients and probabilities in float32."""
     from spec_mcts_amd import kernels as K
