@@ -268,14 +268,16 @@ int smh_prefill_attn(const void *q, const void *k, const void *v, void *out, int
  *                (0, 0 = token-major [P, Hkv, D]; a head-major pool [Hkv, rows, D] is (D, rows * D))
  *   pool         SMH_KV_FP16: pool_k/v fp16 with pool_row_stride / pool_head_stride as above;
  *                SMH_KV_Q40: the model's cache rows, bytes [rows, Hkv, 64] + scales fp16 [rows, Hkv, 2] (strides 0)
- *   pages        page ids [B, pages_stride] of page_bytes = 2, 4 or 8 bytes each (int16 as in the reference, int32, int64)
+ *   pages        page ids [B, pages_stride] of page_bytes = 2, 4 or 8 bytes each (int16 as in the reference, int32, int64);
+ *                the pool has pool_rows rows: an id outside 0 .. pool_rows-1 is read as the nearest valid row (a wrong
+ *                result for that branch, never an access outside the pool)
  *   lens         int32 [B] (lens_stride 1) or one shared int32 (lens_stride 0): pages of the branch that are valid
  *   single_launch, workspace: as smh_shared_prefix_attn_one (counters zeroed once) when != 0, else as smh_shared_prefix_attn
  * smh_page_fork: table[curr + i, 0..n-1] = table[origin, 0..n-1] for i < forks; table int32 [rows, stride]. */
 int smh_paged_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int D,
                           const void *prefix_k, const void *prefix_v, int P, long prefix_row_stride, long prefix_head_stride,
                           int pool_format, const void *pool_k, const void *pool_v, const void *pool_ks, const void *pool_vs,
-                          long pool_row_stride, long pool_head_stride,
+                          long pool_row_stride, long pool_head_stride, long pool_rows,
                           const void *pages, int page_bytes, long pages_stride, const int32_t *lens, int lens_stride,
                           const void *cur_k, const void *cur_v, int single_launch,
                           void *workspace, size_t workspace_bytes, smh_stream_t stream);

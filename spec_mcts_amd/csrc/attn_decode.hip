@@ -47,6 +47,7 @@ struct AttnParams {
     const void *pages;
     long pages_stride;
     int page_bytes;
+    long pool_rows;          // rows of the pool the page ids point into: an id outside 0 .. pool_rows-1 reads the nearest row, never past the pool
     // element strides of the fp16 K/V tensors: between consecutive rows (tokens) and between kv heads.  Token-major
     // [rows, Hkv, 128] is (Hkv * 128, 128); a head-major pool [Hkv, rows, 128] is (128, rows * 128).  Q4_0 rows are token-major.
     long pfx_row_stride, pfx_head_stride;
@@ -496,9 +497,11 @@ __device__ __forceinline__ void attn_suffix_body(const AttnParams &p, int b, int
     auto row_of = [&](int t) -> long {
         if (p.pages == nullptr) return row0 + t;
         const long i = (long)b * p.pages_stride + t;
-        if (p.page_bytes == 4) return reinterpret_cast<const int32_t *>(p.pages)[i];
-        if (p.page_bytes == 2) return reinterpret_cast<const int16_t *>(p.pages)[i];
-        return reinterpret_cast<const int64_t *>(p.pages)[i];
+        long id;
+        if (p.page_bytes == 4) id = reinterpret_cast<const int32_t *>(p.pages)[i];
+        else if (p.page_bytes == 2) id = reinterpret_cast<const int16_t *>(p.pages)[i];
+        else id = reinterpret_cast<const int64_t *>(p.pages)[i];
+        return min(max(id, 0L), p.pool_rows - 1);
     };
     // ---- Q4_0 suffix rows: a wave takes Q4_ROWS rows per pass (row slot Q4_DW g + rl) and Q4_CH passes per chunk; wave
     // `sub` of the nsub that share a query takes every nsub-th pass.  All loads of a chunk are requested together, and
@@ -984,6 +987,7 @@ struct AttnExtras {
     const void *pages = nullptr;
     long pages_stride = 0;
     int page_bytes = 4;
+    long pool_rows = 0;
     long pfx_row = 0, pfx_head = 0, sfx_row = 0, sfx_head = 0;
 };
 
@@ -1015,7 +1019,7 @@ static int shared_prefix_attn(const char *who, bool one, const void *q, void *ou
     p.lens = lens; p.lens_stride = lens_stride;
     p.cur_k = (const half_t *)cur_k; p.cur_v = (const half_t *)cur_v;
     p.suffix_batch_stride_rows = Smax;
-    p.pages = ex.pages; p.pages_stride = ex.pages_stride; p.page_bytes = ex.page_bytes;
+    p.pages = ex.pages; p.pages_stride = ex.pages_stride; p.page_bytes = ex.page_bytes; p.pool_rows = ex.pool_rows;
     p.pfx_row_stride = ex.pfx_row ? ex.pfx_row : (long)Hkv * ATT_D; p.pfx_head_stride = ex.pfx_head ? ex.pfx_head : ATT_D;
     p.sfx_row_stride = ex.sfx_row ? ex.sfx_row : (long)Hkv * ATT_D; p.sfx_head_stride = ex.sfx_head ? ex.sfx_head : ATT_D;
     p.B = B; p.H = H; p.Hkv = Hkv; p.n_rep = H / Hkv; p.Bq = B * p.n_rep;
@@ -1064,7 +1068,7 @@ extern "C" int smh_shared_prefix_attn(const void *q, void *out, int B, int H, in
 extern "C" int smh_paged_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int D,
                                      const void *prefix_k, const void *prefix_v, int P, long prefix_row_stride, long prefix_head_stride,
                                      int pool_format, const void *pool_k, const void *pool_v, const void *pool_ks, const void *pool_vs,
-                                     long pool_row_stride, long pool_head_stride,
+                                     long pool_row_stride, long pool_head_stride, long pool_rows,
                                      const void *pages, int page_bytes, long pages_stride, const int32_t *lens, int lens_stride,
                                      const void *cur_k, const void *cur_v, int single_launch,
                                      void *workspace, size_t workspace_bytes, smh_stream_t stream) {
@@ -1074,12 +1078,13 @@ extern "C" int smh_paged_prefix_attn(const void *q, void *out, int B, int H, int
     SMH_REQUIRE(pages != nullptr && (page_bytes == 2 || page_bytes == 4 || page_bytes == 8) && pages_stride >= 1,
                 "%s: pages=%p page_bytes=%d (2, 4 or 8) pages_stride=%ld", who, pages, page_bytes, pages_stride);
     SMH_REQUIRE(pages_stride <= 0x7fffffffL, "%s: pages_stride=%ld", who, pages_stride);
+    SMH_REQUIRE(pool_rows >= 1, "%s: pool_rows=%ld", who, pool_rows);
     SMH_REQUIRE(prefix_row_stride >= 0 && prefix_head_stride >= 0 && pool_row_stride >= 0 && pool_head_stride >= 0 &&
                 prefix_row_stride % 8 == 0 && prefix_head_stride % 8 == 0 && pool_row_stride % 4 == 0 && pool_head_stride % 4 == 0,
                 "%s: strides must be non-negative (0 = token-major), prefix strides multiples of 8 and pool strides multiples of 4 elements", who);
     SMH_REQUIRE(pool_format != SMH_KV_Q40 || (pool_row_stride == 0 && pool_head_stride == 0), "%s: Q4_0 pools are token-major (strides 0)", who);
     AttnExtras ex;
-    ex.pages = pages; ex.page_bytes = page_bytes; ex.pages_stride = pages_stride;
+    ex.pages = pages; ex.page_bytes = page_bytes; ex.pages_stride = pages_stride; ex.pool_rows = pool_rows;
     ex.pfx_row = prefix_row_stride; ex.pfx_head = prefix_head_stride; ex.sfx_row = pool_row_stride; ex.sfx_head = pool_head_stride;
     return shared_prefix_attn(who, single_launch != 0, q, out, B, H, Hkv, D, prefix_k, prefix_v, P, pool_format, pool_k, pool_v, pool_ks, pool_vs,
                               (int)pages_stride, lens, lens_stride, cur_k, cur_v, workspace, workspace_bytes, stream, ex);
@@ -1199,7 +1204,7 @@ extern "C" int smh_shared_prefix_attn_qkv(const void *qkv_partial, int ksplit, v
     p.suffix_ks = (const half_t *)cache_ks; p.suffix_vs = (const half_t *)cache_vs;
     p.lens = t_dev; p.lens_stride = 0;
     p.suffix_batch_stride_rows = Smax;
-    p.pages = pages; p.pages_stride = pages_stride; p.page_bytes = 4;
+    p.pages = pages; p.pages_stride = pages_stride; p.page_bytes = 4; p.pool_rows = (long)B * Smax;   // a branch reads its own rows and its ancestors', all below B
     p.pfx_row_stride = (long)Hkv * ATT_D; p.pfx_head_stride = ATT_D;
     p.sfx_row_stride = (long)Hkv * ATT_D; p.sfx_head_stride = ATT_D;
     p.B = B; p.H = H; p.Hkv = Hkv; p.n_rep = H / Hkv; p.Bq = B * p.n_rep;

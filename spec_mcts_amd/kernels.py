@@ -739,6 +739,7 @@ def paged_prefix_attn(q: torch.Tensor, pages: torch.Tensor, lens: torch.Tensor, 
         assert pool_ks.dtype == torch.float16 and pool_vs.dtype == torch.float16 and pool_ks.is_contiguous() and pool_vs.is_contiguous()
         assert pool_k.dim() == 3 and pool_k.shape[2] == 64
         Hkv = pool_k.shape[1]
+        rows = pool_k.shape[0]
         row_stride = head_stride = 0
     assert H % Hkv == 0
     p_row = p_head = 0
@@ -758,7 +759,7 @@ def paged_prefix_attn(q: torch.Tensor, pages: torch.Tensor, lens: torch.Tensor, 
     ws = attn_qkv_workspace(q.device, B, H, P) if one else attn_workspace(q.device, B, H, P)
     check(lib.smh_paged_prefix_attn(q.data_ptr(), out.data_ptr(), B, H, Hkv, D, _ptr(prefix_k) if P else None, _ptr(prefix_v) if P else None,
                                     int(P), p_row, p_head, fmt, pool_k.data_ptr(), pool_v.data_ptr(), _ptr(pool_ks), _ptr(pool_vs),
-                                    row_stride, head_stride, pages.data_ptr(), pages.element_size(), pages.stride(0),
+                                    row_stride, head_stride, int(rows), pages.data_ptr(), pages.element_size(), pages.stride(0),
                                     lens.data_ptr(), int(lens_stride), _ptr(cur_k), _ptr(cur_v), int(one), ws.data_ptr(), ws.numel(), _stream()),
           "smh_paged_prefix_attn")
     return out

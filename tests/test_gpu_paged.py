@@ -116,6 +116,25 @@ def test_paged_q40_pool_ragged_lengths_and_current_token(dtype, single_launch):
     assert torch.equal(a, b_)
 
 
+def test_page_ids_outside_the_pool_read_the_nearest_row():
+    """A page id below 0 or past the pool (a corrupted table) is read as row 0 or the last row: the affected branch's
+    result is that of the cut table, bit for bit, and nothing outside the pool is touched."""
+    from spec_mcts_amd import kernels as K
+    B, H, Hkv, D, S, rows = 4, 4, 2, 128, 24, 64
+    g = torch.Generator().manual_seed(78)
+    q = torch.randn((B, H, D), generator=g).half()
+    kw, ks = O.quantize_q40(torch.randn((rows, Hkv, D), generator=g).half(), 64)
+    vw, vs = O.quantize_q40(torch.randn((rows, Hkv, D), generator=g).half(), 64)
+    pages = torch.randint(0, rows, (B, S), generator=g).to(torch.int32)
+    bad = pages.clone()
+    bad[1, 3], bad[2, 0], bad[3, 20] = -7, rows + 1000, 2 ** 30
+    lens = torch.tensor([24, 24, 10, 21], dtype=torch.int32)
+    args = (kw.view(rows, Hkv, 64).cuda(), vw.view(rows, Hkv, 64).cuda(), ks.view(rows, Hkv, 2).cuda(), vs.view(rows, Hkv, 2).cuda())
+    got = K.paged_prefix_attn(q.cuda(), bad.cuda(), lens.cuda(), *args)
+    want = K.paged_prefix_attn(q.cuda(), bad.clamp(0, rows - 1).cuda(), lens.cuda(), *args)
+    assert torch.equal(got, want) and bool(torch.isfinite(got.float()).all())
+
+
 def test_page_fork_copies_page_ids():
     from spec_mcts_amd import kernels as K
     table = torch.arange(8 * 300, dtype=torch.int32).view(8, 300).cuda()
