@@ -83,10 +83,9 @@ int smh_q40_matmul(const void *a, int M, int K, long lda, const void *b_w, const
  * partial[ksplit][M][n_total]; the operator that FOLLOWS the linear in the model adds the slabs
  * (in fp32, in slice order), rounds once to fp16 - the value matmul_q40 returns - and carries on, so no
  * kernel waits for another workgroup and a decode layer needs 4 weight-streaming launches.
- * The slabs are opaque to the caller: they hold fp32 when M <= SMH_GEMV_MAX_M and fp16 above (at those
- * batch sizes slab traffic would otherwise exceed the weight traffic); producer and consumer derive the
- * type from M (B for the rope operator), so the consumer must be given the M the producer was given.
- * Sizes below are upper bounds in bytes for either type.
+ * The slabs hold fp32 at every batch size (a partial sum rounded to fp16 before the final addition is a cast point
+ * the reference does not have); the consumer must be given the M (B for the rope operator) and the ksplit the
+ * producer used.  Sizes below are in bytes.
  * Up to 3 weights that share the input (wq|wk|wv of Attention.forward,
  * hf_model_q40_kv_shared.py:313; w1|w3 of FeedForward.forward, :434) run as segments of one
  * launch; their outputs are concatenated along the columns (n_total = sum of n[i]).

@@ -1,6 +1,6 @@
 // Consumers of the Q4_0 matmul's K-slice slabs.
 //
-// The matmul kernels leave `ksplit` slabs partial[s][m][n] (fp32 up to 16 rows, fp16 above: slab_is_half);
+// The matmul kernels leave `ksplit` slabs partial[s][m][n] (fp32);
 // every kernel here first forms acc = sum_s partial[s][m][n] in fp32 (slice order, so the result does not depend on scheduling), rounds
 // it ONCE to fp16 - the value the reference's matmul_q40 returns - and then applies the operator
 // that follows the linear in the model:
@@ -23,7 +23,7 @@ __global__ __launch_bounds__(256) void partial_reduce_kernel(const void *__restr
     const long i = ((long)blockIdx.x * 256 + threadIdx.x) * 4;
     if (i >= (long)M * N) return;
     const int m = (int)(i / N), n = (int)(i % N);          // N % 4 == 0: the 4 columns share a row
-    const f4 acc = slab_sum4(partial, (long)m * n_total + col0 + n, (long)M * n_total, ksplit, slab_is_half(M));
+    const f4 acc = slab_sum4(partial, (long)m * n_total + col0 + n, (long)M * n_total, ksplit);
     h4 out;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -58,7 +58,7 @@ __global__ __launch_bounds__(1024) void partial_rmsnorm_kernel(const void *__res
         if (n < N) {
             h4 v;
             if (partial != nullptr) {
-                const f4 acc = slab_sum4(partial, (long)m * N + n, slab, ksplit, slab_is_half(M));
+                const f4 acc = slab_sum4(partial, (long)m * N + n, slab, ksplit);
 #pragma unroll
                 for (int j = 0; j < 4; ++j) v[j] = (half_t)acc[j];
                 if (h_in != nullptr) {
@@ -115,7 +115,7 @@ __global__ __launch_bounds__(64) void partial_residual_sumsq_kernel(const void *
     for (int ps = 0; ps < MAXPASS; ++ps) {
         const int n = (ps * 1024 + vt) * 4;
         if (n < N) {
-            acc[ps] = slab_sum4(partial, (long)m * N + n, slab, ksplit, slab_is_half(M));
+            acc[ps] = slab_sum4(partial, (long)m * N + n, slab, ksplit);
             if (h_in != nullptr) res[ps] = *reinterpret_cast<const h4 *>(h_in + (long)m * N + n);
         }
     }
@@ -147,8 +147,8 @@ __global__ __launch_bounds__(256) void partial_silu_mul_kernel(const void *__res
     const int m = blockIdx.y, n = (blockIdx.x * 256 + threadIdx.x) * 4;
     if (n >= n_half) return;
     const long slab = (long)M * 2 * n_half;
-    const f4 ga = slab_sum4(partial, (long)m * 2 * n_half + n, slab, ksplit, slab_is_half(M));
-    const f4 ua = slab_sum4(partial, (long)m * 2 * n_half + n_half + n, slab, ksplit, slab_is_half(M));
+    const f4 ga = slab_sum4(partial, (long)m * 2 * n_half + n, slab, ksplit);
+    const f4 ua = slab_sum4(partial, (long)m * 2 * n_half + n_half + n, slab, ksplit);
     h4 o;
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
@@ -185,7 +185,7 @@ __global__ __launch_bounds__(256) void partial_rope_append_kernel(const void *__
     const int pos = *pos_dev;
     const half_t cos_l = cos_tab[(long)pos * 64 + lane], sin_l = sin_tab[(long)pos * 64 + lane];
     if (live) {
-        const f2 sum = slab_sum2(partial, (long)b * n_total + (long)h * 128 + 2 * lane, (long)B * n_total, ksplit, slab_is_half(B));
+        const f2 sum = slab_sum2(partial, (long)b * n_total + (long)h * 128 + 2 * lane, (long)B * n_total, ksplit);
         *reinterpret_cast<f2 *>(&s_row[wave][2 * lane]) = sum;
     }
     __syncthreads();
@@ -241,7 +241,6 @@ static int fill_params(MatmulParams &p, const void *a, int M, int K, long lda, i
         p.seg[i].N = n[i];
     }
     if (M <= SMH_GEMV_MAX_M) gemv_fill_plan(p); else gemm_fill_plan(p);
-    p.slab_half = slab_is_half(M);
     return 0;
 }
 

@@ -419,20 +419,6 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
                         *reinterpret_cast<h8 *>(p.c + (long)m * p.ldc + n) = o;
                     }
                 }
-            } else if (p.slab_half) {
-                half_t *dst = reinterpret_cast<half_t *>(p.partial) + ((long)slice * p.M + m) * p.n_total + seg.col0 + col0;
-#pragma unroll
-                for (int q = (WAVES == 8 ? o_half : 0); q < (WAVES == 8 ? o_half + 1 : 2); ++q) {
-                    const int cq = 128 * q + 8 * o_lane;
-                    if (col0 + cq < seg.N) {
-                        const f4 v0 = *reinterpret_cast<const f4 *>(otile + o_row * OP + cq);
-                        const f4 v1 = *reinterpret_cast<const f4 *>(otile + o_row * OP + cq + 4);
-                        h8 o;
-#pragma unroll
-                        for (int e = 0; e < 4; ++e) { o[e] = (half_t)v0[e]; o[4 + e] = (half_t)v1[e]; }
-                        *reinterpret_cast<h8 *>(dst + cq) = o;
-                    }
-                }
             } else {
                 float *dst = slab + (long)m * p.n_total + seg.col0 + col0;
 #pragma unroll

@@ -348,8 +348,8 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void q40_gemv_kernel(MatmulParams 
             if (idx < total) {
                 const int m = row_of(idx), k = slice_k0 + 4 * (idx - m * quads);
                 if (k < p.K) {
-                    ga[i] = slab_sum4(p.gu_partial, (long)m * 2 * p.K + k, gu_slab, p.gu_ksplit, false);
-                    ua[i] = slab_sum4(p.gu_partial, (long)m * 2 * p.K + p.K + k, gu_slab, p.gu_ksplit, false);
+                    ga[i] = slab_sum4(p.gu_partial, (long)m * 2 * p.K + k, gu_slab, p.gu_ksplit);
+                    ua[i] = slab_sum4(p.gu_partial, (long)m * 2 * p.K + p.K + k, gu_slab, p.gu_ksplit);
                 } else {
                     ga[i] = f4{0.f, 0.f, 0.f, 0.f};
                     ua[i] = f4{0.f, 0.f, 0.f, 0.f};

@@ -61,7 +61,6 @@ struct MatmulParams {
     int mblocks;             // GEMM: 128-row blocks
     int ksplit, steps_per_slice;
     int epilogue, direct;
-    int slab_half;           // slabs hold fp16 instead of fp32 (see slab_is_half)
     int tiled;               // the segments' weights are in the tiled layout
     // GEMV, at most SMH_SILU_IN_MAX_M rows: the activations are not read from `a` but made by every workgroup for
     // its own K-slice from the slabs of the gate|up product, a[m][k] = silu(gate[m][k]) * up[m][k] (gate = columns
@@ -81,9 +80,6 @@ __device__ __forceinline__ half_t matmul_epilogue(const MatmulParams &p, float a
     if (p.epilogue == SMH_EPI_RESIDUAL) v = (half_t)((float)p.resid[(long)m * p.ldr + n] + (float)v);
     return v;
 }
-
-// The dtype of the slabs follows from the row count alone, so producer and consumer agree without a flag.
-__host__ __device__ inline bool slab_is_half(int M) { (void)M; return false; }
 
 void gemv_fill_plan(MatmulParams &p);
 int gemv_launch(const MatmulParams &p, hipStream_t stream);
