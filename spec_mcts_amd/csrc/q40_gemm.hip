@@ -145,6 +145,17 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
     const uint32_t s_voff = (uint32_t)(s_lrow * s_row + s_lcol);
     const uint32_t a_voff0 = (uint32_t)(a_r0 + 16 * a_chunk), a_voff1 = (uint32_t)(a_r1 + 16 * a_chunk);
 
+    // eight waves: the two DMA instructions of a wave and stage separately, so that the A rows' (no branch around it)
+    // can go between the MFMAs of a step
+    auto issue_ws8 = [&](int step, int slot_) {
+        uint8_t *st = lds + slot_ * GS_BYTES;
+        const uint8_t *tile = w_base + (long)step * TILE_BYTES;
+        if (hh == 0) __builtin_amdgcn_global_load_lds((gptr_t)(tile + wave * 1024 + lane * 16), (lptr_t)(st + wave * 1024), 16, 0, 0);
+        else if (lane < 16) __builtin_amdgcn_global_load_lds((gptr_t)(tile + TILE_W_BYTES + (16 * wave + lane) * 4), (lptr_t)(st + GS_W + wave * 64), 4, 0, 0);
+    };
+    auto issue_a8 = [&](int step, int slot_) {
+        __builtin_amdgcn_global_load_lds((gptr_t)(a_base + (long)step * 64 + a_voff0), (lptr_t)(lds + slot_ * GS_BYTES + GS_W + GS_S + wave8 * 1024), 16, 0, 0);
+    };
     auto issue = [&](int step, int slot_) {
         uint8_t *st = lds + slot_ * GS_BYTES;
         const long k0 = (long)step * 32;
@@ -354,10 +365,45 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
         for (; i + 5 < n_steps; i += 2) {      // both refills exist: the body is one basic block
             gemm_wait_dma<DMA_PER>(1);
             gemm_barrier();
-            fetch_next(back(2));
-            fetch_next(back(1));
-            one_step();
-            one_step();
+            if constexpr (TILED && WAVES == 8) {
+                // the nibbles and scales of the two refills now, their A rows from inside the steps: the address unit takes
+                // 16 cycles per instruction, and between MFMAs the wave has them to spare (2 % off a launch at 100 rows;
+                // the nibbles and scales too from inside the steps, behind their branches: 4 % slower)
+                const int sa = back(2), sb = back(1);
+                const int fa = fetch, fb = fetch + 1 == step1 ? step0 : fetch + 1;
+                fetch = fb + 1 == step1 ? step0 : fb + 1;
+                issue_ws8(fa, sa);
+                issue_ws8(fb, sb);
+                for (int half = 0; half < 2; ++half) {
+                    const uint8_t *st = lds + slot * GS_BYTES;
+                    slot = slot == GEMM_STAGES - 1 ? 0 : slot + 1;
+                    cur = cur + 1 == step1 ? step0 : cur + 1;
+                    uint32_t wv[8], sv[8];
+                    h8 av[TILES], bn[NB];
+                    load_a(st, av);
+                    load_ws(lds + slot * GS_BYTES, wv, sv);
+                    constexpr int T0 = TILES / 2;
+#pragma unroll
+                    for (int t = 0; t < T0; ++t)
+#pragma unroll
+                        for (int o = 0; o < NB; ++o) acc[o][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], bq[o], acc[o][t], 0, 0, 0);
+                    __builtin_amdgcn_sched_barrier(0);
+                    issue_a8(half == 0 ? fa : fb, half == 0 ? sa : sb);
+                    __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+                    for (int t = T0; t < TILES; ++t)
+#pragma unroll
+                        for (int o = 0; o < NB; ++o) acc[o][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], bq[o], acc[o][t], 0, 0, 0);
+                    decode(wv, sv, k_dead(cur), bn);
+#pragma unroll
+                    for (int o = 0; o < NB; ++o) bq[o] = bn[o];
+                }
+            } else {
+                fetch_next(back(2));
+                fetch_next(back(1));
+                one_step();
+                one_step();
+            }
         }
 #pragma unroll 1
         for (; i < n_steps; i += 2) {
