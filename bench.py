@@ -42,7 +42,7 @@ ARCHS = {
 GEMV_TRAFFIC_BYTES_PER_LAUNCH = 27457461
 # the same for q40_gemm_kernel at M=100 (profiles/q40_gemm_m100_hbm_traffic.md): 37.29 MB read + 30.26 MB written
 # (the fp32 partial sums of the K-slices are most of the writes)
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 67551731
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 67528753
 # the same for one call of the decode attention leg (profiles/attn_decode_hbm_traffic.md): 65.6 MB read + 9.0 MB written
 ATTN_TRAFFIC_BYTES_PER_CALL = 74601580
 

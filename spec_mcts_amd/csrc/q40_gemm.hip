@@ -365,7 +365,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
         for (; i + 5 < n_steps; i += 2) {      // both refills exist: the body is one basic block
             gemm_wait_dma<DMA_PER>(1);
             gemm_barrier();
-            if constexpr (TILED && WAVES == 8) {
+            if constexpr (TILED && WAVES == 8 && TILES < 8) {       // (with all 8 row tiles, the prefill, this form measured 5-8 % slower)
                 // the nibbles and scales of the two refills now, their A rows from inside the steps: the address unit takes
                 // 16 cycles per instruction, and between MFMAs the wave has them to spare (2 % off a launch at 100 rows;
                 // the nibbles and scales too from inside the steps, behind their branches: 4 % slower)
