@@ -78,6 +78,16 @@ int smh_q40_matmul(const void *a, int M, int K, long lda, const void *b_w, const
                    void *c, long ldc, int epilogue, const void *residual, long ldr,
                    void *workspace, size_t workspace_bytes, smh_stream_t stream);
 
+/* The block-of-32 flavour of Q4_0 that the benchmark's first configuration describes in words (32-weight blocks along the
+ * input dimension, one fp16 scale = absmax / 8 per block, nibbles q in [0, 15], value = (q - 8) * scale).  The reference's
+ * code has no such format (fp16_to_int4.py:52-96 is the 64-group, absmax / 7, signed-nibble layout above); these two entry
+ * points exist so that that configuration can be run as written: smh_gq40_quantize packs fp16 values [blocks, 32] into
+ * 16 bytes per block (element j in the low nibble of byte j, element j + 16 in the high nibble) + one fp16 scale, with the
+ * reference quantiser's roundings (scale = fp16(absmax / 8), q = rint(fp16(x / scale)) + 8 cut to 0..15, 0 / 0 -> 8);
+ * smh_gq40_dequant is its inverse, one fp16 multiply per weight.  Pointers 16-byte aligned. */
+int smh_gq40_quantize(const void *in, void *packed, void *scale, long blocks, smh_stream_t stream);
+int smh_gq40_dequant(const void *packed, const void *scale, void *out, long blocks, smh_stream_t stream);
+
 /* ---- fused decode-layer operators ------------------------------------------------------------
  * The matmul kernels cut K into `ksplit` slices and leave one slab per slice,
  * partial[ksplit][M][n_total]; the operator that FOLLOWS the linear in the model adds the slabs

@@ -13,6 +13,10 @@ live in tests/test_oracle_*.py):
                                  integer-only C restatement (oracle/q40_ref.c) and numpy float16;
                                  quantiser invariants (code range, |err| <= scale/2, idempotence),
                                  brute force on tiny groups with exact rationals.
+  quantize_gq40 / dequantize_gq40  (the block-of-32 flavour of the benchmark's first configuration; no counterpart in the
+                                 reference's code) every (nibble, fp16 scale) pair against integer arithmetic on the
+                                 bit patterns; |error| <= scale / 2 except at +absmax (cut from 16 to 15: one scale);
+                                 re-quantising a dequantised tensor reproduces the codes.
   weight layout                  closed-form byte map  byte(k, (n//128)*64 + n%64), high nibble
                                  iff n%128 < 64, scale s[k, n//64]  checked element by element.
   matmul_q40                     float64 dense matmul of the dequantised matrix; one-hot inputs
@@ -83,6 +87,40 @@ def dequantize_q40(w: torch.Tensor, scale: torch.Tensor, group_size: int, shape,
     lsb = (w << 4) >> 4
     q = torch.hstack((msb, lsb)).view(-1, group_size)
     return (q * scale.view(-1, 1)).type(ptdtype).reshape(shape)
+
+
+# The OTHER Q4_0 flavour: the one the benchmark's first configuration spells out in words (32-weight blocks along the input
+# dimension, one fp16 scale = absmax / 8 per block, nibbles q in [0, 15] packed two per byte, value = (q - 8) * scale).
+# The reference's code has no such format (its Q4_0 is the 64-group, absmax / 7, signed-nibble layout above); this is a
+# restatement of that text, with the arithmetic conventions of the reference's own quantiser where the text is silent:
+# the scale is fp16(absmax / 8.0), the quotient w / scale is an fp16 division, codes round half to even, 0 / 0 gives q = 8,
+# and element j of a block shares byte j with element j + 16 (low nibble, high nibble) as the widespread block format does.
+GQ_BLOCK = 32
+
+
+def quantize_gq40(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """w fp16 [..., K] with K % 32 == 0 -> (packed uint8 [numel/32, 16], scale fp16 [numel/32])."""
+    assert w.dtype == DTYPE and w.shape[-1] % GQ_BLOCK == 0
+    blocks = w.reshape(-1, GQ_BLOCK)
+    scale = (blocks.abs().max(dim=1).values / 8.0).type(DTYPE)
+    quot = blocks / scale[:, None]                                   # fp16 / fp16
+    # (a scale that underflows to 0 under a non-zero block gives +-inf: cut like any quotient outside the code range)
+    q = torch.nan_to_num(torch.round(quot).float(), nan=0.0, posinf=8.0, neginf=-8.0).clamp(-8.0, 8.0).to(torch.int32) + 8
+    q = q.clamp(0, 15)                                               # +absmax maps to 16: cut to 15
+    packed = (q[:, :16] | (q[:, 16:] << 4)).to(torch.uint8)
+    return packed.contiguous(), scale
+
+
+def dequantize_gq40(packed: torch.Tensor, scale: torch.Tensor, shape) -> torch.Tensor:
+    """value = (q - 8) * scale, ONE fp16 multiply per weight."""
+    p32 = packed.to(torch.int32)
+    q = torch.cat((p32 & 15, p32 >> 4), dim=1) - 8                   # [blocks, 32]
+    return (q.to(torch.int8) * scale.view(-1, 1)).type(DTYPE).reshape(shape)
+
+
+def linear_gq40(x: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor, shape) -> torch.Tensor:
+    """y = x . W^T with W [N, K] held in the block format: dequantise to fp16, accumulate in fp32, round once."""
+    return (x.float() @ dequantize_gq40(packed, scale, shape).float().t()).to(DTYPE)
 
 
 def unpack_codes(w: torch.Tensor) -> torch.Tensor:

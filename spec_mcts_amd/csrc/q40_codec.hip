@@ -221,6 +221,90 @@ extern "C" int smh_q40_dequant(const void *w, const void *s, void *out, long row
     return launch_status();
 }
 
+// ---- the block-of-32 flavour (scale = absmax / 8, codes 0..15 with offset 8, elements j and j + 16 share byte j) ----
+// one thread per block: 16 bytes + one fp16 scale <-> 32 fp16 values
+namespace smh {
+__global__ __launch_bounds__(256) void gq40_dequant_kernel(const u32x4 *__restrict__ packed, const half_t *__restrict__ scale,
+                                                           half_t *__restrict__ out, long blocks) {
+    const long b = (long)blockIdx.x * 256 + threadIdx.x;
+    if (b >= blocks) return;
+    const u32x4 v = packed[b];
+    const half_t sc = scale[b];
+    half_t lo[16], hi[16];
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const uint32_t byte = (v[j >> 2] >> (8 * (j & 3))) & 255u;
+        lo[j] = (half_t)(float)((int)(byte & 15u) - 8) * sc;         // exact small integer times the scale: one fp16 rounding
+        hi[j] = (half_t)(float)((int)(byte >> 4) - 8) * sc;
+    }
+    u32x4 *o = reinterpret_cast<u32x4 *>(out + b * 32);
+#pragma unroll
+    for (int q = 0; q < 2; ++q) {
+        o[q] = u32x4{as_u32(h2{lo[8 * q], lo[8 * q + 1]}), as_u32(h2{lo[8 * q + 2], lo[8 * q + 3]}),
+                     as_u32(h2{lo[8 * q + 4], lo[8 * q + 5]}), as_u32(h2{lo[8 * q + 6], lo[8 * q + 7]})};
+        o[2 + q] = u32x4{as_u32(h2{hi[8 * q], hi[8 * q + 1]}), as_u32(h2{hi[8 * q + 2], hi[8 * q + 3]}),
+                         as_u32(h2{hi[8 * q + 4], hi[8 * q + 5]}), as_u32(h2{hi[8 * q + 6], hi[8 * q + 7]})};
+    }
+}
+
+// rint(fp16(x / scale)) cut to -8 .. 8 while still a float (a scale that underflowed to 0 gives +-inf), NaN (0 / 0) -> 0
+__device__ __forceinline__ int gq40_code(half_t x, float scale) {
+    const float qf = (float)(half_t)((float)x / scale);
+    if (!(qf == qf)) return 0;
+    return (int)__builtin_rintf(fminf(fmaxf(qf, -8.0f), 8.0f));
+}
+
+__global__ __launch_bounds__(256) void gq40_quantize_kernel(const u32x4 *__restrict__ in, u32x4 *__restrict__ packed,
+                                                            half_t *__restrict__ scale, long blocks) {
+    const long b = (long)blockIdx.x * 256 + threadIdx.x;
+    if (b >= blocks) return;
+    half_t x[32];
+    uint32_t amax = 0;
+#pragma unroll
+    for (int q = 0; q < 4; ++q) {
+        const u32x4 r = in[b * 4 + q];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const h2 pr = as_h2(r[j]);
+            x[8 * q + 2 * j] = pr.x;
+            x[8 * q + 2 * j + 1] = pr.y;
+            const uint32_t a = r[j] & 0x7FFF7FFFu;                  // |x| as bit patterns: integer order = magnitude order
+            amax = max(amax, max(a & 0xFFFFu, a >> 16));
+        }
+    }
+    const half_t scale_h = (half_t)((float)__builtin_bit_cast(half_t, (uint16_t)amax) / 8.0f);
+    const float sf = (float)scale_h;
+    uint32_t w[4] = {0, 0, 0, 0};
+#pragma unroll
+    for (int j = 0; j < 16; ++j) {
+        const int ql = min(gq40_code(x[j], sf) + 8, 15), qh = min(gq40_code(x[j + 16], sf) + 8, 15);
+        w[j >> 2] |= (uint32_t)(ql | (qh << 4)) << (8 * (j & 3));
+    }
+    packed[b] = u32x4{w[0], w[1], w[2], w[3]};
+    scale[b] = scale_h;
+}
+}  // namespace smh
+
+extern "C" int smh_gq40_dequant(const void *packed, const void *scale, void *out, long blocks, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(blocks >= 0, "smh_gq40_dequant: blocks=%ld", blocks);
+    if (blocks == 0) return 0;
+    SMH_REQUIRE(packed && scale && out && (((uintptr_t)packed | (uintptr_t)out) & 15) == 0, "smh_gq40_dequant: null or misaligned pointer");
+    hipLaunchKernelGGL(gq40_dequant_kernel, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4 *)packed, (const half_t *)scale, (half_t *)out, blocks);
+    return launch_status();
+}
+
+extern "C" int smh_gq40_quantize(const void *in, void *packed, void *scale, long blocks, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(blocks >= 0, "smh_gq40_quantize: blocks=%ld", blocks);
+    if (blocks == 0) return 0;
+    SMH_REQUIRE(in && packed && scale && (((uintptr_t)in | (uintptr_t)packed) & 15) == 0, "smh_gq40_quantize: null or misaligned pointer");
+    hipLaunchKernelGGL(gq40_quantize_kernel, dim3((unsigned)((blocks + 255) / 256)), dim3(256), 0, (hipStream_t)stream,
+                       (const u32x4 *)in, (u32x4 *)packed, (half_t *)scale, blocks);
+    return launch_status();
+}
+
 extern "C" int smh_q40_quantize(const void *in, void *w, void *s, long groups, smh_stream_t stream) {
     using namespace smh;
     SMH_REQUIRE(groups >= 0 && (groups & 1) == 0, "smh_q40_quantize: groups=%ld must be even", groups);

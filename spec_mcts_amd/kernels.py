@@ -359,6 +359,37 @@ def q_int40(w: torch.Tensor, group_size: int = GROUP_SIZE) -> Tuple[torch.Tensor
     return q, s
 
 
+def quantize_gq40(w: torch.Tensor) -> Tuple[torch.Tensor, torch.Tensor]:
+    """The block-of-32 Q4_0 flavour of the benchmark's first configuration (scale = absmax / 8, q in [0, 15], value =
+    (q - 8) * scale; not a format of the reference's code): fp16 [..., K], K % 32 == 0 -> (uint8 [numel/32, 16], fp16 [numel/32])."""
+    lib = _lib.load()
+    _need_gpu(w)
+    assert w.dtype == torch.float16 and w.shape[-1] % 32 == 0
+    w = w.contiguous()
+    blocks = w.numel() // 32
+    packed = torch.empty((blocks, 16), device=w.device, dtype=torch.uint8)
+    scale = torch.empty(blocks, device=w.device, dtype=torch.float16)
+    check(lib.smh_gq40_quantize(w.data_ptr(), packed.data_ptr(), scale.data_ptr(), blocks, _stream()), "smh_gq40_quantize")
+    return packed, scale
+
+
+def dequantize_gq40(packed: torch.Tensor, scale: torch.Tensor, shape) -> torch.Tensor:
+    """Inverse of quantize_gq40: fp16 tensor of `shape`, one fp16 multiply per weight."""
+    lib = _lib.load()
+    _need_gpu(packed, scale)
+    assert packed.dtype == torch.uint8 and packed.is_contiguous() and packed.dim() == 2 and packed.shape[1] == 16
+    assert scale.dtype == torch.float16 and scale.is_contiguous() and scale.numel() == packed.shape[0]
+    out = torch.empty(tuple(shape), device=packed.device, dtype=torch.float16)
+    assert out.numel() == packed.shape[0] * 32
+    check(lib.smh_gq40_dequant(packed.data_ptr(), scale.data_ptr(), out.data_ptr(), packed.shape[0], _stream()), "smh_gq40_dequant")
+    return out
+
+
+def linear_gq40(x: torch.Tensor, packed: torch.Tensor, scale: torch.Tensor, shape) -> torch.Tensor:
+    """y = x . W^T for W [N, K] held in the block-of-32 flavour: dequantise, then the fp16 linear kernel (fp32 sums, one rounding)."""
+    return f16_linear(x, dequantize_gq40(packed, scale, shape))
+
+
 def q_int40_wide(w: torch.Tensor, group_size: int = GROUP_SIZE) -> Tuple[torch.Tensor, torch.Tensor]:
     """bfloat16 or fp32 -> Q4_0 on the GPU with the roundings torch's CPU quantiser has for those types (scale through
     the tensor's own type, quotient in fp32): what converting a bfloat16 HF checkpoint on the host produces."""

@@ -45,6 +45,33 @@ def test_config0_single_linear():
     _check(y, O.linear_q40_cpu_path(x, w, s, (N, Kd)))
 
 
+def test_config0_as_worded_block32_flavour():
+    """The first configuration as its text words it: W [11008, 4096] in 32-weight blocks, scale = absmax / 8, q in [0, 15],
+    value = (q - 8) * scale (a format the reference's code does not have).  GPU quantiser = oracle quantiser byte for
+    byte, dequant bit-exact, y = x . W^T within tolerance."""
+    from spec_mcts_amd import kernels as K
+    N, Kd = 11008, 4096
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((1, Kd), generator=g).to(torch.float16)
+    v = (torch.randn((N, Kd), generator=g) * 0.02).to(torch.float16)
+    packed, scale = O.quantize_gq40(v)
+    pd, sd_ = K.quantize_gq40(v.cuda())
+    assert torch.equal(pd.cpu(), packed) and torch.equal(sd_.cpu().view(torch.int16), scale.view(torch.int16))
+    deq = K.dequantize_gq40(pd, sd_, (N, Kd))
+    want = O.dequantize_gq40(packed, scale, (N, Kd))
+    assert torch.equal(deq.cpu().view(torch.int16), want.view(torch.int16))
+    assert float((want.float() - v.float()).abs().max()) <= float(scale.float().max())            # it is a quantisation of v
+    y = K.linear_gq40(x.cuda(), pd, sd_, (N, Kd))
+    _check(y, O.linear_gq40(x, packed, scale, (N, Kd)))
+    # zeros, a lone spike and the largest fp16 value survive the round trip's edge cases
+    e = torch.zeros((4, 64), dtype=torch.float16)
+    e[1, 5], e[2, 40], e[3, :] = 3.0, -65504.0, 1e-7
+    pe, se = K.quantize_gq40(e.cuda())
+    po, so = O.quantize_gq40(e)
+    assert torch.equal(pe.cpu(), po) and torch.equal(se.cpu().view(torch.int16), so.view(torch.int16))
+    assert torch.equal(K.dequantize_gq40(pe, se, e.shape).cpu().view(torch.int16), O.dequantize_gq40(po, so, e.shape).view(torch.int16))
+
+
 SHAPES = [(4096, 4096), (11008, 4096), (4096, 11008), (32128, 4096)]   # 32016 padded to 251*128
 
 

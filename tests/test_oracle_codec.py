@@ -136,3 +136,55 @@ def test_weight_layout_byte_map():
             assert _bits(want.reshape(1))[0] == _bits(deq[k, n].reshape(1))[0]
     # and the dequantised matrix approximates v^T
     assert (deq.float() - v.t().float()).abs().max() <= s.float().max() * 0.51
+
+
+# ---- the block-of-32 flavour that the benchmark's first configuration spells out ----------------------------------
+def test_block32_dequant_every_nibble_and_scale():
+    """(q - 8) * scale for all 16 nibbles x all 65536 fp16 scale patterns, against numpy float16 (an independent fp16
+    multiply) - and against exact integer arithmetic where the product needs no rounding."""
+    scales = torch.arange(65536, dtype=torch.int32).to(torch.int16).view(torch.float16)          # every bit pattern
+    for q in range(16):
+        byte = torch.full((65536, 16), q | (q << 4), dtype=torch.uint8)
+        got = O.dequantize_gq40(byte, scales, (65536, 32))
+        with np.errstate(over="ignore", invalid="ignore"):
+            want = (np.float16(q - 8) * scales.numpy().astype(np.float16)).astype(np.float16)
+        g = got[:, 0].numpy()
+        same = (g.view(np.uint16) == want.view(np.uint16)) | (np.isnan(g) & np.isnan(want))
+        assert same.all(), q
+        assert torch.equal(got[:, 0].view(torch.int16), got[:, 31].view(torch.int16))              # both nibbles, every position
+    # powers of two: the product is exact, so it must equal plain integer scaling
+    s2 = torch.tensor([2.0 ** e for e in range(-10, 6)], dtype=torch.float16)
+    by = torch.arange(16, dtype=torch.uint8).repeat(16, 1)                                        # low nibble j, high nibble 0
+    d = O.dequantize_gq40(by.contiguous(), s2, (16, 32))
+    for i in range(16):
+        assert d[i, :16].tolist() == [(j - 8) * float(s2[i]) for j in range(16)]
+        assert d[i, 16:].tolist() == [-8 * float(s2[i])] * 16
+
+
+def test_block32_quantiser_invariants_and_layout():
+    g = torch.Generator().manual_seed(5)
+    w = (torch.randn((64, 128), generator=g) * 0.02).half()
+    w[3] = 0                                                                                      # an all-zero block row: 0 / 0
+    packed, scale = O.quantize_gq40(w)
+    assert packed.shape == (64 * 4, 16) and packed.dtype == torch.uint8 and scale.shape == (256,)
+    blocks = w.reshape(-1, 32)
+    assert torch.equal(scale, (blocks.abs().max(1).values.float() / 8.0).half())                   # true division, one rounding
+    deq = O.dequantize_gq40(packed, scale, w.shape)
+    err = (deq.float() - w.float()).abs().reshape(-1, 32)
+    sc = scale.float()[:, None]
+    at_top = blocks.float() >= 7.5 * sc                                                           # would round to 16: cut to 15
+    slack = blocks.float().abs() * 2.0 ** -10 + 1e-7                    # the fp16 roundings of the quotient and of the product
+    assert bool((err[~at_top] <= (sc.expand_as(err) * 0.5 + slack)[~at_top]).all())
+    assert bool((err[at_top] <= (sc.expand_as(err) * 1.0 + slack)[at_top]).all()) and int(at_top.sum()) > 0
+    assert bool((deq[3] == 0).all()) and bool((packed[12:16] == 0x88).all())                       # 0 / 0 -> q = 8 -> value 0
+    # element j in the low nibble of byte j, element j + 16 in the high nibble
+    q = torch.round(blocks / scale[:, None]).float().nan_to_num(0.0, posinf=8.0, neginf=-8.0).to(torch.int32).add(8).clamp(0, 15)
+    assert torch.equal(packed.to(torch.int32) & 15, q[:, :16]) and torch.equal(packed.to(torch.int32) >> 4, q[:, 16:])
+    # the negative end is exact: -absmax -> q = 0 -> value -8 * scale
+    lo = blocks.float().min(1).values
+    neg = lo <= -blocks.abs().max(1).values.float()
+    assert bool(((packed.to(torch.int32) & 15).min(1).values.minimum((packed.to(torch.int32) >> 4).min(1).values)[neg & (scale > 0)] == 0).all())
+    # re-quantising what was dequantised reproduces codes and scales where the block's extreme code is -8 (scale recoverable)
+    p2, s2 = O.quantize_gq40(deq)
+    keep = neg & (scale > 0)
+    assert torch.equal(p2[keep], packed[keep]) and torch.equal(s2[keep], scale[keep])
