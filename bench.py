@@ -260,6 +260,22 @@ def cpu_baseline(torch, args_kw, budget_s=20.0):
     return out, cores, res
 
 
+def single_linear_cpu_ms(torch):
+    """The first configuration's case on the host: x [1, 4096] through one Q4_0 linear W [11008, 4096] with the reference's CPU
+    recipe (dequantise the whole weight, then F.linear): median of 5 calls, milliseconds."""
+    from oracle import q40_oracle as O
+    g = torch.Generator().manual_seed(0)
+    x = torch.randn((1, 4096), generator=g).half()
+    v = (torch.randn((11008, 4096), generator=g) * 0.02).half()
+    w, s, shape = O.quantize_weight(v)
+    times = []
+    for _ in range(5):
+        t0 = time.perf_counter()
+        O.linear_q40_cpu_path(x, w, s, shape)
+        times.append(time.perf_counter() - t0)
+    return round(sorted(times)[2] * 1e3, 3)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -403,7 +419,8 @@ def main():
                                   "sample": "oracle CPU path (torch dequantise + F.linear, fp32 compute): one layer + lm_head, "
                                             "median of 3 decode steps at B=1, 10 and 100, 64-token prompt, layer time x n_layers; "
                                             "value is the B=%d figure" % head_b,
-                                  "by_batch": {str(B): round(v, 4) for B, v in cpu.items()}}
+                                  "by_batch": {str(B): round(v, 4) for B, v in cpu.items()},
+                                  "single_linear_ms": single_linear_cpu_ms(torch)}
     print(json.dumps(result))
 
 
