@@ -172,22 +172,33 @@ def matmul_sweep(torch, iters=3):
             for _ in range(3):
                 graph.replay()
             us = time_region(torch, graph.replay, iters) * 1e3 / copies
+            del graph
+            # the same launch over ONE weight copy, repeated: the weights stay in the 256 MB Infinity Cache ("hot")
+            hot = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(hot):
+                for _ in range(8):
+                    K.matmul_q40_partial(x, [tiled[0]])
+            for _ in range(3):
+                hot.replay()
+            hot_us = time_region(torch, hot.replay, iters) * 1e3 / 8
+            del hot
             nbytes = q40_bytes(M, N, Kd)
             flops = 2.0 * M * N * Kd
             out.append({"M": M, "N": N, "K": Kd, "us": round(us, 2), "bytes": nbytes, "gbs": round(nbytes / us / 1e3, 1),
                         "hbm_frac": round(nbytes / us / 1e3 / HBM_PEAK_GBS, 4), "tflops": round(flops / us / 1e6, 1),
-                        "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "weight_copies": copies})
-            del graph
+                        "mfma_frac": round(flops / us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4), "weight_copies": copies,
+                        "hot_cache_us": round(hot_us, 2)})
         del tiled
         torch.cuda.empty_cache()
     return out
 
 
-def attention_roofline(torch, iters=5, copies=3):
+def attention_roofline(torch, iters=5, copies=3, fp16_suffix=False):
     """The shared-prefix decode attention alone on the reference's tree-attention shape: 64 branches, 32 heads,
     head_dim 128, one 1024-token fp16 prefix shared by all branches, ragged suffixes of 0..256 rows per branch held
-    as the model stores them (Q4_0 rows + scales), seed 2.  Algorithmic bytes: the prefix once, every valid suffix
-    row once, q and out.  `copies` distinct caches alternate so that the suffix does not stay in the Infinity Cache."""
+    as the model stores them (Q4_0 rows + scales) or, with fp16_suffix, as fp16 rows (the shape as the reference's own
+    check draws it), seed 2.  Algorithmic bytes: the prefix once, every valid suffix row once, q and out.  `copies`
+    distinct caches alternate so that the suffix does not stay in the Infinity Cache."""
     from spec_mcts_amd import kernels as K
     dev = torch.device("cuda:0")
     B, H, D, P, S = 64, 32, 128, 1024, 256
@@ -197,9 +208,13 @@ def attention_roofline(torch, iters=5, copies=3):
     sets = []
     for _ in range(copies):
         pk, pv = torch.randn((P, H, D), device=dev).half(), torch.randn((P, H, D), device=dev).half()
-        sk = torch.randint(-128, 128, (B, S, H, 64), device=dev, dtype=torch.int16).to(torch.int8)
-        sv = torch.randint(-128, 128, (B, S, H, 64), device=dev, dtype=torch.int16).to(torch.int8)
-        sks, svs = (torch.rand((B, S, H, 2), device=dev) * 0.1).half(), (torch.rand((B, S, H, 2), device=dev) * 0.1).half()
+        if fp16_suffix:
+            sk, sv = torch.randn((B, S, H, D), device=dev).half(), torch.randn((B, S, H, D), device=dev).half()
+            sks = svs = None
+        else:
+            sk = torch.randint(-128, 128, (B, S, H, 64), device=dev, dtype=torch.int16).to(torch.int8)
+            sv = torch.randint(-128, 128, (B, S, H, 64), device=dev, dtype=torch.int16).to(torch.int8)
+            sks, svs = (torch.rand((B, S, H, 2), device=dev) * 0.1).half(), (torch.rand((B, S, H, 2), device=dev) * 0.1).half()
         sets.append((pk, pv, sk, sv, sks, svs))
     lens_d = lens.to(dev)
 
@@ -216,7 +231,7 @@ def attention_roofline(torch, iters=5, copies=3):
         graph.replay()
     ms = time_region(torch, graph.replay, iters) / copies
     rows = int(lens.sum())
-    nbytes = 2 * P * H * D * 2 + rows * H * 2 * (64 + 4) + 2 * B * H * D * 2
+    nbytes = 2 * P * H * D * 2 + rows * H * 2 * (2 * D if fp16_suffix else 64 + 4) + 2 * B * H * D * 2
     return {"us": ms * 1e3, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9, "suffix_rows": rows}
 
 
@@ -411,6 +426,12 @@ def main():
                        "suffixes of 0..256 rows (the two launches of one call)",
              "bound": "hbm", "achieved": round(att["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
              "frac": round(att["gbs"] / HBM_PEAK_GBS, 4), "avg_call_us": round(att["us"], 2), "bytes_per_call": att["bytes"], "traffic": ATTN_TRAFFIC_BYTES_PER_CALL})
+        att16 = attention_roofline(torch, fp16_suffix=True)
+        result["rooflines_other"].append(
+            {"kernel": "attn_prefix_kernel + attn_suffix_kernel: the same shape with the suffixes as fp16 rows (512 B per row and head "
+                       "instead of 136 B)",
+             "bound": "hbm", "achieved": round(att16["gbs"], 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+             "frac": round(att16["gbs"] / HBM_PEAK_GBS, 4), "avg_call_us": round(att16["us"], 2), "bytes_per_call": att16["bytes"], "traffic": None})
     if not a.no_sweep and a.arch == "7b":
         result["matmul_sweep"] = matmul_sweep(torch)
     if not a.no_cpu_baseline:
