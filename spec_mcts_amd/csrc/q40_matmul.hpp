@@ -3,9 +3,7 @@
 // Both kernels cut K into slices for occupancy and write one [M, n_total] slab per slice into
 // the caller's `partial` buffer; the slabs are added in slice order (in fp32) by the consuming kernel
 // (partial_ops.hip).  With a single slice and a plain epilogue the product is written directly.
-// Slabs of a product with at most SMH_GEMV_MAX_M rows hold fp32; above that they hold fp16: at those
-// batch sizes writing and re-reading the slabs costs as much HBM traffic as the weights themselves,
-// and a partial sum rounded to fp16 carries the same relative error as the fp16 result it ends up in.
+// The slabs hold fp32 at every batch size.
 #pragma once
 
 #include "smh_common.hpp"
