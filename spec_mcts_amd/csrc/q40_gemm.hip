@@ -45,6 +45,13 @@ constexpr int GEMM_THREADS = GEMM_WAVES * 64;
 #define SMH_GEMM_STAGES 6
 #endif
 constexpr int GEMM_STAGES = SMH_GEMM_STAGES;
+// slots of the ring in the variant with a DMA wave, and the most workgroups of a launch that takes it
+#ifndef SMH_GEMM_PSLOTS
+#define SMH_GEMM_PSLOTS 6
+#endif
+#ifndef SMH_GEMM_PMAX
+#define SMH_GEMM_PMAX 256
+#endif
 constexpr int GS_WBLOCK = 8 * 128 + 64;        // the 8 rows one wave fetches, padded by 16 banks: the four row groups a
                                                // ds_read_b32 touches (lanes 16g..16g+15 read row 8g+r) then sit in different banks
 constexpr int GS_W = 4 * GS_WBLOCK;            // nibbles
@@ -60,27 +67,17 @@ typedef __attribute__((address_space(3))) void *lptr_t;
 
 // Waits until at most `stages` younger stages (PER DMA instructions each: 4 with four waves, 2 with eight) of this wave
 // are still in flight.
+template <int N>
+__device__ __forceinline__ void gemm_wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N < 63 ? N : 63) : "memory"); }
 template <int PER>
 __device__ __forceinline__ void gemm_wait_dma(int stages) {
-    static_assert(PER == 4 || PER == 2, "DMA instructions per wave and stage");
-    if (PER == 4) {
-        switch (stages) {
-            case 5: asm volatile("s_waitcnt vmcnt(20)" ::: "memory"); break;
-            case 4: asm volatile("s_waitcnt vmcnt(16)" ::: "memory"); break;
-            case 3: asm volatile("s_waitcnt vmcnt(12)" ::: "memory"); break;
-            case 2: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
-            case 1: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
-            default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-        }
-    } else {
-        switch (stages) {
-            case 5: asm volatile("s_waitcnt vmcnt(10)" ::: "memory"); break;
-            case 4: asm volatile("s_waitcnt vmcnt(8)" ::: "memory"); break;
-            case 3: asm volatile("s_waitcnt vmcnt(6)" ::: "memory"); break;
-            case 2: asm volatile("s_waitcnt vmcnt(4)" ::: "memory"); break;
-            case 1: asm volatile("s_waitcnt vmcnt(2)" ::: "memory"); break;
-            default: asm volatile("s_waitcnt vmcnt(0)" ::: "memory"); break;
-        }
+    switch (stages) {
+        case 5: gemm_wait_vm<5 * PER>(); break;
+        case 4: gemm_wait_vm<4 * PER>(); break;
+        case 3: gemm_wait_vm<3 * PER>(); break;
+        case 2: gemm_wait_vm<2 * PER>(); break;
+        case 1: gemm_wait_vm<1 * PER>(); break;
+        default: gemm_wait_vm<0>(); break;
     }
 }
 
@@ -94,9 +91,15 @@ __device__ __forceinline__ void gemm_barrier() { asm volatile("s_waitcnt lgkmcnt
 // WAVES = 8 (tiled weights only): waves w and w + 4 share piece w of a tile; wave w multiplies the columns of its HIGH
 // nibbles, wave w + 4 those of the low nibbles (two B operands and half the accumulators each, the same A tiles), so
 // that every SIMD holds two waves of the workgroup and the decode of one runs under the MFMAs of the other.
-template <int TILES, bool RAGGED, bool TILED, int WAVES>
-__global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kernel(MatmulParams p) {
+// PRODUCER (eight waves only): a ninth wave issues every DMA instruction of the workgroup and waits for them; the eight
+// others only meet it at the barriers.  The compute unit's address unit takes 16 cycles per DMA instruction, during which
+// the issuing wave stands still: ~0.28 us per pair of steps off the multiplying waves' path.  For launches with one
+// workgroup per compute unit (a ninth and tenth wave on a SIMD that already holds four would cap the registers below
+// what the kernel needs).  SLOTS: slots of the ring.
+template <int TILES, bool RAGGED, bool TILED, int WAVES, int SLOTS = GEMM_STAGES, bool PRODUCER = false>
+__global__ __launch_bounds__(64 * (WAVES + (PRODUCER ? 1 : 0)), WAVES == 8 ? 1 : 2) void q40_gemm_kernel(MatmulParams p) {
     static_assert(WAVES == 4 || (WAVES == 8 && TILED && !RAGGED), "eight waves: tiled weights, K a multiple of 32");
+    static_assert(SLOTS >= 6 && SLOTS <= 10 && (SLOTS == GEMM_STAGES || PRODUCER) && (!PRODUCER || WAVES == 8), "ring depth");
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int NB = WAVES == 8 ? 2 : 4;     // B operands (16 columns each) per wave
     constexpr int DMA_PER = WAVES == 8 ? 2 : 4;
@@ -213,9 +216,64 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
         issue(fetch, slot_);
         fetch = fetch + 1 == step1 ? step0 : fetch + 1;
     };
+    if constexpr (PRODUCER) {
+        if (wave8 == 8) {
+            // ---- the DMA wave: 5 + TILES instructions a stage (four pieces of nibbles, the scales, one per 16 rows of A) ----
+            constexpr int PER = 5 + TILES;
+            __builtin_amdgcn_s_setprio(3);      // its few instructions first: the others wait for what it requests (3 % of a launch)
+            uint32_t a_voff[TILES];
 #pragma unroll
-    for (int i = 0; i < 4; ++i)
-        if (i < n_steps) fetch_next(i);
+            for (int t = 0; t < TILES; ++t)
+                a_voff[t] = (uint32_t)((long)min(m0 + 16 * t + (lane >> 2), p.M - 1) * p.lda * 2 + 16 * a_chunk);
+            auto issue_all = [&](int slot_) {
+                uint8_t *st = lds + slot_ * GS_BYTES;
+                const uint8_t *tile = w_base + (long)fetch * TILE_BYTES;
+                const uint8_t *arow = a_base + (long)fetch * 64;
+#pragma unroll
+                for (int q = 0; q < 4; ++q)
+                    __builtin_amdgcn_global_load_lds((gptr_t)(tile + q * 1024 + lane * 16), (lptr_t)(st + q * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr_t)(tile + TILE_W_BYTES + lane * 4), (lptr_t)(st + GS_W), 4, 0, 0);
+#pragma unroll
+                for (int t = 0; t < TILES; ++t)
+                    __builtin_amdgcn_global_load_lds((gptr_t)(arow + a_voff[t]), (lptr_t)(st + GS_W + GS_S + t * 1024), 16, 0, 0);
+                fetch = fetch + 1 == step1 ? step0 : fetch + 1;
+            };
+#pragma unroll
+            for (int i = 0; i < SLOTS - 2; ++i)
+                if (i < n_steps) issue_all(i);
+            if (n_steps > 0) {
+                gemm_wait_dma<PER>(min(SLOTS - 3, n_steps - 1));
+                gemm_barrier();
+                int slot = 0;
+                auto back = [&](int k) { return slot >= k ? slot - k : slot + SLOTS - k; };
+                int i = 0;
+#pragma unroll 1
+                for (; i + SLOTS - 1 < n_steps; i += 2) {
+                    gemm_wait_vm<PER * (SLOTS - 5)>();
+                    gemm_barrier();
+                    issue_all(back(2));
+                    issue_all(back(1));
+                    slot = slot + 2 >= SLOTS ? slot + 2 - SLOTS : slot + 2;
+                }
+#pragma unroll 1
+                for (; i < n_steps; i += 2) {
+                    gemm_wait_dma<PER>(max(0, min(n_steps - 1, i + SLOTS - 3) - (i + 2)));      // stages issued past step i + 2
+                    gemm_barrier();
+                    if (i + SLOTS - 2 < n_steps) issue_all(back(2));
+                    if (i + SLOTS - 1 < n_steps) issue_all(back(1));
+                    slot = slot + 2 >= SLOTS ? slot + 2 - SLOTS : slot + 2;
+                }
+            }
+            // the barriers of the epilogue: one that frees the ring, one per row tile
+#pragma unroll 1
+            for (int t = 0; t < 1 + TILES; ++t) gemm_barrier();
+            return;
+        }
+    } else {
+#pragma unroll
+        for (int i = 0; i < SLOTS - 2; ++i)
+            if (i < n_steps) fetch_next(i);
+    }
 
     // the eight dwords of this lane's column bytes and of their scales, for one step
     auto load_ws = [&](const uint8_t *st, uint32_t (&wv)[8], uint32_t (&sv)[8]) {
@@ -328,17 +386,16 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
             for (int o = 0; o < NB; ++o) acc[o][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], b[o], acc[o][t], 0, 0, 0);
         }
     };
-    // Steps go in pairs: ONE wait + barrier per two steps.  Six slots; at the barrier before steps i, i+1 the stages of
-    // steps i .. i+2 have landed (the B operands of step i+2 are decoded during step i+1), step i+3 may be in flight, and
-    // the slots of steps i-2, i-1 are refilled with steps i+4, i+5.  A stage has the same two steps of time to land as
+    // Steps go in pairs: ONE wait + barrier per two steps.  With S slots (six; more only with the DMA wave): at the barrier
+    // before steps i, i+1 the stages of steps i .. i+2 have landed (the B operands of step i+2 are decoded during step i+1),
+    // steps i+3 .. i+S-3 may be in flight, and the slots of steps i-2, i-1 are refilled with steps i+S-2, i+S-1.  A stage has the same two steps of time to land as
     // with a barrier per step; the waves meet half as often.
     if (n_steps > 0) {
-        static_assert(GEMM_STAGES == 6, "the paired loop counts on six slots");
         h8 bq[NB];
         int cur = step0 + rot;                 // step being multiplied
         int slot = 0;                          // its ring slot
         {
-            gemm_wait_dma<DMA_PER>(min(3, n_steps - 1));
+            if constexpr (!PRODUCER) gemm_wait_dma<DMA_PER>(min(SLOTS - 3, n_steps - 1));
             gemm_barrier();
             uint32_t wv[8], sv[8];
             load_ws(lds, wv, sv);
@@ -347,7 +404,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
         // multiply the step in `slot` with bq while the B operands of the next step are decoded
         auto one_step = [&]() {
             const uint8_t *st = lds + slot * GS_BYTES;
-            slot = slot == GEMM_STAGES - 1 ? 0 : slot + 1;
+            slot = slot == SLOTS - 1 ? 0 : slot + 1;
             cur = cur + 1 == step1 ? step0 : cur + 1;
             // past the last step the next slot holds stale bytes: read, decoded and never used
             uint32_t wv[8], sv[8];
@@ -359,13 +416,16 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
 #pragma unroll
             for (int o = 0; o < NB; ++o) bq[o] = bn[o];
         };
-        auto back = [&](int k) { return slot >= k ? slot - k : slot + GEMM_STAGES - k; };
+        auto back = [&](int k) { return slot >= k ? slot - k : slot + SLOTS - k; };
         int i = 0;
 #pragma unroll 1
-        for (; i + 5 < n_steps; i += 2) {      // both refills exist: the body is one basic block
-            gemm_wait_dma<DMA_PER>(1);
+        for (; i + SLOTS - 1 < n_steps; i += 2) {      // both refills exist: the body is one basic block
+            if constexpr (!PRODUCER) gemm_wait_vm<DMA_PER * (SLOTS - 5)>();
             gemm_barrier();
-            if constexpr (TILED && WAVES == 8 && TILES < 8) {       // (with all 8 row tiles, the prefill, this form measured 5-8 % slower)
+            if constexpr (PRODUCER) {
+                one_step();
+                one_step();
+            } else if constexpr (TILED && WAVES == 8 && TILES < 8) {       // (with all 8 row tiles, the prefill, this form measured 5-8 % slower)
                 // the nibbles and scales of the two refills now, their A rows from inside the steps: the address unit takes
                 // 16 cycles per instruction, and between MFMAs the wave has them to spare (2 % off a launch at 100 rows;
                 // the nibbles and scales too from inside the steps, behind their branches: 4 % slower)
@@ -376,7 +436,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
                 issue_ws8(fb, sb);
                 for (int half = 0; half < 2; ++half) {
                     const uint8_t *st = lds + slot * GS_BYTES;
-                    slot = slot == GEMM_STAGES - 1 ? 0 : slot + 1;
+                    slot = slot == SLOTS - 1 ? 0 : slot + 1;
                     cur = cur + 1 == step1 ? step0 : cur + 1;
                     uint32_t wv[8], sv[8];
                     h8 av[TILES], bn[NB];
@@ -407,10 +467,12 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
         }
 #pragma unroll 1
         for (; i < n_steps; i += 2) {
-            gemm_wait_dma<DMA_PER>(i + 3 <= n_steps - 1 ? 1 : 0);
+            if constexpr (!PRODUCER) gemm_wait_dma<DMA_PER>(max(0, min(n_steps - 1, i + SLOTS - 3) - (i + 2)));      // stages issued past step i + 2
             gemm_barrier();
-            if (i + 4 < n_steps) fetch_next(back(2));
-            if (i + 5 < n_steps) fetch_next(back(1));
+            if constexpr (!PRODUCER) {
+                if (i + SLOTS - 2 < n_steps) fetch_next(back(2));
+                if (i + SLOTS - 1 < n_steps) fetch_next(back(1));
+            }
             one_step();
             if (i + 1 < n_steps) one_step();
         }
@@ -423,7 +485,7 @@ __global__ __launch_bounds__(64 * WAVES, WAVES == 8 ? 1 : 2) void q40_gemm_kerne
     // that every wave reaches only when its reads of that buffer have returned.
     constexpr int OP = GEMM_COLS + 4;
     constexpr int OTILE_BYTES = 16 * OP * 4;
-    static_assert(2 * OTILE_BYTES <= GEMM_LDS, "two output tiles must fit in the ring");
+    static_assert(2 * OTILE_BYTES <= SLOTS * GS_BYTES, "two output tiles must fit in the ring");
     float *slab = p.partial + (long)slice * p.M * p.n_total;
     const int o_row = (tid & 255) >> 4;         // 0..15
     const int o_half = tid >> 8;                // eight waves: the second 256 threads store the second half of the columns
@@ -518,6 +580,14 @@ static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
                                            q40_gemm_kernel<3, false, TILED, W>, q40_gemm_kernel<4, false, TILED, W>,
                                            q40_gemm_kernel<5, false, TILED, W>, q40_gemm_kernel<6, false, TILED, W>,
                                            q40_gemm_kernel<7, false, TILED, W>, q40_gemm_kernel<8, false, TILED, W>};
+    // one workgroup per compute unit: the variant with the DMA wave
+    constexpr bool HAS_DMA_WAVE = W == 8;
+    constexpr int PS = HAS_DMA_WAVE ? SMH_GEMM_PSLOTS : GEMM_STAGES;
+    static const gemm_kernel_t with_dma_wave[9] = {
+        nullptr, q40_gemm_kernel<2, false, TILED, W, PS, HAS_DMA_WAVE>, q40_gemm_kernel<2, false, TILED, W, PS, HAS_DMA_WAVE>,
+        q40_gemm_kernel<3, false, TILED, W, PS, HAS_DMA_WAVE>, q40_gemm_kernel<4, false, TILED, W, PS, HAS_DMA_WAVE>,
+        q40_gemm_kernel<5, false, TILED, W, PS, HAS_DMA_WAVE>, q40_gemm_kernel<6, false, TILED, W, PS, HAS_DMA_WAVE>,
+        q40_gemm_kernel<7, false, TILED, W, PS, HAS_DMA_WAVE>, q40_gemm_kernel<8, false, TILED, W, PS, HAS_DMA_WAVE>};
     static const gemm_kernel_t ragged = q40_gemm_kernel<8, true, TILED, 4>;
     // more than 64 KB of dynamic LDS has to be allowed once per kernel (the attribute is not stream work,
     // so a launch under graph capture is not affected)
@@ -525,14 +595,17 @@ static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
         hipError_t e = hipFuncSetAttribute((const void *)ragged, hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS);
         for (int t = 2; t <= 8 && e == hipSuccess; ++t)
             e = hipFuncSetAttribute((const void *)exact[t], hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS);
+        for (int t = 2; t <= 8 && e == hipSuccess && HAS_DMA_WAVE; ++t)
+            e = hipFuncSetAttribute((const void *)with_dma_wave[t], hipFuncAttributeMaxDynamicSharedMemorySize, PS * GS_BYTES);
         return e;
     }();
     if (lds_ok != hipSuccess) return (int)lds_ok;
     if ((long)p.M * p.lda * 2 >= (1L << 32)) return (int)hipErrorInvalidValue;     // lane offsets of A are 32-bit
     const int tiles = p.mblocks > 1 ? 8 : (p.M + 15) / 16;
-    const gemm_kernel_t kern = (p.K % 32 != 0) ? ragged : exact[tiles < 2 ? 2 : tiles];
+    const bool one_each = HAS_DMA_WAVE && p.K % 32 == 0 && (long)p.units * p.mblocks * p.ksplit <= SMH_GEMM_PMAX;
+    const gemm_kernel_t kern = (p.K % 32 != 0) ? ragged : (one_each ? with_dma_wave : exact)[tiles < 2 ? 2 : tiles];
     dim3 grid((unsigned)((long)p.units_pad * p.mblocks * p.ksplit));
-    hipLaunchKernelGGL(kern, grid, dim3(kern == ragged ? GEMM_THREADS : 64 * W), GEMM_LDS, stream, p);
+    hipLaunchKernelGGL(kern, grid, dim3(kern == ragged ? GEMM_THREADS : 64 * W + (one_each ? 64 : 0)), one_each ? PS * GS_BYTES : GEMM_LDS, stream, p);
     return launch_status();
 }
 
