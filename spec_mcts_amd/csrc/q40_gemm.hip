@@ -49,6 +49,9 @@ constexpr int GEMM_STAGES = SMH_GEMM_STAGES;
 #ifndef SMH_GEMM_PSLOTS
 #define SMH_GEMM_PSLOTS 6
 #endif
+#ifndef SMH_GEMM_RANGE_CUT
+#define SMH_GEMM_RANGE_CUT 1
+#endif
 #ifndef SMH_GEMM_PMAX
 #define SMH_GEMM_PMAX 256
 #endif
@@ -91,33 +94,24 @@ __device__ __forceinline__ void gemm_barrier() { asm volatile("s_waitcnt lgkmcnt
 // WAVES = 8 (tiled weights only): waves w and w + 4 share piece w of a tile; wave w multiplies the columns of its HIGH
 // nibbles, wave w + 4 those of the low nibbles (two B operands and half the accumulators each, the same A tiles), so
 // that every SIMD holds two waves of the workgroup and the decode of one runs under the MFMAs of the other.
-// PRODUCER (eight waves only): a ninth wave issues every DMA instruction of the workgroup and waits for them; the eight
-// others only meet it at the barriers.  The compute unit's address unit takes 16 cycles per DMA instruction, during which
-// the issuing wave stands still: ~0.28 us per pair of steps off the multiplying waves' path.  For launches with one
-// workgroup per compute unit (a ninth and tenth wave on a SIMD that already holds four would cap the registers below
-// what the kernel needs).  SLOTS: slots of the ring.
-template <int TILES, bool RAGGED, bool TILED, int WAVES, int SLOTS = GEMM_STAGES, bool PRODUCER = false>
-__global__ __launch_bounds__(64 * (WAVES + (PRODUCER ? 1 : 0)), WAVES == 8 ? 1 : 2) void q40_gemm_kernel(MatmulParams p) {
-    static_assert(WAVES == 4 || (WAVES == 8 && TILED && !RAGGED), "eight waves: tiled weights, K a multiple of 32");
-    static_assert(SLOTS >= 6 && SLOTS <= 10 && (SLOTS == GEMM_STAGES || PRODUCER) && (!PRODUCER || WAVES == 8), "ring depth");
+// One piece of a workgroup's work: steps [step0, step1) of column unit `unit` (row block mb), accumulated and left as slab
+// `slice`.  zero_rest: the piece ends its unit, and the slabs past `slice` (the unit has no piece for them) are written as
+// zeros.  more: another piece follows in this workgroup (one more barrier, after which the ring may be refilled).
+// tid_bias: zero (a range cut passes one the compiler cannot see, see there).
+template <int TILES, bool RAGGED, bool TILED, int WAVES, int SLOTS, bool PRODUCER>
+__device__ __forceinline__ void gemm_piece(const MatmulParams &p, int unit, int mb, int slice, int step0, int step1, bool zero_rest, bool more,
+                                           int tid_bias) {
     extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
     constexpr int NB = WAVES == 8 ? 2 : 4;     // B operands (16 columns each) per wave
     constexpr int DMA_PER = WAVES == 8 ? 2 : 4;
 
-    const int tid = threadIdx.x;
+    const int tid = threadIdx.x + tid_bias;
     const int wave8 = tid >> 6;                // 0 .. WAVES-1
     const int wave = wave8 & 3;                // piece of the tile / rows of the ring this wave serves
     const int hh = wave8 >> 2;                 // eight waves: 0 = high nibbles (columns c), 1 = low nibbles (columns c + 64)
     const int lane = tid & 63;
     const int c = lane & 15;
     const int g = lane >> 4;
-    int bid = blockIdx.x;
-    // slot -> unit: each XCD (blockIdx % 8) takes a contiguous run of column units, which share scale lines
-    const int slot = bid % p.units_pad;  bid /= p.units_pad;
-    const int unit = (slot & 7) * (p.units_pad >> 3) + (slot >> 3);
-    if (unit >= p.units) return;
-    const int mb = bid % p.mblocks;
-    const int slice = bid / p.mblocks;
     int sg = 0;
     if (p.nseg > 1 && unit >= p.seg[1].unit0) sg = 1;
     if (p.nseg > 2 && unit >= p.seg[2].unit0) sg = 2;
@@ -205,8 +199,6 @@ __global__ __launch_bounds__(64 * (WAVES + (PRODUCER ? 1 : 0)), WAVES == 8 ? 1 :
 #pragma unroll
         for (int t = 0; t < TILES; ++t) acc[h][t] = f4{0.f, 0.f, 0.f, 0.f};
 
-    const int step0 = slice * p.steps_per_slice;
-    const int step1 = min(step0 + p.steps_per_slice, (p.K + 31) / 32);
     const int n_steps = max(step1 - step0, 0);
     // workgroups that share a K-slice read the same A tiles; each starts at a different step of the
     // slice (and wraps) so that they do not all pull the same L2 lines at the same time
@@ -266,7 +258,7 @@ __global__ __launch_bounds__(64 * (WAVES + (PRODUCER ? 1 : 0)), WAVES == 8 ? 1 :
             }
             // the barriers of the epilogue: one that frees the ring, one per row tile
 #pragma unroll 1
-            for (int t = 0; t < 1 + TILES; ++t) gemm_barrier();
+            for (int t = 0; t < 1 + TILES + (more ? 1 : 0); ++t) gemm_barrier();
             return;
         }
     } else {
@@ -537,6 +529,65 @@ __global__ __launch_bounds__(64 * (WAVES + (PRODUCER ? 1 : 0)), WAVES == 8 ? 1 :
             }
         }
     }
+    if (zero_rest) {
+        for (int sl = slice + 1; sl < p.ksplit; ++sl) {
+            float *zslab = p.partial + (long)sl * p.M * p.n_total;
+            for (int t = 0; t < TILES; ++t) {
+                const int m = m0 + 16 * t + o_row;
+                if (m < p.M) {
+                    float *dst = zslab + (long)m * p.n_total + seg.col0 + col0;
+#pragma unroll
+                    for (int q = (WAVES == 8 ? 2 * o_half : 0); q < (WAVES == 8 ? 2 * o_half + 2 : 4); ++q) {
+                        const int cq = 64 * q + 4 * o_lane;
+                        if (col0 + cq < seg.N) *reinterpret_cast<f4 *>(dst + cq) = f4{0.f, 0.f, 0.f, 0.f};
+                    }
+                }
+            }
+        }
+    }
+    if (more) gemm_barrier();                   // the next piece refills the ring the last row tile left through
+}
+
+// PRODUCER (eight waves only): a ninth wave issues every DMA instruction of the workgroup and waits for them; the eight
+// others only meet it at the barriers.  The compute unit's address unit takes 16 cycles per DMA instruction, during which
+// the issuing wave stands still: ~0.28 us per pair of steps off the multiplying waves' path.  For launches with one
+// workgroup per compute unit (a ninth and tenth wave on a SIMD that already holds four would cap the registers below
+// what the kernel needs).  SLOTS: slots of the ring.
+// RANGE (p.chunk > 0): the steps of all column units, laid end to end, are dealt in runs of p.chunk to the workgroups, one
+// workgroup per compute unit, so a workgroup may finish one unit and begin the next: up to two pieces, one after the other.
+template <int TILES, bool RAGGED, bool TILED, int WAVES, int SLOTS = GEMM_STAGES, bool PRODUCER = false, bool RANGE = false>
+__global__ __launch_bounds__(64 * (WAVES + (PRODUCER ? 1 : 0)), WAVES == 8 ? 1 : 2) void q40_gemm_kernel(MatmulParams p) {
+    static_assert(WAVES == 4 || (WAVES == 8 && TILED && !RAGGED), "eight waves: tiled weights, K a multiple of 32");
+    static_assert(SLOTS >= 6 && SLOTS <= 10 && (SLOTS == GEMM_STAGES || PRODUCER) && (!PRODUCER || WAVES == 8), "ring depth");
+    const int steps_total = (p.K + 31) / 32;
+    if constexpr (RANGE) {
+        int run0 = (int)blockIdx.x * p.chunk;                  // (units x steps is far below 2^31)
+        const int run1 = min(run0 + p.chunk, p.units * steps_total);
+#pragma unroll 1
+        for (bool more = true; more;) {                        // (a loop, not two calls: the second piece runs code that is warm)
+            const int unit = run0 / steps_total;
+            const int s0 = run0 - unit * steps_total;
+            const int s1 = min(steps_total, s0 + (run1 - run0));
+            const int first = (unit * steps_total) / p.chunk;  // the workgroup that holds the unit's first piece
+            run0 += s1 - s0;
+            more = run0 < run1;
+            // a zero the compiler cannot see keeps everything derived from the thread index inside the piece: hoisted out of
+            // this loop those values stay live through it and the kernel spills
+            int opaque_zero;
+            asm volatile("s_mov_b32 %0, 0" : "=s"(opaque_zero));
+            gemm_piece<TILES, RAGGED, TILED, WAVES, SLOTS, PRODUCER>(p, unit, 0, (int)blockIdx.x - first, s0, s1, s1 == steps_total, more, opaque_zero);
+        }
+    } else {
+        int bid = blockIdx.x;
+        // slot -> unit: each XCD (blockIdx % 8) takes a contiguous run of column units, which share scale lines
+        const int slot = bid % p.units_pad;  bid /= p.units_pad;
+        const int unit = (slot & 7) * (p.units_pad >> 3) + (slot >> 3);
+        if (unit >= p.units) return;
+        const int mb = bid % p.mblocks;
+        const int slice = bid / p.mblocks;
+        const int s0 = slice * p.steps_per_slice;
+        gemm_piece<TILES, RAGGED, TILED, WAVES, SLOTS, PRODUCER>(p, unit, mb, slice, s0, min(s0 + p.steps_per_slice, steps_total), false, false, 0);
+    }
 }
 
 void gemm_fill_plan(MatmulParams &p) {
@@ -567,6 +618,26 @@ void gemm_fill_plan(MatmulParams &p) {
     if (ks < 1) ks = 1;
     p.steps_per_slice = (steps + ks - 1) / ks;
     p.ksplit = (steps + p.steps_per_slice - 1) / p.steps_per_slice;
+    // Range cut: a launch that would put two workgroups on some compute units and one on others (256 < workgroups <= 512)
+    // deals runs of steps instead, one workgroup per compute unit, crossing unit boundaries.
+    p.chunk = 0;
+    const long wgs = tiles * p.ksplit;
+    if (SMH_GEMM_RANGE_CUT && p.mblocks == 1 && p.K % 32 == 0 && wgs > 256 && wgs <= 512) {
+        const long total = (long)p.units * steps;
+        const int chunk = (int)((total + 255) / 256);
+        if (chunk <= steps && chunk >= 2 * GEMM_STAGES) {
+            int pieces = 0;
+            for (int u = 0; u < p.units; ++u) {
+                const int n = (int)(((long)u * steps + steps - 1) / chunk - ((long)u * steps) / chunk) + 1;
+                if (n > pieces) pieces = n;
+            }
+            if (pieces <= p.ksplit) {           // never more slabs than the even split leaves
+                p.chunk = chunk;
+                p.ksplit = pieces;
+                p.steps_per_slice = chunk;
+            }
+        }
+    }
 }
 
 typedef void (*gemm_kernel_t)(MatmulParams);
@@ -588,6 +659,11 @@ static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
         q40_gemm_kernel<3, false, TILED, W, PS, HAS_DMA_WAVE>, q40_gemm_kernel<4, false, TILED, W, PS, HAS_DMA_WAVE>,
         q40_gemm_kernel<5, false, TILED, W, PS, HAS_DMA_WAVE>, q40_gemm_kernel<6, false, TILED, W, PS, HAS_DMA_WAVE>,
         q40_gemm_kernel<7, false, TILED, W, PS, HAS_DMA_WAVE>, q40_gemm_kernel<8, false, TILED, W, PS, HAS_DMA_WAVE>};
+    static const gemm_kernel_t range_cut[9] = {
+        nullptr, q40_gemm_kernel<2, false, TILED, W, PS, HAS_DMA_WAVE, true>, q40_gemm_kernel<2, false, TILED, W, PS, HAS_DMA_WAVE, true>,
+        q40_gemm_kernel<3, false, TILED, W, PS, HAS_DMA_WAVE, true>, q40_gemm_kernel<4, false, TILED, W, PS, HAS_DMA_WAVE, true>,
+        q40_gemm_kernel<5, false, TILED, W, PS, HAS_DMA_WAVE, true>, q40_gemm_kernel<6, false, TILED, W, PS, HAS_DMA_WAVE, true>,
+        q40_gemm_kernel<7, false, TILED, W, PS, HAS_DMA_WAVE, true>, q40_gemm_kernel<8, false, TILED, W, PS, HAS_DMA_WAVE, true>};
     static const gemm_kernel_t ragged = q40_gemm_kernel<8, true, TILED, 4>;
     // more than 64 KB of dynamic LDS has to be allowed once per kernel (the attribute is not stream work,
     // so a launch under graph capture is not affected)
@@ -597,14 +673,17 @@ static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
             e = hipFuncSetAttribute((const void *)exact[t], hipFuncAttributeMaxDynamicSharedMemorySize, GEMM_LDS);
         for (int t = 2; t <= 8 && e == hipSuccess && HAS_DMA_WAVE; ++t)
             e = hipFuncSetAttribute((const void *)with_dma_wave[t], hipFuncAttributeMaxDynamicSharedMemorySize, PS * GS_BYTES);
+        for (int t = 2; t <= 8 && e == hipSuccess; ++t)
+            e = hipFuncSetAttribute((const void *)range_cut[t], hipFuncAttributeMaxDynamicSharedMemorySize, PS * GS_BYTES);
         return e;
     }();
     if (lds_ok != hipSuccess) return (int)lds_ok;
     if ((long)p.M * p.lda * 2 >= (1L << 32)) return (int)hipErrorInvalidValue;     // lane offsets of A are 32-bit
     const int tiles = p.mblocks > 1 ? 8 : (p.M + 15) / 16;
-    const bool one_each = HAS_DMA_WAVE && p.K % 32 == 0 && (long)p.units * p.mblocks * p.ksplit <= SMH_GEMM_PMAX;
-    const gemm_kernel_t kern = (p.K % 32 != 0) ? ragged : (one_each ? with_dma_wave : exact)[tiles < 2 ? 2 : tiles];
-    dim3 grid((unsigned)((long)p.units_pad * p.mblocks * p.ksplit));
+    const bool one_each = HAS_DMA_WAVE && p.K % 32 == 0 && (p.chunk > 0 || (long)p.units * p.mblocks * p.ksplit <= SMH_GEMM_PMAX);
+    const gemm_kernel_t kern = (p.K % 32 != 0) ? ragged : (p.chunk > 0 ? range_cut : one_each ? with_dma_wave : exact)[tiles < 2 ? 2 : tiles];
+    const long total_steps = (long)p.units * ((p.K + 31) / 32);
+    dim3 grid((unsigned)(p.chunk > 0 ? (total_steps + p.chunk - 1) / p.chunk : (long)p.units_pad * p.mblocks * p.ksplit));
     hipLaunchKernelGGL(kern, grid, dim3(kern == ragged ? GEMM_THREADS : 64 * W + (one_each ? 64 : 0)), one_each ? PS * GS_BYTES : GEMM_LDS, stream, p);
     return launch_status();
 }

@@ -58,6 +58,7 @@ struct MatmulParams {
     int units, units_pad;    // column units over all segments (GEMV: padded to a multiple of 8)
     int mblocks;             // GEMM: 128-row blocks
     int ksplit, steps_per_slice;
+    int chunk;               // GEMM, > 0: range cut - workgroup j takes steps [j * chunk, (j + 1) * chunk) of the column units laid end to end
     int epilogue, direct;
     int tiled;               // the segments' weights are in the tiled layout
     // GEMV, at most SMH_SILU_IN_MAX_M rows: the activations are not read from `a` but made by every workgroup for

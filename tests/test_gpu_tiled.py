@@ -79,6 +79,37 @@ def test_tiled_products_equal_checkpoint_layout_products(M, K, ns):
         col += nn
 
 
+@pytest.mark.parametrize("M", [17, 100, 128])
+@pytest.mark.parametrize("K,ns,slabs", [(4096, [11008, 11008], 4), (2048, [16640, 16640], 3), (1024, [7680, 7680, 7680], 4)])
+def test_range_cut_products(M, K, ns, slabs):
+    """launches whose even split would put two workgroups on some compute units and one on others deal runs of steps
+    instead: a workgroup may end one column unit and begin the next (also across two weights of the launch), and a unit
+    with fewer pieces than slabs gets zeros for the rest.  Slab count as planned, slabs equal in both layouts bit for
+    bit, sums against the oracle."""
+    from spec_mcts_amd import kernels as Kn
+    assert Kn.matmul_plan(M, K, ns) == slabs
+    ws = [_weight(K, n, 960 + i + K) for i, n in enumerate(ns)]
+    a = (torch.randn((M, K), generator=torch.Generator().manual_seed(970 + M)) * 0.5).half().cuda()
+    lin = [(w.cuda(), s.cuda(), n) for (w, s), n in zip(ws, ns)]
+    tiled = [Kn.tile_q40(w, s, K, n) for (w, s, n) in lin]
+    # slabs full of NaNs before the launch: a column no piece or zero fill writes would show
+    n = slabs * M * sum(ns)
+    out0 = torch.full((n,), float("nan"), dtype=torch.float32, device="cuda")
+    out1 = out0.clone()
+    p0 = Kn.matmul_q40_partial(a, lin, out0)
+    p1 = Kn.matmul_q40_partial(a, tiled, out1)
+    torch.cuda.synchronize()
+    assert p0.ksplit == slabs and p1.ksplit == slabs
+    assert not torch.isnan(p1.buf[:n]).any()
+    assert torch.equal(p0.buf[:n].view(torch.int32), p1.buf[:n].view(torch.int32))
+    got = Kn.partial_reduce(p1).cpu()
+    col = 0
+    for (w, s), nn in zip(ws, ns):
+        want = O.matmul_q40(a.cpu(), w, s, (K, nn))
+        assert torch.allclose(got[:, col:col + nn].float(), want.float(), rtol=1e-2, atol=2e-3)
+        col += nn
+
+
 def test_model_logits_do_not_depend_on_the_weight_layout():
     """the fused forward on tiled copies against the same forward on the checkpoint tensors: equal bit for bit,
     at prefill (GEMM), at decode (GEMV) and again after a weight has been replaced"""
