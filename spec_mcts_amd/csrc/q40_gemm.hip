@@ -1,8 +1,9 @@
 // Q4_0 dequant + matmul for large batches (decode at B = 100, prefill): c[M,N] = a[M,K] . deq(W)[K,N].
 //
-// A workgroup of 4 waves (8 on tiled weights, see the kernel) owns 128 rows of A, two adjacent 128-column blocks
-// of the weight (one full 128-byte line of packed nibbles per k) and a slice of K; two workgroups share a
-// compute unit.  Everything a 32-row step needs - 4 KB of nibbles, 256 B of scales, the 128 x 32 tile of A -
+// A workgroup of 4 waves (8 on tiled weights, plus one that only issues DMA in launches with one workgroup per compute
+// unit, see the kernel) owns 128 rows of A, two adjacent 128-column blocks of the weight (one full 128-byte line of
+// packed nibbles per k) and a slice of K - or, under a range cut, a run of steps that may end one column unit and begin
+// the next; up to two workgroups share a compute unit.  Everything a 32-row step needs - 4 KB of nibbles, 256 B of scales, the 128 x 32 tile of A -
 // goes global -> LDS by DMA (global_load_lds) into a 6-slot ring shared by the workgroup; one bare s_barrier
 // per TWO steps both publishes stages and frees the oldest ones.  (__syncthreads() would wait for every
 // outstanding DMA first, because they write LDS, and so empty the ring at every barrier.)
@@ -45,15 +46,16 @@ constexpr int GEMM_THREADS = GEMM_WAVES * 64;
 #define SMH_GEMM_STAGES 6
 #endif
 constexpr int GEMM_STAGES = SMH_GEMM_STAGES;
-// slots of the ring in the variant with a DMA wave, and the most workgroups of a launch that takes it
+// slots of the ring in the variant with a DMA wave (eight measured like six), the most workgroups of a launch that
+// takes it (one per compute unit), and whether the plan may cut ranges (gemm_fill_plan)
 #ifndef SMH_GEMM_PSLOTS
 #define SMH_GEMM_PSLOTS 6
 #endif
-#ifndef SMH_GEMM_RANGE_CUT
-#define SMH_GEMM_RANGE_CUT 1
-#endif
 #ifndef SMH_GEMM_PMAX
 #define SMH_GEMM_PMAX 256
+#endif
+#ifndef SMH_GEMM_RANGE_CUT
+#define SMH_GEMM_RANGE_CUT 1
 #endif
 constexpr int GS_WBLOCK = 8 * 128 + 64;        // the 8 rows one wave fetches, padded by 16 banks: the four row groups a
                                                // ds_read_b32 touches (lanes 16g..16g+15 read row 8g+r) then sit in different banks
@@ -61,17 +63,18 @@ constexpr int GS_W = 4 * GS_WBLOCK;            // nibbles
 constexpr int GS_S = 32 * 8;                   // scales
 constexpr int GS_A = GEMM_BM * 64;             // A tile, 64 B per row, 16-byte chunks XOR-swizzled
 constexpr int GS_BYTES = GS_W + GS_S + GS_A;               // 12800
-constexpr int GEMM_LDS = GEMM_STAGES * GS_BYTES;           // 51200
+constexpr int GEMM_LDS = GEMM_STAGES * GS_BYTES;           // 76800
 constexpr int GEMM_COLS = 256;
 
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
 
 
-// Waits until at most `stages` younger stages (PER DMA instructions each: 4 with four waves, 2 with eight) of this wave
-// are still in flight.
+// Waits until at most N DMA instructions of this wave are still in flight (the counter has six bits).
 template <int N>
 __device__ __forceinline__ void gemm_wait_vm() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N < 63 ? N : 63) : "memory"); }
+// ... at most `stages` younger stages of PER DMA instructions each (4 with four waves, 2 with eight, 5 + row tiles in
+// the DMA wave).
 template <int PER>
 __device__ __forceinline__ void gemm_wait_dma(int stages) {
     switch (stages) {
@@ -94,6 +97,7 @@ __device__ __forceinline__ void gemm_barrier() { asm volatile("s_waitcnt lgkmcnt
 // WAVES = 8 (tiled weights only): waves w and w + 4 share piece w of a tile; wave w multiplies the columns of its HIGH
 // nibbles, wave w + 4 those of the low nibbles (two B operands and half the accumulators each, the same A tiles), so
 // that every SIMD holds two waves of the workgroup and the decode of one runs under the MFMAs of the other.
+//
 // One piece of a workgroup's work: steps [step0, step1) of column unit `unit` (row block mb), accumulated and left as slab
 // `slice`.  zero_rest: the piece ends its unit, and the slabs past `slice` (the unit has no piece for them) are written as
 // zeros.  more: another piece follows in this workgroup (one more barrier, after which the ring may be refilled).
