@@ -50,6 +50,25 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert st < 0 and b"static array holds" in lib.smh_last_error_string()
 
 
+def test_matmul_plans_fit_the_workspace_the_library_asks_for():
+    """the slabs of any planned launch (even split, or runs of steps across column units above 16 rows) fit the bytes
+    smh_q40_matmul_workspace_bytes returns for the largest batch and width, and never exceed 16 slices"""
+    from spec_mcts_amd import _lib
+    lib = _lib.load()
+    widths = ([4096], [4096, 4096, 4096], [11008, 11008], [11008], [32128], [8192, 1024, 1024], [28672, 28672], [16640, 16640],
+              [7680, 7680, 7680], [128], [256, 128, 128])
+    for K in (32, 256, 1024, 2048, 4096, 8192, 11008, 28672):
+        for ns in widths:
+            n = (ctypes.c_int * len(ns))(*ns)
+            for M in (1, 2, 10, 16, 17, 64, 100, 128):
+                ks = lib.smh_q40_matmul_plan(M, K, len(ns), n)
+                assert 1 <= ks <= 16, (M, K, ns, ks)
+                assert ks * M * sum(ns) * 4 <= lib.smh_q40_matmul_workspace_bytes(M, sum(ns)), (M, K, ns, ks)
+    # the two plans the GPU tests and the design notes name
+    assert lib.smh_q40_matmul_plan(100, 4096, 2, (ctypes.c_int * 2)(11008, 11008)) == 4      # range cut: 256 runs of 43 steps
+    assert lib.smh_q40_matmul_plan(100, 4096, 3, (ctypes.c_int * 3)(4096, 4096, 4096)) == 5
+
+
 def test_host_quantiser_matches_oracle():
     """spec_mcts_amd.quant (the converter's quantiser) against the oracle on the host"""
     import torch
