@@ -6,13 +6,14 @@ Every path the benchmark times is held against the fixture: one branch (tiled GE
 the matmul launches, the one-launch attention), ten branches (GEMV, separate small kernels) and a hundred (the MFMA
 GEMM, the two-launch attention).  Two runs per path:
   teacher-forced  the GPU model is fed the ORACLE's previous token, so each of the 64 steps is checked on its own.  A step
-                  counts when the oracle's top-1/top-2 logit margin is at least the fixture's `near_tie`; below it the
-                  argmax is only reported.  near_tie comes from the oracle alone: twice the largest change of that margin
-                  between the fp32 oracle and the same oracle accumulating in double precision (two faithful evaluations
-                  of the reference's cast points drift that far apart on this chaotic 32-layer random model).
-  free-running    the GPU model is fed its own tokens, as the benchmark runs it; the length of the common prefix with the
-                  oracle's tokens is printed (after the first near-tie that falls the other way the sequences are unrelated)
-                  and must reach the first step whose margin is below near_tie."""
+                  may differ only where the oracle itself cannot decide it: its top-1/top-2 margin there is at most twice
+                  what the same oracle accumulating in double precision moves that margin AT THAT STEP, or one fp16 ulp of
+                  the logit (two faithful evaluations of the reference's cast points drift that far apart on this chaotic
+                  32-layer random model).  At most one of the 64 steps may differ per path.
+  free-running    the GPU model is fed its own tokens, as the benchmark runs it; the common prefix with the oracle's tokens
+                  must reach the path's first differing teacher-forced step (all 64 tokens when none differs).
+The per-path lines (matches, differing steps with their margins and bounds, free-run length) are also written to
+gpurun_out/greedy_7b_paths.md."""
 import json
 import os
 
@@ -24,40 +25,47 @@ pytestmark = pytest.mark.gpu
 FIXTURE = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "greedy_7b.json")
 
 
+def _fp16_ulp(x: float) -> float:
+    import math
+    x = abs(float(x))
+    return 2.0 ** (max(math.floor(math.log2(x)), -14) - 10) if x > 0 else 2.0 ** -24
+
+
 def test_7b_greedy_tokens_match_oracle():
     import bench
     from spec_mcts_amd import kernels as K
     fx = json.load(open(FIXTURE))
     seed, P, steps = fx["seed"], fx["prompt_len"], fx["steps"]
-    near_tie = fx["near_tie"]
-    assert near_tie == pytest.approx(2.0 * max(fx["noise"]["acc64"]["gap_shift"]), abs=1e-4)
+    assert fx["near_tie"] == pytest.approx(2.0 * max(fx["noise"]["acc64"]["gap_shift"]), abs=1e-4)
     want = torch.tensor(fx["tokens"], dtype=torch.int64)
-    margins = fx["margins"]
+    margins, shift64 = fx["margins"], fx["noise"]["acc64"]["gap_shift"]
     torch.manual_seed(seed)
     model = bench.build_model(torch, dict(fx["args"], max_batch_size=100), seed=seed)
     prompt = torch.randint(0, fx["args"]["vocab_size"], (1, P), generator=torch.Generator().manual_seed(seed)).cuda()
-    decidable = [i for i, m in enumerate(margins) if m >= near_tie]
-    first_near_tie = next(i for i, m in enumerate(margins) if m < near_tie)
-    assert len(decidable) >= steps * 2 // 3, "fixture has too many near-ties to be a test"
-    print(f"near_tie {near_tie}: {len(decidable)} of {steps} steps decidable, first near-tie at step {first_near_tie}", flush=True)
+    report = ["# Greedy tokens of the 7B-architecture model against the oracle's (tests/test_gpu_model_7b.py)\n",
+              f"Fixture: seed {seed}, {P}-token prompt, {steps} greedy steps; smallest oracle margins: "
+              + ", ".join(f"step {i}: {margins[i]}" for i in sorted(range(steps), key=lambda i: margins[i])[:4]) + ".\n",
+              "| branches | teacher-forced equal | differing steps (oracle margin, bound) | free-running equal |", "|---:|---:|---|---:|"]
     for B in (1, 10, 100):
         # ---- teacher-forced ----
         model.resetSeq()
         logits = model(prompt, 0)[:, -1]
         got = torch.zeros((B, steps), dtype=torch.int64)
+        top = torch.zeros(steps)
         got[:, 0] = int(K.argmax(logits.contiguous())[0])
+        top[0] = float(logits[0].max())
         for s in range(1, steps):
             tok = want[s - 1].expand(B, 1).contiguous().cuda()            # the oracle's token, not the model's own
             lg = model(tok, P + s - 1)[:, -1]
             got[:, s] = K.argmax(lg.contiguous()).cpu()
+            top[s] = float(lg[0].max())
         torch.cuda.synchronize()
         for b in range(1, B):
             assert torch.equal(got[b], got[0]), "identical branches must produce identical tokens"
         differing = [i for i in range(steps) if int(got[0, i]) != int(want[i])]
-        print(f"B={B} teacher-forced: {steps - len(differing)}/{steps} tokens equal the oracle's; differing steps and their oracle margins "
-              f"{[(i, margins[i]) for i in differing]}", flush=True)
-        wrong = [i for i in differing if margins[i] >= near_tie]
-        assert not wrong, f"B={B}: tokens differ at steps {wrong} where the oracle's margin is {[margins[i] for i in wrong]} >= {near_tie}"
+        bound = {i: max(2.0 * shift64[i], _fp16_ulp(top[i])) for i in differing}
+        print(f"B={B} teacher-forced: {steps - len(differing)}/{steps} tokens equal the oracle's; differing steps (oracle margin, bound) "
+              f"{[(i, margins[i], bound[i]) for i in differing]}", flush=True)
         # ---- free-running ----
         model.resetSeq()
         logits = model(prompt, 0)[:, -1]
@@ -71,4 +79,21 @@ def test_7b_greedy_tokens_match_oracle():
             assert torch.equal(free[b], free[0])
         run = next((i for i in range(steps) if int(free[0, i]) != int(want[i])), steps)
         print(f"B={B} free-running: first {run} tokens equal the oracle's" + (f" (oracle margin at step {run}: {margins[run]})" if run < steps else ""), flush=True)
-        assert run >= first_near_tie, f"B={B}: free-running tokens leave the oracle's at step {run}, before the first near-tie (step {first_near_tie})"
+        report.append(f"| {B} | {steps - len(differing)} / {steps} | " + (", ".join(f"step {i} ({margins[i]}, {bound[i]:.4f})" for i in differing) or "none")
+                      + f" | {run} / {steps} |")
+        _write_report(report)
+        wrong = [i for i in differing if margins[i] > bound[i]]
+        assert not wrong, f"B={B}: tokens differ at steps {wrong} where the oracle's margin {[margins[i] for i in wrong]} exceeds {[bound[i] for i in wrong]}"
+        assert len(differing) <= 1, f"B={B}: {len(differing)} of {steps} teacher-forced tokens differ from the oracle's (at most one may)"
+        first_diff = differing[0] if differing else steps
+        assert run >= first_diff, f"B={B}: free-running tokens leave the oracle's at step {run}, before the first undecidable step ({first_diff})"
+
+
+def _write_report(lines):
+    out = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+    try:
+        os.makedirs(out, exist_ok=True)
+        with open(os.path.join(out, "greedy_7b_paths.md"), "w") as f:
+            f.write("\n".join(lines) + "\n")
+    except OSError:
+        pass
