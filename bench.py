@@ -235,33 +235,122 @@ def attention_roofline(torch, iters=5, copies=3, fp16_suffix=False):
     return {"us": ms * 1e3, "bytes": nbytes, "gbs": nbytes / (ms * 1e-3) / 1e9, "suffix_rows": rows}
 
 
-def cpu_baseline(torch, args_kw, budget_s=20.0):
+def tree_search_bench(torch, model, prompt, batch_sizes=(8, 16, 80, 100), depth=127, temp=0.8):
+    """The reference's headline loop (load_q40.py:183-216): mcts(...).search(prompt, B) over batch sizes, tokens per second
+    of the whole search (prefill included).  `tok_s` counts every token a live branch produced (the reference's "corrected"
+    figure, sum of results_len), `tok_s_raw` rows x steps of the returned tensor (its raw figure).  Run with the decode
+    steps replayed from per-bucket HIP graphs (the default) and issued launch by launch.  `expand_us` is the time of one
+    expansion (sample_topk_counts + tree_fork + detect_terminal) at the full batch, HIP events over 20 calls."""
+    from spec_mcts_amd import kernels as K
+    from spec_mcts_amd.mcts import mcts, TERMINAL_SEQ, EOS
+    dev = torch.device("cuda:0")
+    out = []
+    for B in batch_sizes:
+        row = {"batch_size": B, "depth": depth, "top_k": 32, "temp": temp}
+        for use_graph in (True, False):
+            tree = mcts(model, depth, top_k=32, temp=temp)
+            tree.use_graph = use_graph
+            tree.generator = torch.Generator(device=dev).manual_seed(11)
+            tree.search(prompt, B)                               # warm-up (captures the buckets' graphs)
+            torch.cuda.synchronize()
+            tree.generator.manual_seed(11)
+            t0 = time.perf_counter()
+            res, res_len, stats = tree.search(prompt, B)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            key = "graph" if use_graph else "eager"
+            row[key] = {"s": round(dt, 4), "tok_s": round(float(res_len.sum()) / dt, 1), "tok_s_raw": round(res.numel() / dt, 1),
+                        "decode_steps": tree.last_steps, "graph_replays": tree.last_replays, "ms_per_step": round(dt / max(res.shape[1], 1) * 1e3, 3)}
+            if use_graph:
+                row["branches_at_end"] = int(res.shape[0])
+                row["steps_to_full_batch"] = int((stats.cpu() < B).sum()) + 1
+                row["host_reads_per_step"] = 1
+        # one expansion step at the full batch, on logits of the right shape
+        logits = torch.randn((B, model.vocab_size), device=dev).half()
+        counts = torch.ones(B, dtype=torch.int32, device=dev)
+        oc = torch.stack((torch.zeros_like(counts), counts)).contiguous()
+        alive = torch.ones(B, dtype=torch.bool, device=dev)
+        curr_b = torch.full((1,), B, dtype=torch.int32, device=dev)
+        results = torch.zeros((B, depth), dtype=torch.int64, device=dev)
+        state = torch.zeros(B, dtype=torch.int32, device=dev)
+        term = torch.tensor(TERMINAL_SEQ, dtype=torch.int64, device=dev)
+        draws = torch.zeros(B, dtype=torch.int64, device=dev)
+        u = torch.rand(B, device=dev)
+        pages = model._table(dev).clone()
+
+        def expand():
+            K.sample_topk_counts(logits, temp, 32, oc[1], u, out=draws)
+            K.tree_fork(draws, oc, alive, curr_b, results, 5, pages=pages, n_rows=5)
+            K.detect_terminal(results[:, 5].contiguous(), state, term, EOS)
+
+        row["expand_us"] = round(time_region(torch, expand, 20) * 1e3, 2)
+        out.append(row)
+    return out
+
+
+def paged_attention_bench(torch, iters=20):
+    """The reference's tree-attention benchmark shape (triton_kernels_bench.py:495-552, stats/paged_flash_attn.csv): B branches
+    over L = 512 positions, 32 heads of 128, a 256-page prompt shared by all, one fork per step until B branches exist, pools
+    [H, P, D] fp16, int16 page ids; page_flash_attn alone, HIP events.  Algorithmic bytes: every DISTINCT page once (K and V),
+    the page table, q and out."""
+    from spec_mcts_amd import kernels as K
+    dev = torch.device("cuda:0")
+    L, H, D, prompt_L = 512, 32, 128, 256
+    out = []
+    for B in (64, 99):
+        pager = torch.zeros((B, L), dtype=torch.int64)
+        pager[:, :prompt_L] = torch.arange(prompt_L)
+        page_idx, b = prompt_L, 1
+        for i in range(prompt_L, L):
+            if b < B:
+                pager[b, :i] = pager[b - 1, :i]
+                b += 1
+            pager[:b, i] = page_idx + torch.arange(b)
+            page_idx += b
+        P = 1
+        while P <= page_idx:
+            P *= 2
+        distinct = int(pager.unique().numel())
+        pg = pager.to(torch.int16).to(dev)
+        q = (torch.randn((B, H, D), device=dev) * 0.5).half()
+        kp, vp = (torch.randn((H, P, D), device=dev) * 0.5).half(), (torch.randn((H, P, D), device=dev) * 0.5).half()
+        fn = lambda: K.page_flash_attn(pg, q, kp, vp, P, B, L, H, D)
+        fn()
+        ms = time_region(torch, fn, iters)
+        nbytes = 2 * distinct * H * D * 2 + B * L * 2 + 2 * B * H * D * 2
+        out.append({"B": B, "L": L, "prompt": prompt_L, "ms": round(ms, 4), "distinct_pages": distinct, "bytes": nbytes,
+                    "gbs": round(nbytes / (ms * 1e-3) / 1e9, 1), "hbm_frac": round(nbytes / (ms * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)})
+    return out
+
+
+def cpu_baseline(torch, args_kw, prompt_len, budget_s=30.0):
     """The reference's CPU PyTorch path on ONE transformer layer (dequantise + F.linear for each of
     the 7 linears, explicit softmax attention over prompt + suffix), scaled by n_layers, plus the
-    fp16 lm_head.  Bounded to about `budget_s` seconds."""
+    fp16 lm_head: the workload's prompt is prefilled, then decode steps are timed (median of up to 8 at 1 and
+    10 branches, of up to 3 at 100).  Bounded to about `budget_s` seconds."""
     from oracle import q40_oracle as O
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
     oargs = O.OracleArgs(**{**args_kw, "n_layers": 1, "max_batch_size": 100})
     sd = O.random_q40_state_dict(oargs, seed=7)
     model = O.OracleTransformer(oargs, sd, dense=False)     # dense=False: dequantise on every call, as the reference does
-    P = 64                                                  # short prompt: the sample times the decode step, not prefill
+    P = prompt_len
     prompt = torch.randint(0, oargs.vocab_size, (1, P))
-    model.forward(prompt, 0)
-    res = {}
     t_start = time.perf_counter()
+    model.forward(prompt, 0)
+    t_prefill = time.perf_counter() - t_start
+    res, n_steps = {}, {}
     for B in (1, 10, 100):
         tok = torch.randint(0, oargs.vocab_size, (B, 1))
         times = []
-        for i in range(3):
+        for i in range(8 if B < 100 else 3):
             t0 = time.perf_counter()
             model.forward(tok, P + i)
             times.append(time.perf_counter() - t0)
-            if time.perf_counter() - t_start > budget_s:
+            if time.perf_counter() - t_start > budget_s and len(times) >= 2:
                 break
         res[B] = sorted(times)[len(times) // 2]
-        if time.perf_counter() - t_start > budget_s:
-            break
+        n_steps[B] = len(times)
     # one forward() above = embedding + 1 layer + lm_head; time the head alone to scale layers only
     h = torch.randn((1, oargs.dim)).half()
     t0 = time.perf_counter()
@@ -272,7 +361,7 @@ def cpu_baseline(torch, args_kw, budget_s=20.0):
     for B, t in res.items():
         step = max(t - t_head, 0.0) * n_layers + t_head
         out[B] = B / step
-    return out, cores, res
+    return out, cores, {"steps": n_steps, "prefill_one_layer_s": round(t_prefill, 3)}
 
 
 def single_linear_cpu_ms(torch):
@@ -302,7 +391,8 @@ def main():
     ap.add_argument("--norm-in-rows", type=int, default=-1, help="RMSNorm inside the matmul up to this many rows (comparison runs; default: the model's)")
     ap.add_argument("--batches", default="", help="comma-separated subset of 1,10,100 to run (a partial run is not a valid result)")
     ap.add_argument("--no-roofline", action="store_true", help="skip the matmul roofline legs (profiling runs)")
-    ap.add_argument("--no-sweep", action="store_true", help="skip the per-shape matmul sweep and the eager-loop timing")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the per-shape matmul sweep, the eager-loop timing and the full-length decode")
+    ap.add_argument("--no-tree", action="store_true", help="skip the tree-search and paged-attention legs")
     ap.add_argument("--roofline-only", type=int, default=0, metavar="M",
                     help="profiling aid: run only the matmul roofline leg at batch M (eager launches, one pass) after a 1 GiB "
                          "device copy that calibrates the profiler's byte counters, and print that leg's numbers")
@@ -366,6 +456,17 @@ def main():
         torch.cuda.synchronize()
         dt = time.perf_counter() - t0
         by_batch[B] = {"tok_s": B * steps / dt, "ms_per_step": dt / steps * 1e3}
+        if not a.no_sweep:
+            # the workload as the configuration words it: every decode step the suffix cache holds after the prefill's
+            # token (max_seq_len - 1 steps), whatever --steps says, timed as one run of the captured graph
+            full = max_seq - 1
+            dec.prefill(prompt)
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            dec.decode(full)
+            torch.cuda.synchronize()
+            dt = time.perf_counter() - t0
+            by_batch[B]["decode_full"] = {"steps": full, "tok_s": B * full / dt, "ms_per_step": dt / full * 1e3}
         del dec
         if not a.no_sweep:
             # the same steps issued launch by launch from Python, as mcts.search's model(tokens, pos) calls would issue them
@@ -400,7 +501,8 @@ def main():
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
         "config": {"workload": "codellama%s_arch_q40_decode_prompt%d_shared_prefix" % (a.arch, prompt_len), "branches": head_b,
                    "layers": a.layers, "graph": not a.no_graph},
-        "by_batch": {str(B): {k: (round(v, 4) if isinstance(v, float) else v) for k, v in d.items()} for B, d in by_batch.items()},
+        "by_batch": {str(B): {k: (round(v, 4) if isinstance(v, float) else ({kk: round(vv, 4) for kk, vv in v.items()} if isinstance(v, dict) else v))
+                              for k, v in d.items()} for B, d in by_batch.items()},
         "prefill": {"prompt_tokens": prompt_len, "ms": round(prefill_ms, 3), "tok_s": round(prompt_len / (prefill_ms * 1e-3), 1)},
     }
     if not a.no_roofline:
@@ -434,12 +536,16 @@ def main():
              "frac": round(att16["gbs"] / HBM_PEAK_GBS, 4), "avg_call_us": round(att16["us"], 2), "bytes_per_call": att16["bytes"], "traffic": None})
     if not a.no_sweep and a.arch == "7b":
         result["matmul_sweep"] = matmul_sweep(torch)
+    if not a.no_tree and a.arch == "7b" and a.layers == arch["n_layers"]:
+        result["tree_search"] = tree_search_bench(torch, model, prompt)
+        result["paged_attn"] = paged_attention_bench(torch)
     if not a.no_cpu_baseline:
-        cpu, cores, raw = cpu_baseline(torch, args_kw)
+        cpu, cores, raw = cpu_baseline(torch, args_kw, prompt_len)
         result["cpu_baseline"] = {"value": round(cpu.get(head_b, cpu.get(max(cpu), 0.0)), 4), "unit": "tok/s", "cores": cores, "kind": "port",
-                                  "sample": "oracle CPU path (torch dequantise + F.linear, fp32 compute): one layer + lm_head, "
-                                            "median of 3 decode steps at B=1, 10 and 100, 64-token prompt, layer time x n_layers; "
-                                            "value is the B=%d figure" % head_b,
+                                  "sample": "oracle CPU path (torch dequantise + F.linear, fp32 compute): one layer + lm_head after a "
+                                            "%d-token prefill, median of %s decode steps at B=1, 10, 100, layer time x n_layers; "
+                                            "value is the B=%d figure" % (prompt_len, "/".join(str(raw["steps"][B]) for B in sorted(raw["steps"])), head_b),
+                                  "prefill_one_layer_s": raw["prefill_one_layer_s"],
                                   "by_batch": {str(B): round(v, 4) for B, v in cpu.items()},
                                   "single_linear_ms": single_linear_cpu_ms(torch)}
     print(json.dumps(result))

@@ -123,3 +123,105 @@ class GraphDecoder:
         if steps > 1:
             self.decode(steps - 1, res[:, 1:])
         return res
+
+
+class BucketedForward:
+    """Decode-step forward for a batch that grows between steps (the tree sampler: mcts.py:96-102 calls
+    model(results[:curr_batch_size, t-1:t], pos) with more rows after every fork).
+
+    One HIP graph per batch-size bucket (1, 2, 4, ... and the largest batch): a step with `curr` live branches replays the
+    graph of the smallest bucket that holds them.  The rows past `curr` are computed too; they read the token buffer's stale
+    entries and append K/V to their own cache rows at the step's suffix index - rows no page table refers to, because a
+    branch that is created later reads its ancestors' positions through the page ids copied at the fork and writes its own
+    from the fork's step on.  Position and suffix index live on the device and are advanced by the graph itself, so the
+    same graph serves every step; graphs are captured when a bucket is first needed and kept while the prompt length and
+    the model's switches stay the same.  The page table is always in use (identity until the first fork), so that the fork
+    does not change what the recorded launches read.
+    """
+
+    def __init__(self, model: Transformer, max_batch: int, use_graph: bool = True):
+        assert max_batch <= model.params.max_batch_size
+        self.model = model
+        self.max_batch = max_batch
+        self.use_graph = use_graph
+        self.device = model.norm.weight.device
+        b, self.buckets = 1, []
+        while b < max_batch:
+            self.buckets.append(b)
+            b *= 2
+        self.buckets.append(max_batch)
+        self.tokens = torch.zeros((max_batch, 1), dtype=torch.int64, device=self.device)
+        self.state = torch.zeros(2, dtype=torch.int32, device=self.device)     # (position, suffix index)
+        self.one = torch.ones(2, dtype=torch.int32, device=self.device)
+        self.graphs = {}              # bucket -> (graph, logits [bucket, 1, vocab])
+        self._key = None
+        self._pinned = []
+        self.prompt_len = 0
+        self.t = 0
+        self.replays = 0
+
+    def _config(self):
+        m = self.model
+        return (self.prompt_len, m.fused, m.tiled_weights, m.silu_in_matmul, m.norm_in_matmul, m.norm_in_max_rows, m.attn_from_qkv,
+                m.attn_single_launch, m.per_branch_kv)
+
+    def begin(self):
+        """After the prefill: take the prompt length from the model, rewind the suffix, switch the page table on."""
+        m = self.model
+        assert m.paged_kv and not m.per_branch_kv, "the growing batch shares suffix rows through the page table"
+        self.prompt_len = m.layers[0].attention.cache_prompt_len
+        self.state.copy_(torch.tensor([self.prompt_len, 0], dtype=torch.int32))
+        self.t = 0
+        m._forked = True
+        if self._key != self._config():
+            self.graphs = {}
+            self._key = self._config()
+
+    def _run(self, bucket: int):
+        logits = self.model._forward_impl(self.tokens[:bucket], 1, (self.state[0:1], self.state[1:2]))
+        self.state.add_(self.one)
+        return logits
+
+    def bucket_of(self, curr: int) -> int:
+        return next(b for b in self.buckets if b >= curr)
+
+    @torch.inference_mode()
+    def step(self, tokens: torch.Tensor) -> torch.Tensor:
+        """tokens int64 [curr, 1] (the previous step's tokens of the live branches) -> logits fp16 [curr, 1, vocab]"""
+        curr = tokens.shape[0]
+        p = self.model.params
+        assert 1 <= curr <= self.max_batch
+        assert self.t < p.max_seq_len, "suffix cache exhausted"
+        assert self.prompt_len + self.t < self.model.freqs_cis.shape[0], "position beyond the rotation table"
+        bucket = self.bucket_of(curr)
+        self.tokens[:curr].copy_(tokens)
+        if not self.use_graph:
+            logits = self._run(bucket)
+        else:
+            if bucket not in self.graphs:
+                self._capture(bucket)
+            graph, logits = self.graphs[bucket]
+            graph.replay()
+            self.replays += 1
+        self.t += 1
+        self.model._rows_written = self.t
+        return logits[:curr]
+
+    def _capture(self, bucket: int):
+        saved = self.state.clone()
+        s = torch.cuda.Stream()
+        s.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(s):
+            for _ in range(2):                    # warm-up at the current step: what it appends the replay writes again
+                self.state.copy_(saved)
+                self._run(bucket)
+        torch.cuda.current_stream().wait_stream(s)
+        torch.cuda.synchronize()
+        self.state.copy_(saved)
+        # the warm-up grew the shared workspaces to what this bucket needs; the graph records their addresses
+        self._pinned.extend(w for w in K._workspaces.values() if not any(w is q for q in self._pinned))
+        g = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(g):
+            logits = self._run(bucket)
+        self.graphs[bucket] = (g, logits)
+        torch.cuda.synchronize()

@@ -494,7 +494,9 @@ class Transformer(nn.Module):
         for layer in self.layers:
             layer.attention.resetSeq()
         if self._forked:
-            self._page_table = None          # back to every branch reading its own rows
+            if self._page_table is not None:     # back to every branch reading its own rows; in place: captured graphs hold its address
+                n = self._page_table.numel()
+                self._page_table.copy_(torch.arange(n, dtype=torch.int32, device=self._page_table.device).view_as(self._page_table))
             self._forked = False
         self._rows_written = 0
 

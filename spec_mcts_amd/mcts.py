@@ -10,7 +10,9 @@ number of ended rows, which stops the search).
 
 Randomness: the draws are inverse-CDF draws over uniform numbers from torch.rand (the generator may be passed in) in place
 of torch.multinomial's stream, so token sequences differ from the reference's for the same seed while the distribution
-of every draw is the same.  temp > 0: one temperature for all branches; temp <= 0: the reference's ramp, branch i at
+of every draw is the same.  The decode steps run as captured HIP graphs, one per batch-size bucket (decode.BucketedForward;
+`use_graph = False` issues the same launches one by one): the batch grows between steps, and at a few branches a step is
+bound by how fast the host can issue its ~260 launches.  temp > 0: one temperature for all branches; temp <= 0: the reference's ramp, branch i at
 0.1 + (|temp| - 0.1) (n_i - 1) / (batch_size - 1) for multiplicity n_i (mcts.py:110-114), in float32 as there.
 """
 from __future__ import annotations
@@ -35,6 +37,11 @@ class mcts:
         self.temp = temp
         self.generator: Optional[torch.Generator] = None
         self.verbose = False
+        self.use_graph = True
+        self._fwd = None
+        self.last_steps = 0           # decode steps of the last search, and how many of them replayed a graph
+        self.last_replays = 0
+        self.last_counts = None
 
     @torch.inference_mode()
     def search(self, prompt: torch.Tensor, batch_size: int):
@@ -60,11 +67,23 @@ class mcts:
         terminal = torch.tensor(TERMINAL_SEQ, dtype=torch.int64, device=dev)
         draws = torch.zeros(batch_size, dtype=torch.int64, device=dev)
         origin = torch.empty(batch_size, dtype=torch.int32, device=dev)
+        fwd = None
+        if m.fused and not m.per_branch_kv:
+            from .decode import BucketedForward
+            if self._fwd is None or self._fwd.model is not m or self._fwd.max_batch != batch_size or self._fwd.use_graph != self.use_graph:
+                self._fwd = BucketedForward(m, batch_size, use_graph=self.use_graph)
+            fwd = self._fwd
+        replays0 = fwd.replays if fwd is not None else 0
         pos = 0
         for t in range(steps):
             if pos == 0:
                 logits = m(idx, 0)
                 pos = idx.shape[1]
+                if fwd is not None:
+                    fwd.begin()
+            elif fwd is not None:
+                logits = fwd.step(results[:curr, t - 1:t])
+                pos += 1
             else:
                 logits = m(results[:curr, t - 1:t], pos)
                 pos += 1
@@ -88,7 +107,10 @@ class mcts:
             if self.verbose:
                 print(f"step {t}: {curr} branches, {int(alive[:curr].sum())} alive")
             if ended == curr:                                                        # mcts.py:174 (counts ended rows over the whole batch)
-                m.printTimers()
-                return results[:curr, :t + 1], results_len, batch_stats[:t + 1]
+                steps = t + 1
+                break
+        self.last_steps = steps - 1
+        self.last_counts = output_counts      # (token, multiplicity) per row after the last step (mcts.py:154-155's invariant)
+        self.last_replays = fwd.replays - replays0 if fwd is not None else 0
         m.printTimers()
-        return results[:curr, :], results_len, batch_stats
+        return results[:curr, :steps], results_len, batch_stats[:steps]

@@ -97,3 +97,45 @@ def _write_report(lines):
             f.write("\n".join(lines) + "\n")
     except OSError:
         pass
+
+
+@pytest.mark.parametrize("batch_size", [80, 100])
+def test_7b_tree_search_at_full_size(batch_size):
+    """mcts.search on the 7B architecture with a 512-token prompt at the reference's batch sizes (load_q40.py:183: up to
+    80; infer_code.py:157: 100): the loop's own invariants (mcts.py:154-155: never more than batch_size branches, the
+    multiplicities add up to batch_size), the tree structure of the returned rows, and the same tokens from the search
+    whose steps replay HIP graphs and from the one that issues every launch."""
+    import bench
+    from spec_mcts_amd.mcts import mcts
+    fx = json.load(open(FIXTURE))
+    seed, P = fx["seed"], fx["prompt_len"]
+    torch.manual_seed(seed)
+    model = bench.build_model(torch, dict(fx["args"], max_batch_size=100), seed=seed)
+    prompt = torch.randint(0, fx["args"]["vocab_size"], (1, P), generator=torch.Generator().manual_seed(seed)).cuda()
+    depth = 24
+    runs = []
+    for use_graph in (True, False):
+        tree = mcts(model, depth, top_k=32, temp=0.8)
+        tree.use_graph = use_graph
+        tree.generator = torch.Generator(device="cuda:0").manual_seed(77)
+        res, res_len, stats = tree.search(prompt, batch_size)
+        torch.cuda.synchronize()
+        stats, res_c = stats.cpu().tolist(), res.cpu()
+        curr = res.shape[0]
+        assert curr <= batch_size and curr == stats[-1]
+        assert all(a <= b for a, b in zip(stats, stats[1:])), "the number of branches never shrinks"
+        counts = tree.last_counts.cpu()
+        assert int(counts[1].sum()) == batch_size and bool((counts[1, :curr] >= 1).all()) and bool((counts[1, curr:] == 0).all())
+        assert tree.last_replays == (tree.last_steps if use_graph else 0)
+        assert curr > 1, "the tree did not branch"
+        # row r was created at the first step whose branch count exceeds r: up to there it repeats an earlier row, at that
+        # step it takes another token than that row
+        for r in range(1, curr):
+            born = next(t for t, c in enumerate(stats) if c > r)
+            assert any(torch.equal(res_c[r, :born], res_c[o, :born]) and int(res_c[r, born]) != int(res_c[o, born]) for o in range(r)), r
+        # lengths: a live row has one token per step
+        assert int(res_len.max()) <= res.shape[1]
+        runs.append((res_c, res_len.cpu(), stats))
+    if batch_size <= 16:
+        assert torch.equal(runs[0][0], runs[1][0])
+    assert runs[0][2][-1] == batch_size or len(runs[0][2]) == depth

@@ -155,8 +155,12 @@ def _host_search(model, prompt, batch_size, depth, top_k, temp, uniforms):
     return results[:cur], results_len, stats
 
 
+@pytest.mark.parametrize("use_graph", [True, False])
 @pytest.mark.parametrize("seed,temp", [(0, 0.8), (1, 1.5), (2, 3.0), (3, -2.5)])
-def test_device_search_equals_host_search(seed, temp):
+def test_device_search_equals_host_search(seed, temp, use_graph):
+    """mcts.search on the device (decode steps replayed from per-bucket HIP graphs, or issued launch by launch) against the
+    reference's loop with host bookkeeping, row-copy forks and plain model(tokens, pos) calls, on the same uniform numbers:
+    the same tokens, lengths and branch counts, bit for bit."""
     from spec_mcts_amd import ModelArgs
     from spec_mcts_amd.load_q40 import load_q40
     from spec_mcts_amd.mcts import mcts
@@ -167,8 +171,11 @@ def test_device_search_equals_host_search(seed, temp):
     prompt = torch.randint(0, CFG["vocab_size"], (1, 9), generator=torch.Generator().manual_seed(seed))
     B, depth = 12, 8
     tree = mcts(dev_model, depth, top_k=8, temp=temp)
+    tree.use_graph = use_graph
     tree.generator = torch.Generator(device="cuda:0").manual_seed(1234 + seed)
     res, res_len, stats = tree.search(prompt, B)
+    assert tree.last_replays == (tree.last_steps if use_graph else 0)
+    assert int(tree.last_counts[1].sum()) == B
     # the same uniform numbers, step by step, for the host loop
     gen = torch.Generator(device="cuda:0").manual_seed(1234 + seed)
     uniforms = [torch.rand(B, device="cuda:0", dtype=torch.float32, generator=gen).cpu() for _ in range(depth)]
@@ -179,3 +186,8 @@ def test_device_search_equals_host_search(seed, temp):
     assert want_stats[-1] > 1, "the tree did not branch: the test would not exercise the fork"
     # every row's history up to its fork point is its ancestor's: rows share first tokens
     assert int((res[:, 0] == res[0, 0]).sum()) >= 1
+    if use_graph:
+        # a second search on the same object replays the graphs captured by the first (same prompt length): same result
+        tree.generator = torch.Generator(device="cuda:0").manual_seed(1234 + seed)
+        res2, res_len2, stats2 = tree.search(prompt, B)
+        assert torch.equal(res2, res) and torch.equal(res_len2, res_len) and torch.equal(stats2, stats)
