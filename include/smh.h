@@ -201,8 +201,9 @@ int smh_sample_topk(const void *logits, int rows, int vocab, long ld, float temp
  *   batch_size <= 1024. */
 int smh_sample_topk_counts(const void *logits, int rows, int vocab, long ld, float temperature, int top_k,
                            const float *uniform, const int32_t *counts, int64_t *out, int n_draws, smh_stream_t stream);
-/* smh_sample_topk_rowtemp: smh_sample_topk_counts with a temperature per row, row_temps fp32 [rows] on the device, all
- * positive - the tree sampler's temp <= 0 mode, where the logits of branch i are divided by a ramp of its multiplicity
+/* smh_sample_topk_rowtemp: smh_sample_topk_counts with a temperature per row, row_temps fp32 [rows] on the device (a row
+ * whose temperature is not positive draws its largest logit every time, lowest index first among equals: the limit of the
+ * distribution) - the tree sampler's temp <= 0 mode, where the logits of branch i are divided by a ramp of its multiplicity
  * (mcts.py:110-114).  There the divisor is a float32 TENSOR, which promotes the fp16 logits: quotients, softmax and
  * probabilities are fp32 here too (no fp16 rounding of x or p); the candidates are the top_k largest logits. */
 int smh_sample_topk_rowtemp(const void *logits, int rows, int vocab, long ld, const float *row_temps, int top_k,
@@ -277,7 +278,9 @@ int smh_prefill_attn(const void *q, const void *k, const void *v, void *out, int
  *                (0, 0 = token-major [P, Hkv, D]; a head-major pool [Hkv, rows, D] is (D, rows * D))
  *   pool         SMH_KV_FP16: pool_k/v fp16 with pool_row_stride / pool_head_stride as above;
  *                SMH_KV_Q40: the model's cache rows, bytes [rows, Hkv, 64] + scales fp16 [rows, Hkv, 2] (strides 0)
- *   pages        page ids [B, pages_stride] of page_bytes = 2, 4 or 8 bytes each (int16 as in the reference, int32, int64);
+ *   pages        page ids of page_bytes = 2, 4 or 8 bytes each (int16 as in the reference, int32, int64): row b starts at
+ *                element b * pages_stride and holds pages_cols ids (a column slice of a wider table has pages_cols <
+ *                pages_stride); lens[b] is cut to pages_cols, so no id past a row's end is read;
  *                the pool has pool_rows rows: an id outside 0 .. pool_rows-1 is read as the nearest valid row (a wrong
  *                result for that branch, never an access outside the pool)
  *   lens         int32 [B] (lens_stride 1) or one shared int32 (lens_stride 0): pages of the branch that are valid
@@ -287,7 +290,7 @@ int smh_paged_prefix_attn(const void *q, void *out, int B, int H, int Hkv, int D
                           const void *prefix_k, const void *prefix_v, int P, long prefix_row_stride, long prefix_head_stride,
                           int pool_format, const void *pool_k, const void *pool_v, const void *pool_ks, const void *pool_vs,
                           long pool_row_stride, long pool_head_stride, long pool_rows,
-                          const void *pages, int page_bytes, long pages_stride, const int32_t *lens, int lens_stride,
+                          const void *pages, int page_bytes, long pages_stride, int pages_cols, const int32_t *lens, int lens_stride,
                           const void *cur_k, const void *cur_v, int single_launch,
                           void *workspace, size_t workspace_bytes, smh_stream_t stream);
 int smh_page_fork(int32_t *table, int rows, long stride, int origin, int curr, int forks, int n, smh_stream_t stream);

@@ -71,7 +71,7 @@ SIGNATURES = {
     "smh_shared_prefix_attn_qkv": (c_int, [_P, c_int, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, c_int,
                                            _P, _P, _P, _P, c_int, _P, _P, c_int, c_int, _P, c_size_t, _P]),
     "smh_paged_prefix_attn": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, c_long, c_long,
-                                      c_int, _P, _P, _P, _P, c_long, c_long, c_long, _P, c_int, c_long, _P, c_int, _P, _P, c_int,
+                                      c_int, _P, _P, _P, _P, c_long, c_long, c_long, _P, c_int, c_long, c_int, _P, c_int, _P, _P, c_int,
                                       _P, c_size_t, _P]),
     "smh_page_fork": (c_int, [_P, c_int, c_long, c_int, c_int, c_int, c_int, _P]),
 }

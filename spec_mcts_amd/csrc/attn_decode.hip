@@ -1069,11 +1069,12 @@ extern "C" int smh_paged_prefix_attn(const void *q, void *out, int B, int H, int
                                      const void *prefix_k, const void *prefix_v, int P, long prefix_row_stride, long prefix_head_stride,
                                      int pool_format, const void *pool_k, const void *pool_v, const void *pool_ks, const void *pool_vs,
                                      long pool_row_stride, long pool_head_stride, long pool_rows,
-                                     const void *pages, int page_bytes, long pages_stride, const int32_t *lens, int lens_stride,
+                                     const void *pages, int page_bytes, long pages_stride, int pages_cols, const int32_t *lens, int lens_stride,
                                      const void *cur_k, const void *cur_v, int single_launch,
                                      void *workspace, size_t workspace_bytes, smh_stream_t stream) {
     using namespace smh;
     const char *who = "smh_paged_prefix_attn";
+    SMH_REQUIRE(pages_cols >= 1 && pages_cols <= pages_stride, "%s: pages_cols=%d must lie in 1 .. pages_stride=%ld", who, pages_cols, pages_stride);
     SMH_REQUIRE(pool_format == SMH_KV_FP16 || pool_format == SMH_KV_Q40, "%s: pool_format=%d", who, pool_format);
     SMH_REQUIRE(pages != nullptr && (page_bytes == 2 || page_bytes == 4 || page_bytes == 8) && pages_stride >= 1,
                 "%s: pages=%p page_bytes=%d (2, 4 or 8) pages_stride=%ld", who, pages, page_bytes, pages_stride);
@@ -1086,8 +1087,9 @@ extern "C" int smh_paged_prefix_attn(const void *q, void *out, int B, int H, int
     AttnExtras ex;
     ex.pages = pages; ex.page_bytes = page_bytes; ex.pages_stride = pages_stride; ex.pool_rows = pool_rows;
     ex.pfx_row = prefix_row_stride; ex.pfx_head = prefix_head_stride; ex.sfx_row = pool_row_stride; ex.sfx_head = pool_head_stride;
+    // (the kernels cut lens[b] to the row count they are given: the ids a table row holds, not the distance between rows)
     return shared_prefix_attn(who, single_launch != 0, q, out, B, H, Hkv, D, prefix_k, prefix_v, P, pool_format, pool_k, pool_v, pool_ks, pool_vs,
-                              (int)pages_stride, lens, lens_stride, cur_k, cur_v, workspace, workspace_bytes, stream, ex);
+                              pages_cols, lens, lens_stride, cur_k, cur_v, workspace, workspace_bytes, stream, ex);
 }
 
 // copies entries 0 .. n - 1 of row `origin` of a page table [rows, stride] to rows curr .. curr + forks - 1
@@ -1148,6 +1150,8 @@ extern "C" int smh_shared_prefix_attn_static(const void *q, void *out, int B, in
                                              smh_stream_t stream) {
     using namespace smh;
     const char *who = "smh_shared_prefix_attn_static";
+    // (every argument check comes before the scratch array's address is asked for: a refused call does not touch the device)
+    SMH_REQUIRE(D == ATT_D, "%s: head dim %d (only 128)", who, D);
     SMH_REQUIRE(B >= 0 && B <= 65535 && H > 0 && Hkv > 0 && H % Hkv == 0 && P >= 0, "%s: B=%d (at most 65535) H=%d Hkv=%d P=%d", who, B, H, Hkv, P);
     // the partials the two launches exchange: one (max, sum, o[128]) per prefix slice and query, as smh_shared_prefix_attn plans them
     int tw = ATT_TW_MAX, qgroups = 1;
@@ -1156,6 +1160,10 @@ extern "C" int smh_shared_prefix_attn_static(const void *q, void *out, int B, in
     const size_t need = splits * (size_t)B * H * (ATT_D + 2) * sizeof(float);
     SMH_REQUIRE(need <= ATT_STATIC_SCRATCH_BYTES, "%s: B=%d H=%d P=%d needs %zu bytes of scratch, the static array holds %zu (use smh_shared_prefix_attn with a workspace)",
                 who, B, H, P, need, ATT_STATIC_SCRATCH_BYTES);
+    SMH_REQUIRE(B == 0 || (q && out), "%s: null q/out", who);
+    SMH_REQUIRE(P == 0 || (prefix_k && prefix_v), "%s: null prefix", who);
+    SMH_REQUIRE(suffix_format == SMH_KV_NONE || (suffix_k && suffix_v && lens && Smax > 0), "%s: suffix arguments incomplete", who);
+    if (B == 0) return 0;
     void *ws = nullptr;
     const int st = static_scratch(&ws);
     if (st) return st;

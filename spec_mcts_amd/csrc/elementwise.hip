@@ -274,6 +274,10 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
     // different fp16 values stay different in fp32), softmax and probabilities in fp32
     const bool wide = row_temps != nullptr;
     if (wide) temperature = row_temps[blockIdx.x];
+    // a row temperature that is not positive (a ramp that reaches 0, a NaN) has no softmax: the row draws its largest logit
+    // every time (the limit of the distribution as the temperature goes to 0), lowest index first among equals
+    const bool greedy_row = wide && !(temperature > 0.f);
+    if (greedy_row) temperature = 1.0f;
     __shared__ int bins[256];
     __shared__ int s_bin, s_above, s_count;
     __shared__ int scan[1024];
@@ -377,6 +381,10 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
         draws = max(counts[blockIdx.x], 0);
         draws = (int)max(min((long)draws, (long)n_draws - first), 0L);       // counts that add up to more than the buffers hold are cut
     }
+    if (greedy_row) {
+        for (int j = tid; j < draws; j += 1024) out[first + j] = o_idx[0];
+        return;
+    }
     if (tid < k) {
         const float before = tid == 0 ? 0.f : cdf[tid - 1];
         for (int j = 0; j < draws; ++j) {
@@ -403,10 +411,14 @@ __global__ __launch_bounds__(256) void tree_fork_kernel(const int64_t *__restric
                                                         int64_t *__restrict__ results, long ld, int t,
                                                         int32_t *__restrict__ pages, long pages_stride, int n_rows,
                                                         int32_t *__restrict__ origin) {
-    __shared__ int64_t u_tok[TREE_MAX_BATCH];      // the draws, then per branch its distinct tokens (at the segment's start)
-    __shared__ int u_cnt[TREE_MAX_BATCH];
+    __shared__ uint64_t keys[TREE_MAX_BATCH];      // (branch, token) of every draw, sorted by the whole workgroup
+    __shared__ int64_t u_tok[TREE_MAX_BATCH];      // per branch its distinct tokens in ascending order (at the segment's start)
+    __shared__ int u_cnt[TREE_MAX_BATCH];          // ... and their multiplicities
     __shared__ int seg_off[TREE_MAX_BATCH + 1];    // first draw of branch i
     __shared__ int seg_uniq[TREE_MAX_BATCH];       // distinct tokens of branch i
+    __shared__ int scan[TREE_MAX_BATCH + 1];       // distinct (branch, token) pairs before position i
+    __shared__ int start[TREE_MAX_BATCH + 1];      // first position of the u-th distinct pair
+    __shared__ int wave_sum[4];
     __shared__ int s_new;                          // branches after the step
     const int tid = threadIdx.x;
     const int c0 = min(max(*curr_b, 0), batch_size);             // (a counter outside the batch is cut, never followed)
@@ -417,24 +429,74 @@ __global__ __launch_bounds__(256) void tree_fork_kernel(const int64_t *__restric
     }
     __syncthreads();
     const int total = min(seg_off[c0], min(n_draws, TREE_MAX_BATCH));   // draws the buffer does not hold do not exist
-    for (int i = tid; i < total; i += 256) u_tok[i] = draws[i];
+    // key of draw i: its branch (the last one whose segment starts at or before i, found by bisection) above its token;
+    // slots past the draws sort to the end
+    for (int i = tid; i < TREE_MAX_BATCH; i += 256) {
+        uint64_t key = ~0ull;
+        if (i < total) {
+            int lo = 0, hi = c0 - 1;
+            while (lo < hi) {
+                const int mid = (lo + hi + 1) >> 1;
+                if (seg_off[mid] <= i) lo = mid; else hi = mid - 1;
+            }
+            key = ((uint64_t)(uint32_t)lo << 32) | (uint64_t)(uint32_t)draws[i];
+        }
+        keys[i] = key;
+    }
     for (int r = tid; r < batch_size; r += 256) origin[r] = -1;
     __syncthreads();
-    // one thread per branch: insertion sort of its draws, then run-length encoding in place
+    // bitonic sort of the 1024 keys: every thread takes two compare-exchanges a pass
+    for (int k = 2; k <= TREE_MAX_BATCH; k <<= 1)
+        for (int j = k >> 1; j > 0; j >>= 1) {
+            for (int x = tid; x < TREE_MAX_BATCH / 2; x += 256) {
+                const int i = ((x & ~(j - 1)) << 1) | (x & (j - 1));        // the lower index of the pair (i, i + j)
+                const uint64_t a = keys[i], b = keys[i + j];
+                const bool up = (i & k) == 0;
+                if ((a > b) == up) { keys[i] = b; keys[i + j] = a; }
+            }
+            __syncthreads();
+        }
+    // run-length encoding by the whole workgroup: a position opens a run when its key differs from its predecessor's
+    // (a new branch always does); an exclusive scan numbers the runs, start[u] is where run u begins
+    {
+        int head[4], local = 0;
+        const int base = tid * 4;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int i = base + e;
+            head[e] = (i < total && (i == 0 || keys[i] != keys[i - 1])) ? 1 : 0;
+            local += head[e];
+        }
+        int incl = local;                                   // inclusive scan over the 256 threads: wave scan, then wave sums
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const int v = __shfl_up(incl, o, 64);
+            if ((tid & 63) >= o) incl += v;
+        }
+        if ((tid & 63) == 63) wave_sum[tid >> 6] = incl;
+        __syncthreads();
+        int before = incl - local;
+        for (int w = 0; w < (tid >> 6); ++w) before += wave_sum[w];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            scan[base + e] = before;
+            if (head[e]) start[before] = base + e;
+            before += head[e];
+        }
+        if (tid == 255) { scan[TREE_MAX_BATCH] = before; start[before] = total; }
+    }
+    __syncthreads();
+    const int n_runs = scan[TREE_MAX_BATCH];
     for (int i = tid; i < c0; i += 256) {
         const int lo = min(seg_off[i], total), hi = min(seg_off[i + 1], total);
-        for (int a = lo + 1; a < hi; ++a) {
-            const int64_t v = u_tok[a];
-            int b = a - 1;
-            while (b >= lo && u_tok[b] > v) { u_tok[b + 1] = u_tok[b]; --b; }
-            u_tok[b + 1] = v;
-        }
-        int n = 0;
-        for (int a = lo; a < hi; ++a) {
-            if (n > 0 && u_tok[lo + n - 1] == u_tok[a]) { ++u_cnt[lo + n - 1]; }
-            else { u_tok[lo + n] = u_tok[a]; u_cnt[lo + n] = 1; ++n; }
-        }
-        seg_uniq[i] = n;
+        seg_uniq[i] = scan[hi] - scan[lo];                  // (scan[total] counts every run: no run opens past the draws)
+    }
+    for (int u = tid; u < n_runs; u += 256) {
+        const int at = start[u];
+        const int br = (int)(keys[at] >> 32);
+        const int slot = min(seg_off[br], total) + (u - scan[min(seg_off[br], total)]);
+        u_tok[slot] = (int64_t)(int32_t)(uint32_t)keys[at];
+        u_cnt[slot] = start[u + 1] - at;
     }
     __syncthreads();
     // rows are handed out in branch order (what is left depends on every earlier branch): one thread walks the branches

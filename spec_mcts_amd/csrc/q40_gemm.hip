@@ -681,8 +681,11 @@ static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
             e = hipFuncSetAttribute((const void *)range_cut[t], hipFuncAttributeMaxDynamicSharedMemorySize, PS * GS_BYTES);
         return e;
     }();
-    if (lds_ok != hipSuccess) return (int)lds_ok;
-    if ((long)p.M * p.lda * 2 >= (1L << 32)) return (int)hipErrorInvalidValue;     // lane offsets of A are 32-bit
+    if (lds_ok != hipSuccess) {
+        set_error("q40 gemm: the kernels' LDS could not be reserved: %s", hipGetErrorString(lds_ok));
+        return (int)lds_ok;
+    }
+    SMH_REQUIRE((long)p.M * p.lda * 2 < (1L << 32), "q40 gemm: M x lda = %d x %ld exceeds the 32-bit lane offsets of A", p.M, p.lda);
     const int tiles = p.mblocks > 1 ? 8 : (p.M + 15) / 16;
     const bool one_each = HAS_DMA_WAVE && p.K % 32 == 0 && (p.chunk > 0 || (long)p.units * p.mblocks * p.ksplit <= SMH_GEMM_PMAX);
     const gemm_kernel_t kern = (p.K % 32 != 0) ? ragged : (p.chunk > 0 ? range_cut : one_each ? with_dma_wave : exact)[tiles < 2 ? 2 : tiles];

@@ -565,7 +565,10 @@ int gemv_launch(const MatmulParams &p, hipStream_t stream) {
             // more than 64 KB of dynamic LDS has to be allowed once (not stream work: fine under graph capture)
             static const hipError_t lds_ok = hipFuncSetAttribute((const void *)q40_gemv_kernel<2>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                                                  80 * 1024);
-            if (lds_ok != hipSuccess) return (int)lds_ok;
+            if (lds_ok != hipSuccess) {
+                set_error("q40 gemv: the kernel's LDS could not be reserved: %s", hipGetErrorString(lds_ok));
+                return (int)lds_ok;
+            }
             hipLaunchKernelGGL((q40_gemv_kernel<2>), grid, dim3(256), lds, stream, p);
         } else if (p.norm_w != nullptr) {
             if (!gemv_norm_in_fits(p)) {
@@ -575,7 +578,10 @@ int gemv_launch(const MatmulParams &p, hipStream_t stream) {
             }
             static const hipError_t lds_ok = hipFuncSetAttribute((const void *)q40_gemv_kernel<3>, hipFuncAttributeMaxDynamicSharedMemorySize,
                                                                  80 * 1024);
-            if (lds_ok != hipSuccess) return (int)lds_ok;
+            if (lds_ok != hipSuccess) {
+                set_error("q40 gemv: the kernel's LDS could not be reserved: %s", hipGetErrorString(lds_ok));
+                return (int)lds_ok;
+            }
             hipLaunchKernelGGL((q40_gemv_kernel<3>), grid, dim3(256), lds, stream, p);
         } else {
             hipLaunchKernelGGL((q40_gemv_kernel<1>), grid, dim3(256), lds, stream, p);

@@ -750,7 +750,8 @@ def paged_prefix_attn(q: torch.Tensor, pages: torch.Tensor, lens: torch.Tensor, 
     """Tree attention: out[b,h] = softmax(q[b,h] . K_b^T / sqrt(D)) . V_b with K_b = prefix[:P] (shared) || the pool rows
     pages[b, :lens[b]] || cur_k[b].  The rows are looked up inside the kernel (nothing is gathered or copied).
     pool: fp16 [rows, Hkv, D] (or [Hkv, rows, D] with head_major) or Q4_0 rows int8 [rows, Hkv, 64] + scales fp16
-    [rows, Hkv, 2]; pages: int16 / int32 / int64 [B, L]; lens int32 on the device."""
+    [rows, Hkv, 2]; pages: int16 / int32 / int64 [B, L] (possibly a column slice of a wider table); lens int32 on the device,
+    cut to L inside the kernel."""
     lib = _lib.load()
     _need_gpu(q, pages, lens, pool_k, pool_v)
     assert q.is_contiguous() and q.dtype == torch.float16 and q.dim() == 3
@@ -790,7 +791,7 @@ def paged_prefix_attn(q: torch.Tensor, pages: torch.Tensor, lens: torch.Tensor, 
     ws = attn_qkv_workspace(q.device, B, H, P) if one else attn_workspace(q.device, B, H, P)
     check(lib.smh_paged_prefix_attn(q.data_ptr(), out.data_ptr(), B, H, Hkv, D, _ptr(prefix_k) if P else None, _ptr(prefix_v) if P else None,
                                     int(P), p_row, p_head, fmt, pool_k.data_ptr(), pool_v.data_ptr(), _ptr(pool_ks), _ptr(pool_vs),
-                                    row_stride, head_stride, int(rows), pages.data_ptr(), pages.element_size(), pages.stride(0),
+                                    row_stride, head_stride, int(rows), pages.data_ptr(), pages.element_size(), pages.stride(0), pages.shape[1],
                                     lens.data_ptr(), int(lens_stride), _ptr(cur_k), _ptr(cur_v), int(one), ws.data_ptr(), ws.numel(), _stream()),
           "smh_paged_prefix_attn")
     return out

@@ -199,3 +199,25 @@ def test_fork_heavy_decode_matches_oracle_and_row_copy(cfg, seed, fused):
     # a new prompt starts from unshared rows again
     models[True].resetSeq()
     assert models[True]._pages(torch.device("cuda:0")) is None
+
+
+def test_lens_are_cut_to_the_columns_of_a_sliced_table():
+    """a column slice of a wider page table: the rows are `stride` apart but hold fewer ids; a length beyond the slice is cut
+    to it inside the kernel (no id of the next columns, or past the last row's end, is read)"""
+    from spec_mcts_amd import kernels as K
+    B, L, H, D, prompt_L = 9, 96, 4, 128, 32
+    P, q, pager, kp, vp = branch_paged(B, L, H, D, prompt_L, seed=77, dtype=torch.int32)
+    off, cols = 40, 30
+    table = pager.cuda()
+    view = table[:, off:off + cols]                                  # stride L, 30 ids a row
+    assert view.stride(0) == L and view.shape[1] == cols
+    over = torch.full((B,), 10 * L, dtype=torch.int32, device="cuda")
+    got = K.paged_prefix_attn(q.cuda(), view, over, kp.cuda(), vp.cuda(), head_major=True).cpu().float()
+    want = sdpa(q, pager[:, off:off + cols], kp, vp)
+    assert torch.allclose(got, want, atol=1e-2, rtol=0)
+    # the last row's slice ends before the table does; with the slice at the very end of the table the cut is what keeps
+    # the reads inside it
+    tail = table[:, L - cols:]
+    got = K.paged_prefix_attn(q.cuda(), tail, over, kp.cuda(), vp.cuda(), head_major=True).cpu().float()
+    want = sdpa(q, pager[:, L - cols:], kp, vp)
+    assert torch.allclose(got, want, atol=1e-2, rtol=0)

@@ -191,3 +191,51 @@ def test_device_search_equals_host_search(seed, temp, use_graph):
         tree.generator = torch.Generator(device="cuda:0").manual_seed(1234 + seed)
         res2, res_len2, stats2 = tree.search(prompt, B)
         assert torch.equal(res2, res) and torch.equal(res_len2, res_len) and torch.equal(stats2, stats)
+
+
+def test_row_temperature_that_is_not_positive_draws_the_largest_logit():
+    """a ramp that reaches 0 (or a NaN) has no softmax: the row returns its argmax for every draw, the other rows are unaffected"""
+    from spec_mcts_amd import kernels as K
+    g = torch.Generator().manual_seed(5)
+    logits = torch.randn((4, 500), generator=g).half().cuda()
+    counts = torch.tensor([3, 2, 4, 1], dtype=torch.int32).cuda()
+    u = torch.rand(10, generator=g).cuda()
+    temps = torch.tensor([0.7, 0.0, float("nan"), -1.0]).cuda()
+    good = torch.tensor([0.7, 0.7, 0.7, 0.7]).cuda()
+    got = K.sample_topk_counts(logits, temps, 8, counts, u).cpu()
+    ref = K.sample_topk_counts(logits, good, 8, counts, u).cpu()
+    top = logits.float().argmax(1).cpu()
+    assert torch.equal(got[:3], ref[:3])
+    assert got[3:5].tolist() == [int(top[1])] * 2 and got[5:9].tolist() == [int(top[2])] * 4 and got[9:].tolist() == [int(top[3])]
+
+
+@pytest.mark.parametrize("seed", range(4))
+def test_tree_fork_first_step_of_a_wide_search(seed):
+    """the first step: one branch owns all batch_size draws (up to 1024), the case the workgroup-wide sort is for; and a
+    later step with many branches, empty segments and dead branches"""
+    from spec_mcts_amd import kernels as K
+    g = torch.Generator().manual_seed(300 + seed)
+    for B, cur, hot in ((1024, 1, 40), (777, 1, 3), (1000, 37, 12)):
+        steps = 6
+        results = torch.randint(1, 1000, (B, steps), generator=g)
+        oc = torch.zeros((2, B), dtype=torch.int32)
+        if cur == 1:
+            oc[1, 0] = B
+        else:
+            cut = torch.sort(torch.randint(0, B + 1, (cur - 1,), generator=g)).values
+            edges = torch.cat((torch.tensor([0]), cut, torch.tensor([B])))
+            oc[1, :cur] = (edges[1:] - edges[:-1]).int()                 # some multiplicities are 0
+        alive = torch.ones(B, dtype=torch.bool)
+        if cur > 1:
+            alive[torch.randint(0, cur, (5,), generator=g)] = False
+        n = int(oc[1, :cur].sum())
+        draws = torch.randint(0, hot, (n,), generator=g)
+        t = 3
+        want_oc, want_res = oc.clone(), results.clone()
+        want_cur, want_origin = O.tree_fork(draws, want_oc, alive, cur, B, want_res, t)
+        d_oc, d_res, d_cur = oc.cuda(), results.cuda(), torch.tensor([cur], dtype=torch.int32).cuda()
+        origin = K.tree_fork(draws.cuda(), d_oc, alive.cuda(), d_cur, d_res, t)
+        assert int(d_cur) == want_cur
+        assert origin.cpu().tolist() == want_origin
+        assert torch.equal(d_oc.cpu(), want_oc)
+        assert torch.equal(d_res.cpu(), want_res)
