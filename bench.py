@@ -240,7 +240,8 @@ def tree_search_bench(torch, model, prompt, batch_sizes=(8, 16, 80, 100), depth=
     of the whole search (prefill included).  `tok_s` counts every token a live branch produced (the reference's "corrected"
     figure, sum of results_len), `tok_s_raw` rows x steps of the returned tensor (its raw figure).  Run with the decode
     steps replayed from per-bucket HIP graphs (the default) and issued launch by launch.  `expand_us` is the time of one
-    expansion (sample_topk_counts + tree_fork + detect_terminal) at the full batch, HIP events over 20 calls."""
+    expansion (sample_topk_counts + tree_step: draws, fork, terminal state machine, bookkeeping) at the full batch, HIP events
+    over 20 calls."""
     from spec_mcts_amd import kernels as K
     from spec_mcts_amd.mcts import mcts, TERMINAL_SEQ, EOS
     dev = torch.device("cuda:0")
@@ -269,7 +270,7 @@ def tree_search_bench(torch, model, prompt, batch_sizes=(8, 16, 80, 100), depth=
         logits = torch.randn((B, model.vocab_size), device=dev).half()
         counts = torch.ones(B, dtype=torch.int32, device=dev)
         oc = torch.stack((torch.zeros_like(counts), counts)).contiguous()
-        alive = torch.ones(B, dtype=torch.bool, device=dev)
+        alive = torch.ones(B, dtype=torch.uint8, device=dev)
         curr_b = torch.full((1,), B, dtype=torch.int32, device=dev)
         results = torch.zeros((B, depth), dtype=torch.int64, device=dev)
         state = torch.zeros(B, dtype=torch.int32, device=dev)
@@ -277,11 +278,13 @@ def tree_search_bench(torch, model, prompt, batch_sizes=(8, 16, 80, 100), depth=
         draws = torch.zeros(B, dtype=torch.int64, device=dev)
         u = torch.rand(B, device=dev)
         pages = model._table(dev).clone()
+        t_dev = torch.full((1,), 5, dtype=torch.int32, device=dev)
+        origin, res_len = torch.empty(B, dtype=torch.int32, device=dev), torch.zeros(B, dtype=torch.int32, device=dev)
+        nxt, summary = torch.zeros(B, dtype=torch.int64, device=dev), torch.zeros(2, dtype=torch.int32, device=dev)
 
         def expand():
             K.sample_topk_counts(logits, temp, 32, oc[1], u, out=draws)
-            K.tree_fork(draws, oc, alive, curr_b, results, 5, pages=pages, n_rows=5)
-            K.detect_terminal(results[:, 5].contiguous(), state, term, EOS)
+            K.tree_step(draws, oc, alive, curr_b, results, t_dev, pages, origin, state, term, res_len, nxt, summary, EOS)
 
         row["expand_us"] = round(time_region(torch, expand, 20) * 1e3, 2)
         out.append(row)

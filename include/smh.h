@@ -211,6 +211,17 @@ int smh_sample_topk_rowtemp(const void *logits, int rows, int vocab, long ld, co
 int smh_tree_fork(const int64_t *draws, int n_draws, int32_t *tok, int32_t *cnt, const uint8_t *alive, int32_t *curr_b, int batch_size,
                   int64_t *results, long ld, int t, int32_t *pages, long pages_stride, int n_rows, int32_t *origin,
                   smh_stream_t stream);
+/* smh_tree_step: one whole step of the search loop after the draws (mcts.py:127-175) in one launch, with the step index read
+ * on the device so that the launch can be replayed from a captured HIP graph: smh_tree_fork with column t = *t_dev and
+ * n_rows = *t_dev (search step t follows t decode steps; a counter outside the row is cut), then smh_detect_terminal on
+ * that column (:162), results_len += alive, alive &= !ended (:163-164, alive is updated in place), next_tokens[r] =
+ * results[r, t] (the next forward's input, :102) and summary[0] = branches after the step, summary[1] = rows of the whole
+ * batch that have ended (:174's two numbers, the only ones the host reads per step).
+ *   state int32 [batch_size] = end_stateMachine; results_len int32 [batch_size]; next_tokens int64 [batch_size]; summary int32 [2]. */
+int smh_tree_step(const int64_t *draws, int n_draws, int32_t *tok, int32_t *cnt, uint8_t *alive, int32_t *curr_b, int batch_size,
+                  int64_t *results, long ld, const int32_t *t_dev, int32_t *pages, long pages_stride, int32_t *origin,
+                  int32_t *state, const int64_t *terminal_seq, int seq_len, int64_t eos, int32_t *results_len,
+                  int64_t *next_tokens, int32_t *summary, smh_stream_t stream);
 /* smh_detect_terminal: detectTerminal (mcts.py:14-28) for `rows` branches in place: state[b] counts the tokens of
  * terminal_seq (int64 [seq_len], "[/PYTHON]" in the reference, mcts.py:12) produced in a row, any other token sends it
  * back to 0; end[b] = 1 when the sequence is complete or token[b] == eos (2 in the reference), and the state of an ended

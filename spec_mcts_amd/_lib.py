@@ -39,6 +39,7 @@ SIGNATURES = {
     "smh_q40_matmul_partial_tiled_norm": (c_int, [_P, c_long, _P, _P, c_float, c_int, c_int, c_int, _P, _P, _P, c_size_t, _P]),
     "smh_sample_topk_counts": (c_int, [_P, c_int, c_int, c_long, c_float, c_int, _P, _P, _P, c_int, _P]),
     "smh_tree_fork": (c_int, [_P, c_int, _P, _P, _P, _P, c_int, _P, c_long, c_int, _P, c_long, c_int, _P, _P]),
+    "smh_tree_step": (c_int, [_P, c_int, _P, _P, _P, _P, c_int, _P, c_long, _P, _P, c_long, _P, _P, _P, c_int, ctypes.c_int64, _P, _P, _P, _P]),
     "smh_detect_terminal": (c_int, [_P, _P, _P, _P, c_int, ctypes.c_int64, c_int, _P]),
     "smh_partial_reduce": (c_int, [_P, c_int, c_int, c_int, c_int, c_int, _P, c_long, c_int, _P, c_long, _P]),
     "smh_partial_rmsnorm": (c_int, [_P, c_int, c_int, c_int, _P, _P, c_float, _P, _P, _P]),

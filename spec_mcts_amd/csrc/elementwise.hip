@@ -406,11 +406,29 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
 //           zeroed (:160).
 //   tok / cnt = output_counts[0] / [1] of the reference; origin[r] = the branch row r was forked from in this step, else -1.
 constexpr int TREE_MAX_BATCH = 1024;
+// What follows the fork in a step of the search loop (mcts.py:160-175), for the variant that does the whole step in one launch:
+// the terminal state machine on the step's column, the lengths and the mask of live rows, the tokens the next forward
+// reads, and the two numbers the host needs (branches, ended rows).
+struct TreeFinish {
+    int32_t *state;              // end_stateMachine [batch_size]
+    const int64_t *seq;          // the terminal sequence
+    int seq_len;
+    int64_t eos;
+    int32_t *results_len;        // [batch_size]
+    int64_t *next_tokens;        // [batch_size]: column t of results, the next decode step's input
+    int32_t *summary;            // [2]: branches after the step, rows that have ended
+};
+// t_dev != nullptr: the step's column AND the suffix rows written so far are *t_dev (a search step t follows t decode steps),
+// read on the device so that one captured launch serves every step.
 __global__ __launch_bounds__(256) void tree_fork_kernel(const int64_t *__restrict__ draws, int n_draws, int32_t *__restrict__ tok, int32_t *__restrict__ cnt,
-                                                        const uint8_t *__restrict__ alive, int32_t *__restrict__ curr_b, int batch_size,
+                                                        uint8_t *__restrict__ alive, int32_t *__restrict__ curr_b, int batch_size,
                                                         int64_t *__restrict__ results, long ld, int t,
                                                         int32_t *__restrict__ pages, long pages_stride, int n_rows,
-                                                        int32_t *__restrict__ origin) {
+                                                        int32_t *__restrict__ origin, const int32_t *__restrict__ t_dev, TreeFinish fin) {
+    if (t_dev != nullptr) {
+        t = min(max(*t_dev, 0), (int)ld - 1);                    // (a counter outside the row is cut, never followed)
+        n_rows = (int)min((long)t, pages_stride);
+    }
     __shared__ uint64_t keys[TREE_MAX_BATCH];      // (branch, token) of every draw, sorted by the whole workgroup
     __shared__ int64_t u_tok[TREE_MAX_BATCH];      // per branch its distinct tokens in ascending order (at the segment's start)
     __shared__ int u_cnt[TREE_MAX_BATCH];          // ... and their multiplicities
@@ -445,10 +463,13 @@ __global__ __launch_bounds__(256) void tree_fork_kernel(const int64_t *__restric
     }
     for (int r = tid; r < batch_size; r += 256) origin[r] = -1;
     __syncthreads();
-    // bitonic sort of the 1024 keys: every thread takes two compare-exchanges a pass
-    for (int k = 2; k <= TREE_MAX_BATCH; k <<= 1)
+    // bitonic sort of the keys by the whole workgroup, over the smallest power of two that holds the draws (the slots
+    // past them hold the largest key and stay behind)
+    int n_sort = 2;
+    while (n_sort < total) n_sort <<= 1;
+    for (int k = 2; k <= n_sort; k <<= 1)
         for (int j = k >> 1; j > 0; j >>= 1) {
-            for (int x = tid; x < TREE_MAX_BATCH / 2; x += 256) {
+            for (int x = tid; x < n_sort / 2; x += 256) {
                 const int i = ((x & ~(j - 1)) << 1) | (x & (j - 1));        // the lower index of the pair (i, i + j)
                 const uint64_t a = keys[i], b = keys[i + j];
                 const bool up = (i & k) == 0;
@@ -528,9 +549,36 @@ __global__ __launch_bounds__(256) void tree_fork_kernel(const int64_t *__restric
             for (int j = tid; j < n_rows; j += 256) pages[(long)r * pages_stride + j] = pages[(long)o * pages_stride + j];
     }
     __syncthreads();
+    int ended = 0;
     for (int r = tid; r < batch_size; r += 256) {
-        if (!alive[r]) results[(long)r * ld + t] = 0;
-        else if (r < c1 && (r >= c0 || seg_uniq[r] > 0)) results[(long)r * ld + t] = tok[r];
+        int64_t token = results[(long)r * ld + t];
+        if (!alive[r]) token = 0;
+        else if (r < c1 && (r >= c0 || seg_uniq[r] > 0)) token = tok[r];
+        results[(long)r * ld + t] = token;
+        if (fin.state != nullptr) {
+            // detectTerminal on the step's column (mcts.py:14-28, :162), lengths and mask (:163-164)
+            const int32_t st = fin.state[r];
+            const int32_t match = (st >= 0 && st < fin.seq_len && fin.seq[st] == token) ? 1 : 0;
+            const int32_t nxt = (st + match) * match;
+            const bool done = nxt == fin.seq_len || token == fin.eos;
+            fin.state[r] = done ? 0 : nxt;
+            const bool was = alive[r] != 0;
+            fin.results_len[r] += was ? 1 : 0;
+            const bool now = was && !done;
+            alive[r] = now ? 1 : 0;
+            ended += now ? 0 : 1;
+            fin.next_tokens[r] = token;
+        }
+    }
+    if (fin.state != nullptr) {
+        __syncthreads();                            // (scan[] is free again)
+        scan[tid] = ended;
+        __syncthreads();
+        for (int o = 128; o > 0; o >>= 1) {
+            if (tid < o) scan[tid] += scan[tid + o];
+            __syncthreads();
+        }
+        if (tid == 0) { fin.summary[0] = c1; fin.summary[1] = scan[0]; }
     }
 }
 
@@ -582,8 +630,23 @@ extern "C" int smh_tree_fork(const int64_t *draws, int n_draws, int32_t *tok, in
     SMH_REQUIRE(draws && n_draws >= 0 && tok && cnt && alive && curr_b && results && origin, "smh_tree_fork: null pointer or n_draws=%d", n_draws);
     SMH_REQUIRE(ld >= 1 && t >= 0 && t < ld, "smh_tree_fork: column %d outside the %ld of a row", t, ld);
     SMH_REQUIRE(pages == nullptr || (pages_stride >= n_rows && n_rows >= 0), "smh_tree_fork: n_rows=%d pages_stride=%ld", n_rows, pages_stride);
-    hipLaunchKernelGGL(tree_fork_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, draws, n_draws, tok, cnt, alive, curr_b, batch_size, results, ld, t,
-                       pages, pages_stride, n_rows, origin);
+    hipLaunchKernelGGL(tree_fork_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, draws, n_draws, tok, cnt, const_cast<uint8_t *>(alive), curr_b, batch_size,
+                       results, ld, t, pages, pages_stride, n_rows, origin, (const int32_t *)nullptr, TreeFinish{});
+    return launch_status();
+}
+
+extern "C" int smh_tree_step(const int64_t *draws, int n_draws, int32_t *tok, int32_t *cnt, uint8_t *alive, int32_t *curr_b, int batch_size,
+                             int64_t *results, long ld, const int32_t *t_dev, int32_t *pages, long pages_stride, int32_t *origin,
+                             int32_t *state, const int64_t *terminal_seq, int seq_len, int64_t eos, int32_t *results_len,
+                             int64_t *next_tokens, int32_t *summary, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(batch_size >= 1 && batch_size <= TREE_MAX_BATCH, "smh_tree_step: batch_size=%d outside [1,%d]", batch_size, TREE_MAX_BATCH);
+    SMH_REQUIRE(draws && n_draws >= 0 && tok && cnt && alive && curr_b && results && origin && t_dev, "smh_tree_step: null pointer or n_draws=%d", n_draws);
+    SMH_REQUIRE(ld >= 1 && (pages == nullptr || pages_stride >= 1), "smh_tree_step: ld=%ld pages_stride=%ld", ld, pages_stride);
+    SMH_REQUIRE(state && terminal_seq && seq_len >= 1 && results_len && next_tokens && summary, "smh_tree_step: null pointer or seq_len=%d", seq_len);
+    TreeFinish fin{state, terminal_seq, seq_len, eos, results_len, next_tokens, summary};
+    hipLaunchKernelGGL(tree_fork_kernel, dim3(1), dim3(256), 0, (hipStream_t)stream, draws, n_draws, tok, cnt, alive, curr_b, batch_size, results, ld, 0,
+                       pages, pages_stride, 0, origin, t_dev, fin);
     return launch_status();
 }
 

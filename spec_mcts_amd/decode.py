@@ -136,7 +136,9 @@ class BucketedForward:
     from the fork's step on.  Position and suffix index live on the device and are advanced by the graph itself, so the
     same graph serves every step; graphs are captured when a bucket is first needed and kept while the prompt length and
     the model's switches stay the same.  The page table is always in use (identity until the first fork), so that the fork
-    does not change what the recorded launches read.
+    does not change what the recorded launches read.  `post(logits)` - set by the caller, None for none - is issued right
+    behind the forward and recorded with it (the tree sampler's draws and bookkeeping: they take the step index from
+    `state[1]` and leave the next step's tokens in `tokens`), so a whole search step is one replay.
     """
 
     def __init__(self, model: Transformer, max_batch: int, use_graph: bool = True):
@@ -159,6 +161,8 @@ class BucketedForward:
         self.prompt_len = 0
         self.t = 0
         self.replays = 0
+        self.post = None
+        self.post_key = None
 
     def _config(self):
         m = self.model
@@ -180,21 +184,25 @@ class BucketedForward:
     def _run(self, bucket: int):
         logits = self.model._forward_impl(self.tokens[:bucket], 1, (self.state[0:1], self.state[1:2]))
         self.state.add_(self.one)
+        if self.post is not None:
+            self.post(logits)
         return logits
 
     def bucket_of(self, curr: int) -> int:
         return next(b for b in self.buckets if b >= curr)
 
     @torch.inference_mode()
-    def step(self, tokens: torch.Tensor) -> torch.Tensor:
-        """tokens int64 [curr, 1] (the previous step's tokens of the live branches) -> logits fp16 [curr, 1, vocab]"""
-        curr = tokens.shape[0]
+    def step(self, tokens: Optional[torch.Tensor], curr: int = 0) -> torch.Tensor:
+        """tokens int64 [curr, 1] (the previous step's tokens of the live branches; None: `curr` rows of the token buffer
+        are already in place) -> logits fp16 [curr, 1, vocab]"""
+        curr = tokens.shape[0] if tokens is not None else curr
         p = self.model.params
         assert 1 <= curr <= self.max_batch
         assert self.t < p.max_seq_len, "suffix cache exhausted"
         assert self.prompt_len + self.t < self.model.freqs_cis.shape[0], "position beyond the rotation table"
         bucket = self.bucket_of(curr)
-        self.tokens[:curr].copy_(tokens)
+        if tokens is not None:
+            self.tokens[:curr].copy_(tokens)
         if not self.use_graph:
             logits = self._run(bucket)
         else:
@@ -209,6 +217,7 @@ class BucketedForward:
 
     def _capture(self, bucket: int):
         saved = self.state.clone()
+        post, self.post = self.post, None         # the warm-up runs the forward only: `post` changes the caller's state
         s = torch.cuda.Stream()
         s.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(s):
@@ -218,6 +227,7 @@ class BucketedForward:
         torch.cuda.current_stream().wait_stream(s)
         torch.cuda.synchronize()
         self.state.copy_(saved)
+        self.post = post
         # the warm-up grew the shared workspaces to what this bucket needs; the graph records their addresses
         self._pinned.extend(w for w in K._workspaces.values() if not any(w is q for q in self._pinned))
         g = torch.cuda.CUDAGraph()

@@ -528,6 +528,33 @@ def tree_fork(draws: torch.Tensor, output_counts: torch.Tensor, alive: torch.Ten
     return origin
 
 
+def tree_step(draws: torch.Tensor, output_counts: torch.Tensor, alive: torch.Tensor, curr_b: torch.Tensor, results: torch.Tensor,
+              t_dev: torch.Tensor, pages: Optional[torch.Tensor], origin: torch.Tensor, state: torch.Tensor, terminal_seq: torch.Tensor,
+              results_len: torch.Tensor, next_tokens: torch.Tensor, summary: torch.Tensor, eos: int = 2) -> None:
+    """One whole step of the tree sampler after the draws (mcts.py:127-175) in one launch, everything in place and the step
+    index read from the device (t_dev int32 [1]: the column of `results` and the suffix rows written so far), so that the
+    launch can sit in a captured graph: tree_fork, then detect_terminal on the step's column, results_len += alive,
+    alive &= ~ended, next_tokens = results[:, t], summary = (branches, ended rows).  alive is uint8 [batch]."""
+    lib = _lib.load()
+    _need_gpu(draws, output_counts, alive, curr_b, results, t_dev, origin, state, terminal_seq, results_len, next_tokens, summary)
+    B, ld = results.shape
+    assert draws.dtype == torch.int64 and draws.is_contiguous()
+    assert output_counts.dtype == torch.int32 and output_counts.shape == (2, B) and output_counts.is_contiguous()
+    assert alive.dtype == torch.uint8 and alive.numel() == B and alive.is_contiguous()
+    assert curr_b.dtype == torch.int32 and t_dev.dtype == torch.int32 and summary.dtype == torch.int32 and summary.numel() >= 2
+    assert results.dtype == torch.int64 and results.is_contiguous()
+    assert origin.dtype == torch.int32 and origin.numel() >= B and state.dtype == torch.int32 and state.numel() == B
+    assert results_len.dtype == torch.int32 and results_len.numel() == B and next_tokens.dtype == torch.int64 and next_tokens.numel() >= B
+    assert terminal_seq.dtype == torch.int64 and terminal_seq.is_contiguous()
+    if pages is not None:
+        _need_gpu(pages)
+        assert pages.dtype == torch.int32 and pages.dim() == 2 and pages.shape[0] >= B and pages.stride(1) == 1
+    check(lib.smh_tree_step(draws.data_ptr(), draws.numel(), output_counts[0].data_ptr(), output_counts[1].data_ptr(), alive.data_ptr(),
+                            curr_b.data_ptr(), B, results.data_ptr(), ld, t_dev.data_ptr(), _ptr(pages), pages.stride(0) if pages is not None else 0,
+                            origin.data_ptr(), state.data_ptr(), terminal_seq.data_ptr(), terminal_seq.numel(), int(eos), results_len.data_ptr(),
+                            next_tokens.data_ptr(), summary.data_ptr(), _stream()), "smh_tree_step")
+
+
 def detect_terminal(token: torch.Tensor, state: torch.Tensor, terminal_seq: torch.Tensor, eos: int = 2):
     """detectTerminal of the reference's tree sampler (mcts.py:14-28) on the device in one launch.
     token int64 [B], state int32 [B], terminal_seq int64 [L] -> (end bool [B], state int32 [B]); `state` is not modified."""
