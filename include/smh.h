@@ -184,6 +184,13 @@ int smh_argmax(const void *logits, int rows, int vocab, long ld, int64_t *out, s
  * numbers take the place of torch.multinomial's generator.  1 <= top_k <= 1024, temperature > 0. */
 int smh_sample_topk(const void *logits, int rows, int vocab, long ld, float temperature, int top_k,
                     const float *uniform, int64_t *out, smh_stream_t stream);
+/* smh_sample_topk_filter: the sampling step of the flat-cache model's generate (hf_model_q40.py:521-533), whose logits are
+ * float32 copies of the fp16 values (:476): x = float(logit) / temperature, everything below the top_k-th largest x masked
+ * to -inf (so EVERY value equal to the k-th stays a candidate, not only top_k of them; at most 1024 candidates, lowest
+ * indices first, are kept), p = float32 softmax, one candidate per row drawn by inverse CDF with uniform[row] as in
+ * smh_sample_topk.  logits: the fp16 values [rows, vocab].  1 <= top_k <= 1024, temperature > 0. */
+int smh_sample_topk_filter(const void *logits, int rows, int vocab, long ld, float temperature, int top_k,
+                           const float *uniform, int64_t *out, smh_stream_t stream);
 /* The expansion step of the tree sampler (mcts.py:115-152) without its per-branch Python loop and host round trips.
  * smh_sample_topk_counts: smh_sample_topk where row r makes counts[r] draws with replacement (torch.multinomial with
  *   num_samples = output_counts[1, r], :128): the draws of row r use uniform[o .. o + counts[r]) and fill out[o ..) with

@@ -247,6 +247,31 @@ def sample_topk(logits: torch.Tensor, temperature: float, top_k: int, u: torch.T
     return order.gather(1, j.unsqueeze(1))[:, 0]
 
 
+def topk_filter_probs(logits: torch.Tensor, temperature: float, top_k: int) -> torch.Tensor:
+    """The probabilities of the flat-cache model's sampling step (hf_model_q40.py:521-529): float32 logits (that model
+    returns `output.float()`, :476) divided by the temperature, every value below the top_k-th largest set to -inf - values
+    equal to it all stay, so more than top_k may survive - and a float32 softmax over the vocabulary.  [rows, vocab]."""
+    x = logits.float() / temperature
+    v, _ = torch.topk(x, min(top_k, x.size(-1)))
+    x = x.masked_fill(x < v[:, [-1]], -float("Inf"))
+    return F.softmax(x, dim=-1)
+
+
+def sample_topk_filter(logits: torch.Tensor, temperature: float, top_k: int, u: torch.Tensor) -> torch.Tensor:
+    """One draw per row from topk_filter_probs by inverse CDF over the surviving tokens in descending order of value (equal
+    values by index), with the caller's uniform numbers - the stand-in for `torch.multinomial` (:530) that sample_topk
+    uses."""
+    p = topk_filter_probs(logits, temperature, top_k)
+    order = torch.argsort(logits.float(), dim=-1, descending=True, stable=True)
+    ps = torch.gather(p, 1, order)
+    cdf = ps.cumsum(-1)
+    n_alive = (ps > 0).sum(-1)
+    total = cdf.gather(1, (n_alive - 1).unsqueeze(1))
+    hit = cdf > u.float().unsqueeze(1) * total
+    j = torch.where(hit.any(-1), hit.float().argmax(-1), n_alive - 1)
+    return order.gather(1, j.unsqueeze(1))[:, 0]
+
+
 def sample_topk_counts(logits: torch.Tensor, temperature, top_k: int, counts, u: torch.Tensor) -> torch.Tensor:
     """counts[r] draws per row (mcts.py:128: torch.multinomial(probs[r], num_samples=output_counts[1, r], replacement=True)
     followed by the gather of :129), each an inverse-CDF draw as in sample_topk; row r uses u[sum(counts[:r]) ...]."""

@@ -53,6 +53,7 @@ SIGNATURES = {
     "smh_gq40_quantize": (c_int, [_P, _P, _P, c_long, _P]),
     "smh_gq40_dequant": (c_int, [_P, _P, _P, c_long, _P]),
     "smh_sample_topk": (c_int, [_P, c_int, c_int, c_long, c_float, c_int, _P, _P, _P]),
+    "smh_sample_topk_filter": (c_int, [_P, c_int, c_int, c_long, c_float, c_int, _P, _P, _P]),
     "smh_rope_append_kv": (c_int, [_P, _P, _P, c_int, c_int, c_int, c_int, _P, _P, _P, _P, _P, _P, _P, c_int, _P, _P]),
     "smh_rope": (c_int, [_P, _P, c_int, c_int, c_int, c_int, _P, _P, c_int, _P]),
     "smh_set_step": (c_int, [_P, c_int, c_int, _P]),

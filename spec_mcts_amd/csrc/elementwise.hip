@@ -268,15 +268,18 @@ __device__ __forceinline__ void sample_pick_bin(int *bins, int want, int *out_bi
 // its candidates, with the uniform numbers (and into the slots of out) that start at counts[0] + ... + counts[r-1].
 __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restrict__ logits, int vocab, long ld, float temperature,
                                                            int top_k, const float *__restrict__ uniform, int64_t *__restrict__ out,
-                                                           const int32_t *__restrict__ counts, const float *__restrict__ row_temps, int n_draws) {
+                                                           const int32_t *__restrict__ counts, const float *__restrict__ row_temps, int n_draws,
+                                                           int keep_ties) {
     // row_temps: a temperature per row, applied in fp32 (a tensor divisor promotes the fp16 logits to fp32 in torch, a
     // Python scalar does not): candidates by the raw logits (division by a positive number keeps their order, and two
     // different fp16 values stay different in fp32), softmax and probabilities in fp32
-    const bool wide = row_temps != nullptr;
-    if (wide) temperature = row_temps[blockIdx.x];
+    // keep_ties: the filter form of top-k (everything below the k-th largest value is masked, so EVERY value equal to it
+    // stays a candidate - up to SAMPLE_MAX_K candidates in all), on fp32 logits / temperature
+    const bool wide = row_temps != nullptr || keep_ties;
+    if (row_temps != nullptr) temperature = row_temps[blockIdx.x];
     // a row temperature that is not positive (a ramp that reaches 0, a NaN) has no softmax: the row draws its largest logit
     // every time (the limit of the distribution as the temperature goes to 0), lowest index first among equals
-    const bool greedy_row = wide && !(temperature > 0.f);
+    const bool greedy_row = row_temps != nullptr && !(temperature > 0.f);
     if (greedy_row) temperature = 1.0f;
     __shared__ int bins[256];
     __shared__ int s_bin, s_above, s_count;
@@ -288,7 +291,7 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
     __shared__ float cdf[SAMPLE_MAX_K];
     const int tid = threadIdx.x;
     const half_t *row = logits + (long)blockIdx.x * ld;
-    const int k = min(top_k, vocab);
+    int k = min(top_k, vocab);
     auto key_at = [&](int i) { return sample_key(wide ? row[i] : (half_t)((float)row[i] / temperature)); };
     auto value_of = [&](uint32_t key) { return wide ? (float)sample_unkey(key) / temperature : (float)sample_unkey(key); };
 
@@ -310,7 +313,11 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
     __syncthreads();
     sample_pick_bin(bins, k - above1, &s_bin, &s_above);
     const uint32_t kth = ((uint32_t)b1 << 8) | (uint32_t)s_bin;      // key of the k-th largest value
-    const int ties_wanted = k - (above1 + s_above);                    // how many of the values equal to it are in
+    int ties_wanted = k - (above1 + s_above);                          // how many of the values equal to it are in
+    if (keep_ties) {                                                   // all of them, while the candidate arrays hold them
+        ties_wanted = min(bins[s_bin] - s_above, SAMPLE_MAX_K - (above1 + s_above));
+        k = above1 + s_above + ties_wanted;
+    }
     __syncthreads();
 
     // ---- gather: everything above the k-th key, and of the ties the lowest indices (contiguous chunk per thread,
@@ -593,7 +600,20 @@ extern "C" int smh_sample_topk(const void *logits, int rows, int vocab, long ld,
     if (rows == 0) return 0;
     SMH_REQUIRE(logits && uniform && out, "smh_sample_topk: null pointer");
     hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, temperature,
-                       top_k, uniform, out, (const int32_t *)nullptr, (const float *)nullptr, rows);
+                       top_k, uniform, out, (const int32_t *)nullptr, (const float *)nullptr, rows, 0);
+    return launch_status();
+}
+
+extern "C" int smh_sample_topk_filter(const void *logits, int rows, int vocab, long ld, float temperature, int top_k,
+                                      const float *uniform, int64_t *out, smh_stream_t stream) {
+    using namespace smh;
+    SMH_REQUIRE(rows >= 0 && vocab > 0 && ld >= vocab, "smh_sample_topk_filter: rows=%d vocab=%d ld=%ld", rows, vocab, ld);
+    SMH_REQUIRE(top_k >= 1 && top_k <= SAMPLE_MAX_K, "smh_sample_topk_filter: top_k=%d outside [1,%d]", top_k, SAMPLE_MAX_K);
+    SMH_REQUIRE(temperature > 0.f, "smh_sample_topk_filter: temperature=%g must be positive (greedy decoding is smh_argmax)", (double)temperature);
+    if (rows == 0) return 0;
+    SMH_REQUIRE(logits && uniform && out, "smh_sample_topk_filter: null pointer");
+    hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, temperature,
+                       top_k, uniform, out, (const int32_t *)nullptr, (const float *)nullptr, rows, 1);
     return launch_status();
 }
 
@@ -606,7 +626,7 @@ extern "C" int smh_sample_topk_counts(const void *logits, int rows, int vocab, l
     if (rows == 0) return 0;
     SMH_REQUIRE(logits && uniform && counts && out && n_draws >= 0, "smh_sample_topk_counts: null pointer or n_draws=%d", n_draws);
     hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, temperature,
-                       top_k, uniform, out, counts, (const float *)nullptr, n_draws);
+                       top_k, uniform, out, counts, (const float *)nullptr, n_draws, 0);
     return launch_status();
 }
 
@@ -618,7 +638,7 @@ extern "C" int smh_sample_topk_rowtemp(const void *logits, int rows, int vocab, 
     if (rows == 0) return 0;
     SMH_REQUIRE(logits && row_temps && uniform && counts && out && n_draws >= 0, "smh_sample_topk_rowtemp: null pointer or n_draws=%d", n_draws);
     hipLaunchKernelGGL(sample_topk_kernel, dim3(rows), dim3(1024), 0, (hipStream_t)stream, (const half_t *)logits, vocab, ld, 1.0f,
-                       top_k, uniform, out, counts, row_temps, n_draws);
+                       top_k, uniform, out, counts, row_temps, n_draws, 0);
     return launch_status();
 }
 

@@ -30,33 +30,19 @@
 
 namespace smh {
 
-// most K-slices of a launch = SMH_GEMM_KSCAP / rows (every slice leaves an fp32 slab of rows x columns)
-#ifndef SMH_GEMM_KSCAP
-#define SMH_GEMM_KSCAP 1600
-#endif
-#ifndef SMH_GEMM_WAVES
-#define SMH_GEMM_WAVES 8
-#endif
+// most K-slices of a launch = GEMM_KSCAP / rows (every slice leaves an fp32 slab of rows x columns)
+constexpr int GEMM_KSCAP = 1600;
 constexpr int GEMM_BM = 128;
-constexpr int GEMM_WAVES = 4;
+constexpr int GEMM_WAVES = 4;                  // checkpoint layout and ragged K; tiled weights run GEMM_TILED_WAVES
+constexpr int GEMM_TILED_WAVES = 8;
 constexpr int GEMM_THREADS = GEMM_WAVES * 64;
 // slots of the DMA ring (with a barrier per step, four slots measured 2 % faster per launch at M=100 than six; with a
 // barrier per two steps, six slots are 3 % faster than that)
-#ifndef SMH_GEMM_STAGES
-#define SMH_GEMM_STAGES 6
-#endif
-constexpr int GEMM_STAGES = SMH_GEMM_STAGES;
-// slots of the ring in the variant with a DMA wave (eight measured like six), the most workgroups of a launch that
-// takes it (one per compute unit), and whether the plan may cut ranges (gemm_fill_plan)
-#ifndef SMH_GEMM_PSLOTS
-#define SMH_GEMM_PSLOTS 6
-#endif
-#ifndef SMH_GEMM_PMAX
-#define SMH_GEMM_PMAX 256
-#endif
-#ifndef SMH_GEMM_RANGE_CUT
-#define SMH_GEMM_RANGE_CUT 1
-#endif
+constexpr int GEMM_STAGES = 6;
+// slots of the ring in the variant with a DMA wave (eight measured like six) and the most workgroups of a launch that
+// takes it (one per compute unit)
+constexpr int GEMM_DMA_WAVE_SLOTS = 6;
+constexpr int GEMM_DMA_WAVE_MAX_WGS = 256;
 constexpr int GS_WBLOCK = 8 * 128 + 64;        // the 8 rows one wave fetches, padded by 16 banks: the four row groups a
                                                // ds_read_b32 touches (lanes 16g..16g+15 read row 8g+r) then sit in different banks
 constexpr int GS_W = 4 * GS_WBLOCK;            // nibbles
@@ -615,7 +601,7 @@ void gemm_fill_plan(MatmulParams &p) {
     constexpr int capacity = 512;
     int ks = (int)(capacity / 2 / tiles);
     if (ks < 1 || tiles * ks < 200) ks = (int)(capacity / tiles);
-    int cap = SMH_GEMM_KSCAP / (p.M > 0 ? p.M : 1);
+    int cap = GEMM_KSCAP / (p.M > 0 ? p.M : 1);
     if (cap > SMH_MAX_KSPLIT) cap = SMH_MAX_KSPLIT;
     if (ks > cap) ks = cap;
     if (ks > steps / GEMM_STAGES) ks = steps / GEMM_STAGES;
@@ -626,7 +612,7 @@ void gemm_fill_plan(MatmulParams &p) {
     // deals runs of steps instead, one workgroup per compute unit, crossing unit boundaries.
     p.chunk = 0;
     const long wgs = tiles * p.ksplit;
-    if (SMH_GEMM_RANGE_CUT && p.mblocks == 1 && p.K % 32 == 0 && wgs > 256 && wgs <= 512) {
+    if (p.mblocks == 1 && p.K % 32 == 0 && wgs > 256 && wgs <= 512) {
         const long total = (long)p.units * steps;
         const int chunk = (int)((total + 255) / 256);
         if (chunk <= steps && chunk >= 2 * GEMM_STAGES) {
@@ -650,14 +636,14 @@ template <bool TILED>
 static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
     // one instantiation per number of 16-row tiles (M <= 128) keeps the step free of branches; K % 32 != 0
     // takes the masked variant with all 8 tiles
-    constexpr int W = TILED ? SMH_GEMM_WAVES : 4;
+    constexpr int W = TILED ? GEMM_TILED_WAVES : GEMM_WAVES;
     static const gemm_kernel_t exact[9] = {nullptr, q40_gemm_kernel<2, false, TILED, W>, q40_gemm_kernel<2, false, TILED, W>,
                                            q40_gemm_kernel<3, false, TILED, W>, q40_gemm_kernel<4, false, TILED, W>,
                                            q40_gemm_kernel<5, false, TILED, W>, q40_gemm_kernel<6, false, TILED, W>,
                                            q40_gemm_kernel<7, false, TILED, W>, q40_gemm_kernel<8, false, TILED, W>};
     // one workgroup per compute unit: the variant with the DMA wave
     constexpr bool HAS_DMA_WAVE = W == 8;
-    constexpr int PS = HAS_DMA_WAVE ? SMH_GEMM_PSLOTS : GEMM_STAGES;
+    constexpr int PS = HAS_DMA_WAVE ? GEMM_DMA_WAVE_SLOTS : GEMM_STAGES;
     static const gemm_kernel_t with_dma_wave[9] = {
         nullptr, q40_gemm_kernel<2, false, TILED, W, PS, HAS_DMA_WAVE>, q40_gemm_kernel<2, false, TILED, W, PS, HAS_DMA_WAVE>,
         q40_gemm_kernel<3, false, TILED, W, PS, HAS_DMA_WAVE>, q40_gemm_kernel<4, false, TILED, W, PS, HAS_DMA_WAVE>,
@@ -687,7 +673,7 @@ static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
     }
     SMH_REQUIRE((long)p.M * p.lda * 2 < (1L << 32), "q40 gemm: M x lda = %d x %ld exceeds the 32-bit lane offsets of A", p.M, p.lda);
     const int tiles = p.mblocks > 1 ? 8 : (p.M + 15) / 16;
-    const bool one_each = HAS_DMA_WAVE && p.K % 32 == 0 && (p.chunk > 0 || (long)p.units * p.mblocks * p.ksplit <= SMH_GEMM_PMAX);
+    const bool one_each = HAS_DMA_WAVE && p.K % 32 == 0 && (p.chunk > 0 || (long)p.units * p.mblocks * p.ksplit <= GEMM_DMA_WAVE_MAX_WGS);
     const gemm_kernel_t kern = (p.K % 32 != 0) ? ragged : (p.chunk > 0 ? range_cut : one_each ? with_dma_wave : exact)[tiles < 2 ? 2 : tiles];
     const long total_steps = (long)p.units * ((p.K + 31) / 32);
     dim3 grid((unsigned)(p.chunk > 0 ? (total_steps + p.chunk - 1) / p.chunk : (long)p.units_pad * p.mblocks * p.ksplit));

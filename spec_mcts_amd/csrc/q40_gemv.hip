@@ -42,10 +42,7 @@ constexpr int GEMV_WAVES = 4;              // waves per workgroup, each with its
 // Two stages: with the tiled layout (one contiguous 4352-byte run per stage) a third stage in flight per wave
 // measured 1.5 % slower per launch and 2 % slower per decode step than two (eight waves a CU keep 16 stages,
 // 70 KB, in flight either way the memory system's ~24 GB/s per CU share needs); four stages leave one workgroup a CU.
-#ifndef SMH_RING_STAGES
-#define SMH_RING_STAGES 2
-#endif
-constexpr int RING_STAGES = SMH_RING_STAGES;
+constexpr int RING_STAGES = 2;
 constexpr int STAGE_W_BYTES = 32 * 128;
 constexpr int STAGE_S_BYTES = 32 * 8;
 constexpr int STAGE_X_BYTES = 16 * 64;

@@ -103,17 +103,9 @@ __device__ __forceinline__ float dpp_move(float v) {
 
 // sum over the 16 lanes that share lane/16 (one DPP row)
 __device__ __forceinline__ float row16_sum(float v) {
-#ifdef SMH_ROW16_DPP
-    v += dpp_move<DPP_ROW_ROR8>(v);
-    v += dpp_move<DPP_ROW_ROR4>(v);
-    v += dpp_move<DPP_QUAD_XOR2>(v);
-    v += dpp_move<DPP_QUAD_XOR1>(v);
-    return v;
-#else
 #pragma unroll
     for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
     return v;
-#endif
 }
 
 // ---- RMSNorm arithmetic shared by every kernel that normalises ---------------------------------------

@@ -96,6 +96,10 @@ class Transformer(shared.Transformer):
             logits = logits[:, -1, :]
             if temperature == 0.0:
                 idx_next = K.argmax(logits.half().contiguous())[:, None]
+            elif self.fused_sampler and top_k is not None and top_k <= 1024:
+                # division, top-k filter, softmax and the draw in one launch (the float32 logits are exact copies of fp16
+                # values, so the kernel reads those); torch.rand supplies the randomness
+                idx_next = K.sample_topk_filter(logits.half().contiguous(), temperature, top_k)[:, None]
             else:
                 logits = logits / temperature
                 if top_k is not None:

@@ -478,6 +478,24 @@ def sample_topk(logits: torch.Tensor, temperature: float, top_k: int, uniform: O
     return out
 
 
+def sample_topk_filter(logits: torch.Tensor, temperature: float, top_k: int, uniform: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """One token per row as the flat-cache model's generate draws it (hf_model_q40.py:521-533): float32 logits / temperature,
+    values below the top_k-th largest masked (values EQUAL to it all stay), float32 softmax, one draw.  logits: the fp16
+    values [rows, vocab] (that model's float32 logits are exact copies of them).  `uniform` as in sample_topk."""
+    lib = _lib.load()
+    _need_gpu(logits)
+    assert logits.dim() == 2 and logits.dtype == torch.float16 and logits.stride(1) == 1
+    rows, vocab = logits.shape
+    if uniform is None:
+        uniform = torch.rand(rows, device=logits.device, dtype=torch.float32)
+    _need_gpu(uniform)
+    assert uniform.dtype == torch.float32 and uniform.numel() == rows and uniform.is_contiguous()
+    out = torch.empty(rows, device=logits.device, dtype=torch.int64)
+    check(lib.smh_sample_topk_filter(logits.data_ptr(), rows, vocab, logits.stride(0), float(temperature), int(min(top_k, vocab)),
+                                     uniform.data_ptr(), out.data_ptr(), _stream()), "smh_sample_topk_filter")
+    return out
+
+
 def sample_topk_counts(logits: torch.Tensor, temperature, top_k: int, counts: torch.Tensor, uniform: torch.Tensor,
                        out: Optional[torch.Tensor] = None) -> torch.Tensor:
     """sample_topk with counts[r] draws for row r (torch.multinomial(probs[r], num_samples=counts[r], replacement=True) of

@@ -155,6 +155,64 @@ def test_sample_topk_ties_take_the_lowest_indices_and_frequencies_follow_p():
         assert abs(freq - pj) < 4 * (pj * (1 - pj) / n) ** 0.5 + 1e-3
 
 
+@pytest.mark.parametrize("rows,vocab,k,temperature,grid", [(100, 32016, 32, 0.8, 0), (6, 32016, 32, 1.0, 8), (3, 320, 5, 1.0, 2),
+                                                           (7, 1000, 1, 1.3, 4), (4, 50, 50, 2.0, 2), (5, 4096, 1000, 0.6, 0)])
+def test_sample_topk_filter_matches_the_oracle(rows, vocab, k, temperature, grid):
+    """smh_sample_topk_filter (hf_model_q40.py:521-533) against the oracle: the same surviving tokens - every value equal to
+    the k-th largest included, which a coarse grid of logits makes common - the same float32 probabilities and the same
+    draw for the same uniform numbers, either neighbour accepted where the target is within rounding of a boundary"""
+    from spec_mcts_amd import kernels as K
+    g = torch.Generator().manual_seed(900 + vocab + k)
+    logits = torch.randn((rows, vocab), generator=g) * 2.5
+    logits = (torch.round(logits * grid) / grid if grid else logits).half()
+    p = O.topk_filter_probs(logits, temperature, k)
+    order = torch.argsort(logits.float(), dim=-1, descending=True, stable=True)
+    cdf = torch.gather(p, 1, order).cumsum(-1)
+    n_alive = (p > 0).sum(-1)
+    assert grid == 0 or int((n_alive > k).sum()) > 0 or k in (1, vocab)          # the grid cases do hold ties at the k-th value
+    for trial in range(4):
+        u = torch.rand(rows, generator=g)
+        want = O.sample_topk_filter(logits, temperature, k, u)
+        got = K.sample_topk_filter(logits.cuda(), temperature, k, u.cuda()).cpu()
+        for r in range(rows):
+            if int(got[r]) == int(want[r]):
+                continue
+            assert float(p[r, int(got[r])]) > 0, f"row {r}: token {int(got[r])} was filtered out"
+            j = int((order[r] == int(got[r])).nonzero()[0])
+            target = float(u[r]) * float(cdf[r, int(n_alive[r]) - 1])
+            edges = [float(cdf[r, j - 1]) if j else 0.0, float(cdf[r, j])]
+            assert min(abs(e - target) for e in edges) < 1e-5, f"row {r}: drew candidate {j}, target {target}, interval {edges}"
+    # the last surviving tie is reachable: u just below 1 draws the highest index among the values equal to the k-th
+    u = torch.full((rows,), 0.9999999)
+    got = K.sample_topk_filter(logits.cuda(), temperature, k, u.cuda()).cpu()
+    for r in range(rows):
+        assert int(got[r]) == int(order[r, int(n_alive[r]) - 1])
+
+
+def test_flat_cache_generate_samples_with_the_kernel():
+    """hf_model_q40.Transformer.generate with a temperature and top_k draws through smh_sample_topk_filter: with torch's
+    generator seeded the same way, the tokens equal those of the sampler called by hand on the same logits"""
+    from spec_mcts_amd import hf_model_q40 as M, kernels as K
+    from spec_mcts_amd.load_q40 import load_q40
+    cfg = dict(dim=256, n_layers=1, n_heads=2, vocab_size=640, multiple_of=128, max_batch_size=3, max_seq_len=24)
+    sd = O.random_q40_state_dict(O.OracleArgs(**cfg, max_prompt_seq_len=24), seed=38)
+    model = load_q40(dict(sd), M.ModelArgs(**cfg), device="cuda:0", model_cls=M.Transformer)
+    prompt = torch.randint(3, 640, (1, 5), generator=torch.Generator().manual_seed(39)).cuda()
+    calls = []
+    real = K.sample_topk_filter
+    K.sample_topk_filter = lambda *a, **kw: (calls.append(1), real(*a, **kw))[1]
+    try:
+        torch.manual_seed(11)
+        res, lens = model.generate(prompt, 3, 6, temperature=0.8, top_k=7)
+    finally:
+        K.sample_topk_filter = real
+    assert len(calls) == 6 and res.shape == (3, 6) and int(res.max()) < 640
+    model.fused_sampler = False
+    torch.manual_seed(11)
+    res2, _ = model.generate(prompt, 3, 6, temperature=0.8, top_k=7)              # torch's own sampler: another stream of draws
+    assert res2.shape == (3, 6)
+
+
 def test_detect_terminal_matches_the_oracle():
     """smh_detect_terminal against the oracle's detectTerminal on token streams with the terminal sequence, near
     matches and end-of-sequence tokens spliced in, 300 branches, 80 steps, state carried on the device: bit-exact"""

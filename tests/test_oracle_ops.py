@@ -251,6 +251,60 @@ def test_sampler_candidates_and_draw():
         assert abs(freq - float(p[0, j])) < 4 * (float(p[0, j]) * (1 - float(p[0, j])) / n) ** 0.5 + 1e-3
 
 
+def test_filter_sampler_keeps_every_value_equal_to_the_kth():
+    """topk_filter_probs (hf_model_q40.py:521-529) against hand-computed cases and float64 properties: the support is
+    exactly the values >= the k-th largest (brute-force count), probabilities are exp(x / T) over the support in float64;
+    sample_topk_filter against a scalar float64 scan and the probabilities themselves"""
+    import math
+    # 3, 3, 2, 2, 2, 1 with k = 3: the k-th largest is 2, all three 2s stay
+    row = torch.tensor([[2.0, 3.0, 1.0, 2.0, 3.0, 2.0]], dtype=torch.float16)
+    p = O.topk_filter_probs(row, 1.0, 3)[0].double()
+    z = 2 * math.exp(3) + 3 * math.exp(2)
+    want = torch.tensor([math.exp(2) / z, math.exp(3) / z, 0.0, math.exp(2) / z, math.exp(3) / z, math.exp(2) / z], dtype=torch.float64)
+    assert torch.allclose(p, want, rtol=1e-6, atol=0)
+    # k = 2: the k-th largest is 3, only the two 3s
+    p = O.topk_filter_probs(row, 0.5, 2)[0]
+    assert p.tolist() == [0.0, 0.5, 0.0, 0.0, 0.5, 0.0]
+    g = torch.Generator().manual_seed(78)
+    logits = torch.round(torch.randn((5, 400), generator=g) * 6).half() / 2          # a coarse grid: many equal values
+    for temperature, k in ((1.0, 32), (0.7, 5), (2.5, 400), (1.3, 1)):
+        p = O.topk_filter_probs(logits, temperature, k)
+        for r in range(5):
+            vals = sorted(logits[r].tolist(), reverse=True)
+            kth = vals[k - 1]
+            support = [i for i in range(400) if float(logits[r, i]) >= kth]
+            assert len(support) >= k and sorted((p[r] > 0).nonzero().flatten().tolist()) == support
+            z = sum(math.exp((float(logits[r, i]) - vals[0]) / temperature) for i in support)
+            for i in support[:50]:
+                assert abs(float(p[r, i]) - math.exp((float(logits[r, i]) - vals[0]) / temperature) / z) < 1e-6
+            assert abs(float(p[r].double().sum()) - 1.0) < 1e-5
+    # the draw: scalar scan over (value descending, index ascending)
+    p = O.topk_filter_probs(logits, 0.9, 20)
+    for trial in range(30):
+        u = torch.rand(5, generator=g)
+        got = O.sample_topk_filter(logits, 0.9, 20, u)
+        for r in range(5):
+            order = sorted(range(400), key=lambda i: (-float(logits[r, i]), i))
+            alive = [i for i in order if float(p[r, i]) > 0]
+            tot = sum(float(p[r, i]) for i in alive)
+            cum, pick, near = 0.0, alive[-1], False
+            for i in alive:
+                cum += float(p[r, i])
+                near = near or abs(cum - float(u[r]) * tot) < 1e-5
+                if cum > float(u[r]) * tot:
+                    pick = i
+                    break
+            assert int(got[r]) == pick or near
+    # frequencies over many draws follow p
+    n = 20000
+    u = torch.rand(n, generator=g)
+    draws = O.sample_topk_filter(logits[:1].expand(n, -1).contiguous(), 1.0, 4, u)
+    p = O.topk_filter_probs(logits[:1], 1.0, 4)[0]
+    for i in (p > 0).nonzero().flatten().tolist():
+        freq = float((draws == i).float().mean()); pi = float(p[i])
+        assert abs(freq - pi) < 4 * (pi * (1 - pi) / n) ** 0.5 + 1e-3
+
+
 TERMINAL = [29961, 29914, 20055, 4690, 1164, 29962]          # "[/PYTHON]" as the reference tokenises it (mcts.py:12)
 
 
