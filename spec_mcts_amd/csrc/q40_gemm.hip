@@ -109,7 +109,7 @@ __device__ __forceinline__ void gemm_piece(const MatmulParams &p, int unit, int 
     const int pair = unit - seg.unit0;
     const int col0 = pair * GEMM_COLS;
     const bool two_blocks = col0 + 128 < seg.N;
-    const int m0 = mb * GEMM_BM;
+    const int m0 = mb * p.block_rows;
     const int blk = wave >> 1;                 // block of the pair this wave decodes
     const int bp = wave & 1;                   // ... and its pair of byte positions
     const uint32_t sel0 = 0x0c000c00u | (uint32_t)(2 * bp) | ((uint32_t)(4 + 2 * bp) << 16);
@@ -591,7 +591,13 @@ void gemm_fill_plan(MatmulParams &p) {
     p.units = unit0;
     p.units_pad = (unit0 + 7) / 8 * 8;
     p.n_total = col0;
-    p.mblocks = (p.M + GEMM_BM - 1) / GEMM_BM;
+    p.block_rows = GEMM_BM;
+    // 65 .. 128 rows of a matrix with few column units and a short K (wo at 100 branches): two 64-row blocks per unit take
+    // half as many K-slices to fill the GPU, so half the slab bytes are written here and read by the consumer.  The blocks
+    // of a unit read the same weights at the same time in the same XCD.  (Measured at 100 rows: wo and the RMSNorm behind
+    // it 17.1 us against 19.8; with K = 11008 the launch itself loses what the consumer gains, 43 steps a workgroup.)
+    if (p.M > 64 && p.M <= 128 && p.units <= 16 && p.K % 32 == 0 && p.K <= 4096) p.block_rows = 64;
+    p.mblocks = (p.M + p.block_rows - 1) / p.block_rows;
     const int steps = (p.K + 31) / 32;
     const long tiles = (long)p.units * p.mblocks;
     // One round of workgroups.  One workgroup per compute unit when the column units divide the GPU well
@@ -672,7 +678,7 @@ static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
         return (int)lds_ok;
     }
     SMH_REQUIRE((long)p.M * p.lda * 2 < (1L << 32), "q40 gemm: M x lda = %d x %ld exceeds the 32-bit lane offsets of A", p.M, p.lda);
-    const int tiles = p.mblocks > 1 ? 8 : (p.M + 15) / 16;
+    const int tiles = p.mblocks > 1 ? p.block_rows / 16 : (p.M + 15) / 16;
     const bool one_each = HAS_DMA_WAVE && p.K % 32 == 0 && (p.chunk > 0 || (long)p.units * p.mblocks * p.ksplit <= GEMM_DMA_WAVE_MAX_WGS);
     const gemm_kernel_t kern = (p.K % 32 != 0) ? ragged : (p.chunk > 0 ? range_cut : one_each ? with_dma_wave : exact)[tiles < 2 ? 2 : tiles];
     const long total_steps = (long)p.units * ((p.K + 31) / 32);

@@ -101,11 +101,26 @@ class LinearQ4_0(torch.nn.Module):
         self.shape = (out_features, in_features)
         self._tiled = None
         self._tiled_key = None
+        self._released = False
+
+    def release_checkpoint(self):
+        """Keep only the tiled copy of this weight on the device: `.w` and `.s` become empty tensors (`.shape` stays), which
+        halves the weight bytes the model holds.  The module still multiplies (forward and the model's fused path read the
+        tiled copy); operators that take the checkpoint tensors themselves (matmul_q40, triton_deq_int40) no longer can."""
+        assert self.w.is_cuda, "the tiled copy lives on the GPU"
+        self.operand(True)
+        dev = self.w.device
+        self.w = torch.empty((0, self.group_size), dtype=torch.int8, device=dev)
+        self.s = torch.empty(0, dtype=DTYPE, device=dev)
+        self._released = True
 
     def operand(self, tiled: bool = True):
         """What matmul_q40_partial takes for this weight: (w, s, N) in the checkpoint layout, or - the default
         on the GPU - its tiled copy, made on first use (before any graph capture) and remade when `.w` / `.s`
         are replaced; after changing them in place call `invalidate()`."""
+        if self._released:
+            assert tiled, "this linear holds only its tiled copy (release_checkpoint)"
+            return self._tiled
         if not tiled or not self.w.is_cuda:
             return (self.w, self.s, self.shape[0])
         key = (self.w.data_ptr(), self.s.data_ptr())
@@ -123,7 +138,10 @@ class LinearQ4_0(torch.nn.Module):
         t0 = _tick()
         if residual is not None:
             residual = residual.reshape(shape[0] * shape[1], -1)
-        result = K.matmul_q40(x, self.w, self.s, (self.shape[1], self.shape[0]), residual=residual)
+        if self._released:
+            result = K.partial_reduce(K.matmul_q40_partial(x.contiguous(), [self._tiled]), residual=residual)
+        else:
+            result = K.matmul_q40(x, self.w, self.s, (self.shape[1], self.shape[0]), residual=residual)
         if PROFILE:
             global COMP_TIME
             COMP_TIME += _tick() - t0
@@ -499,6 +517,17 @@ class Transformer(nn.Module):
                 self._page_table.copy_(torch.arange(n, dtype=torch.int32, device=self._page_table.device).view_as(self._page_table))
             self._forked = False
         self._rows_written = 0
+
+    def release_checkpoint_weights(self):
+        """Drop every linear's checkpoint-layout tensors once their tiled copies exist (LinearQ4_0.release_checkpoint): the model
+        then holds one copy of the weights (3.6 GB less at 7B, 38 GB less at the 70B architecture).  Not in the reference,
+        whose kernels read the checkpoint layout; call it when nothing outside the model needs `.w` / `.s`."""
+        assert self.tiled_weights, "the model must be running on tiled weights"
+        for layer in self.layers:
+            a, f = layer.attention, layer.feed_forward
+            for lin in (a.wq, a.wk, a.wv, a.wo, f.w1, f.w2, f.w3):
+                lin.release_checkpoint()
+        torch.cuda.empty_cache()
 
     def resetTimers(self):
         global COMP_TIME, DEQ_TIME, QKVO_TIME, ATTN_TIME, MLP_TIME, Q_TIME, DQ_TIME

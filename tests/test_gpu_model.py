@@ -131,6 +131,35 @@ def test_fused_and_module_paths_agree():
         assert torch.allclose(x.float(), y.float(), rtol=1e-2, atol=1e-2)
 
 
+def test_model_runs_on_the_tiled_weights_alone():
+    """release_checkpoint_weights drops `.w` / `.s` of every linear: prefill and decode logits stay bit-identical (the
+    fused path never read them), a linear called as a module still multiplies, and the device holds fewer bytes"""
+    oargs, sd, model = _build(SMALL, 45)
+    prompt = torch.randint(0, SMALL["vocab_size"], (1, 19), generator=torch.Generator().manual_seed(145)).cuda()
+    tok = torch.randint(0, SMALL["vocab_size"], (3, 1), generator=torch.Generator().manual_seed(146)).cuda()
+
+    def run():
+        model.resetSeq()
+        a = model(prompt, 0).clone()
+        model.fork(0, 1, 2)
+        return a, model(tok, 19).clone()
+
+    before = run()
+    lin = model.layers[0].feed_forward.w2
+    x = torch.randn((1, 5, lin.shape[1]), generator=torch.Generator().manual_seed(147)).half().cuda()
+    y_before = lin(x).clone()
+    torch.cuda.synchronize()
+    held = torch.cuda.memory_allocated()
+    model.release_checkpoint_weights()
+    assert lin.w.numel() == 0 and lin.s.numel() == 0 and tuple(lin.shape) == (SMALL["dim"], 768)
+    assert torch.cuda.memory_allocated() < held
+    after = run()
+    assert torch.equal(before[0], after[0]) and torch.equal(before[1], after[1])
+    assert torch.equal(lin(x), y_before)
+    with pytest.raises(AssertionError):
+        lin.operand(False)
+
+
 def test_hf_model_q40_flavour_matches_oracle():
     """hf_model_q40.Transformer: per-row Q4_0 cache for every position, B distinct prompt rows prefilled
     together, fp32 logits; decode steps run the same kernels with an empty shared prefix"""
