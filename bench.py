@@ -40,9 +40,9 @@ ARCHS = {
 # HBM bytes per q40_gemv_kernel launch at M=1: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by a 1 GiB copy
 # (profiles/q40_gemv_m1_hbm_traffic.md has the commands and the factors: 2.0 for reads, 1.0 for writes)
 GEMV_TRAFFIC_BYTES_PER_LAUNCH = 27457381
-# the same for q40_gemm_kernel at M=100 (profiles/q40_gemm_m100_hbm_traffic.md): 37.37 MB read + 28.06 MB written
-# (the fp32 partial sums of the K-slices are most of the writes)
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 65425312
+# the same for q40_gemm_kernel at M=100 (profiles/q40_gemm_m100_hbm_traffic.md): 37.34 MB read + 24.78 MB written
+# (the fp32 partial sums of the K-slices are the writes)
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 62123956
 # the same for one call of the decode attention leg (profiles/attn_decode_hbm_traffic.md): 65.6 MB read + 9.0 MB written
 ATTN_TRAFFIC_BYTES_PER_CALL = 74610046
 
