@@ -402,6 +402,9 @@ def main():
     ap.add_argument("--attention-only", action="store_true",
                     help="profiling aid: run only the decode attention leg (64 branches, 1024-token shared prefix, ragged Q4_0 suffixes) "
                          "after the same 1 GiB calibration copy, and print that leg's numbers")
+    ap.add_argument("--tree-only", action="store_true",
+                    help="profiling aid: run only the tree-search leg (mcts.search, 512-token prompt, 8 .. 100 branches) and the paged "
+                         "attention leg, and print their numbers")
     ap.add_argument("--layers", type=int, default=0, help="fewer layers for a quick functional run (INVALID as a result)")
     ap.add_argument("--arch", choices=sorted(ARCHS), default="7b",
                     help="7b is the headline workload; 70b is the 80-layer GQA architecture with a 2048-token prompt (about 38 GB of Q4_0 "
@@ -436,6 +439,9 @@ def main():
         torch.cuda.synchronize()
         del src, dst
         print(json.dumps(attention_roofline(torch) if a.attention_only else matmul_roofline(torch, model, a.roofline_only, 3)))
+        return
+    if a.tree_only:
+        print(json.dumps({"tree_search": tree_search_bench(torch, model, prompt), "paged_attn": paged_attention_bench(torch)}))
         return
     batches = tuple(int(x) for x in a.batches.split(",")) if a.batches else BATCHES
     # the prefill of the shared prompt (once per tree, outside the timed decode steps): reported next to them
