@@ -16,8 +16,8 @@ near_tie = 2 x the largest change of the top-1/top-2 gap between the fp32 and th
 below it can be decided either way by implementations that both follow the reference exactly.
 
 Needs a GPU (the weights are generated and quantised there by bench.build_model, then copied to the host) and about
-90 GB of host memory.  Run from the repository root on the GPU box; results land in gpurun_out/greedy_7b.json (copy
-it to tests/golden/):
+90 GB of host memory.  Run from the repository root on the GPU box; results land in greedy_7b.json next to this
+script and in the run's output folder (OUT_DIR below):
 
     python tests/golden/make_7b_greedy.py [--seed 3] [--variants acc64,scale_on_x,p_half,slab_half]
 
@@ -34,6 +34,7 @@ import time
 import torch
 
 ROOT = os.path.dirname(os.path.dirname(os.path.dirname(os.path.abspath(__file__))))
+OUT_DIR = "gpurun_out"
 sys.path.insert(0, ROOT)
 import bench                                  # noqa: E402  (build_model: the generator of the 7B random weights)
 from oracle import q40_oracle as O            # noqa: E402
@@ -136,8 +137,8 @@ def main():
             out["noise"]["acc64"] = study("acc64", oargs, sd, prompt, tokens, base_logits, None)
     if "acc64" in out["noise"]:
         out["near_tie"] = round(2.0 * max(out["noise"]["acc64"]["gap_shift"]), 5)
-    os.makedirs(os.path.join(ROOT, "gpurun_out"), exist_ok=True)
-    for dst in (path, os.path.join(ROOT, "gpurun_out", "greedy_7b.json")):
+    os.makedirs(os.path.join(ROOT, OUT_DIR), exist_ok=True)
+    for dst in (path, os.path.join(ROOT, OUT_DIR, "greedy_7b.json")):
         with open(dst, "w") as f:
             json.dump(out, f)
     print(json.dumps({k: v for k, v in out.items() if k != "noise"})[:600])

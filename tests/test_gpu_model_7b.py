@@ -13,9 +13,11 @@ GEMM, the two-launch attention).  Two runs per path:
   free-running    the GPU model is fed its own tokens, as the benchmark runs it; the common prefix with the oracle's tokens
                   must reach the path's first differing teacher-forced step (all 64 tokens when none differs).
 The per-path lines (matches, differing steps with their margins and bounds, free-run length) are also written to
-gpurun_out/greedy_7b_paths.md."""
+greedy_7b_paths.md in the run's output folder (REPORT_DIR below)."""
 import json
 import os
+
+REPORT_DIR = "gpurun_out"
 
 import pytest
 import torch
@@ -90,7 +92,7 @@ def test_7b_greedy_tokens_match_oracle():
 
 
 def _write_report(lines):
-    out = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "gpurun_out")
+    out = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), REPORT_DIR)
     try:
         os.makedirs(out, exist_ok=True)
         with open(os.path.join(out, "greedy_7b_paths.md"), "w") as f:
