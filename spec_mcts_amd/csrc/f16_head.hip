@@ -25,9 +25,15 @@ constexpr int HEAD_BN = 128;                   // outputs (rows of W) per workgr
 constexpr int HEAD_BM = 128;                   // rows of x per workgroup
 constexpr int HEAD_WAVES = 4;
 constexpr int HEAD_KS = 64;                    // K values per stage (128 bytes per row)
-constexpr int HEAD_STAGES = 4;
-static_assert(HEAD_STAGES == 4, "the drain loop's waits are written for four stages");
 constexpr int HEAD_W_BYTES = HEAD_BN * 128;    // 16 KB per stage
+constexpr int HEAD_LDS_MAX = 160 * 1024;
+// ring slots for TILES 16-row tiles of x: four (six and eight, where the compute unit's LDS holds them, measured 2-3 % slower:
+// the kernel does not wait on memory latency)
+constexpr int HEAD_MAX_STAGES = 4;
+constexpr int head_stages(int tiles) {
+    const int fit = HEAD_LDS_MAX / (HEAD_W_BYTES + tiles * 16 * 128);
+    return fit > HEAD_MAX_STAGES ? HEAD_MAX_STAGES : fit;
+}
 
 typedef const __attribute__((address_space(1))) void *gptr_t;
 typedef __attribute__((address_space(3))) void *lptr_t;
@@ -43,6 +49,15 @@ struct HeadParams {
 
 template <int N_>
 __device__ __forceinline__ void head_wait_dma() { asm volatile("s_waitcnt vmcnt(%0)" ::"n"(N_) : "memory"); }
+// at most `left` (0 .. MAX) stages of PER instructions may stay in flight
+template <int PER, int MAX>
+__device__ __forceinline__ void head_wait_stages(int left) {
+    if constexpr (MAX == 0) head_wait_dma<0>();
+    else {
+        if (left >= MAX) head_wait_dma<MAX * PER>();
+        else head_wait_stages<PER, MAX - 1>(left);
+    }
+}
 
 // TILES: 16-row tiles of x a workgroup multiplies (1..8); XD = DMA instructions of the x tile per wave and stage
 template <int TILES>
@@ -52,7 +67,8 @@ __global__ __launch_bounds__(HEAD_WAVES * 64) void f16_head_kernel(HeadParams p)
     constexpr int STAGE = HEAD_W_BYTES + X_BYTES;
     constexpr int XD = (2 * TILES + HEAD_WAVES - 1) / HEAD_WAVES;
     constexpr int PER = 4 + XD;                       // DMA instructions per wave and stage
-    static_assert((HEAD_STAGES - 2) * PER <= 63, "vmcnt is a 6-bit counter");
+    constexpr int HEAD_STAGES = head_stages(TILES);
+    static_assert(HEAD_STAGES >= 3 && (HEAD_STAGES - 2) * PER <= 63, "vmcnt is a 6-bit counter");
 
     const int tid = threadIdx.x;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -85,8 +101,16 @@ __global__ __launch_bounds__(HEAD_WAVES * 64) void f16_head_kernel(HeadParams p)
     }
     const uint8_t *x_base = reinterpret_cast<const uint8_t *>(p.x);
 
-    auto issue = [&](int stage_k, int slot) {
+    // Workgroup j starts at stage j of K and wraps.  The rows of W are K * 2 bytes apart (8 KB at the 7B shape), so with every
+    // workgroup on the same stage all 128 x 251 row pieces in flight have the same low address bits and fall on a few memory
+    // channels: 59.6 us per launch at the 7B shape; staggered, 47.8 us (5.5 TB/s).  The order of the fp32 additions of an output
+    // then depends on its block of 128 outputs, not on anything that varies between runs.
+    const int n_stages = p.K / HEAD_KS;
+    const int rot = (int)(blockIdx.x % (unsigned)n_stages);
+    auto issue = [&](int stage_i, int slot) {
         uint8_t *st = lds + slot * STAGE;
+        int stage_k = stage_i + rot;
+        if (stage_k >= n_stages) stage_k -= n_stages;
         const long kb = (long)stage_k * HEAD_KS * 2;
 #pragma unroll
         for (int i = 0; i < 4; ++i)
@@ -102,7 +126,6 @@ __global__ __launch_bounds__(HEAD_WAVES * 64) void f16_head_kernel(HeadParams p)
 #pragma unroll
         for (int t = 0; t < TILES; ++t) acc[a][t] = f4{0.f, 0.f, 0.f, 0.f};
 
-    const int n_stages = p.K / HEAD_KS;
 #pragma unroll
     for (int i = 0; i < HEAD_STAGES - 1; ++i)
         if (i < n_stages) issue(i, i);
@@ -143,10 +166,7 @@ __global__ __launch_bounds__(HEAD_WAVES * 64) void f16_head_kernel(HeadParams p)
     // drain: no refills; `left` younger stages are still in flight
 #pragma unroll 1
     for (; i < n_stages; ++i) {
-        const int left = n_stages - 1 - i;
-        if (left >= 2) head_wait_dma<2 * PER>();
-        else if (left == 1) head_wait_dma<PER>();
-        else head_wait_dma<0>();
+        head_wait_stages<PER, HEAD_STAGES - 2>(n_stages - 1 - i);
         asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
         compute(lds + slot * STAGE);
         slot = slot == HEAD_STAGES - 1 ? 0 : slot + 1;
@@ -204,7 +224,7 @@ extern "C" int smh_f16_linear(const void *x, int M, int K, long ldx, const void 
     static const hipError_t lds_ok = [] {
         hipError_t e = hipSuccess;
         for (int t = 1; t <= 8 && e == hipSuccess; ++t)
-            e = hipFuncSetAttribute((const void *)kern[t], hipFuncAttributeMaxDynamicSharedMemorySize, HEAD_STAGES * (HEAD_W_BYTES + 8 * 16 * 128));
+            e = hipFuncSetAttribute((const void *)kern[t], hipFuncAttributeMaxDynamicSharedMemorySize, head_stages(t) * (HEAD_W_BYTES + t * 16 * 128));
         return e;
     }();
     if (lds_ok != hipSuccess) { set_error("%s: hipFuncSetAttribute: %s", who, hipGetErrorString(lds_ok)); return (int)lds_ok; }
@@ -213,7 +233,7 @@ extern "C" int smh_f16_linear(const void *x, int M, int K, long ldx, const void 
     p.ldx = ldx; p.ldo = ldo; p.M = M; p.N = N; p.K = K;
     p.vec_store = (ldo % 4 == 0) && (((uintptr_t)out & 7) == 0);
     const int tiles = M >= HEAD_BM ? 8 : (M + 15) / 16;
-    const size_t lds = (size_t)HEAD_STAGES * (HEAD_W_BYTES + tiles * 16 * 128);
+    const size_t lds = (size_t)head_stages(tiles) * (HEAD_W_BYTES + tiles * 16 * 128);
     dim3 grid((unsigned)((N + HEAD_BN - 1) / HEAD_BN), (unsigned)((M + HEAD_BM - 1) / HEAD_BM));
     hipLaunchKernelGGL(kern[tiles], grid, dim3(HEAD_WAVES * 64), lds, (hipStream_t)stream, p);
     return launch_status();
