@@ -247,16 +247,31 @@ __device__ __forceinline__ half_t sample_unkey(uint32_t k) {
     return __builtin_bit_cast(half_t, b);
 }
 
-// bins[t] <- sum of bins[t..255]; then the bin where the count from the top reaches `want` and the count above it
-__device__ __forceinline__ void sample_pick_bin(int *bins, int want, int *out_bin, int *out_above) {
-    const int t = threadIdx.x;
-    for (int off = 1; off < 256; off <<= 1) {
-        int v = 0;
-        if (t < 256 && t + off < 256) v = bins[t + off];
-        __syncthreads();
-        if (t < 256) bins[t] += v;
-        __syncthreads();
+// Inclusive prefix sums over the 1024 threads of the workgroup (thread order): inside a wave by lane shifts, across waves
+// through s_w[16]; two barriers.  Every thread of the workgroup must call.
+template <class T>
+__device__ __forceinline__ T sample_block_scan(T v, T *s_w) {
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const T t = __shfl_up(v, o, 64);
+        if (lane >= o) v += t;
     }
+    if (lane == 63) s_w[wave] = v;
+    __syncthreads();
+    T base = 0;
+    for (int w = 0; w < wave; ++w) base += s_w[w];
+    __syncthreads();
+    return v + base;
+}
+
+// bins[t] <- sum of bins[t..255]; then the bin where the count from the top reaches `want` and the count above it
+__device__ __forceinline__ void sample_pick_bin(int *bins, int *s_w, int want, int *out_bin, int *out_above) {
+    const int t = threadIdx.x;
+    const int mine = t < 256 ? bins[255 - t] : 0;                 // thread t holds bin 255 - t: a prefix sum from the top
+    const int upto = sample_block_scan(mine, s_w);
+    if (t < 256) bins[255 - t] = upto;
+    __syncthreads();
     if (t < 256) {
         const int above = t == 255 ? 0 : bins[t + 1];
         if (bins[t] >= want && above < want) { *out_bin = t; *out_above = above; }
@@ -266,6 +281,9 @@ __device__ __forceinline__ void sample_pick_bin(int *bins, int want, int *out_bi
 
 // counts == nullptr: one draw per row, uniform[row] -> out[row].  Otherwise row r makes counts[r] draws with replacement from
 // its candidates, with the uniform numbers (and into the slots of out) that start at counts[0] + ... + counts[r-1].
+// Thread t owns the contiguous chunk of ceil(vocab / 1024) logits that starts at t times that.  Up to 32768 logits (a multiple
+// of 8, rows 16-byte aligned) the chunk is read ONCE, as four 16-byte loads, and its 32 sixteen-bit keys stay in registers for
+// the two histogram passes, the tie count and the gather; otherwise every pass reads the logits again.
 __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restrict__ logits, int vocab, long ld, float temperature,
                                                            int top_k, const float *__restrict__ uniform, int64_t *__restrict__ out,
                                                            const int32_t *__restrict__ counts, const float *__restrict__ row_temps, int n_draws,
@@ -282,8 +300,10 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
     const bool greedy_row = row_temps != nullptr && !(temperature > 0.f);
     if (greedy_row) temperature = 1.0f;
     __shared__ int bins[256];
+    __shared__ int wbins[256 * 16];
+    __shared__ int s_wi[16];
+    __shared__ float s_wf[16];
     __shared__ int s_bin, s_above, s_count;
-    __shared__ int scan[1024];
     __shared__ uint32_t c_key[SAMPLE_MAX_K];
     __shared__ int c_idx[SAMPLE_MAX_K];
     __shared__ uint32_t o_key[SAMPLE_MAX_K];
@@ -292,26 +312,70 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
     const int tid = threadIdx.x;
     const half_t *row = logits + (long)blockIdx.x * ld;
     int k = min(top_k, vocab);
-    auto key_at = [&](int i) { return sample_key(wide ? row[i] : (half_t)((float)row[i] / temperature)); };
+    auto key_of = [&](half_t x) { return sample_key(wide ? x : (half_t)((float)x / temperature)); };
     auto value_of = [&](uint32_t key) { return wide ? (float)sample_unkey(key) / temperature : (float)sample_unkey(key); };
 
+    constexpr int CH = 32;
+    const bool in_regs = vocab <= 1024 * CH && vocab % 8 == 0 && (reinterpret_cast<uintptr_t>(row) & 15) == 0;     // (uniform)
+    const int chunk = in_regs ? CH : (vocab + 1023) / 1024;
+    const int lo = min(tid * chunk, vocab), hi = min(vocab, lo + chunk);
+    uint32_t kr[CH / 2];                       // in_regs: keys of elements lo + 2 j (low half) and lo + 2 j + 1
+    if (in_regs) {
+        u32x4 raw[CH / 8];
+#pragma unroll
+        for (int q = 0; q < CH / 8; ++q) {
+            raw[q] = u32x4{0u, 0u, 0u, 0u};
+            if (lo + 8 * q < hi) raw[q] = *reinterpret_cast<const u32x4 *>(row + lo + 8 * q);
+        }
+#pragma unroll
+        for (int j = 0; j < CH / 2; ++j) {
+            const uint32_t two = raw[j >> 2][j & 3];
+            const uint32_t k0 = key_of(__builtin_bit_cast(half_t, (uint16_t)(two & 0xFFFFu)));
+            const uint32_t k1 = key_of(__builtin_bit_cast(half_t, (uint16_t)(two >> 16)));
+            kr[j] = k0 | (k1 << 16);
+        }
+    }
+    // f(index, key) for every logit of this thread's chunk, in index order
+    auto for_each = [&](auto f) {
+        if (in_regs) {
+#pragma unroll
+            for (int j = 0; j < CH; ++j)
+                if (lo + j < hi) f(lo + j, (kr[j >> 1] >> (16 * (j & 1))) & 0xFFFFu);
+        } else {
+            for (int i = lo; i < hi; ++i) f(i, key_of(row[i]));
+        }
+    };
+
     // ---- the k-th largest key: high byte, then low byte ----
-    if (tid < 256) bins[tid] = 0;
+    // Atomics of different waves on one LDS word take turns, and logits crowd into a few high bytes: every wave counts into a
+    // histogram of its own (word = bin * 16 + wave, the 16 copies of a bin in 16 banks), which are then added.
+    const int wv = tid >> 6;
+    auto fold_bins = [&]() {
+        if (tid < 256) {
+            int n = 0;
+#pragma unroll
+            for (int w = 0; w < 16; ++w) n += wbins[tid * 16 + w];
+            bins[tid] = n;
+        }
+        __syncthreads();
+    };
+    for (int i = tid; i < 256 * 16; i += 1024) wbins[i] = 0;
     if (tid == 0) s_count = 0;
     __syncthreads();
-    for (int i = tid; i < vocab; i += 1024) atomicAdd(&bins[key_at(i) >> 8], 1);
+    for_each([&](int, uint32_t key) { atomicAdd(&wbins[(key >> 8) * 16 + wv], 1); });
     __syncthreads();
-    sample_pick_bin(bins, k, &s_bin, &s_above);
+    fold_bins();
+    sample_pick_bin(bins, s_wi, k, &s_bin, &s_above);
     const int b1 = s_bin, above1 = s_above;
     __syncthreads();
-    if (tid < 256) bins[tid] = 0;
+    for (int i = tid; i < 256 * 16; i += 1024) wbins[i] = 0;
     __syncthreads();
-    for (int i = tid; i < vocab; i += 1024) {
-        const uint32_t key = key_at(i);
-        if ((int)(key >> 8) == b1) atomicAdd(&bins[key & 255], 1);
-    }
+    for_each([&](int, uint32_t key) {
+        if ((int)(key >> 8) == b1) atomicAdd(&wbins[(key & 255u) * 16 + wv], 1);
+    });
     __syncthreads();
-    sample_pick_bin(bins, k - above1, &s_bin, &s_above);
+    fold_bins();
+    sample_pick_bin(bins, s_wi, k - above1, &s_bin, &s_above);
     const uint32_t kth = ((uint32_t)b1 << 8) | (uint32_t)s_bin;      // key of the k-th largest value
     int ties_wanted = k - (above1 + s_above);                          // how many of the values equal to it are in
     if (keep_ties) {                                                   // all of them, while the candidate arrays hold them
@@ -320,23 +384,12 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
     }
     __syncthreads();
 
-    // ---- gather: everything above the k-th key, and of the ties the lowest indices (contiguous chunk per thread,
-    //      exclusive scan of the per-thread tie counts gives each tie its rank by index) ----
-    const int chunk = (vocab + 1023) / 1024;
-    const int lo = tid * chunk, hi = min(vocab, lo + chunk);
+    // ---- gather: everything above the k-th key, and of the ties the lowest indices (the chunks are in index order, so a
+    //      prefix sum of the per-thread tie counts gives each tie its rank by index) ----
     int my_ties = 0;
-    for (int i = lo; i < hi; ++i) my_ties += key_at(i) == kth;
-    scan[tid] = my_ties;
-    __syncthreads();
-    for (int off = 1; off < 1024; off <<= 1) {
-        const int v = tid >= off ? scan[tid - off] : 0;
-        __syncthreads();
-        scan[tid] += v;
-        __syncthreads();
-    }
-    int tie_rank = scan[tid] - my_ties;                                // ties at lower indices
-    for (int i = lo; i < hi; ++i) {
-        const uint32_t key = key_at(i);
+    for_each([&](int, uint32_t key) { my_ties += key == kth; });
+    int tie_rank = sample_block_scan(my_ties, s_wi) - my_ties;         // ties at lower indices
+    for_each([&](int i, uint32_t key) {
         bool take = key > kth;
         if (key == kth) { take = tie_rank < ties_wanted; ++tie_rank; }
         if (take) {
@@ -344,7 +397,7 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
             c_key[slot] = key;
             c_idx[slot] = i;
         }
-    }
+    });
     __syncthreads();
 
     // ---- order the k candidates: rank = number of candidates that come before ----
@@ -358,28 +411,16 @@ __global__ __launch_bounds__(1024) void sample_topk_kernel(const half_t *__restr
     }
     __syncthreads();
 
-    // ---- p = fp16(softmax), inverse CDF ----
+    // ---- p = fp16(softmax) (fp32 with a row temperature or the filter form), inverse CDF ----
     const float xmax = value_of(o_key[0]);
     const float e = tid < k ? expf(value_of(o_key[tid]) - xmax) : 0.f;
-    cdf[tid] = e;
+    cdf[tid] = sample_block_scan(e, s_wf);
     __syncthreads();
-    for (int off = 1; off < 1024; off <<= 1) {
-        const float v = tid >= off ? cdf[tid - off] : 0.f;
-        __syncthreads();
-        cdf[tid] += v;
-        __syncthreads();
-    }
     const float total = cdf[k - 1];
     __syncthreads();
     const float pr = tid < k ? (wide ? e / total : (float)(half_t)(e / total)) : 0.f;
-    cdf[tid] = pr;
+    cdf[tid] = sample_block_scan(pr, s_wf);
     __syncthreads();
-    for (int off = 1; off < 1024; off <<= 1) {
-        const float v = tid >= off ? cdf[tid - off] : 0.f;
-        __syncthreads();
-        cdf[tid] += v;
-        __syncthreads();
-    }
     long first = blockIdx.x;
     int draws = 1;
     if (counts != nullptr) {
