@@ -100,7 +100,8 @@ int smh_gq40_dequant(const void *packed, const void *scale, void *out, long bloc
  * hf_model_q40_kv_shared.py:313; w1|w3 of FeedForward.forward, :434) run as segments of one
  * launch; their outputs are concatenated along the columns (n_total = sum of n[i]).
  *
- * smh_q40_matmul_plan         ksplit the kernels will use for these dimensions (depends on M, K, n only)
+ * smh_q40_matmul_plan         ksplit the kernels will use for these dimensions on checkpoint-layout weights (depends on M, K, n only)
+ * smh_q40_matmul_plan_tiled   the same for tiled weights (smh_q40_tile): equal up to 16 rows; above, tiled weights may take fewer slices
  * smh_q40_matmul_partial      produce the slabs; partial_bytes >= ksplit * M * n_total * 4
  * smh_partial_reduce          c[m][j] = fp16(sum) (+ residual) for columns col0 .. col0+N-1
  * smh_partial_rmsnorm         h_out = h_in + fp16(sum) (residual add of TransformerBlock.forward,
@@ -113,6 +114,7 @@ int smh_gq40_dequant(const void *packed, const void *scale, void *out, long bloc
  *                             *t_dev of every branch's suffix cache (:365-371); cache_k may be NULL
  */
 int smh_q40_matmul_plan(int M, int K, int nseg, const int *n);
+int smh_q40_matmul_plan_tiled(int M, int K, int nseg, const int *n);
 int smh_q40_matmul_partial(const void *a, int M, int K, long lda, int nseg, const void *const *w,
                            const void *const *s, const int *n, void *partial, size_t partial_bytes,
                            smh_stream_t stream);

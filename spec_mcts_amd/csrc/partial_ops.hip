@@ -226,7 +226,7 @@ using namespace smh;
 
 // ---- host side: plan, produce, consume ----------------------------------------------------------------
 static int fill_params(MatmulParams &p, const void *a, int M, int K, long lda, int nseg, const void *const *w,
-                       const void *const *s, const int *n, const char *who) {
+                       const void *const *s, const int *n, const char *who, bool tiled = false) {
     SMH_REQUIRE(M >= 0, "%s: M=%d", who, M);
     SMH_REQUIRE(K > 0 && K % 8 == 0, "%s: K=%d must be a positive multiple of 8", who, K);
     SMH_REQUIRE(nseg >= 1 && nseg <= SMH_MAX_SEGMENTS && n != nullptr, "%s: nseg=%d outside [1,%d]", who, nseg, SMH_MAX_SEGMENTS);
@@ -240,6 +240,7 @@ static int fill_params(MatmulParams &p, const void *a, int M, int K, long lda, i
         p.seg[i].s = s ? (const half_t *)s[i] : nullptr;
         p.seg[i].N = n[i];
     }
+    p.tiled = tiled ? 1 : 0;                   // (the plan above 16 rows depends on the layout)
     if (M <= SMH_GEMV_MAX_M) gemv_fill_plan(p); else gemm_fill_plan(p);
     return 0;
 }
@@ -248,6 +249,13 @@ extern "C" int smh_q40_matmul_plan(int M, int K, int nseg, const int *n) {
     MatmulParams p;
     if (M <= 0) return 1;
     int st = fill_params(p, nullptr, M, K, (K + 7) / 8 * 8, nseg, nullptr, nullptr, n, "smh_q40_matmul_plan");
+    return st < 0 ? st : p.ksplit;
+}
+
+extern "C" int smh_q40_matmul_plan_tiled(int M, int K, int nseg, const int *n) {
+    MatmulParams p;
+    if (M <= 0) return 1;
+    int st = fill_params(p, nullptr, M, K, (K + 7) / 8 * 8, nseg, nullptr, nullptr, n, "smh_q40_matmul_plan_tiled", true);
     return st < 0 ? st : p.ksplit;
 }
 
@@ -280,7 +288,7 @@ extern "C" int smh_q40_matmul_partial(const void *a, int M, int K, long lda, int
 extern "C" int smh_q40_matmul_partial_tiled(const void *a, int M, int K, long lda, int nseg, const void *const *tiled,
                                             const int *n, void *partial, size_t partial_bytes, smh_stream_t stream) {
     MatmulParams p;
-    int st = fill_params(p, a, M, K, lda, nseg, tiled, nullptr, n, "smh_q40_matmul_partial_tiled");
+    int st = fill_params(p, a, M, K, lda, nseg, tiled, nullptr, n, "smh_q40_matmul_partial_tiled", true);
     if (st) return st;
     if (M == 0) return 0;
     SMH_REQUIRE(a && tiled && partial, "smh_q40_matmul_partial_tiled: null pointer");
@@ -298,7 +306,7 @@ extern "C" int smh_q40_matmul_partial_tiled_silu(const void *gate_up_partial, in
                                                  const void *const *tiled, const int *n, void *partial, size_t partial_bytes,
                                                  smh_stream_t stream) {
     MatmulParams p;
-    int st = fill_params(p, nullptr, M, K, (K + 7) / 8 * 8, nseg, tiled, nullptr, n, "smh_q40_matmul_partial_tiled_silu");
+    int st = fill_params(p, nullptr, M, K, (K + 7) / 8 * 8, nseg, tiled, nullptr, n, "smh_q40_matmul_partial_tiled_silu", true);
     if (st) return st;
     if (M == 0) return 0;
     SMH_REQUIRE(M <= SMH_SILU_IN_MAX_M, "smh_q40_matmul_partial_tiled_silu: M=%d (at most %d rows; use smh_partial_silu_mul above)", M, SMH_SILU_IN_MAX_M);
@@ -321,7 +329,7 @@ extern "C" int smh_q40_matmul_partial_tiled_silu(const void *gate_up_partial, in
 extern "C" int smh_q40_norm_in_fits(int M, int K, int nseg, const int *n) {
     MatmulParams p;
     if (M <= 0 || M > SMH_GEMV_MAX_M || K % 32 != 0) return 0;
-    int st = fill_params(p, nullptr, M, K, (K + 7) / 8 * 8, nseg, nullptr, nullptr, n, "smh_q40_norm_in_fits");
+    int st = fill_params(p, nullptr, M, K, (K + 7) / 8 * 8, nseg, nullptr, nullptr, n, "smh_q40_norm_in_fits", true);
     return st < 0 ? st : (gemv_norm_in_fits(p) ? 1 : 0);
 }
 
@@ -330,7 +338,7 @@ extern "C" int smh_q40_matmul_partial_tiled_norm(const void *h, long ldh, const 
                                                  void *partial, size_t partial_bytes, smh_stream_t stream) {
     const char *who = "smh_q40_matmul_partial_tiled_norm";
     MatmulParams p;
-    int st = fill_params(p, h, M, K, ldh, nseg, tiled, nullptr, n, who);
+    int st = fill_params(p, h, M, K, ldh, nseg, tiled, nullptr, n, who, true);
     if (st) return st;
     if (M == 0) return 0;
     SMH_REQUIRE(M <= SMH_GEMV_MAX_M, "%s: M=%d (at most %d rows; use smh_partial_rmsnorm above)", who, M, SMH_GEMV_MAX_M);

@@ -580,6 +580,233 @@ __global__ __launch_bounds__(64 * (WAVES + (PRODUCER ? 1 : 0)), WAVES == 8 ? 1 :
     }
 }
 
+// ---- two K-groups in one workgroup (tiled weights, K a multiple of 64, one workgroup per compute unit) ----------------
+// A workgroup owns ONE 128-column block (pieces 2 blk, 2 blk + 1 of the unit's tiles), a block of rows and a K-slice, and
+// its eight multiplying waves form two groups: group kk takes the steps 2 i + kk of the slice.  Wave (kk, hh, bp)
+// multiplies the columns of nibble hh of piece 2 blk + bp of its group's steps with all row tiles of A - the same two B
+// operands and 14 MFMAs per step as in q40_gemm_kernel - so a ring stage holds TWO steps: both pieces of the block and the
+// scales of either step, and either step's rows of A.  The groups' accumulators are added through LDS at the end (group 0
+// + group 1, a fixed order), and the first four waves write the slab.  Against q40_gemm_kernel's 256-column units this
+// fills the GPU with half as many K-slices, i.e. half the slab bytes written here and read back by the consumer; the
+// price is that a row of A is staged for 128 columns instead of 256.
+constexpr int KG_W = 4096;                     // [group kk][piece bp] x 1024
+constexpr int KG_S = 512;                      // [group kk] x 256 (the whole scale block of the step)
+template <int TILES> struct KgShape {
+    static constexpr int STAGE = KG_W + KG_S + 2 * TILES * 1024;
+    static constexpr int SLOTS = GEMM_DMA_WAVE_SLOTS;
+    static constexpr int LDS = SLOTS * STAGE;
+    static constexpr int PER = 2 * (3 + TILES);                    // DMA instructions of a stage
+    static constexpr int RED = 4 * TILES * 2 * 1024;               // the second group's accumulators: [wave][t][o][lane] x 16 B
+    static constexpr int OP = 128 + 4;
+    static constexpr int OTILE = 16 * OP * 4;
+    static_assert(RED + 2 * OTILE <= LDS, "the sums of the second group and two output tiles must fit in the ring");
+    static_assert(PER * (SLOTS - 5) <= 63 && LDS <= 160 * 1024, "ring");
+};
+
+template <int TILES>
+__global__ __launch_bounds__(576, 1) void q40_gemm_kg_kernel(MatmulParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    typedef KgShape<TILES> S;
+    constexpr int SLOTS = S::SLOTS, PER = S::PER, STAGE = S::STAGE;
+    const int tid = threadIdx.x;
+    const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);       // 0..7 multiply, 8 issues the DMA
+    const int lane = tid & 63, c = lane & 15, g = lane >> 4;
+    // blockIdx -> (128-column block, row block, K-slice); blocks of one unit are neighbours (same XCD every 8)
+    int bid = blockIdx.x;
+    const int hb = bid % (2 * p.units_pad);  bid /= 2 * p.units_pad;
+    const int slot_u = hb >> 1, blk = hb & 1;
+    const int unit = (slot_u & 7) * (p.units_pad >> 3) + (slot_u >> 3);
+    if (unit >= p.units) return;
+    const int mb = bid % p.mblocks, slice = bid / p.mblocks;
+    int sg = 0;
+    if (p.nseg > 1 && unit >= p.seg[1].unit0) sg = 1;
+    if (p.nseg > 2 && unit >= p.seg[2].unit0) sg = 2;
+    const MatmulSegment seg = p.seg[sg];
+    const int pair = unit - seg.unit0;
+    const int col0 = pair * GEMM_COLS + 128 * blk;
+    if (col0 >= seg.N) return;                                         // a weight with an odd number of 128-column blocks
+    const int m0 = mb * p.block_rows;
+    const int steps_total = p.K / 32;
+    const int step0 = slice * p.steps_per_slice, step1 = min(step0 + p.steps_per_slice, steps_total);
+    const int n_st = max(step1 - step0, 0) / 2;                        // stages (two steps each; slices are even)
+    const uint8_t *w_base = seg.w + (long)pair * tiled_steps(p.K) * TILE_BYTES + (long)step0 * TILE_BYTES;
+    const uint8_t *a_base = reinterpret_cast<const uint8_t *>(p.a) + (long)step0 * 64;
+    const int rot = n_st > 0 ? (hb * 5) % n_st : 0;                   // workgroups of a K-slice start at different stages
+
+    if (wave8 == 8) {
+        // ---- the DMA wave ----
+        __builtin_amdgcn_s_setprio(3);
+        const int a_chunk = (lane & 3) ^ ((lane >> 4) & 3);
+        uint32_t a_voff[TILES];
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+            a_voff[t] = (uint32_t)((long)min(m0 + 16 * t + (lane >> 2), p.M - 1) * p.lda * 2 + 16 * a_chunk);
+        int fetch = rot;
+        auto issue_stage = [&](int slot_) {
+            uint8_t *st = lds + slot_ * STAGE;
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+                const uint8_t *tile = w_base + (long)(2 * fetch + kk) * TILE_BYTES;
+                const uint8_t *arow = a_base + (long)(2 * fetch + kk) * 64;
+#pragma unroll
+                for (int bp = 0; bp < 2; ++bp)
+                    __builtin_amdgcn_global_load_lds((gptr_t)(tile + (2 * blk + bp) * 1024 + lane * 16), (lptr_t)(st + (2 * kk + bp) * 1024), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr_t)(tile + TILE_W_BYTES + lane * 4), (lptr_t)(st + KG_W + kk * 256), 4, 0, 0);
+#pragma unroll
+                for (int t = 0; t < TILES; ++t)
+                    __builtin_amdgcn_global_load_lds((gptr_t)(arow + a_voff[t]), (lptr_t)(st + KG_W + KG_S + (kk * TILES + t) * 1024), 16, 0, 0);
+            }
+            fetch = fetch + 1 == n_st ? 0 : fetch + 1;
+        };
+#pragma unroll
+        for (int i = 0; i < SLOTS - 2; ++i)
+            if (i < n_st) issue_stage(i);
+        if (n_st > 0) {
+            gemm_wait_dma<PER>(min(SLOTS - 3, n_st - 1));
+            gemm_barrier();
+            int slot = 0;
+            auto back = [&](int k) { return slot >= k ? slot - k : slot + SLOTS - k; };
+            int i = 0;
+#pragma unroll 1
+            for (; i + SLOTS - 1 < n_st; i += 2) {
+                gemm_wait_vm<PER * (SLOTS - 5)>();
+                gemm_barrier();
+                issue_stage(back(2));
+                issue_stage(back(1));
+                slot = slot + 2 >= SLOTS ? slot + 2 - SLOTS : slot + 2;
+            }
+#pragma unroll 1
+            for (; i < n_st; i += 2) {
+                gemm_wait_dma<PER>(max(0, min(n_st - 1, i + SLOTS - 3) - (i + 2)));
+                gemm_barrier();
+                if (i + SLOTS - 2 < n_st) issue_stage(back(2));
+                if (i + SLOTS - 1 < n_st) issue_stage(back(1));
+                slot = slot + 2 >= SLOTS ? slot + 2 - SLOTS : slot + 2;
+            }
+        }
+        // the barriers of the epilogue: ring free, second group's sums in place, one per row tile
+#pragma unroll 1
+        for (int t = 0; t < 2 + TILES; ++t) gemm_barrier();
+        return;
+    }
+
+    const int kk = wave8 >> 2, hh = (wave8 >> 1) & 1, bp = wave8 & 1;
+    const uint32_t nib_mask = hh == 0 ? 0x00F000F0u : 0x000F000Fu;
+    const h2 nib_mul = hh == 0 ? h2{(half_t)0.0625f, (half_t)0.0625f} : h2{(half_t)1.0f, (half_t)1.0f};
+    const h2 nib_off = hh == 0 ? h2{(half_t)-72.0f, (half_t)-72.0f} : h2{(half_t)-1032.0f, (half_t)-1032.0f};
+    struct Raw { u32x4 wq, sc; };
+    auto load_ws = [&](const uint8_t *st, Raw &r) {
+        r.wq = *reinterpret_cast<const u32x4 *>(st + (2 * kk + bp) * 1024 + lane * 16);
+        r.sc = *reinterpret_cast<const u32x4 *>(st + KG_W + kk * 256 + g * 64 + (2 * blk + hh) * 16);
+    };
+    auto decode = [&](const Raw &r, h8 (&b)[2]) {
+        u32x4 v0, v1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t pr0 = j < 2 ? r.wq[j] : r.wq[j - 2] >> 8;       // rows (2j, 2j+1) of byte 2bp, codes + 8
+            const uint32_t pr1 = j < 2 ? r.wq[2 + j] : r.wq[j] >> 8;       // ... of byte 2bp+1
+            const h2 sc = as_h2(r.sc[j]);
+            v0[j] = as_u32(__builtin_elementwise_fma(as_h2((pr0 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
+            v1[j] = as_u32(__builtin_elementwise_fma(as_h2((pr1 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
+        }
+        b[0] = __builtin_bit_cast(h8, v0);
+        b[1] = __builtin_bit_cast(h8, v1);
+    };
+    auto load_a = [&](const uint8_t *st, h8 (&av)[TILES]) {
+        const uint8_t *at = st + KG_W + KG_S + kk * TILES * 1024;
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            const int r = 16 * t + c;
+            av[t] = *reinterpret_cast<const h8 *>(at + r * 64 + ((g ^ ((r >> 2) & 3)) << 4));
+        }
+    };
+    f4 acc[2][TILES];
+#pragma unroll
+    for (int o = 0; o < 2; ++o)
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) acc[o][t] = f4{0.f, 0.f, 0.f, 0.f};
+
+    if (n_st > 0) {
+        h8 bq[2];
+        int slot = 0;
+        gemm_barrier();
+        {
+            Raw r;
+            load_ws(lds, r);
+            decode(r, bq);
+        }
+        auto one_stage = [&]() {
+            const uint8_t *st = lds + slot * STAGE;
+            slot = slot == SLOTS - 1 ? 0 : slot + 1;
+            Raw r;
+            h8 av[TILES], bn[2];
+            load_a(st, av);
+            load_ws(lds + slot * STAGE, r);                    // (past the last stage: stale bytes, decoded and never used)
+#pragma unroll
+            for (int t = 0; t < TILES; ++t)
+#pragma unroll
+                for (int o = 0; o < 2; ++o) acc[o][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], bq[o], acc[o][t], 0, 0, 0);
+            decode(r, bn);
+            bq[0] = bn[0];
+            bq[1] = bn[1];
+        };
+        int i = 0;
+#pragma unroll 1
+        for (; i + 1 < n_st; i += 2) {
+            gemm_barrier();
+            one_stage();
+            one_stage();
+        }
+        if (i < n_st) {
+            gemm_barrier();
+            one_stage();
+        }
+    }
+
+    // ---- group 0 + group 1 through LDS, then the slab one row tile at a time ----
+    gemm_barrier();                                            // every wave has left the loop: the ring is free
+    if (kk == 1) {
+        uint8_t *dst = lds + (wave8 - 4) * (TILES * 2 * 1024) + lane * 16;
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+            for (int o = 0; o < 2; ++o) *reinterpret_cast<f4 *>(dst + (t * 2 + o) * 1024) = acc[o][t];
+    }
+    gemm_barrier();
+    if (kk == 1) {
+#pragma unroll 1
+        for (int t = 0; t < TILES; ++t) gemm_barrier();
+        return;
+    }
+    {
+        const uint8_t *src = lds + wave8 * (TILES * 2 * 1024) + lane * 16;
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+            for (int o = 0; o < 2; ++o) acc[o][t] += *reinterpret_cast<const f4 *>(src + (t * 2 + o) * 1024);
+    }
+    constexpr int OP = S::OP;
+    float *slab = p.partial + (long)slice * p.M * p.n_total;
+    const int o_row = tid >> 4, o_lane = tid & 15;            // tid < 256 here
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        float *otile = reinterpret_cast<float *>(lds + S::RED + (t & 1) * S::OTILE);
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            *reinterpret_cast<f2 *>(&otile[(4 * g + r) * OP + 64 * hh + 4 * c + 2 * bp]) = f2{acc[0][t][r], acc[1][t][r]};
+        gemm_barrier();
+        const int m = m0 + 16 * t + o_row;
+        if (m < p.M && m < m0 + p.block_rows) {
+            float *dst = slab + (long)m * p.n_total + seg.col0 + col0;
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const int cq = 64 * q + 4 * o_lane;
+                *reinterpret_cast<f4 *>(dst + cq) = *reinterpret_cast<const f4 *>(otile + o_row * OP + cq);
+            }
+        }
+    }
+}
+
 void gemm_fill_plan(MatmulParams &p) {
     int unit0 = 0, col0 = 0;
     for (int i = 0; i < p.nseg; ++i) {
@@ -592,6 +819,36 @@ void gemm_fill_plan(MatmulParams &p) {
     p.units_pad = (unit0 + 7) / 8 * 8;
     p.n_total = col0;
     p.block_rows = GEMM_BM;
+    p.kgroups = 0;
+    // Tiled weights, 17 .. 128 rows, K a multiple of 64: 128-column blocks with two K-groups a workgroup (q40_gemm_kg_kernel)
+    // where they fill at least two thirds of the compute units in one round - half the K-slices, or fewer, of the 256-column
+    // units below for the same number of workgroups.  Narrow matrices (at most 32 blocks: wo, w2) at any such row count, and
+    // with two 64-row blocks per column block where K is short (wo at 65 .. 128 rows); wide ones (wq|wk|wv, w1|w3) above
+    // 64 rows only (below, the launch loses more than its consumer gains).  Measured at 100 rows, launch + consumer: wo 15.8
+    // against 17.5 us, w2 24.7 against 26.9, w1|w3 39.7 against 40.9; a decode step at 100 branches 4.30 against 4.43 ms.
+    if (p.tiled && p.M <= 128 && p.K % 64 == 0) {
+        int blocks = 0;
+        for (int i = 0; i < p.nseg; ++i) blocks += p.seg[i].N / 128;
+        const bool narrow = blocks <= 32;
+        const int mblocks = (narrow && p.M > 64 && p.K <= 4096) ? 2 : 1;
+        int ks = 256 / (blocks * mblocks);
+        int cap = GEMM_KSCAP / p.M;
+        if (cap > SMH_MAX_KSPLIT) cap = SMH_MAX_KSPLIT;
+        if (ks > cap) ks = cap;
+        const int steps = p.K / 32;
+        if (ks > steps / 8) ks = steps / 8;                    // at least four stages (of two steps) a slice
+        if (ks >= 1 && (narrow || p.M > 64) && (long)blocks * mblocks * ks >= 170) {
+            p.kgroups = 2;
+            p.mblocks = mblocks;
+            p.block_rows = mblocks == 2 ? 64 : GEMM_BM;
+            p.chunk = 0;
+            int sps = (steps + ks - 1) / ks;
+            sps += sps & 1;                                    // a stage of the ring is two steps
+            p.steps_per_slice = sps;
+            p.ksplit = (steps + sps - 1) / sps;
+            return;
+        }
+    }
     // 65 .. 128 rows of a matrix with few column units and a short K (wo at 100 branches): two 64-row blocks per unit take
     // half as many K-slices to fill the GPU, so half the slab bytes are written here and read by the consumer.  The blocks
     // of a unit read the same weights at the same time in the same XCD.  (Measured at 100 rows: wo and the RMSNorm behind
@@ -687,7 +944,31 @@ static int gemm_launch_layout(const MatmulParams &p, hipStream_t stream) {
     return launch_status();
 }
 
+typedef void (*gemm_kg_kernel_t)(MatmulParams);
+static int gemm_kg_launch(const MatmulParams &p, hipStream_t stream) {
+    static const gemm_kg_kernel_t kern[9] = {nullptr, nullptr, q40_gemm_kg_kernel<2>, q40_gemm_kg_kernel<3>, q40_gemm_kg_kernel<4>, q40_gemm_kg_kernel<5>,
+                                             q40_gemm_kg_kernel<6>, q40_gemm_kg_kernel<7>, q40_gemm_kg_kernel<8>};
+    static const int lds_bytes[9] = {0, 0, KgShape<2>::LDS, KgShape<3>::LDS, KgShape<4>::LDS, KgShape<5>::LDS, KgShape<6>::LDS, KgShape<7>::LDS, KgShape<8>::LDS};
+    static const hipError_t lds_ok = [] {
+        hipError_t e = hipSuccess;
+        for (int t = 2; t <= 8 && e == hipSuccess; ++t)
+            e = hipFuncSetAttribute((const void *)kern[t], hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes[t]);
+        return e;
+    }();
+    if (lds_ok != hipSuccess) {
+        set_error("q40 gemm: the kernels' LDS could not be reserved: %s", hipGetErrorString(lds_ok));
+        return (int)lds_ok;
+    }
+    SMH_REQUIRE((long)p.M * p.lda * 2 < (1L << 32), "q40 gemm: M x lda = %d x %ld exceeds the 32-bit lane offsets of A", p.M, p.lda);
+    int tiles = p.mblocks > 1 ? p.block_rows / 16 : (p.M + 15) / 16;
+    if (tiles < 2) tiles = 2;
+    dim3 grid((unsigned)(2L * p.units_pad * p.mblocks * p.ksplit));
+    hipLaunchKernelGGL(kern[tiles], grid, dim3(576), lds_bytes[tiles], stream, p);
+    return launch_status();
+}
+
 int gemm_launch(const MatmulParams &p, hipStream_t stream) {
+    if (p.kgroups == 2 && p.tiled) return gemm_kg_launch(p, stream);
     return p.tiled ? gemm_launch_layout<true>(p, stream) : gemm_launch_layout<false>(p, stream);
 }
 

@@ -58,6 +58,7 @@ struct MatmulParams {
     int units, units_pad;    // column units over all segments (GEMV: padded to a multiple of 8)
     int mblocks, block_rows; // GEMM: row blocks and the rows of one (128, or 64 where two blocks of a narrow matrix halve its K-slices)
     int ksplit, steps_per_slice;
+    int kgroups;             // GEMM, 2: q40_gemm_kg_kernel (128-column blocks, two K-groups a workgroup)
     int chunk;               // GEMM, > 0: range cut - workgroup j takes steps [j * chunk, (j + 1) * chunk) of the column units laid end to end
     int epilogue, direct;
     int tiled;               // the segments' weights are in the tiled layout

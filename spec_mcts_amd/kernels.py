@@ -104,14 +104,15 @@ def matmul_q40(a: torch.Tensor, b_w: torch.Tensor, b_s: torch.Tensor, b_shape: S
     return c
 
 
-def matmul_plan(M: int, K: int, ns: Sequence[int]) -> int:
-    """Number of K slices the matmul kernels use for a [M,K] x [K, sum(ns)] product."""
+def matmul_plan(M: int, K: int, ns: Sequence[int], tiled: bool = False) -> int:
+    """Number of K slices the matmul kernels use for a [M,K] x [K, sum(ns)] product on checkpoint-layout or on tiled
+    weights (the same up to 16 rows)."""
     import ctypes
     lib = _lib.load()
     arr = (ctypes.c_int * len(ns))(*[int(n) for n in ns])
-    ks = lib.smh_q40_matmul_plan(int(M), int(K), len(ns), arr)
+    ks = (lib.smh_q40_matmul_plan_tiled if tiled else lib.smh_q40_matmul_plan)(int(M), int(K), len(ns), arr)
     if ks < 1:
-        check(ks, "smh_q40_matmul_plan")
+        check(ks, "smh_q40_matmul_plan_tiled" if tiled else "smh_q40_matmul_plan")
     return ks
 
 
@@ -156,7 +157,7 @@ def matmul_q40_partial(a: torch.Tensor, linears, out: Optional[torch.Tensor] = N
     if isinstance(linears[0], TiledQ40):
         assert all(isinstance(t, TiledQ40) and t.K == Kd for t in linears), "tiled and checkpoint-layout weights cannot share a launch"
         ns = [t.N for t in linears]
-        ks = matmul_plan(M, Kd, ns)
+        ks = matmul_plan(M, Kd, ns, tiled=True)
         n_total = sum(ns)
         need = ks * M * n_total
         if out is None:
@@ -200,7 +201,7 @@ def matmul_q40_partial_silu(gu: PartialProduct, linears, out: Optional[torch.Ten
     assert M <= SILU_IN_MAX_M and gu.buf.dtype == torch.float32
     assert all(isinstance(t, TiledQ40) and t.K == Kd for t in linears), "tiled weights with K = half the gate|up columns"
     ns = [t.N for t in linears]
-    ks = matmul_plan(M, Kd, ns)
+    ks = matmul_plan(M, Kd, ns, tiled=True)
     n_total = sum(ns)
     need = ks * M * n_total
     if out is None:
@@ -250,7 +251,7 @@ def matmul_q40_partial_norm(h: torch.Tensor, sums: torch.Tensor, weight: torch.T
     assert weight.numel() == Kd and weight.dtype == torch.float16
     assert all(isinstance(t, TiledQ40) and t.K == Kd for t in linears), "tiled weights with K = the width of h"
     ns = [t.N for t in linears]
-    ks = matmul_plan(M, Kd, ns)
+    ks = matmul_plan(M, Kd, ns, tiled=True)
     n_total = sum(ns)
     need = ks * M * n_total
     if out is None:

@@ -61,12 +61,22 @@ def test_matmul_plans_fit_the_workspace_the_library_asks_for():
         for ns in widths:
             n = (ctypes.c_int * len(ns))(*ns)
             for M in (1, 2, 10, 16, 17, 64, 100, 128):
-                ks = lib.smh_q40_matmul_plan(M, K, len(ns), n)
-                assert 1 <= ks <= 16, (M, K, ns, ks)
-                assert ks * M * sum(ns) * 4 <= lib.smh_q40_matmul_workspace_bytes(M, sum(ns)), (M, K, ns, ks)
-    # the two plans the GPU tests and the design notes name
-    assert lib.smh_q40_matmul_plan(100, 4096, 2, (ctypes.c_int * 2)(11008, 11008)) == 4      # range cut: 256 runs of 43 steps
-    assert lib.smh_q40_matmul_plan(100, 4096, 3, (ctypes.c_int * 3)(4096, 4096, 4096)) == 5
+                for plan in (lib.smh_q40_matmul_plan, lib.smh_q40_matmul_plan_tiled):
+                    ks = plan(M, K, len(ns), n)
+                    assert 1 <= ks <= 16, (M, K, ns, ks)
+                    assert ks * M * sum(ns) * 4 <= lib.smh_q40_matmul_workspace_bytes(M, sum(ns)), (M, K, ns, ks)
+                if M <= 16:
+                    assert lib.smh_q40_matmul_plan(M, K, len(ns), n) == lib.smh_q40_matmul_plan_tiled(M, K, len(ns), n)
+    # the plans the GPU tests and the design notes name: checkpoint layout ...
+    three, two, one = (ctypes.c_int * 3)(4096, 4096, 4096), (ctypes.c_int * 2)(11008, 11008), (ctypes.c_int * 1)(4096)
+    assert lib.smh_q40_matmul_plan(100, 4096, 2, two) == 4      # range cut: 256 runs of 43 steps
+    assert lib.smh_q40_matmul_plan(100, 4096, 3, three) == 5
+    # ... and tiled weights at 100 rows: 128-column blocks with two K-groups a workgroup
+    assert lib.smh_q40_matmul_plan_tiled(100, 4096, 1, one) == 4         # wo: 32 blocks x 2 row blocks x 4 slices
+    assert lib.smh_q40_matmul_plan_tiled(100, 11008, 1, one) == 8        # w2: 32 blocks x 8 slices
+    assert lib.smh_q40_matmul_plan_tiled(100, 4096, 3, three) == 2       # wq|wk|wv: 96 blocks x 2 slices
+    assert lib.smh_q40_matmul_plan_tiled(100, 4096, 2, two) == 1         # w1|w3: 172 blocks, K uncut
+    assert lib.smh_q40_matmul_plan_tiled(32, 4096, 2, two) == 4          # wide and at most 64 rows: the 256-column units' plan
 
 
 def test_host_quantiser_matches_oracle():
