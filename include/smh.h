@@ -115,6 +115,15 @@ int smh_gq40_dequant(const void *packed, const void *scale, void *out, long bloc
  */
 int smh_q40_matmul_plan(int M, int K, int nseg, const int *n);
 int smh_q40_matmul_plan_tiled(int M, int K, int nseg, const int *n);
+/* smh_q40_matmul_tiled_swiglu: out[M, n_half] = fp16(silu(fp16(a . gate))) * fp16(a . up) for tiled gate and up weights
+ * [K, n_half] - `F.silu(self.w1(x)) * self.w3(x)` of FeedForward.forward (hf_model_q40_kv_shared.py:434) in ONE launch, with
+ * the roundings of smh_q40_matmul_partial_tiled + smh_partial_silu_mul (every linear rounded to fp16 first) and no slab
+ * in between.  17 <= M <= 128, K a multiple of 64, n_half a multiple of 128 and at most 16384 (all of K in one workgroup,
+ * one workgroup per compute unit).  smh_q40_swiglu_fits: 1 when the shape is supported AND wide enough (n_half >= 8192) for
+ * this to be the faster way; else use the two launches. */
+int smh_q40_swiglu_fits(int M, int K, int n_half);
+int smh_q40_matmul_tiled_swiglu(const void *a, int M, int K, long lda, const void *tiled_gate, const void *tiled_up, int n_half,
+                                void *out, long ldo, smh_stream_t stream);
 int smh_q40_matmul_partial(const void *a, int M, int K, long lda, int nseg, const void *const *w,
                            const void *const *s, const int *n, void *partial, size_t partial_bytes,
                            smh_stream_t stream);

@@ -30,6 +30,8 @@ SIGNATURES = {
     "smh_q40_matmul": (c_int, [_P, c_int, c_int, c_long, _P, _P, c_int, _P, c_long, c_int, _P, c_long, _P, c_size_t, _P]),
     "smh_q40_matmul_plan": (c_int, [c_int, c_int, c_int, _P]),
     "smh_q40_matmul_plan_tiled": (c_int, [c_int, c_int, c_int, _P]),
+    "smh_q40_swiglu_fits": (c_int, [c_int, c_int, c_int]),
+    "smh_q40_matmul_tiled_swiglu": (c_int, [_P, c_int, c_int, c_long, _P, _P, c_int, _P, c_long, _P]),
     "smh_q40_matmul_partial": (c_int, [_P, c_int, c_int, c_long, c_int, _P, _P, _P, _P, c_size_t, _P]),
     "smh_q40_tiled_bytes": (c_size_t, [c_int, c_int]),
     "smh_q40_tile": (c_int, [_P, _P, c_int, c_int, _P, c_size_t, _P]),

@@ -252,6 +252,25 @@ extern "C" int smh_q40_matmul_plan(int M, int K, int nseg, const int *n) {
     return st < 0 ? st : p.ksplit;
 }
 
+extern "C" int smh_q40_swiglu_fits(int M, int K, int n_half) { return smh::gemm_swiglu_fits(M, K, n_half, true) ? 1 : 0; }
+
+extern "C" int smh_q40_matmul_tiled_swiglu(const void *a, int M, int K, long lda, const void *tiled_gate, const void *tiled_up, int n_half,
+                                           void *out, long ldo, smh_stream_t stream) {
+    const char *who = "smh_q40_matmul_tiled_swiglu";
+    SMH_REQUIRE(gemm_swiglu_fits(M, K, n_half, false),
+                "%s: M=%d (17 .. 128) K=%d (a multiple of 64) n_half=%d (a multiple of 128, at most 16384)", who, M, K, n_half);
+    SMH_REQUIRE(a && tiled_gate && tiled_up && out, "%s: null pointer", who);
+    SMH_REQUIRE(lda >= K && lda % 8 == 0 && ldo >= n_half && ldo % 2 == 0, "%s: lda=%ld (>= K, a multiple of 8) ldo=%ld (>= n_half, even)", who, lda, ldo);
+    SMH_REQUIRE(((uintptr_t)a & 15) == 0 && ((uintptr_t)out & 3) == 0 && ((uintptr_t)tiled_gate & 127) == 0 && ((uintptr_t)tiled_up & 127) == 0,
+                "%s: misaligned pointer", who);
+    MatmulParams p = MatmulParams{};
+    p.a = (const half_t *)a; p.M = M; p.K = K; p.lda = lda; p.nseg = 2;
+    p.seg[0].w = (const uint8_t *)tiled_gate; p.seg[0].N = n_half;
+    p.seg[1].w = (const uint8_t *)tiled_up; p.seg[1].N = n_half;
+    p.c = (half_t *)out; p.ldc = ldo; p.tiled = 1;
+    return gemm_swiglu_launch(p, (hipStream_t)stream);
+}
+
 extern "C" int smh_q40_matmul_plan_tiled(int M, int K, int nseg, const int *n) {
     MatmulParams p;
     if (M <= 0) return 1;

@@ -807,6 +807,229 @@ __global__ __launch_bounds__(576, 1) void q40_gemm_kg_kernel(MatmulParams p) {
     }
 }
 
+// ---- SwiGLU inside the launch of w1|w3 (tiled weights, 17 .. 128 rows, all of K in one workgroup) -----------------------
+// q40_gemm_kg_kernel with the roles of a workgroup's waves changed: instead of the two pieces of one 128-column block, a
+// workgroup takes piece bp of block j of the GATE weight and the same piece of the UP weight (64 columns each, the same
+// columns), so its wave (kk, hh, gu) holds, after the K-groups are added, gate or up for exactly the columns its neighbour
+// holds the other for.  The epilogue forms fp16(silu(fp16(gate))) * fp16(up) with the roundings of partial_silu_mul_kernel
+// and stores the activations of w2: no slab leaves the launch and the SiLU launch is gone.
+template <int TILES> struct SwigluShape {
+    static constexpr int SC = 1024;                                  // scales: [group kk][gate | up] x 256
+    static constexpr int STAGE = KG_W + SC + 2 * TILES * 1024;
+    static constexpr int SLOTS = GEMM_DMA_WAVE_SLOTS;
+    static constexpr int LDS = SLOTS * STAGE;
+    static constexpr int PER = 2 * (4 + TILES);
+    static constexpr int RED = 4 * TILES * 2 * 1024;
+    static constexpr int OP = 64 + 4;
+    static constexpr int OTILE = 2 * 16 * OP * 4;
+    static_assert(RED + 2 * OTILE <= LDS, "the sums of the second group and two output tiles must fit in the ring");
+    static_assert(PER * (SLOTS - 5) <= 63 && LDS <= 160 * 1024, "ring");
+};
+
+template <int TILES>
+__global__ __launch_bounds__(576, 1) void q40_gemm_swiglu_kernel(MatmulParams p) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t lds[];
+    typedef SwigluShape<TILES> S;
+    constexpr int SLOTS = S::SLOTS, PER = S::PER, STAGE = S::STAGE;
+    const int tid = threadIdx.x;
+    const int wave8 = __builtin_amdgcn_readfirstlane(tid >> 6);       // 0..7 multiply, 8 issues the DMA
+    const int lane = tid & 63, c = lane & 15, g = lane >> 4;
+    // blockIdx -> (128-column block j of the gate and of the up weight, piece bp of that block)
+    const int hb = blockIdx.x;
+    const int blockj = hb >> 1, bp = hb & 1;
+    const int pair = blockj >> 1, blk = blockj & 1;
+    const int n_half = p.seg[0].N;
+    if (128 * blockj >= n_half) return;
+    constexpr int m0 = 0;
+    const int n_st = p.K / 64;                                         // stages (two steps each), all of K
+    const uint8_t *w_gate = p.seg[0].w + (long)pair * tiled_steps(p.K) * TILE_BYTES;
+    const uint8_t *w_up = p.seg[1].w + (long)pair * tiled_steps(p.K) * TILE_BYTES;
+    const uint8_t *a_base = reinterpret_cast<const uint8_t *>(p.a);
+    const int rot = n_st > 0 ? (hb * 5) % n_st : 0;                   // workgroups of a K-slice start at different stages
+
+    if (wave8 == 8) {
+        // ---- the DMA wave ----
+        __builtin_amdgcn_s_setprio(3);
+        const int a_chunk = (lane & 3) ^ ((lane >> 4) & 3);
+        uint32_t a_voff[TILES];
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+            a_voff[t] = (uint32_t)((long)min(m0 + 16 * t + (lane >> 2), p.M - 1) * p.lda * 2 + 16 * a_chunk);
+        int fetch = rot;
+        auto issue_stage = [&](int slot_) {
+            uint8_t *st = lds + slot_ * STAGE;
+#pragma unroll
+            for (int kk = 0; kk < 2; ++kk) {
+                const long off = (long)(2 * fetch + kk) * TILE_BYTES;
+                const uint8_t *arow = a_base + (long)(2 * fetch + kk) * 64;
+#pragma unroll
+                for (int gu = 0; gu < 2; ++gu) {
+                    const uint8_t *tile = (gu == 0 ? w_gate : w_up) + off;
+                    __builtin_amdgcn_global_load_lds((gptr_t)(tile + (2 * blk + bp) * 1024 + lane * 16), (lptr_t)(st + (2 * kk + gu) * 1024), 16, 0, 0);
+                    __builtin_amdgcn_global_load_lds((gptr_t)(tile + TILE_W_BYTES + lane * 4), (lptr_t)(st + KG_W + (2 * kk + gu) * 256), 4, 0, 0);
+                }
+#pragma unroll
+                for (int t = 0; t < TILES; ++t)
+                    __builtin_amdgcn_global_load_lds((gptr_t)(arow + a_voff[t]), (lptr_t)(st + KG_W + S::SC + (kk * TILES + t) * 1024), 16, 0, 0);
+            }
+            fetch = fetch + 1 == n_st ? 0 : fetch + 1;
+        };
+#pragma unroll
+        for (int i = 0; i < SLOTS - 2; ++i)
+            if (i < n_st) issue_stage(i);
+        if (n_st > 0) {
+            gemm_wait_dma<PER>(min(SLOTS - 3, n_st - 1));
+            gemm_barrier();
+            int slot = 0;
+            auto back = [&](int k) { return slot >= k ? slot - k : slot + SLOTS - k; };
+            int i = 0;
+#pragma unroll 1
+            for (; i + SLOTS - 1 < n_st; i += 2) {
+                gemm_wait_vm<PER * (SLOTS - 5)>();
+                gemm_barrier();
+                issue_stage(back(2));
+                issue_stage(back(1));
+                slot = slot + 2 >= SLOTS ? slot + 2 - SLOTS : slot + 2;
+            }
+#pragma unroll 1
+            for (; i < n_st; i += 2) {
+                gemm_wait_dma<PER>(max(0, min(n_st - 1, i + SLOTS - 3) - (i + 2)));
+                gemm_barrier();
+                if (i + SLOTS - 2 < n_st) issue_stage(back(2));
+                if (i + SLOTS - 1 < n_st) issue_stage(back(1));
+                slot = slot + 2 >= SLOTS ? slot + 2 - SLOTS : slot + 2;
+            }
+        }
+        // the barriers of the epilogue: ring free, second group's sums in place, one per row tile
+#pragma unroll 1
+        for (int t = 0; t < 2 + TILES; ++t) gemm_barrier();
+        return;
+    }
+
+    const int kk = wave8 >> 2, hh = (wave8 >> 1) & 1, gu = wave8 & 1;       // K-group, nibble, gate (0) or up (1)
+    const uint32_t nib_mask = hh == 0 ? 0x00F000F0u : 0x000F000Fu;
+    const h2 nib_mul = hh == 0 ? h2{(half_t)0.0625f, (half_t)0.0625f} : h2{(half_t)1.0f, (half_t)1.0f};
+    const h2 nib_off = hh == 0 ? h2{(half_t)-72.0f, (half_t)-72.0f} : h2{(half_t)-1032.0f, (half_t)-1032.0f};
+    struct Raw { u32x4 wq, sc; };
+    auto load_ws = [&](const uint8_t *st, Raw &r) {
+        r.wq = *reinterpret_cast<const u32x4 *>(st + (2 * kk + gu) * 1024 + lane * 16);
+        r.sc = *reinterpret_cast<const u32x4 *>(st + KG_W + (2 * kk + gu) * 256 + g * 64 + (2 * blk + hh) * 16);
+    };
+    auto decode = [&](const Raw &r, h8 (&b)[2]) {
+        u32x4 v0, v1;
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+            const uint32_t pr0 = j < 2 ? r.wq[j] : r.wq[j - 2] >> 8;       // rows (2j, 2j+1) of byte 2bp, codes + 8
+            const uint32_t pr1 = j < 2 ? r.wq[2 + j] : r.wq[j] >> 8;       // ... of byte 2bp+1
+            const h2 sc = as_h2(r.sc[j]);
+            v0[j] = as_u32(__builtin_elementwise_fma(as_h2((pr0 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
+            v1[j] = as_u32(__builtin_elementwise_fma(as_h2((pr1 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
+        }
+        b[0] = __builtin_bit_cast(h8, v0);
+        b[1] = __builtin_bit_cast(h8, v1);
+    };
+    auto load_a = [&](const uint8_t *st, h8 (&av)[TILES]) {
+        const uint8_t *at = st + KG_W + S::SC + kk * TILES * 1024;
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) {
+            const int r = 16 * t + c;
+            av[t] = *reinterpret_cast<const h8 *>(at + r * 64 + ((g ^ ((r >> 2) & 3)) << 4));
+        }
+    };
+    f4 acc[2][TILES];
+#pragma unroll
+    for (int o = 0; o < 2; ++o)
+#pragma unroll
+        for (int t = 0; t < TILES; ++t) acc[o][t] = f4{0.f, 0.f, 0.f, 0.f};
+
+    if (n_st > 0) {
+        h8 bq[2];
+        int slot = 0;
+        gemm_barrier();
+        {
+            Raw r;
+            load_ws(lds, r);
+            decode(r, bq);
+        }
+        auto one_stage = [&]() {
+            const uint8_t *st = lds + slot * STAGE;
+            slot = slot == SLOTS - 1 ? 0 : slot + 1;
+            Raw r;
+            h8 av[TILES], bn[2];
+            load_a(st, av);
+            load_ws(lds + slot * STAGE, r);                    // (past the last stage: stale bytes, decoded and never used)
+#pragma unroll
+            for (int t = 0; t < TILES; ++t)
+#pragma unroll
+                for (int o = 0; o < 2; ++o) acc[o][t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(av[t], bq[o], acc[o][t], 0, 0, 0);
+            decode(r, bn);
+            bq[0] = bn[0];
+            bq[1] = bn[1];
+        };
+        int i = 0;
+#pragma unroll 1
+        for (; i + 1 < n_st; i += 2) {
+            gemm_barrier();
+            one_stage();
+            one_stage();
+        }
+        if (i < n_st) {
+            gemm_barrier();
+            one_stage();
+        }
+    }
+
+    // ---- group 0 + group 1 through LDS, then the slab one row tile at a time ----
+    gemm_barrier();                                            // every wave has left the loop: the ring is free
+    if (kk == 1) {
+        uint8_t *dst = lds + (wave8 - 4) * (TILES * 2 * 1024) + lane * 16;
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+            for (int o = 0; o < 2; ++o) *reinterpret_cast<f4 *>(dst + (t * 2 + o) * 1024) = acc[o][t];
+    }
+    gemm_barrier();
+    if (kk == 1) {
+#pragma unroll 1
+        for (int t = 0; t < TILES; ++t) gemm_barrier();
+        return;
+    }
+    {
+        const uint8_t *src = lds + wave8 * (TILES * 2 * 1024) + lane * 16;
+#pragma unroll
+        for (int t = 0; t < TILES; ++t)
+#pragma unroll
+            for (int o = 0; o < 2; ++o) acc[o][t] += *reinterpret_cast<const f4 *>(src + (t * 2 + o) * 1024);
+    }
+    // rows of 64 columns: local column 32 hh + 2 c + o is column 128 blockj + 64 hh + 4 c + 2 bp + o of the weights
+    constexpr int OP = S::OP;
+    const int o_row = tid >> 4, o_lane = tid & 15;            // tid < 256 here
+    const int st_hh = o_lane >> 3, st_c = 2 * (o_lane & 7);   // this thread's four local columns 4 o_lane .. + 3 when storing
+#pragma unroll
+    for (int t = 0; t < TILES; ++t) {
+        float *otile = reinterpret_cast<float *>(lds + S::RED + (t & 1) * S::OTILE);      // [gate | up][16][OP]
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            *reinterpret_cast<f2 *>(&otile[gu * 16 * OP + (4 * g + r) * OP + 32 * hh + 2 * c]) = f2{acc[0][t][r], acc[1][t][r]};
+        gemm_barrier();
+        const int m = 16 * t + o_row;
+        if (m < p.M) {
+            const f4 gv = *reinterpret_cast<const f4 *>(otile + o_row * OP + 4 * o_lane);
+            const f4 uv = *reinterpret_cast<const f4 *>(otile + 16 * OP + o_row * OP + 4 * o_lane);
+            half_t ov[4];
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {                      // the roundings of partial_silu_mul_kernel
+                const float gf = (float)(half_t)gv[e];
+                const half_t sl = (half_t)(gf / (1.0f + expf(-gf)));
+                ov[e] = sl * (half_t)uv[e];
+            }
+            half_t *dst = p.c + (long)m * p.ldc + 128 * blockj + 64 * st_hh + 4 * st_c + 2 * bp;
+            *reinterpret_cast<h2 *>(dst) = h2{ov[0], ov[1]};
+            *reinterpret_cast<h2 *>(dst + 4) = h2{ov[2], ov[3]};
+        }
+    }
+}
+
 void gemm_fill_plan(MatmulParams &p) {
     int unit0 = 0, col0 = 0;
     for (int i = 0; i < p.nseg; ++i) {
@@ -824,9 +1047,11 @@ void gemm_fill_plan(MatmulParams &p) {
     // where they fill at least two thirds of the compute units in one round - half the K-slices, or fewer, of the 256-column
     // units below for the same number of workgroups.  Narrow matrices (at most 32 blocks: wo, w2) at any such row count, and
     // with two 64-row blocks per column block where K is short (wo at 65 .. 128 rows); wide ones (wq|wk|wv, w1|w3) above
-    // 64 rows only (below, the launch loses more than its consumer gains).  Measured at 100 rows, launch + consumer: wo 15.8
-    // against 17.5 us, w2 24.7 against 26.9, w1|w3 39.7 against 40.9; a decode step at 100 branches 4.30 against 4.43 ms.
-    if (p.tiled && p.M <= 128 && p.K % 64 == 0) {
+    // 64 rows only (below, the launch loses more than its consumer gains); K up to 16384 (a row of A is staged for 128 columns
+    // instead of 256, which makes the loop ~12 % slower per step: with K = 28672 that outweighs the slabs).  Measured at 100
+    // rows, launch + consumer: wo 15.8 against 17.5 us, w2 24.7 against 26.9, w1|w3 39.7 against 40.9; a decode step at 100
+    // branches 4.06 against 4.29 ms.
+    if (p.tiled && p.M <= 128 && p.K % 64 == 0 && p.K <= 16384) {
         int blocks = 0;
         for (int i = 0; i < p.nseg; ++i) blocks += p.seg[i].N / 128;
         const bool narrow = blocks <= 32;
@@ -964,6 +1189,40 @@ static int gemm_kg_launch(const MatmulParams &p, hipStream_t stream) {
     if (tiles < 2) tiles = 2;
     dim3 grid((unsigned)(2L * p.units_pad * p.mblocks * p.ksplit));
     hipLaunchKernelGGL(kern[tiles], grid, dim3(576), lds_bytes[tiles], stream, p);
+    return launch_status();
+}
+
+// Can w1|w3 of these dimensions run with SwiGLU inside the launch, and is it the faster way?  17 .. 128 rows, K a multiple of
+// 64, two weights of n_half columns (a multiple of 128) whose 2 * n_half / 128 workgroups fit the compute units in one round;
+// `worth_it`: and fill at least half of them (narrower weights are faster as two kernels with a K-split), above 32 rows
+// (measured at the 7B shape, w1|w3 + SiLU: 38.1 against 44.9 us at 100 rows, 29.1 against 31.5 at 64, level at 32).
+bool gemm_swiglu_fits(int M, int K, int n_half, bool worth_it) {
+    if (M <= SMH_GEMV_MAX_M || M > 128 || K <= 0 || K % 64 != 0 || n_half <= 0 || n_half % 128 != 0) return false;
+    const int wgs = 2 * (n_half / 128);
+    return wgs <= 256 && (!worth_it || (wgs >= 128 && M > 32));
+}
+
+typedef void (*gemm_swiglu_kernel_t)(MatmulParams);
+int gemm_swiglu_launch(const MatmulParams &p, hipStream_t stream) {
+    static const gemm_swiglu_kernel_t kern[9] = {nullptr, nullptr, q40_gemm_swiglu_kernel<2>, q40_gemm_swiglu_kernel<3>, q40_gemm_swiglu_kernel<4>,
+                                                 q40_gemm_swiglu_kernel<5>, q40_gemm_swiglu_kernel<6>, q40_gemm_swiglu_kernel<7>,
+                                                 q40_gemm_swiglu_kernel<8>};
+    static const int lds_bytes[9] = {0, 0, SwigluShape<2>::LDS, SwigluShape<3>::LDS, SwigluShape<4>::LDS, SwigluShape<5>::LDS, SwigluShape<6>::LDS,
+                                     SwigluShape<7>::LDS, SwigluShape<8>::LDS};
+    static const hipError_t lds_ok = [] {
+        hipError_t e = hipSuccess;
+        for (int t = 2; t <= 8 && e == hipSuccess; ++t)
+            e = hipFuncSetAttribute((const void *)kern[t], hipFuncAttributeMaxDynamicSharedMemorySize, lds_bytes[t]);
+        return e;
+    }();
+    if (lds_ok != hipSuccess) {
+        set_error("q40 gemm: the kernels' LDS could not be reserved: %s", hipGetErrorString(lds_ok));
+        return (int)lds_ok;
+    }
+    SMH_REQUIRE((long)p.M * p.lda * 2 < (1L << 32), "q40 gemm: M x lda = %d x %ld exceeds the 32-bit lane offsets of A", p.M, p.lda);
+    int tiles = (p.M + 15) / 16;
+    if (tiles < 2) tiles = 2;
+    hipLaunchKernelGGL(kern[tiles], dim3((unsigned)(2 * (p.seg[0].N / 128))), dim3(576), lds_bytes[tiles], stream, p);
     return launch_status();
 }
 

@@ -86,5 +86,7 @@ int gemv_launch(const MatmulParams &p, hipStream_t stream);
 bool gemv_norm_in_fits(const MatmulParams &p);     // after gemv_fill_plan: can RMSNorm be made inside the launch
 void gemm_fill_plan(MatmulParams &p);
 int gemm_launch(const MatmulParams &p, hipStream_t stream);
+bool gemm_swiglu_fits(int M, int K, int n_half, bool worth_it);
+int gemm_swiglu_launch(const MatmulParams &p, hipStream_t stream);     // seg[0] = gate, seg[1] = up (tiled), c / ldc = the activations
 
 }  // namespace smh

@@ -60,7 +60,7 @@ class GraphDecoder:
 
     def _key(self):
         m = self.model
-        return (self.prompt_len, self.B, m.fused, m.tiled_weights, m.silu_in_matmul, m.norm_in_matmul, m.norm_in_max_rows,
+        return (self.prompt_len, self.B, m.fused, m.tiled_weights, m.silu_in_matmul, m.swiglu_in_matmul, m.norm_in_matmul, m.norm_in_max_rows,
                 m.attn_from_qkv, m.attn_single_launch, m.per_branch_kv, m._forked)
 
     def _reset_state(self):
@@ -166,7 +166,7 @@ class BucketedForward:
 
     def _config(self):
         m = self.model
-        return (self.prompt_len, m.fused, m.tiled_weights, m.silu_in_matmul, m.norm_in_matmul, m.norm_in_max_rows, m.attn_from_qkv,
+        return (self.prompt_len, m.fused, m.tiled_weights, m.silu_in_matmul, m.swiglu_in_matmul, m.norm_in_matmul, m.norm_in_max_rows, m.attn_from_qkv,
                 m.attn_single_launch, m.per_branch_kv)
 
     def begin(self):

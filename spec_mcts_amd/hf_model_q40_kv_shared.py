@@ -306,6 +306,7 @@ class Transformer(nn.Module):
         self.per_branch_kv = False    # True: hf_model_q40's protocol (every position in the branch's own Q4_0 cache)
         self.fused_sampler = True          # generate(): temperature / top-k / draw as one kernel instead of five torch ops
         self.silu_in_matmul = True         # up to 2 rows: w2's launch makes its own SiLU(gate)*up activations
+        self.swiglu_in_matmul = True       # 33 .. 128 rows, wide FFN: SiLU(gate) * up inside w1|w3's launch (kernels.matmul_q40_swiglu)
         self.tiled_weights = True          # the fused path streams tiled copies of the weights (LinearQ4_0.operand)
         self.attn_single_launch = True     # up to 16 queries per kv head: prefix slices, suffix passes and the merge in one launch
                                            # (above, the one workgroup that merges a kv head's query tiles takes longer than a launch)
@@ -412,6 +413,11 @@ class Transformer(nn.Module):
                     o = att.decode_attention(q, k, v, t_dev, pages, self.attn_single_launch and M * (H // Hkv) <= 16).view(M, H * D)
             po = K.matmul_q40_partial(o, [att.wo.operand(tiled)])
             gu_ops = [ff.w1.operand(tiled), ff.w3.operand(tiled)]
+            if tiled and self.swiglu_in_matmul and K.swiglu_fits(M, p.dim, ff.w1.shape[0]):
+                # 33 .. 128 rows and a wide FFN: SiLU(gate) * up leaves w1|w3's launch as the activations of w2
+                h, xn = K.partial_rmsnorm(po, h, layer.ffn_norm.weight, layer.ffn_norm.eps)
+                pending = K.matmul_q40_partial(K.matmul_q40_swiglu(xn, gu_ops[0], gu_ops[1]), [ff.w2.operand(True)])
+                continue
             if self._norm_in(M, p.dim, gu_ops):
                 h, sums = K.partial_residual_sumsq(po, h)
                 gu = K.matmul_q40_partial_norm(h, sums, layer.ffn_norm.weight, layer.ffn_norm.eps, gu_ops)

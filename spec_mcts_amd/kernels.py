@@ -189,6 +189,28 @@ def matmul_q40_partial(a: torch.Tensor, linears, out: Optional[torch.Tensor] = N
     return PartialProduct(out, ks, M, n_total)
 
 
+def swiglu_fits(M: int, K: int, n_half: int) -> bool:
+    """Is matmul_q40_swiglu the faster way for these dimensions (17 .. 128 rows, a wide gate / up pair)?"""
+    return bool(_lib.load().smh_q40_swiglu_fits(int(M), int(K), int(n_half)))
+
+
+def matmul_q40_swiglu(a: torch.Tensor, gate: "TiledQ40", up: "TiledQ40", out: Optional[torch.Tensor] = None) -> torch.Tensor:
+    """fp16(silu(fp16(a . gate))) * fp16(a . up) in one launch (FeedForward's `F.silu(self.w1(x)) * self.w3(x)`,
+    hf_model_q40_kv_shared.py:434) for tiled weights: what partial_silu_mul(matmul_q40_partial(a, [gate, up])) returns, without
+    the slabs.  17 <= M <= 128, K a multiple of 64, n_half a multiple of 128 up to 16384."""
+    lib = _lib.load()
+    assert a.is_contiguous() and a.dtype == torch.float16 and a.dim() == 2 and a.data_ptr() % 16 == 0
+    _need_gpu(a)
+    M, Kd = a.shape
+    assert isinstance(gate, TiledQ40) and isinstance(up, TiledQ40) and gate.K == Kd and up.K == Kd and gate.N == up.N
+    if out is None:
+        out = torch.empty((M, gate.N), dtype=torch.float16, device=a.device)
+    assert out.shape == (M, gate.N) and out.dtype == torch.float16 and out.is_contiguous()
+    check(lib.smh_q40_matmul_tiled_swiglu(a.data_ptr(), M, Kd, Kd, gate.buf.data_ptr(), up.buf.data_ptr(), gate.N, out.data_ptr(), gate.N,
+                                          _stream()), "smh_q40_matmul_tiled_swiglu")
+    return out
+
+
 SILU_IN_MAX_M = 2
 
 

@@ -43,6 +43,11 @@ def test_argument_errors_are_reported_without_a_gpu():
     assert 1 <= ks <= 16
     assert lib.smh_q40_matmul_plan(1, 4096, 1, (ctypes.c_int * 1)(100)) < 0      # N not a multiple of 128
     assert lib.smh_attn_workspace_bytes(64, 32, 1024) >= 32 * 64 * 32 * 130 * 4
+    # SwiGLU inside the gate|up launch: 17 .. 128 rows, K a multiple of 64, at most 16384 columns per weight
+    assert lib.smh_q40_swiglu_fits(100, 4096, 11008) == 1 and lib.smh_q40_swiglu_fits(16, 4096, 11008) == 0
+    assert lib.smh_q40_swiglu_fits(100, 4096, 28672) == 0 and lib.smh_q40_swiglu_fits(100, 4096, 1024) == 0
+    st = lib.smh_q40_matmul_tiled_swiglu(None, 5, 4096, 4096, None, None, 11008, None, 11008, None)
+    assert st < 0 and b"17 .. 128" in lib.smh_last_error_string()
     # the entry point without a workspace refuses shapes beyond its static array before anything touches the device
     assert lib.smh_attn_static_scratch_bytes() == 16 << 20
     st = lib.smh_shared_prefix_attn_static(None, None, 4096, 64, 64, 128, None, None, 4096, 0, None, None, None, None, 0, None, 0,

@@ -121,6 +121,29 @@ def test_range_cut_products(M, K, ns, slabs):
             col += nn
 
 
+@pytest.mark.parametrize("M", [17, 33, 64, 100, 128])
+@pytest.mark.parametrize("K,n_half", [(4096, 11008), (256, 384), (8192, 1024), (128, 128), (1024, 16384)])
+def test_swiglu_inside_the_gate_up_launch(M, K, n_half):
+    """smh_q40_matmul_tiled_swiglu (hf_model_q40_kv_shared.py:434, `F.silu(self.w1(x)) * self.w3(x)`) against the oracle's two
+    linears, SiLU and product with their fp16 roundings, and against the two launches it replaces (smh_q40_matmul_partial_tiled
+    + smh_partial_silu_mul: the same roundings, another order of the fp32 additions, so single fp16 ulps may differ)"""
+    import torch.nn.functional as F
+    from spec_mcts_amd import kernels as Kn
+    w1, w3 = _weight(K, n_half, 980 + K), _weight(K, n_half, 981 + K)
+    x = (torch.randn((M, K), generator=torch.Generator().manual_seed(982 + M)) * 0.5).half()
+    t1, t3 = Kn.tile_q40(w1[0].cuda(), w1[1].cuda(), K, n_half), Kn.tile_q40(w3[0].cuda(), w3[1].cuda(), K, n_half)
+    got = Kn.matmul_q40_swiglu(x.cuda(), t1, t3)
+    two = Kn.partial_silu_mul(Kn.matmul_q40_partial(x.cuda(), [t1, t3]))
+    torch.cuda.synchronize()
+    g16, u16 = O.matmul_q40(x, w1[0], w1[1], (K, n_half)), O.matmul_q40(x, w3[0], w3[1], (K, n_half))
+    want = F.silu(g16.float()).half() * u16
+    assert got.shape == (M, n_half) and got.dtype == torch.float16
+    assert torch.allclose(got.cpu().float(), want.float(), rtol=1e-2, atol=2e-3)
+    assert torch.allclose(got.float(), two.float(), rtol=4e-3, atol=1e-4)
+    assert float((got != two).float().mean()) < 0.02
+    assert Kn.swiglu_fits(M, K, n_half) == (M > 32 and n_half >= 8192)
+
+
 def test_model_logits_do_not_depend_on_the_weight_layout():
     """the fused forward on tiled copies against the same forward on the checkpoint tensors: equal bit for bit,
     at prefill (GEMM), at decode (GEMV) and again after a weight has been replaced"""
