@@ -40,9 +40,9 @@ ARCHS = {
 # HBM bytes per q40_gemv_kernel launch at M=1: rocprofv3 FETCH_SIZE + WRITE_SIZE, each scaled by a 1 GiB copy
 # (profiles/q40_gemv_m1_hbm_traffic.md has the commands and the factors: 2.0 for reads, 1.0 for writes)
 GEMV_TRAFFIC_BYTES_PER_LAUNCH = 27457381
-# the same for q40_gemm_kernel at M=100 (profiles/q40_gemm_m100_hbm_traffic.md): 37.34 MB read + 24.78 MB written
-# (the fp32 partial sums of the K-slices are the writes)
-GEMM_TRAFFIC_BYTES_PER_LAUNCH = 62123956
+# the same for the GEMM kernels at M=100 (profiles/q40_gemm_m100_hbm_traffic.md): 39.68 MB read + 8.47 MB written
+# (the fp32 partial sums of the K-slices and the activations of w2 are the writes)
+GEMM_TRAFFIC_BYTES_PER_LAUNCH = 48156518
 # the same for one call of the decode attention leg (profiles/attn_decode_hbm_traffic.md): 65.6 MB read + 9.0 MB written
 ATTN_TRAFFIC_BYTES_PER_CALL = 74610046
 
@@ -107,7 +107,8 @@ def step_matmuls(model):
 
 
 def matmul_roofline(torch, model, M, iters):
-    """Only the Q4_0 matmul kernel (q40_gemv_kernel for M <= 16, q40_gemm_kernel above), launched once per
+    """Only the Q4_0 matmul kernels (q40_gemv_kernel for M <= 16; above, the kernels the model launches at that batch:
+    q40_gemm_kg_kernel, q40_gemm_swiglu_kernel for w1|w3 where it applies, q40_gemm_kernel otherwise), launched once per
     weight launch of a decode step at batch M, back to back in one HIP graph; timed with HIP events on the
     stream the graph runs on.  Every launch reads different weights (3.4 GB per pass, the Infinity Cache
     holds 256 MB)."""
@@ -118,7 +119,10 @@ def matmul_roofline(torch, model, M, iters):
 
     def run():
         for k_in, segs in launches:
-            K.matmul_q40_partial(xs[k_in], [op for op, _ in segs])
+            if len(segs) == 2 and model.swiglu_in_matmul and K.swiglu_fits(M, k_in, segs[0][1]):
+                K.matmul_q40_swiglu(xs[k_in], segs[0][0], segs[1][0])       # w1|w3 as the model launches it at this batch
+            else:
+                K.matmul_q40_partial(xs[k_in], [op for op, _ in segs])
 
     run()
     torch.cuda.synchronize()
@@ -527,7 +531,7 @@ def main():
         result["rooflines_other"] = [
             {"kernel": "q40_gemv_kernel at M=10", "bound": "hbm", "achieved": round(rf10["gbs"], 1), "peak": HBM_PEAK_GBS,
              "unit": "GB/s", "frac": round(rf10["gbs"] / HBM_PEAK_GBS, 4), "avg_launch_us": round(rf10["avg_us"], 3)},
-            {"kernel": "q40_gemm_kernel at M=100", "bound": "mfma", "achieved": round(rf100["tflops"], 1),
+            {"kernel": "Q4_0 GEMM at M=100: q40_gemm_kg_kernel (wq|wk|wv, wo, w2) and q40_gemm_swiglu_kernel (w1|w3), the 128 weight launches of a step", "bound": "mfma", "achieved": round(rf100["tflops"], 1),
              "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s", "frac": round(rf100["tflops"] / MFMA_F16_PEAK_TFLOPS, 4),
              "hbm_gbs": round(rf100["gbs"], 1), "avg_launch_us": round(rf100["avg_us"], 3), "traffic": GEMM_TRAFFIC_BYTES_PER_LAUNCH if a.arch == "7b" else None},
         ]
