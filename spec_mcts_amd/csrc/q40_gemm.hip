@@ -586,7 +586,7 @@ __global__ __launch_bounds__(64 * (WAVES + (PRODUCER ? 1 : 0)), WAVES == 8 ? 1 :
 // multiplies the columns of nibble hh of piece 2 blk + bp of its group's steps with all row tiles of A - the same two B
 // operands and 14 MFMAs per step as in q40_gemm_kernel - so a ring stage holds TWO steps: both pieces of the block and the
 // scales of either step, and either step's rows of A.  The groups' accumulators are added through LDS at the end (group 0
-// + group 1, a fixed order), and the first four waves write the slab.  Against q40_gemm_kernel's 256-column units this
+// + group 1, a fixed order), and all eight waves write the slab.  Against q40_gemm_kernel's 256-column units this
 // fills the GPU with half as many K-slices, i.e. half the slab bytes written here and read back by the consumer; the
 // price is that a row of A is staged for 128 columns instead of 256.
 constexpr int KG_W = 4096;                     // [group kk][piece bp] x 1024
@@ -594,12 +594,11 @@ constexpr int KG_S = 512;                      // [group kk] x 256 (the whole sc
 template <int TILES> struct KgShape {
     static constexpr int STAGE = KG_W + KG_S + 2 * TILES * 1024;
     static constexpr int SLOTS = GEMM_DMA_WAVE_SLOTS;
-    static constexpr int LDS = SLOTS * STAGE;
+    static constexpr int RING = SLOTS * STAGE;
     static constexpr int PER = 2 * (3 + TILES);                    // DMA instructions of a stage
-    static constexpr int RED = 4 * TILES * 2 * 1024;               // the second group's accumulators: [wave][t][o][lane] x 16 B
-    static constexpr int OP = 128 + 4;
-    static constexpr int OTILE = 16 * OP * 4;
-    static_assert(RED + 2 * OTILE <= LDS, "the sums of the second group and two output tiles must fit in the ring");
+    static constexpr int OP = 128 + 4;                             // floats per row of a group's sums in LDS
+    static constexpr int SUMS = TILES * 16 * OP * 4;               // one K-group's sums: [row][OP] fp32
+    static constexpr int LDS = RING > 2 * SUMS ? RING : 2 * SUMS;
     static_assert(PER * (SLOTS - 5) <= 63 && LDS <= 160 * 1024, "ring");
 };
 
@@ -684,9 +683,8 @@ __global__ __launch_bounds__(576, 1) void q40_gemm_kg_kernel(MatmulParams p) {
                 slot = slot + 2 >= SLOTS ? slot + 2 - SLOTS : slot + 2;
             }
         }
-        // the barriers of the epilogue: ring free, second group's sums in place, one per row tile
-#pragma unroll 1
-        for (int t = 0; t < 2 + TILES; ++t) gemm_barrier();
+        gemm_barrier();                                        // the epilogue's two barriers: ring free, sums in place
+        gemm_barrier();
         return;
     }
 
@@ -763,46 +761,29 @@ __global__ __launch_bounds__(576, 1) void q40_gemm_kg_kernel(MatmulParams p) {
         }
     }
 
-    // ---- group 0 + group 1 through LDS, then the slab one row tile at a time ----
+    // ---- both groups' sums as rows of 128 floats in LDS; then every thread adds group 0 + group 1 (a fixed order) for
+    // 16-byte runs of whole rows and writes the slab: one pass, two barriers, all eight waves storing ----
     gemm_barrier();                                            // every wave has left the loop: the ring is free
-    if (kk == 1) {
-        uint8_t *dst = lds + (wave8 - 4) * (TILES * 2 * 1024) + lane * 16;
+    constexpr int OP = S::OP;
+    {
+        float *sums = reinterpret_cast<float *>(lds + kk * S::SUMS);
 #pragma unroll
         for (int t = 0; t < TILES; ++t)
 #pragma unroll
-            for (int o = 0; o < 2; ++o) *reinterpret_cast<f4 *>(dst + (t * 2 + o) * 1024) = acc[o][t];
+            for (int r = 0; r < 4; ++r)
+                *reinterpret_cast<f2 *>(&sums[(16 * t + 4 * g + r) * OP + 64 * hh + 4 * c + 2 * bp]) = f2{acc[0][t][r], acc[1][t][r]};
     }
     gemm_barrier();
-    if (kk == 1) {
-#pragma unroll 1
-        for (int t = 0; t < TILES; ++t) gemm_barrier();
-        return;
-    }
-    {
-        const uint8_t *src = lds + wave8 * (TILES * 2 * 1024) + lane * 16;
+    const float *sum0 = reinterpret_cast<const float *>(lds), *sum1 = reinterpret_cast<const float *>(lds + S::SUMS);
+    float *slab = p.partial + (long)slice * p.M * p.n_total + seg.col0 + col0;
 #pragma unroll
-        for (int t = 0; t < TILES; ++t)
-#pragma unroll
-            for (int o = 0; o < 2; ++o) acc[o][t] += *reinterpret_cast<const f4 *>(src + (t * 2 + o) * 1024);
-    }
-    constexpr int OP = S::OP;
-    float *slab = p.partial + (long)slice * p.M * p.n_total;
-    const int o_row = tid >> 4, o_lane = tid & 15;            // tid < 256 here
-#pragma unroll
-    for (int t = 0; t < TILES; ++t) {
-        float *otile = reinterpret_cast<float *>(lds + S::RED + (t & 1) * S::OTILE);
-#pragma unroll
-        for (int r = 0; r < 4; ++r)
-            *reinterpret_cast<f2 *>(&otile[(4 * g + r) * OP + 64 * hh + 4 * c + 2 * bp]) = f2{acc[0][t][r], acc[1][t][r]};
-        gemm_barrier();
-        const int m = m0 + 16 * t + o_row;
-        if (m < p.M && m < m0 + p.block_rows) {
-            float *dst = slab + (long)m * p.n_total + seg.col0 + col0;
-#pragma unroll
-            for (int q = 0; q < 2; ++q) {
-                const int cq = 64 * q + 4 * o_lane;
-                *reinterpret_cast<f4 *>(dst + cq) = *reinterpret_cast<const f4 *>(otile + o_row * OP + cq);
-            }
+    for (int it = 0; it < TILES; ++it) {
+        const int idx = tid + 512 * it;                        // tid < 512 here: (row, run of four columns)
+        const int row = idx >> 5, cq = 4 * (idx & 31);
+        const int m = m0 + row;
+        if (m < p.M && row < p.block_rows) {
+            const f4 v = *reinterpret_cast<const f4 *>(sum0 + row * OP + cq) + *reinterpret_cast<const f4 *>(sum1 + row * OP + cq);
+            *reinterpret_cast<f4 *>(slab + (long)m * p.n_total + cq) = v;
         }
     }
 }
