@@ -52,7 +52,7 @@ def test_tiles_match_the_layout_definition(K, N):
     assert np.array_equal(got, want)
 
 
-@pytest.mark.parametrize("M", [1, 3, 10, 16, 17, 100, 130])
+@pytest.mark.parametrize("M", [1, 3, 10, 16, 17, 65, 100, 128, 130])
 @pytest.mark.parametrize("K,ns", [(64, [128]), (40, [384]), (4096, [4096]), (1000, [256, 128, 128]), (4096, [1024, 256, 256]),
                                   (11008, [4096]), (4096, [11008, 11008]),
                                   # 1, 3, 5 and 7 steps of 32 rows: the ends of a loop that takes its steps in pairs
