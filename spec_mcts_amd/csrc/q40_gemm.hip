@@ -294,6 +294,8 @@ __device__ __forceinline__ void gemm_piece(const MatmulParams &p, int unit, int 
     // exact fp16 code * scale, as the four B operands (byte 2bp high / low, byte 2bp+1 high / low)
     // eight waves: the nibble this wave decodes, as constants of one and-or + one packed fma (code = fp16 bits * mul + off)
     const uint32_t nib_mask = hh == 0 ? 0x00F000F0u : 0x000F000Fu;
+    uint32_t nib_magic = MAGIC_1024;                             // in a register the compiler cannot see through: (bits & mask) | magic is
+    asm volatile("" : "+v"(nib_magic));                       // then ONE v_and_or_b32 (no literal operands there), not an AND and an OR
     const h2 nib_mul = hh == 0 ? h2{(half_t)0.0625f, (half_t)0.0625f} : h2{(half_t)1.0f, (half_t)1.0f};
     const h2 nib_off = hh == 0 ? h2{(half_t)-72.0f, (half_t)-72.0f} : h2{(half_t)-1032.0f, (half_t)-1032.0f};
     auto decode = [&](const uint32_t (&wv)[8], const uint32_t (&sv)[8], bool dead, h8 (&b)[NB]) {
@@ -304,8 +306,8 @@ __device__ __forceinline__ void gemm_piece(const MatmulParams &p, int unit, int 
                 const uint32_t pr0 = j < 2 ? wv[j] : wv[j - 2] >> 8;           // rows (2j, 2j+1) of byte 2bp, codes + 8
                 const uint32_t pr1 = j < 2 ? wv[2 + j] : wv[j] >> 8;           // ... of byte 2bp+1
                 const h2 sc = as_h2(sv[j]);
-                v0h[j] = as_u32(__builtin_elementwise_fma(as_h2((pr0 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
-                v1h[j] = as_u32(__builtin_elementwise_fma(as_h2((pr1 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
+                v0h[j] = as_u32(__builtin_elementwise_fma(as_h2((pr0 & nib_mask) | nib_magic), nib_mul, nib_off) * sc);
+                v1h[j] = as_u32(__builtin_elementwise_fma(as_h2((pr1 & nib_mask) | nib_magic), nib_mul, nib_off) * sc);
             }
             b[0] = __builtin_bit_cast(h8, v0h);
             b[1] = __builtin_bit_cast(h8, v1h);
@@ -690,6 +692,8 @@ __global__ __launch_bounds__(576, 1) void q40_gemm_kg_kernel(MatmulParams p) {
 
     const int kk = wave8 >> 2, hh = (wave8 >> 1) & 1, bp = wave8 & 1;
     const uint32_t nib_mask = hh == 0 ? 0x00F000F0u : 0x000F000Fu;
+    uint32_t nib_magic = MAGIC_1024;                             // in a register the compiler cannot see through: (bits & mask) | magic is
+    asm volatile("" : "+v"(nib_magic));                       // then ONE v_and_or_b32 (no literal operands there), not an AND and an OR
     const h2 nib_mul = hh == 0 ? h2{(half_t)0.0625f, (half_t)0.0625f} : h2{(half_t)1.0f, (half_t)1.0f};
     const h2 nib_off = hh == 0 ? h2{(half_t)-72.0f, (half_t)-72.0f} : h2{(half_t)-1032.0f, (half_t)-1032.0f};
     struct Raw { u32x4 wq, sc; };
@@ -704,8 +708,8 @@ __global__ __launch_bounds__(576, 1) void q40_gemm_kg_kernel(MatmulParams p) {
             const uint32_t pr0 = j < 2 ? r.wq[j] : r.wq[j - 2] >> 8;       // rows (2j, 2j+1) of byte 2bp, codes + 8
             const uint32_t pr1 = j < 2 ? r.wq[2 + j] : r.wq[j] >> 8;       // ... of byte 2bp+1
             const h2 sc = as_h2(r.sc[j]);
-            v0[j] = as_u32(__builtin_elementwise_fma(as_h2((pr0 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
-            v1[j] = as_u32(__builtin_elementwise_fma(as_h2((pr1 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
+            v0[j] = as_u32(__builtin_elementwise_fma(as_h2((pr0 & nib_mask) | nib_magic), nib_mul, nib_off) * sc);
+            v1[j] = as_u32(__builtin_elementwise_fma(as_h2((pr1 & nib_mask) | nib_magic), nib_mul, nib_off) * sc);
         }
         b[0] = __builtin_bit_cast(h8, v0);
         b[1] = __builtin_bit_cast(h8, v1);
@@ -889,6 +893,8 @@ __global__ __launch_bounds__(576, 1) void q40_gemm_swiglu_kernel(MatmulParams p)
 
     const int kk = wave8 >> 2, hh = (wave8 >> 1) & 1, gu = wave8 & 1;       // K-group, nibble, gate (0) or up (1)
     const uint32_t nib_mask = hh == 0 ? 0x00F000F0u : 0x000F000Fu;
+    uint32_t nib_magic = MAGIC_1024;                             // in a register the compiler cannot see through: (bits & mask) | magic is
+    asm volatile("" : "+v"(nib_magic));                       // then ONE v_and_or_b32 (no literal operands there), not an AND and an OR
     const h2 nib_mul = hh == 0 ? h2{(half_t)0.0625f, (half_t)0.0625f} : h2{(half_t)1.0f, (half_t)1.0f};
     const h2 nib_off = hh == 0 ? h2{(half_t)-72.0f, (half_t)-72.0f} : h2{(half_t)-1032.0f, (half_t)-1032.0f};
     struct Raw { u32x4 wq, sc; };
@@ -903,8 +909,8 @@ __global__ __launch_bounds__(576, 1) void q40_gemm_swiglu_kernel(MatmulParams p)
             const uint32_t pr0 = j < 2 ? r.wq[j] : r.wq[j - 2] >> 8;       // rows (2j, 2j+1) of byte 2bp, codes + 8
             const uint32_t pr1 = j < 2 ? r.wq[2 + j] : r.wq[j] >> 8;       // ... of byte 2bp+1
             const h2 sc = as_h2(r.sc[j]);
-            v0[j] = as_u32(__builtin_elementwise_fma(as_h2((pr0 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
-            v1[j] = as_u32(__builtin_elementwise_fma(as_h2((pr1 & nib_mask) | MAGIC_1024), nib_mul, nib_off) * sc);
+            v0[j] = as_u32(__builtin_elementwise_fma(as_h2((pr0 & nib_mask) | nib_magic), nib_mul, nib_off) * sc);
+            v1[j] = as_u32(__builtin_elementwise_fma(as_h2((pr1 & nib_mask) | nib_magic), nib_mul, nib_off) * sc);
         }
         b[0] = __builtin_bit_cast(h8, v0);
         b[1] = __builtin_bit_cast(h8, v1);
